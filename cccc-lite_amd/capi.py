@@ -1,0 +1,115 @@
+"""ctypes binding of include/cccc_hip_quant.h (the drop-in C-ABI)."""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+
+
+class DataType:
+    """cccc::DataType values (reference cccc/types.h:24-34)."""
+    FLOAT = 0
+    DOUBLE = 1
+    HALF = 2
+    BFLOAT16 = 3
+    FP8_E4M3 = 4
+    FP8_E5M2 = 5
+    FP4_E2M1 = 6
+
+
+NO_TRANS, TRANS = 0, 1
+
+EXPORTS = (
+    "hip_convert",
+    "hip_fp4_blockscale_to_bf16",
+    "hip_float_to_fp4_blockscale",
+    "hip_quant_gemm",
+    "hip_quant_set_sync",
+    "hip_quant_set_stream",
+    "hip_quant_last_kernel",
+)
+
+
+def library_path() -> Path:
+    return HERE / "libcccc_hip_quant.so"
+
+
+class QuantLibrary:
+    """The loaded shared library with typed entry points.  Pointers are plain integers (device
+    addresses, e.g. torch.Tensor.data_ptr())."""
+
+    def __init__(self, path: Path | None = None):
+        path = Path(path) if path else library_path()
+        if not path.exists():
+            raise FileNotFoundError(
+                f"{path} is missing: build it with `make -C {HERE}` (or __graft_entry__.build()); "
+                "there is no CPU or PyTorch fallback for this path")
+        self.path = path
+        L = ctypes.CDLL(str(path))
+        vp, i32, u32, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint, ctypes.c_float
+        L.hip_convert.restype = i32
+        L.hip_convert.argtypes = [vp, i32, vp, i32, u32, f32]
+        L.hip_fp4_blockscale_to_bf16.restype = i32
+        L.hip_fp4_blockscale_to_bf16.argtypes = [vp, vp, vp, u32, u32]
+        L.hip_float_to_fp4_blockscale.restype = i32
+        L.hip_float_to_fp4_blockscale.argtypes = [vp, vp, vp, u32, u32]
+        L.hip_quant_gemm.restype = i32
+        L.hip_quant_gemm.argtypes = [i32, i32, i32, i32, i32, f32,
+                                     vp, i32, i32, f32,
+                                     vp, i32, i32, f32,
+                                     f32, vp, i32, i32, f32,
+                                     vp, vp, u32]
+        L.hip_quant_set_sync.restype = i32
+        L.hip_quant_set_sync.argtypes = [i32]
+        L.hip_quant_set_stream.restype = i32
+        L.hip_quant_set_stream.argtypes = [vp]
+        L.hip_quant_last_kernel.restype = ctypes.c_char_p
+        L.hip_quant_last_kernel.argtypes = []
+        self.c = L
+
+    # -- thin, argument-for-argument wrappers ------------------------------------------------
+    def convert(self, src, src_type, dst, dst_type, n, scale=1.0) -> int:
+        return self.c.hip_convert(src, src_type, dst, dst_type, n, scale)
+
+    def fp4_blockscale_to_bf16(self, nibbles, scales, dst, n_elems, block_size=16) -> int:
+        return self.c.hip_fp4_blockscale_to_bf16(nibbles, scales, dst, n_elems, block_size)
+
+    def float_to_fp4_blockscale(self, src, nibbles, scales, n_elems, block_size=16) -> int:
+        return self.c.hip_float_to_fp4_blockscale(src, nibbles, scales, n_elems, block_size)
+
+    def quant_gemm(self, transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
+                   B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale=0.0,
+                   blk_scA=None, blk_scB=None, block_size=16) -> int:
+        return self.c.hip_quant_gemm(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
+                                     B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale,
+                                     blk_scA, blk_scB, block_size)
+
+    def set_sync(self, enabled: bool) -> int:
+        return self.c.hip_quant_set_sync(1 if enabled else 0)
+
+    def set_stream(self, stream_handle: int | None) -> int:
+        return self.c.hip_quant_set_stream(stream_handle)
+
+    def last_kernel(self) -> str:
+        return (self.c.hip_quant_last_kernel() or b"").decode()
+
+    # -- the call the LLM graph makes --------------------------------------------------------
+    def linear(self, W, w_type, X, Y, n_out, tokens, K, inv_scale=1.0, blk_sc=None, block_size=16,
+               alpha=1.0, beta=0.0) -> int:
+        """y[t][o] = sum_k W[o][k] x[t][k], argument layout of Matrix::mulBatched(W, X, Y, TRANS,
+        NO_TRANS) for a linear layer (reference cccc/Matrix.cpp:1162-1203): BLAS M = n_out,
+        BLAS N = tokens, lda = ldb = K, ldc = n_out."""
+        return self.quant_gemm(TRANS, NO_TRANS, n_out, tokens, K, alpha, W, w_type, K, inv_scale,
+                               X, DataType.BFLOAT16, K, 1.0, beta, Y, DataType.BFLOAT16, n_out, 0.0,
+                               blk_sc, None, block_size)
+
+
+_library = None
+
+
+def library() -> QuantLibrary:
+    global _library
+    if _library is None:
+        _library = QuantLibrary()
+    return _library

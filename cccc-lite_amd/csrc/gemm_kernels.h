@@ -1,0 +1,275 @@
+// Prefill GEMM for gfx950 (tokens > 16): weight tiles are dequantised to BF16 on their way into
+// LDS and both operands feed v_mfma_f32_32x32x16_bf16 with FP32 accumulation; one rounding to
+// BF16 in the epilogue.  Same numerics as the reference's dequantise-then-BF16-GEMM
+// (cccc/cublas_real.h:943-964): the weight value entering a product is bf16(decode(w) * scale).
+//
+// Tiling: a 256-thread workgroup (4 waves, 2 x 2) owns BM output features x BN tokens and walks K
+// in steps of 64.  LDS holds one X tile [BN][64] and one dequantised W tile [BM][64], rows of 128
+// bytes whose 16-byte chunks are XOR-swizzled with (row / 2) % 8 so that the 128-bit fragment
+// reads of 16 consecutive rows hit 16 distinct bank groups.  The next k-tile is fetched from
+// global memory into registers while the current one is multiplied.
+//   A operand (rows)    = tokens,          lane (r = lane % 32, h = lane / 32) holds k = 8 h .. 8 h + 7
+//   B operand (columns) = output features, same k split
+//   D: lane holds column lane % 32; register v is row 8 (v / 4) + 4 (lane / 32) + v % 4
+#pragma once
+#include "linear_args.h"
+#include "quant_device.h"
+#include "runtime.h"
+
+namespace ccq
+{
+
+__device__ __forceinline__ int swizzled_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+// 16 FP8 codes -> 16 BF16 (two 16-byte LDS chunks)
+template <int WT, bool SCALED>
+__device__ __forceinline__ void dequant16_fp8(const u32x4& w, float scale, u32x4& lo, u32x4& hi)
+{
+    uint32_t out[8];
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        bf16x2 p, q;
+        if (!SCALED)
+        {
+            if (WT == DT_E5M2)
+            {
+                p = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w[d], 1.0f, false);
+                q = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w[d], 1.0f, true);
+            }
+            else
+            {
+                p = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[d], 1.0f, false);
+                q = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[d], 1.0f, true);
+            }
+        }
+        else
+        {
+            f32x2 a, b;
+            if (WT == DT_E5M2)
+            {
+                a = __builtin_amdgcn_cvt_pk_f32_bf8(w[d], false);
+                b = __builtin_amdgcn_cvt_pk_f32_bf8(w[d], true);
+            }
+            else
+            {
+                a = __builtin_amdgcn_cvt_pk_f32_fp8(w[d], false);
+                b = __builtin_amdgcn_cvt_pk_f32_fp8(w[d], true);
+            }
+            p = bf16x2{ (__bf16)(a.x * scale), (__bf16)(a.y * scale) };
+            q = bf16x2{ (__bf16)(b.x * scale), (__bf16)(b.y * scale) };
+        }
+        out[2 * d] = __builtin_bit_cast(uint32_t, p);
+        out[2 * d + 1] = __builtin_bit_cast(uint32_t, q);
+    }
+    lo = u32x4{ out[0], out[1], out[2], out[3] };
+    hi = u32x4{ out[4], out[5], out[6], out[7] };
+}
+
+// 8 FP4 codes (one dword) times a block scale -> 8 BF16 (one 16-byte LDS chunk)
+__device__ __forceinline__ u32x4 dequant8_fp4(uint32_t w, float scale)
+{
+    uint32_t out[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+    {
+        f32x2 v;
+        switch (b)
+        {
+        case 0: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); break;
+        case 1: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); break;
+        case 2: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); break;
+        default: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); break;
+        }
+        const bf16x2 p = { (__bf16)(v.x * scale), (__bf16)(v.y * scale) };
+        out[b] = __builtin_bit_cast(uint32_t, p);
+    }
+    return u32x4{ out[0], out[1], out[2], out[3] };
+}
+
+// WT: DT_E5M2 / DT_E4M3 / DT_FP4.  BLOCK: FP4 block length (16 / 32), unused for FP8.
+// Requires K % 16 == 0 (FP8) or K % 32 == 0 (FP4), and the alignment rules of the GEMV kernels.
+template <int WT, int BLOCK, int BM, int BN, bool SCALED>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
+{
+    constexpr int BK = 64;
+    constexpr int WM = BM / 2;          // output features per wave
+    constexpr int WN = BN / 2;          // tokens per wave
+    constexpr int TM = WM / 32;         // MFMA tiles along output features
+    constexpr int TN = WN / 32;         // MFMA tiles along tokens
+    constexpr bool FP4 = WT == DT_FP4;
+    constexpr int W_CHUNK_K = FP4 ? 32 : 16;                // elements per 16-byte global chunk
+    constexpr int W_CHUNKS = BM * (BK / W_CHUNK_K);         // per k-tile
+    constexpr int W_PER_THREAD = (W_CHUNKS + 255) / 256;
+    constexpr int X_PER_THREAD = BN * 8 / 256;
+
+    __shared__ u32x4 xs[BN * 8];
+    __shared__ u32x4 ws[BM * 8];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave & 1;
+    const int wave_n = wave >> 1;
+    const int out_base = blockIdx.x * BM;
+    const int tok_base = blockIdx.y * BN;
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { acc[tn][tm][v] = 0.0f; }
+
+    u32x4 wreg[W_PER_THREAD];
+    uint32_t sreg[W_PER_THREAD];
+    u32x4 xreg[X_PER_THREAD];
+
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < W_PER_THREAD; i++)
+        {
+            const int q = tid + i * 256;
+            const int row_in_tile = q / (BK / W_CHUNK_K);
+            const int part = q % (BK / W_CHUNK_K);
+            const int k = k0 + part * W_CHUNK_K;
+            wreg[i] = u32x4{ 0u, 0u, 0u, 0u };
+            sreg[i] = 0u;
+            if (q < W_CHUNKS && k < a.K)
+            {
+                const long long row = min(out_base + row_in_tile, a.n_out - 1);
+                const long long flat = row * a.ldw + k;
+                wreg[i] = *(const u32x4*)(a.W + (FP4 ? (flat >> 1) : flat));
+                if (FP4)
+                {
+                    if (BLOCK == 16) { sreg[i] = *(const uint16_t*)(a.blk_sc + flat / 16); }
+                    else { sreg[i] = a.blk_sc[flat / 32]; }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++)
+        {
+            const int q = tid + i * 256;
+            const int row_in_tile = q >> 3;
+            const int chunk = q & 7;
+            const int k = k0 + chunk * 8;
+            xreg[i] = u32x4{ 0u, 0u, 0u, 0u };
+            if (k < a.K)
+            {
+                const long long tok = min(tok_base + row_in_tile, a.tokens - 1);
+                xreg[i] = *(const u32x4*)(a.X + tok * a.ldx + k);
+            }
+        }
+    };
+
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < W_PER_THREAD; i++)
+        {
+            const int q = tid + i * 256;
+            if (q < W_CHUNKS)
+            {
+                const int row = q / (BK / W_CHUNK_K);
+                const int part = q % (BK / W_CHUNK_K);
+                if (FP4)
+                {
+                    const float s0 = __builtin_amdgcn_cvt_f32_fp8(sreg[i], 0);
+                    const float s1 = BLOCK == 16 ? __builtin_amdgcn_cvt_f32_fp8(sreg[i], 1) : s0;
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                    {
+                        ws[row * 8 + swizzled_chunk(row, part * 4 + d)] = dequant8_fp4(wreg[i][d], d < 2 ? s0 : s1);
+                    }
+                }
+                else
+                {
+                    u32x4 lo, hi;
+                    dequant16_fp8<WT, SCALED>(wreg[i], a.w_scale, lo, hi);
+                    ws[row * 8 + swizzled_chunk(row, part * 2)] = lo;
+                    ws[row * 8 + swizzled_chunk(row, part * 2 + 1)] = hi;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++)
+        {
+            const int q = tid + i * 256;
+            const int row = q >> 3;
+            xs[row * 8 + swizzled_chunk(row, q & 7)] = xreg[i];
+        }
+    };
+
+    const int r32 = lane & 31;
+    const int h = lane >> 5;
+
+    fetch(0);
+    for (int k0 = 0; k0 < a.K; k0 += BK)
+    {
+        stage();
+        __syncthreads();
+        if (k0 + BK < a.K) { fetch(k0 + BK); }
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++)
+        {
+            bf16x8 xf[TN], wf[TM];
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+            {
+                const int row = wave_n * WN + tn * 32 + r32;
+                xf[tn] = __builtin_bit_cast(bf16x8, xs[row * 8 + swizzled_chunk(row, ks * 2 + h)]);
+            }
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+            {
+                const int row = wave_m * WM + tm * 32 + r32;
+                wf[tm] = __builtin_bit_cast(bf16x8, ws[row * 8 + swizzled_chunk(row, ks * 2 + h)]);
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) { acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tn], wf[tm], acc[tn][tm], 0, 0, 0); }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+    {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+        {
+            const int out = out_base + wave_m * WM + tm * 32 + r32;
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+            {
+                const int tok = tok_base + wave_n * WN + tn * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (out < a.n_out && tok < a.tokens)
+                {
+                    uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                    *y = finish_output(acc[tn][tm][v], a.alpha, a.beta, y);
+                }
+            }
+        }
+    }
+}
+
+template <int WT, int BLOCK, int BM, int BN>
+void launch_gemm_mfma(const LinearArgs& a)
+{
+    const dim3 grid((a.n_out + BM - 1) / BM, (a.tokens + BN - 1) / BN);
+    if (WT != DT_FP4 && a.w_scale != 1.0f) { gemm_mfma_kernel<WT, BLOCK, BM, BN, true><<<grid, 256, 0, stream()>>>(a); }
+    else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false><<<grid, 256, 0, stream()>>>(a); }
+}
+
+template <int WT, int BLOCK>
+bool gemm_mfma(const LinearArgs& a)
+{
+    const long long tiles_big = (long long)((a.n_out + 127) / 128) * ((a.tokens + 127) / 128);
+    if (tiles_big >= 2LL * cu_count()) { launch_gemm_mfma<WT, BLOCK, 128, 128>(a); }
+    else { launch_gemm_mfma<WT, BLOCK, 128, 64>(a); }
+    return true;
+}
+
+}    // namespace ccq

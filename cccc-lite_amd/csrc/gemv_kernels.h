@@ -1,0 +1,484 @@
+// Decode-time GEMV family for gfx950 (tokens 1..16): streams the packed weight once with 128-bit
+// loads, converts FP8 / FP4 to BF16 in registers with the CDNA4 conversion instructions, multiplies
+// against BF16 activations with FP32 accumulation and rounds once to BF16.
+//
+// Numerics are those of the reference's "dequantise to BF16, then BF16 GEMM with FP32 accumulate"
+// (cccc/cublas_real.h:943-964): the weight value entering each product is bf16(decode(w) * scale).
+//   * scale == 1: every E5M2 / E4M3 / E2M1 value is exactly representable in BF16, so the hardware
+//     conversion is that value.
+//   * scale != 1: decode to FP32, one FP32 multiply, round to nearest even to BF16 (SCALED = true).
+//   * FP4 block scales: fp4 * e4m3 has at most 6 significant bits, so bf16(fp4 * s) == fp4 * s and
+//     sum_k (fp4_k * s_b) * x_k == sum_b s_b * sum_{k in b} fp4_k * x_k; the kernel factors the
+//     scale out of each block.
+#pragma once
+#include "linear_args.h"
+#include "quant_device.h"
+
+namespace ccq
+{
+
+// ------------------------------------------------------------------------------------------
+// register-level conversions
+
+// four FP8 codes in one dword -> two packed BF16 pairs (elements 0,1 and 2,3)
+template <int WT, bool SCALED>
+__device__ __forceinline__ void fp8x4_to_bf16(uint32_t w, float scale, bf16x2& p01, bf16x2& p23)
+{
+    if (!SCALED)
+    {
+        if (WT == DT_E5M2)
+        {
+            p01 = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, false);
+            p23 = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, true);
+        }
+        else
+        {
+            p01 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+            p23 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+        }
+    }
+    else
+    {
+        f32x2 a, b;
+        if (WT == DT_E5M2)
+        {
+            a = __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+            b = __builtin_amdgcn_cvt_pk_f32_bf8(w, true);
+        }
+        else
+        {
+            a = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+            b = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+        }
+        p01 = bf16x2{ (__bf16)(a.x * scale), (__bf16)(a.y * scale) };
+        p23 = bf16x2{ (__bf16)(b.x * scale), (__bf16)(b.y * scale) };
+    }
+}
+
+__device__ __forceinline__ float dot2_bf16(bf16x2 a, uint32_t x, float acc)
+{
+    return __builtin_amdgcn_fdot2_f32_bf16(a, __builtin_bit_cast(bf16x2, x), acc, false);
+}
+
+// ------------------------------------------------------------------------------------------
+// Activations in LDS.  A "k-step" is the span one wave covers with one 128-bit load per lane:
+// KSTEP elements.  Each lane needs KSTEP/64 consecutive BF16 of every token per step; they are
+// stored as PARTS 16-byte pieces, piece p of lane l at [step][token][p][l], so that every
+// ds_read_b128 of a wave hits 64 consecutive 16-byte slots (no bank conflicts).
+//   FP8: KSTEP = 1024, PARTS = 2.   FP4: KSTEP = 2048, PARTS = 4.
+
+template <int MT, int PARTS>
+__device__ __forceinline__ void stage_activations(const LinearArgs& a, u32x4* xs, int n_steps, int threads)
+{
+    constexpr int KSTEP = 64 * 8 * PARTS;
+    const int chunks_per_token = n_steps * 64 * PARTS;    // 16-byte chunks, zero padded beyond K
+    for (int c = threadIdx.x; c < chunks_per_token * MT; c += threads)
+    {
+        const int t = c / chunks_per_token;
+        const int r = c - t * chunks_per_token;    // chunk index along k
+        const int k = r * 8;
+        u32x4 v = { 0u, 0u, 0u, 0u };
+        if (k < a.K) { v = *(const u32x4*)(a.X + (long long)t * a.ldx + k); }
+        const int step = k / KSTEP;
+        const int in_step = r - step * (64 * PARTS);
+        const int lane = in_step / PARTS;
+        const int part = in_step - lane * PARTS;
+        xs[((step * MT + t) * PARTS + part) * 64 + lane] = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// FP8 GEMV, dot2 + DPP reduction.  One wave owns R consecutive output rows; lanes stride along K.
+//   WT      DT_E5M2 / DT_E4M3
+//   MT      tokens handled (1..4), compile time so the accumulators stay in registers
+//   R       rows per wave
+//   U       k-steps in flight per loop trip (loads issued before any is consumed)
+//   WAVES   waves per workgroup
+// Requires: K % 16 == 0, ldw % 16 == 0, W 16-byte aligned, ldx % 8 == 0, X 16-byte aligned.
+// Dynamic LDS: MT * ceil(K / 1024) * 2048 bytes.
+
+template <int WT, int MT, int R, int U, int WAVES, bool SCALED>
+__global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs a)
+{
+    extern __shared__ u32x4 xs[];
+    const int n_steps = (a.K + 1023) / 1024;
+    stage_activations<MT, 2>(a, xs, n_steps, WAVES * 64);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_groups = (a.n_out + R - 1) / R;
+    const int last_row = a.n_out - 1;
+
+    for (int g = blockIdx.x * WAVES + wave; g < n_groups; g += gridDim.x * WAVES)
+    {
+        const uint8_t* wrow[R];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+        {
+            const int row = min(g * R + r, last_row);    // clamped rows are computed and dropped
+            wrow[r] = a.W + (long long)row * a.ldw + lane * 16;
+        }
+        float acc[R][MT];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) { acc[r][t] = 0.0f; }
+
+        for (int s0 = 0; s0 < n_steps; s0 += U)
+        {
+            u32x4 w[U][R];
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                const int k = (s0 + u) * 1024 + lane * 16;
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                {
+                    w[u][r] = u32x4{ 0u, 0u, 0u, 0u };
+                    if (k < a.K) { w[u][r] = __builtin_nontemporal_load((const u32x4*)(wrow[r] + (s0 + u) * 1024)); }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                if (s0 + u < n_steps)
+                {
+                    u32x4 x[MT][2];
+#pragma unroll
+                    for (int t = 0; t < MT; t++)
+                    {
+                        x[t][0] = xs[(((s0 + u) * MT + t) * 2 + 0) * 64 + lane];
+                        x[t][1] = xs[(((s0 + u) * MT + t) * 2 + 1) * 64 + lane];
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                    {
+#pragma unroll
+                        for (int d = 0; d < 4; d++)
+                        {
+                            bf16x2 p01, p23;
+                            fp8x4_to_bf16<WT, SCALED>(w[u][r][d], a.w_scale, p01, p23);
+#pragma unroll
+                            for (int t = 0; t < MT; t++)
+                            {
+                                acc[r][t] = dot2_bf16(p01, x[t][d >> 1][(d & 1) * 2 + 0], acc[r][t]);
+                                acc[r][t] = dot2_bf16(p23, x[t][d >> 1][(d & 1) * 2 + 1], acc[r][t]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; r++)
+        {
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+            {
+                const float total = wave_sum(acc[r][t]);
+                const int row = g * R + r;
+                if (lane == 0 && row < a.n_out)
+                {
+                    uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)row * a.y_stride_out;
+                    *y = finish_output(total, a.alpha, a.beta, y);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// FP4 block-scale GEMV, dot2 + DPP reduction.  One 128-bit load = 32 nibbles = 32 consecutive
+// elements of one row = 32 / BLOCK blocks (BLOCK = 16 or 32); the block scales of a k-step are
+// 64 * 32 / BLOCK consecutive bytes of the scale array.
+// Requires: K % 32 == 0, ldw == K (blocks run over the flat index), W 16-byte aligned,
+// (row * K) % BLOCK == 0, ldx % 8 == 0, X 16-byte aligned.
+// Dynamic LDS: MT * ceil(K / 2048) * 4096 bytes.
+
+__device__ __forceinline__ float e4m3_byte_to_f32(uint32_t word, int byte_index)
+{
+    return byte_index == 0 ? __builtin_amdgcn_cvt_f32_fp8(word, 0) : __builtin_amdgcn_cvt_f32_fp8(word, 1);
+}
+
+template <int MT, int R, int U, int WAVES, int BLOCK>
+__global__ __launch_bounds__(WAVES * 64) void gemv4_dot2_kernel(const LinearArgs a)
+{
+    static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    extern __shared__ u32x4 xs[];
+    const int n_steps = (a.K + 2047) / 2048;
+    stage_activations<MT, 4>(a, xs, n_steps, WAVES * 64);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_groups = (a.n_out + R - 1) / R;
+    const int last_row = a.n_out - 1;
+
+    for (int g = blockIdx.x * WAVES + wave; g < n_groups; g += gridDim.x * WAVES)
+    {
+        const uint8_t* wrow[R];
+        const uint8_t* srow[R];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+        {
+            const long long row = min(g * R + r, last_row);
+            wrow[r] = a.W + ((row * a.ldw) >> 1) + lane * 16;
+            srow[r] = a.blk_sc + (row * a.ldw) / BLOCK + lane * (32 / BLOCK);
+        }
+        float acc[R][MT];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) { acc[r][t] = 0.0f; }
+
+        for (int s0 = 0; s0 < n_steps; s0 += U)
+        {
+            u32x4 w[U][R];
+            uint32_t sc[U][R];
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                const int k = (s0 + u) * 2048 + lane * 32;
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                {
+                    w[u][r] = u32x4{ 0u, 0u, 0u, 0u };
+                    sc[u][r] = 0u;
+                    if (k < a.K)
+                    {
+                        w[u][r] = __builtin_nontemporal_load((const u32x4*)(wrow[r] + (s0 + u) * 1024));
+                        if (BLOCK == 16) { sc[u][r] = *(const uint16_t*)(srow[r] + (s0 + u) * 128); }
+                        else { sc[u][r] = *(srow[r] + (s0 + u) * 64); }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                if (s0 + u < n_steps)
+                {
+                    u32x4 x[MT][4];
+#pragma unroll
+                    for (int t = 0; t < MT; t++)
+#pragma unroll
+                        for (int p = 0; p < 4; p++) { x[t][p] = xs[(((s0 + u) * MT + t) * 4 + p) * 64 + lane]; }
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                    {
+                        const float s_lo = e4m3_byte_to_f32(sc[u][r], 0);
+                        const float s_hi = BLOCK == 16 ? e4m3_byte_to_f32(sc[u][r], 1) : s_lo;
+                        float part[MT][2];
+#pragma unroll
+                        for (int t = 0; t < MT; t++) { part[t][0] = part[t][1] = 0.0f; }
+#pragma unroll
+                        for (int d = 0; d < 4; d++)
+                        {
+                            // dword d holds elements 8d .. 8d+7; byte b holds elements 8d+2b, 8d+2b+1
+                            const bf16x2 q0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[u][r][d], 1.0f, 0);
+                            const bf16x2 q1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[u][r][d], 1.0f, 1);
+                            const bf16x2 q2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[u][r][d], 1.0f, 2);
+                            const bf16x2 q3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[u][r][d], 1.0f, 3);
+#pragma unroll
+                            for (int t = 0; t < MT; t++)
+                            {
+                                float p = part[t][d >> 1];
+                                p = dot2_bf16(q0, x[t][d][0], p);
+                                p = dot2_bf16(q1, x[t][d][1], p);
+                                p = dot2_bf16(q2, x[t][d][2], p);
+                                p = dot2_bf16(q3, x[t][d][3], p);
+                                part[t][d >> 1] = p;
+                            }
+                        }
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+                        {
+                            acc[r][t] = fmaf(s_lo, part[t][0], acc[r][t]);
+                            acc[r][t] = fmaf(s_hi, part[t][1], acc[r][t]);
+                        }
+                    }
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; r++)
+        {
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+            {
+                const float total = wave_sum(acc[r][t]);
+                const int row = g * R + r;
+                if (lane == 0 && row < a.n_out)
+                {
+                    uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)row * a.y_stride_out;
+                    *y = finish_output(total, a.alpha, a.beta, y);
+                }
+            }
+        }
+    }
+}
+
+}    // namespace ccq
+
+namespace ccq
+{
+
+// ------------------------------------------------------------------------------------------
+// FP8 GEMV on the matrix cores, tokens 1..16 (v_mfma_f32_16x16x32_bf16).
+//
+// A workgroup owns RT tiles of 16 consecutive output rows and splits K over its WAVES waves in
+// interleaved spans of 64 * U elements; partial 16x16 tiles meet in LDS.  Within a 64-element
+// chunk lane (i = lane % 16, g = lane / 16) loads the 16 codes W[row i][chunk + 16 g ..] with one
+// 128-bit load (a wave touches 16 rows x 64 contiguous bytes) and feeds two MFMAs: codes 0..7 and
+// codes 8..15.  The activation operand of lane (j, g) is x[token j][chunk + 16 g ..] for the same
+// two halves, so both operands agree on which k each register slot means.
+//   A operand = weights: row i = output row, 8 k per lane.
+//   B operand = activations: column j = token.
+//   D: lane holds column j = lane % 16 (token), rows 4 g .. 4 g + 3 (output rows).
+// Requires: K % 16 == 0, ldw % 16 == 0, W 16-byte aligned, ldx % 8 == 0, X 16-byte aligned.
+// Static LDS: WAVES * RT * 1 KiB.
+
+template <int WT, int RT, int U, int WAVES, bool SCALED>
+__global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs a)
+{
+    __shared__ float partial[WAVES][RT][64][4];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int i = lane & 15;
+    const int g = lane >> 4;
+    const int row_base = blockIdx.x * (16 * RT);
+    const int last_row = a.n_out - 1;
+
+    const uint8_t* wrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+    {
+        const int row = min(row_base + rt * 16 + i, last_row);
+        wrow[rt] = a.W + (long long)row * a.ldw + g * 16;
+    }
+    const bool has_token = i < a.tokens;
+    const uint16_t* xrow = a.X + (long long)(has_token ? i : 0) * a.ldx + g * 16;
+
+    f32x4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) { acc[rt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+
+    const int span = 64 * U;
+    for (int kb = wave * span; kb < a.K; kb += WAVES * span)
+    {
+        u32x4 w[U][RT];
+        u32x4 x[U][2];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int k = kb + u * 64 + g * 16;
+            const bool in_k = k < a.K;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+            {
+                w[u][rt] = u32x4{ 0u, 0u, 0u, 0u };
+                if (in_k) { w[u][rt] = __builtin_nontemporal_load((const u32x4*)(wrow[rt] + kb + u * 64)); }
+            }
+            x[u][0] = x[u][1] = u32x4{ 0u, 0u, 0u, 0u };
+            if (in_k && has_token)
+            {
+                x[u][0] = *(const u32x4*)(xrow + kb + u * 64);
+                x[u][1] = *(const u32x4*)(xrow + kb + u * 64 + 8);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+            {
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                {
+                    bf16x2 p0, p1, p2, p3;
+                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h], a.w_scale, p0, p1);
+                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h + 1], a.w_scale, p2, p3);
+                    const bf16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
+                    const bf16x8 xb = __builtin_bit_cast(bf16x8, x[u][h]);
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb, acc[rt], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) { partial[wave][rt][lane][c] = acc[rt][c]; }
+    __syncthreads();
+
+    for (int v = threadIdx.x; v < RT * 256; v += WAVES * 64)
+    {
+        const int c = v & 3;
+        const int src_lane = (v >> 2) & 63;
+        const int rt = v >> 8;
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) { total += partial[w][rt][src_lane][c]; }
+        const int token = src_lane & 15;
+        const int row = row_base + rt * 16 + 4 * (src_lane >> 4) + c;
+        if (token < a.tokens && row < a.n_out)
+        {
+            uint16_t* y = a.Y + (long long)token * a.y_stride_tok + (long long)row * a.y_stride_out;
+            *y = finish_output(total, a.alpha, a.beta, y);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Fallback for any layout / type / size the fast kernels do not take: one lane per output element,
+// software decode of the flat element index exactly as the reference's dequant kernels index it.
+//   element (o, k) of the weight is at flat index  o * w_stride_out + k * w_stride_k
+//   element (t, k) of the activation is at         t * x_stride_tok + k * x_stride_k
+struct GenericArgs
+{
+    const uint8_t* W;
+    const uint8_t* blk_sc;
+    const uint16_t* X;
+    uint16_t* Y;
+    long long w_stride_out, w_stride_k, x_stride_tok, x_stride_k, y_stride_tok, y_stride_out;
+    int n_out, tokens, K, w_type;
+    unsigned block_size;
+    float w_scale, alpha, beta;
+};
+
+__global__ __launch_bounds__(256) void generic_linear_kernel(const GenericArgs a)
+{
+    const long long total = (long long)a.n_out * a.tokens;
+    for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256)
+    {
+        const int o = (int)(idx % a.n_out);
+        const int t = (int)(idx / a.n_out);
+        float acc = 0.0f;
+        for (int k = 0; k < a.K; k++)
+        {
+            const long long fi = (long long)o * a.w_stride_out + (long long)k * a.w_stride_k;
+            float wv;
+            if (a.w_type == DT_FP4)
+            {
+                const uint32_t byte = a.W[fi >> 1];
+                const float s = a.blk_sc ? e4m3_to_f32(a.blk_sc[fi / a.block_size]) : a.w_scale;
+                wv = fp4_to_f32((fi & 1) ? (byte >> 4) : (byte & 0xFu)) * s;
+            }
+            else
+            {
+                wv = (a.w_type == DT_E5M2 ? e5m2_to_f32(a.W[fi]) : e4m3_to_f32(a.W[fi])) * a.w_scale;
+            }
+            const float wq = bf16_bits_to_f32(f32_to_bf16_bits(wv));
+            const float xv = bf16_bits_to_f32(a.X[(long long)t * a.x_stride_tok + (long long)k * a.x_stride_k]);
+            acc = fmaf(wq, xv, acc);
+        }
+        uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)o * a.y_stride_out;
+        *y = finish_output(acc, a.alpha, a.beta, y);
+    }
+}
+
+}    // namespace ccq

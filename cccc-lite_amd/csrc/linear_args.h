@@ -1,0 +1,28 @@
+// One quantized linear, normalised from the BLAS-style call of the unified dispatcher
+// (cccc/cublas_real.h:875-880): y[t][o] = alpha * sum_k dequant(W)[o][k] * x[t][k] + beta * y[t][o].
+#pragma once
+#include <stdint.h>
+
+namespace ccq
+{
+
+struct LinearArgs
+{
+    const uint8_t* W;         // quantized weight, row o starts at element o * ldw (FP4: two elements per byte)
+    const uint8_t* blk_sc;    // FP4 per-block E4M3 scales over the flat element index, or nullptr
+    const uint16_t* X;        // bf16 activations, token t starts at element t * ldx
+    uint16_t* Y;              // bf16 output, element (t, o) at t * y_stride_tok + o * y_stride_out
+    long long ldw;
+    long long ldx;
+    long long y_stride_tok;
+    long long y_stride_out;
+    int n_out;
+    int tokens;
+    int K;
+    unsigned block_size;      // FP4 block length (elements)
+    float w_scale;            // per-tensor dequant multiplier (invScale); ignored when blk_sc is set
+    float alpha;
+    float beta;
+};
+
+}    // namespace ccq

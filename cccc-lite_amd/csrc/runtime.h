@@ -1,0 +1,21 @@
+// Host-side state shared by the entry points: the stream work is enqueued on, the
+// synchronise-after-launch switch, and the error convention of the reference's HIP library
+// (cccc-hip/hip_functions.cpp:32-42: 0 ok, 1 runtime error with a message on stderr).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace ccq
+{
+
+hipStream_t stream();
+bool sync_enabled();
+void note_kernel(const char* name);
+
+// Called after every launch: picks up launch errors, and when the sync switch is on also waits
+// for the device like the reference does after each kernel.
+int finish(const char* what);
+
+// Number of compute units of the current device (cached per device).
+int cu_count();
+
+}    // namespace ccq

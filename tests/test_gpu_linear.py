@@ -1,0 +1,316 @@
+"""Parity of hip_quant_gemm (decode GEMV family, prefill GEMM, generic fallback) against the
+oracle, through the C-ABI.  Expected values are the exact float64 contraction of the bit-exact
+dequantized BF16 weights (oracle.linear_exact); tolerances are the benchmark's (gpu_util)."""
+import numpy as np
+import pytest
+
+from gpu_util import check_bf16_close, check_rows, from_dev, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_f64(oracle, bits):
+    return oracle.bf16_to_f32(bits).astype(np.float64)
+
+
+def run_linear(gpu, pkg, W, w_type, X, n_out, tokens, K, inv_scale=1.0, blk_sc=None, block=16, alpha=1.0, beta=0.0, Y0=None):
+    torch, dev, lib = gpu
+    wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+    sd = to_dev(torch, dev, blk_sc) if blk_sc is not None else None
+    y0 = Y0 if Y0 is not None else np.zeros((tokens, n_out), dtype=np.uint16)
+    yd = to_dev(torch, dev, np.concatenate([y0.ravel(), np.zeros(64, dtype=np.uint16)]))
+    rc = lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, inv_scale,
+                    sd.data_ptr() if sd is not None else None, block, alpha, beta)
+    assert rc == 0
+    out = from_dev(yd, np.uint16)
+    assert not out[tokens * n_out:].any(), "wrote past the end"
+    return out[: tokens * n_out].reshape(tokens, n_out), lib.last_kernel()
+
+
+# ------------------------------------------------------------------------------------------ golden
+
+def test_golden_linear_cases(gpu, pkg, oracle, golden_linear):
+    g = golden_linear
+    for name, n_out, K, tokens in (("fp8_a", 24, 64, 1), ("fp8_b", 17, 48, 3)):
+        y, _ = run_linear(gpu, pkg, g[name + "_w"], oracle.E5M2, g[name + "_x"], n_out, tokens, K)
+        check_rows(bf16_f64(oracle, y), g[name + "_y_f64"], name)
+        check_bf16_close(y, g[name + "_y_f64"], name, slack_ulp=1.0, abs_floor=1e-6)
+    y, _ = run_linear(gpu, pkg, g["fp4_a_w"], oracle.FP4, g["fp4_a_x"], 8, 2, 64, blk_sc=g["fp4_a_s"])
+    check_rows(bf16_f64(oracle, y), g["fp4_a_y_f64"], "fp4_a")
+
+
+# ------------------------------------------------------------------------------------------ FP8 GEMV
+
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4, 5, 8, 16])
+@pytest.mark.parametrize("n_out,K", [(4096, 4096), (1024, 4096), (768, 12288), (1000, 2064), (7, 16)])
+def test_fp8_gemv_vs_oracle(gpu, pkg, oracle, tokens, n_out, K):
+    seed = pkg.synth.seed_for(2, n_out % 97 + tokens)
+    W = pkg.synth.weights_e5m2(seed, n_out, K)
+    X = pkg.synth.activations(seed, tokens, K)
+    y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K)
+    want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X)
+    check_rows(bf16_f64(oracle, y), want, f"{kernel} {n_out}x{K} M={tokens}")
+    check_bf16_close(y, want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    assert kernel in ("gemv_dot2", "gemv_mfma")
+
+
+@pytest.mark.parametrize("tokens", [1, 4, 16])
+def test_every_code_dequantizes_exactly_inside_the_gemv(gpu, pkg, oracle, tokens):
+    """One-hot activations pick single dequantized weights out of the GEMV: with x = e_k the output
+    row is bf16(decode(W[:, k])) bit for bit, for all 256 codes (NaN codes: NaN)."""
+    for w_type, K in ((oracle.E5M2, 256), (oracle.E4M3, 256)):
+        n_out = 256
+        W = np.empty((n_out, K), dtype=np.uint8)
+        for o in range(n_out):
+            W[o] = np.roll(np.arange(256, dtype=np.uint8), o)        # W[o][k] = (k - o) mod 256
+        ks = [0, 5, 255][:max(1, min(tokens, 3))]
+        X = np.zeros((tokens, K), dtype=np.uint16)
+        for t in range(tokens):
+            X[t, ks[t % len(ks)]] = 0x3F80                            # 1.0
+        # Inf / NaN codes would poison their whole row through 0 * Inf; give them a separate pass
+        tab = oracle.decode_table(w_type)
+        special = ~np.isfinite(tab)
+        Wf = W.copy()
+        Wf[special[W]] = 0
+        y, kernel = run_linear(gpu, pkg, Wf, w_type, X, n_out, tokens, K)
+        for t in range(tokens):
+            k = ks[t % len(ks)]
+            want = oracle.dequant_fp8_to_bf16(Wf[:, k], w_type, 1.0)
+            got = y[t].copy()
+            got[got == 0x8000] = 0                                    # -0.0 + 0.0 accumulates to +0.0
+            want = want.copy(); want[want == 0x8000] = 0
+            assert np.array_equal(got, want), (kernel, w_type, t)
+    # Inf and NaN codes propagate
+    W = np.full((16, 64), 0x3C, dtype=np.uint8)
+    W[3, 7] = 0x7C; W[5, 9] = 0x7E; W[6, 0] = 0xFC
+    X = np.full((tokens, 64), 0x3F80, dtype=np.uint16)
+    y, _ = run_linear(gpu, pkg, W, oracle.E5M2, X, 16, tokens, 64)
+    f = bf16_f64(oracle, y)
+    assert np.all(f[:, 3] == np.inf) and np.all(np.isnan(f[:, 5])) and np.all(f[:, 6] == -np.inf) and np.all(f[:, 0] == 64.0)
+
+
+@pytest.mark.parametrize("tokens", [1, 3, 16, 40])
+@pytest.mark.parametrize("w_type_name", ["e5m2", "e4m3"])
+def test_per_tensor_scale_rounds_the_weight_to_bf16(gpu, pkg, oracle, tokens, w_type_name):
+    """With invScale != 1 the weight entering the product is bf16(decode * invScale)."""
+    n_out, K = 512, 1024
+    seed = pkg.synth.seed_for(2, 40 + tokens)
+    X = pkg.synth.activations(seed, tokens, K)
+    if w_type_name == "e5m2":
+        wf = pkg.synth.weights_f32(seed, n_out, K)
+        inv = float(np.abs(wf).max()) / 57344.0
+        W, w_type = oracle.encode_e5m2_rne(wf / np.float32(inv)), oracle.E5M2
+    else:
+        W, inv = pkg.synth.weights_e4m3(seed, n_out, K)
+        w_type = oracle.E4M3
+    y, kernel = run_linear(gpu, pkg, W, w_type, X, n_out, tokens, K, inv_scale=inv)
+    want = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K, inv), X)
+    check_rows(bf16_f64(oracle, y), want, kernel)
+    check_bf16_close(y, want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    # and it is measurably different from scaling after the sum (so the rounding point is tested)
+    unrounded = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K, 1.0), X) * inv
+    assert np.abs(unrounded - want).max() > 0
+
+
+def test_alpha_beta_epilogue(gpu, pkg, oracle):
+    n_out, K = 640, 2048
+    for tokens in (1, 4, 12, 48):
+        seed = pkg.synth.seed_for(2, 60 + tokens)
+        W = pkg.synth.weights_e5m2(seed, n_out, K)
+        X = pkg.synth.activations(seed, tokens, K)
+        Y0 = pkg.synth.activations(seed + 1, tokens, n_out)
+        y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K, alpha=0.5, beta=-2.0, Y0=Y0)
+        want = 0.5 * oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X) - 2.0 * bf16_f64(oracle, Y0)
+        check_rows(bf16_f64(oracle, y), want, kernel)
+
+
+# ------------------------------------------------------------------------------------------ FP4
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
+@pytest.mark.parametrize("n_out,K", [(4096, 4096), (1024, 4096), (512, 14336), (33, 64)])
+def test_fp4_gemv_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, block):
+    seed = pkg.synth.seed_for(3, n_out % 89 + tokens + block)
+    nib, sc = pkg.synth.weights_fp4(seed, n_out, K, block)
+    X = pkg.synth.activations(seed, tokens, K)
+    y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, K, blk_sc=sc, block=block)
+    want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block), X)
+    check_rows(bf16_f64(oracle, y), want, f"{kernel} fp4 {n_out}x{K} M={tokens} b={block}")
+    assert kernel == "gemv_dot2"
+
+
+def test_fp4_every_nibble_and_scale_inside_the_gemv(gpu, pkg, oracle):
+    """x = one-hot: the output is bf16(fp4 * e4m3 scale) exactly, for all 16 nibbles x all finite
+    scale bytes."""
+    K, n_out = 64, 256
+    nib_row = (np.arange(16, dtype=np.uint8)[0::2] | (np.arange(16, dtype=np.uint8)[1::2] << 4)).astype(np.uint8)
+    nib = np.tile(nib_row, (n_out, K // 16))                            # element k of every row = nibble k % 16
+    sc = np.repeat(np.arange(256, dtype=np.uint8)[:, None], K // 16, axis=1)
+    sc[sc == 0x7F] = 0x38; sc[sc == 0xFF] = 0xB8
+    Wd = oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=16)
+    for k in (0, 9, 15, 16 + 3, 63):
+        X = np.zeros((1, K), dtype=np.uint16); X[0, k] = 0x3F80
+        y, _ = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, 1, K, blk_sc=sc, block=16)
+        got, want = y[0].copy(), Wd[:, k].copy()
+        got[got == 0x8000] = 0; want[want == 0x8000] = 0
+        assert np.array_equal(got, want), k
+
+
+# ------------------------------------------------------------------------------------------ prefill GEMM
+
+@pytest.mark.parametrize("tokens,n_out,K", [(128, 256, 512), (512, 768, 1024), (130, 200, 144), (17, 128, 64), (2048, 256, 256)])
+@pytest.mark.parametrize("fmt", ["e5m2", "fp4_16", "fp4_32"])
+def test_prefill_gemm_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, fmt):
+    seed = pkg.synth.seed_for(4, tokens % 83 + n_out % 7)
+    X = pkg.synth.activations(seed, tokens, K)
+    if fmt == "e5m2":
+        W = pkg.synth.weights_e5m2(seed, n_out, K)
+        y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K)
+        Wd = oracle.dequant_weight(W, oracle.E5M2, n_out, K)
+    else:
+        block = int(fmt[-2:])
+        if K % 32:
+            pytest.skip("FP4 rows are packed in 32-element loads")
+        nib, sc = pkg.synth.weights_fp4(seed, n_out, K, block)
+        y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, K, blk_sc=sc, block=block)
+        Wd = oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block)
+    want = oracle.linear_exact(Wd, X)
+    check_rows(bf16_f64(oracle, y), want, f"{kernel} {fmt} {tokens}x{n_out}x{K}")
+    check_bf16_close(y, want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    assert kernel == "gemm_mfma"
+
+
+# ------------------------------------------------------------------------------------------ dispatcher
+
+def test_weight_as_B_and_transposed_layouts_match_the_scalar_oracle(gpu, pkg, oracle):
+    """All eight (which operand is quantized) x (transA) x (transB) layouts of the unified call
+    against the scalar C restatement of the dispatcher."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(77)
+    n_out, tokens, K = 48, 5, 64
+    Wq = oracle.encode_e5m2_rne((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32))
+    Xb = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
+    for weight_is_a in (True, False):
+        for ta in (0, 1):
+            for tb in (0, 1):
+                if weight_is_a:
+                    M, N = n_out, tokens
+                    A = Wq if ta else np.ascontiguousarray(Wq.T)           # trans: stored [M][K] (lda=K); no-trans: [K][M] (lda=M)
+                    B = np.ascontiguousarray(Xb.T) if tb else Xb           # no-trans: stored [N][K] (ldb=K); trans: [K][N] (ldb=N)
+                    lda, ldb = (K if ta else M), (N if tb else K)
+                    tA, tB, sA = oracle.E5M2, oracle.BF16, 0.25
+                else:
+                    M, N = tokens, n_out
+                    A = Xb if ta else np.ascontiguousarray(Xb.T)
+                    B = np.ascontiguousarray(Wq.T) if tb else Wq
+                    lda, ldb = (K if ta else M), (N if tb else K)
+                    tA, tB, sA = oracle.BF16, oracle.E5M2, 1.0
+                sB = 0.25 if not weight_is_a else 1.0
+                C0 = oracle.f32_to_bf16(rng.standard_normal((N, M)).astype(np.float32))
+                want = C0.copy()
+                assert oracle.quant_gemm(ta, tb, M, N, K, 1.5, A, tA, lda, sA, B, tB, ldb, sB, 0.5, want, M) == 0
+                Ad, Bd, Cd = to_dev(torch, dev, A), to_dev(torch, dev, B), to_dev(torch, dev, C0)
+                rc = lib.quant_gemm(ta, tb, M, N, K, 1.5, Ad.data_ptr(), tA, lda, sA, Bd.data_ptr(), tB, ldb, sB, 0.5,
+                                    Cd.data_ptr(), oracle.BF16, M)
+                assert rc == 0
+                got = from_dev(Cd, np.uint16).reshape(N, M)
+                diff = np.abs(bf16_f64(oracle, got) - bf16_f64(oracle, want))
+                assert diff.max() <= 2.0 ** -7 * np.abs(bf16_f64(oracle, want)).max(), (weight_is_a, ta, tb, lib.last_kernel())
+
+
+def test_fp4_weight_as_B_with_block_scales(gpu, pkg, oracle):
+    torch, dev, lib = gpu
+    n_out, tokens, K = 64, 3, 128
+    nib, sc = pkg.synth.weights_fp4(5, n_out, K, 16)
+    Xb = pkg.synth.activations(5, tokens, K)
+    C0 = np.zeros((n_out, tokens), dtype=np.uint16)
+    want = C0.copy()
+    assert oracle.quant_gemm(1, 0, tokens, n_out, K, 1.0, Xb, oracle.BF16, K, 1.0, nib, oracle.FP4, K, 1.0, 0.0, want, tokens, None, sc, 16) == 0
+    Ad, Bd, Sd, Cd = to_dev(torch, dev, Xb), to_dev(torch, dev, nib), to_dev(torch, dev, sc), to_dev(torch, dev, C0)
+    rc = lib.quant_gemm(1, 0, tokens, n_out, K, 1.0, Ad.data_ptr(), oracle.BF16, K, 1.0, Bd.data_ptr(), oracle.FP4, K, 1.0, 0.0,
+                        Cd.data_ptr(), oracle.BF16, tokens, 0.0, None, Sd.data_ptr(), 16)
+    assert rc == 0
+    got = from_dev(Cd, np.uint16).reshape(n_out, tokens)
+    diff = np.abs(bf16_f64(oracle, got) - bf16_f64(oracle, want))
+    assert diff.max() <= 2.0 ** -7 * np.abs(bf16_f64(oracle, want)).max()
+
+
+def test_odd_sizes_fall_back_to_the_generic_kernel(gpu, pkg, oracle):
+    rng = np.random.default_rng(78)
+    n_out, tokens, K = 37, 3, 50                                         # K % 16 != 0
+    W = oracle.encode_e5m2_rne((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32))
+    X = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
+    y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K, inv_scale=0.3)
+    assert kernel == "generic"
+    want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K, 0.3), X)
+    check_rows(bf16_f64(oracle, y), want, kernel)
+    # FP4 with a per-tensor scale and no block scales
+    nib = rng.integers(0, 256, size=(n_out, 32), dtype=np.uint8)
+    X = oracle.f32_to_bf16(rng.standard_normal((tokens, 64)).astype(np.float32))
+    y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, 64, inv_scale=0.01)
+    assert kernel == "generic"
+    want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, 64, 0.01), X)
+    check_rows(bf16_f64(oracle, y), want, kernel)
+
+
+def test_rejected_argument_combinations(gpu, oracle):
+    torch, dev, lib = gpu
+    b = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    p = b.data_ptr()
+    BF, E5 = oracle.BF16, oracle.E5M2
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, E5, 16, 1.0, 0.0, p, BF, 16) == -1       # both quantized (W8A8 route)
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, BF, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == -1       # nothing quantized
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, oracle.HALF, 16, 1.0, 0.0, p, oracle.HALF, 16) == -1
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, oracle.FLOAT, 16) == -1
+    assert lib.quant_gemm(2, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == -1
+    assert lib.quant_gemm(1, 0, 0, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == 0         # empty output
+    assert not b.cpu().numpy().any()
+    # K == 0: the sum is empty, C = beta * C
+    c = to_dev(torch, dev, np.full(16, 0x4000, dtype=np.uint16))
+    assert lib.quant_gemm(1, 0, 16, 1, 0, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.5, c.data_ptr(), BF, 16) == 0
+    assert np.all(from_dev(c, np.uint16) == 0x3F80)
+
+
+# ------------------------------------------------------------------------------------------ full-size properties
+
+def test_full_size_gemv_properties(gpu, pkg, oracle):
+    """At the benchmark's real shapes (too big for the scalar oracle in a test): (1) rows sampled at
+    random agree with the exact contraction; (2) linearity in x; (3) all-ones x gives row sums."""
+    torch, dev, lib = gpu
+    for n_out, K in ((12288, 4096), (4096, 12288), (151936, 4096)):
+        g = torch.Generator(device="cpu").manual_seed(n_out + K)
+        W = (torch.randn(n_out, K, generator=g) * 0.02).to(torch.bfloat16).to(torch.float8_e5m2).view(torch.uint8).numpy()
+        wd = to_dev(torch, dev, W)
+        rows = np.random.default_rng(n_out).choice(n_out, size=257, replace=False)
+        Wd_rows = oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2)
+        for tokens in (1, 4, 16):
+            X = pkg.synth.activations(n_out + tokens, tokens, K)
+            xd = to_dev(torch, dev, X)
+            yd = torch.zeros(tokens, n_out, dtype=torch.int16, device=dev)
+            assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
+            y = from_dev(yd, np.uint16)
+            want = oracle.linear_exact(Wd_rows, X)
+            check_rows(bf16_f64(oracle, y[:, rows]), want, f"{lib.last_kernel()} {n_out}x{K} M={tokens}")
+        ones = np.full((1, K), 0x3F80, dtype=np.uint16)
+        yd = torch.zeros(1, n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), oracle.E5M2, to_dev(torch, dev, ones).data_ptr(), yd.data_ptr(), n_out, 1, K) == 0
+        sums = oracle.decode_table(oracle.E5M2).astype(np.float64)[W[rows]].sum(axis=1)
+        got = bf16_f64(oracle, from_dev(yd, np.uint16))[0, rows]
+        assert np.all(np.abs(got - sums) <= 2.0 ** -8 * np.abs(sums) + 1e-5)
+        del wd
+
+
+def test_full_size_prefill_gemm_sampled(gpu, pkg, oracle):
+    torch, dev, lib = gpu
+    for tokens, n_out, K in ((512, 12288, 4096), (2048, 4096, 12288)):
+        g = torch.Generator(device="cpu").manual_seed(tokens + K)
+        W = (torch.randn(n_out, K, generator=g) * 0.02).to(torch.bfloat16).to(torch.float8_e5m2).view(torch.uint8).numpy()
+        X = pkg.synth.activations(tokens, tokens, K)
+        wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+        yd = torch.zeros(tokens, n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
+        assert lib.last_kernel() == "gemm_mfma"
+        y = from_dev(yd, np.uint16)
+        rows = np.random.default_rng(tokens).choice(n_out, size=192, replace=False)
+        want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2), X)
+        check_rows(bf16_f64(oracle, y[:, rows]), want, f"gemm {tokens}x{n_out}x{K}")
