@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X weight-only quantized linear path (one GPU).
+
+A step is one pass of the hot path over one batch of synthetic input.  Default workload: the
+linear layers of one Qwen3-8B W8A16 decode token at batch 1 -- 36 layers x (q, k, v, o, gate, up,
+down) + lm_head = 253 FP8_E5M2 GEMVs over 7,568,097,280 bytes of distinct, HBM-resident weights --
+issued through the C++ host mirror's Matrix::mulBatched exactly as cccc's graph issues them.
+`value` = algorithmic bytes (K*N + 2*M*K + 2*M*N per GEMV) / elapsed.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_linears|gemv|prefill]
+                    [--shape K,N] [--tokens M] [--no-graph] [--no-cpu] [--no-sweep]
+
+Prints ONE JSON line.  `roofline` is measured live on the dominant kernel (the gate/up-shaped
+GEMV, K=4096 N=12288) with HIP events on the stream it runs on; `cpu_baseline` times the CPU
+restatement of the reference's CPU route (scalar dequant of the whole weight + cblas_sgemm) on a
+bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
+
+QWEN3_8B = dict(layers=36, hidden=4096, q_out=4096, kv_out=1024, inter=12288, vocab=151936)
+QWEN_SHAPES = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096), (4096, 151936)]     # (K, N)
+
+
+def gemv_bytes(K, N, M):
+    return K * N + 2 * M * K + 2 * M * N
+
+
+class Workspace:
+    """Weights, activations and outputs of the benchmark as host-mirror matrices on cuda:0."""
+
+    def __init__(self, pkg, torch):
+        self.pkg, self.torch = pkg, torch
+        self.lib = pkg.library()
+        self.host = pkg.host_api.host()
+        self.host.init(0)
+        self.dev = torch.device("cuda:0")
+        self.gen = torch.Generator(device=self.dev).manual_seed(1234)
+        self.keep = []
+
+    def weight_e5m2(self, n_out, K):
+        t = self.torch
+        m = self.host.matrix(K, n_out, 1, 1, E5M2)
+        rows = max(1, min(n_out, (1 << 27) // K))
+        for r0 in range(0, n_out, rows):
+            r = min(rows, n_out - r0)
+            w = (t.randn(r, K, device=self.dev, generator=self.gen) * 0.02).to(t.bfloat16).to(t.float8_e5m2)
+            assert self.lib.convert(w.data_ptr(), E5M2, m.data_ptr + r0 * K, E5M2, r * K, 1.0) == 0
+            t.cuda.synchronize()
+        return m
+
+    def activation(self, tokens, K):
+        t = self.torch
+        m = self.host.matrix(K, tokens, 1, 1, BF16)
+        x = t.randn(tokens, K, device=self.dev, generator=self.gen).to(t.bfloat16)
+        assert self.lib.convert(x.data_ptr(), BF16, m.data_ptr, BF16, tokens * K * 2, 1.0) == 0
+        t.cuda.synchronize()
+        return m
+
+    def output(self, tokens, n_out):
+        return self.host.matrix(n_out, tokens, 1, 1, BF16)
+
+
+def build_decode_model(ws: Workspace, tokens: int):
+    """Returns (ops, weights_by_shape): ops = list of (W, X, Y, K, N) in graph order."""
+    c = QWEN3_8B
+    x_h, x_i = ws.activation(tokens, c["hidden"]), ws.activation(tokens, c["inter"])
+    y = {n: ws.output(tokens, n) for n in (c["q_out"], c["kv_out"], c["inter"], c["vocab"])}
+    y_up = ws.output(tokens, c["inter"])
+    y_v = ws.output(tokens, c["kv_out"])
+    ops, by_shape = [], {}
+
+    def add(K, N, X, Y):
+        W = ws.weight_e5m2(N, K)
+        by_shape.setdefault((K, N), []).append(W)
+        ops.append((W, X, Y, K, N))
+
+    for _ in range(c["layers"]):
+        add(c["hidden"], c["q_out"], x_h, y[c["q_out"]])
+        add(c["hidden"], c["kv_out"], x_h, y[c["kv_out"]])
+        add(c["hidden"], c["kv_out"], x_h, y_v)
+        add(c["hidden"], c["q_out"], x_h, y[c["q_out"]])          # o
+        add(c["hidden"], c["inter"], x_h, y[c["inter"]])          # gate
+        add(c["hidden"], c["inter"], x_h, y_up)                   # up
+        add(c["inter"], c["hidden"], x_i, y[c["q_out"]])          # down
+    add(c["hidden"], c["vocab"], x_h, y[c["vocab"]])              # lm_head
+    return ops, by_shape
+
+
+def time_chain(ws, ops, steps, warmup, use_graph):
+    ms = ws.host.bench_linear_chain([o[0] for o in ops], [o[1] for o in ops], [o[2] for o in ops], steps, warmup, use_graph)
+    if ms < 0:
+        raise RuntimeError(f"bench chain failed with code {ms}")
+    return ms
+
+
+def shape_sweep(ws, by_shape, token_counts, use_graph):
+    """Per-shape GEMV rates with weights rotating over distinct buffers (no cache reuse)."""
+    out = []
+    for (K, N) in QWEN_SHAPES:
+        weights = by_shape[(K, N)]
+        for M in token_counts:
+            X, Y = ws.activation(M, K), ws.output(M, N)
+            reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
+            ops = [(W, X, Y, K, N) for W in weights] * reps
+            ms = time_chain(ws, ops, 3, 1, use_graph)
+            us = ms * 1000.0 / (3 * len(ops))
+            gbs = gemv_bytes(K, N, M) / us * 1e-3
+            assert ws.lib.linear(weights[0].data_ptr, E5M2, X.data_ptr, Y.data_ptr, N, M, K) == 0
+            out.append({"K": K, "N": N, "M": M, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                        "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(K * N * len(weights) / 2 ** 20)})
+    return out
+
+
+def cpu_baseline(pkg, threads):
+    """The reference CPU route on one transformer layer's seven linears at M=1 (bounded sample)."""
+    import numpy as np
+    from oracle import oracle
+    c = QWEN3_8B
+    shapes = [(c["hidden"], c["q_out"]), (c["hidden"], c["kv_out"]), (c["hidden"], c["kv_out"]), (c["hidden"], c["q_out"]),
+              (c["hidden"], c["inter"]), (c["hidden"], c["inter"]), (c["inter"], c["hidden"])]
+    fn, blas = oracle.find_cblas_sgemm()
+    rng = np.random.default_rng(7)
+    data = []
+    for K, N in shapes:
+        W = rng.integers(0, 0x7C, size=(N, K), dtype=np.uint8)
+        X = pkg.synth.activations(7, 1, K)
+        data.append((W, X, K, N))
+    runs = []
+    t_end = time.time() + 25.0
+    for rep in range(6):
+        td = tg = 0.0
+        for W, X, K, N in data:
+            _, a, b = oracle.cpu_linear(W, oracle.E5M2, 1.0, None, 16, X, N, 1, K, sgemm=fn, threads=threads)
+            td, tg = td + a, tg + b
+        if rep:
+            runs.append((td + tg, td, tg))
+        if time.time() > t_end and len(runs) >= 2:
+            break
+    runs.sort()
+    total, td, tg = runs[len(runs) // 2]
+    nbytes = sum(gemv_bytes(K, N, 1) for _, _, K, N in data)
+    return {"value": round(nbytes / total * 1e-9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"one Qwen3-8B layer (q,k,v,o,gate,up,down) at M=1, {nbytes} bytes, median of {len(runs)} runs after one warm-up",
+            "dequant_s": round(td, 4), "gemm_s": round(tg, 4), "blas": blas}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="decode_linears", choices=["decode_linears", "gemv", "prefill"])
+    ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
+    ap.add_argument("--tokens", type=int, default=1)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import __graft_entry__
+    pkg = __graft_entry__.load_package()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    ws = Workspace(pkg, torch)
+    use_graph = not args.no_graph
+    extra = {}
+
+    if args.workload == "decode_linears":
+        ops, by_shape = build_decode_model(ws, 1)
+        step_bytes = sum(gemv_bytes(K, N, 1) for *_, K, N in ops)
+        torch.cuda.synchronize()
+        ms = time_chain(ws, ops, args.steps, args.warmup, use_graph)
+        torch.cuda.synchronize()
+        ms_other = time_chain(ws, ops, args.steps, 1, not use_graph)
+        ms_step = ms / args.steps
+        value = step_bytes / ms_step * 1e-6
+        extra["launch_mode"] = "hipGraph" if use_graph else "stream"
+        extra["ms_per_step_" + ("stream" if use_graph else "hipGraph")] = round(ms_other / args.steps, 4)
+        extra["decode_linears_tok_s"] = round(1000.0 / ms_step, 1)
+        extra["launches_per_step"] = len(ops)
+        workload = "qwen3-8b W8A16 decode linears, batch 1: 36x(q,k,v,o,gate,up,down)+lm_head, 7568097280 B of distinct FP8_E5M2 weights per step"
+        # dominant kernel: gate/up-shaped GEMV over the 72 distinct gate/up weights
+        K, N, M = 4096, 12288, 1
+        dom_ops = [o for o in ops if (o[3], o[4]) == (K, N)]
+        dom_ms = time_chain(ws, dom_ops, 10, 2, False)
+        dom_us = dom_ms * 1000.0 / (10 * len(dom_ops))
+        if not args.no_sweep:
+            extra["sweep"] = shape_sweep(ws, by_shape, (1, 4, 16), False)
+    else:
+        K, N = (int(v) for v in args.shape.split(","))
+        M = args.tokens if args.workload == "gemv" else max(args.tokens, 512)
+        n_w = max(2, min(64, (1 << 30) // (K * N)))
+        weights = [ws.weight_e5m2(N, K) for _ in range(n_w)]
+        X, Y = ws.activation(M, K), ws.output(M, N)
+        ops = [(W, X, Y, K, N) for W in weights]
+        torch.cuda.synchronize()
+        ms = time_chain(ws, ops, args.steps, args.warmup, False)
+        torch.cuda.synchronize()
+        ms_step = ms / args.steps
+        step_bytes = sum(gemv_bytes(K, N, M) for _ in ops)
+        value = step_bytes / ms_step * 1e-6
+        dom_us = ms_step * 1000.0 / len(ops)
+        extra["launch_mode"] = "stream"
+        workload = f"{args.workload} K={K} N={N} M={M} over {n_w} distinct FP8_E5M2 weights"
+
+    assert ws.lib.linear(ops[0][0].data_ptr, E5M2, ops[0][1].data_ptr, ops[0][2].data_ptr, ops[0][4], M if args.workload != "decode_linears" else 1, ops[0][3]) == 0
+    if args.workload == "prefill":
+        flops = 2.0 * M * K * N
+        achieved = flops / dom_us * 1e-6
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                    "kernel": "gemm_mfma_kernel", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3)}
+    else:
+        achieved = gemv_bytes(K, N, M) / dom_us * 1e-3
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "kernel": "gemv8_dot2_kernel", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
+                    "bytes_per_launch": gemv_bytes(K, N, M)}
+
+    line = {
+        "metric": "quant GEMV HBM GB/s (Qwen3-8B W8A16 decode linears, bs=1)" if args.workload != "prefill" else "W8A16 prefill GEMM algorithmic GB/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        threads = min(16, len(os.sched_getaffinity(0)))
+        line["cpu_baseline"] = cpu_baseline(pkg, threads)
+    line.update(extra)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

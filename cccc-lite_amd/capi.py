@@ -24,6 +24,7 @@ EXPORTS = (
     "hip_convert",
     "hip_fp4_blockscale_to_bf16",
     "hip_float_to_fp4_blockscale",
+    "hip_absmax",
     "hip_quant_gemm",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
@@ -54,6 +55,8 @@ class QuantLibrary:
         L.hip_fp4_blockscale_to_bf16.argtypes = [vp, vp, vp, u32, u32]
         L.hip_float_to_fp4_blockscale.restype = i32
         L.hip_float_to_fp4_blockscale.argtypes = [vp, vp, vp, u32, u32]
+        L.hip_absmax.restype = i32
+        L.hip_absmax.argtypes = [vp, i32, u32, vp]
         L.hip_quant_gemm.restype = i32
         L.hip_quant_gemm.argtypes = [i32, i32, i32, i32, i32, f32,
                                      vp, i32, i32, f32,
@@ -77,6 +80,9 @@ class QuantLibrary:
 
     def float_to_fp4_blockscale(self, src, nibbles, scales, n_elems, block_size=16) -> int:
         return self.c.hip_float_to_fp4_blockscale(src, nibbles, scales, n_elems, block_size)
+
+    def absmax(self, src, src_type, n, d_result) -> int:
+        return self.c.hip_absmax(src, src_type, n, d_result)
 
     def quant_gemm(self, transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
                    B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale=0.0,

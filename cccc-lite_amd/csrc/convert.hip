@@ -34,7 +34,8 @@ __device__ __forceinline__ float decode8(uint32_t b)
 __device__ __forceinline__ uint32_t f32_to_half_bits(float f)
 {
     const _Float16 h = (_Float16)f;    // v_cvt_f16_f32, round to nearest even
-    return (uint32_t)__builtin_bit_cast(uint16_t, h);
+    // the sign is carried over explicitly so that -0.0 stays -0.0
+    return ((uint32_t)__builtin_bit_cast(uint16_t, h) & 0x7FFFu) | ((f32_to_bits(f) >> 16) & 0x8000u);
 }
 
 template <int DST>
@@ -295,7 +296,33 @@ __global__ __launch_bounds__(kThreads) void encode4_blockscale_kernel(const floa
     }
 }
 
+// Largest magnitude: per-lane running max, DPP/LDS-free wave reduction through lane reads, one
+// atomic per wave on the bit pattern (non-negative floats order like unsigned integers).
+__global__ __launch_bounds__(kThreads) void absmax_kernel(const void* __restrict__ src, int src_type, size_t n, unsigned int* __restrict__ out)
+{
+    const size_t stride = (size_t)gridDim.x * kThreads;
+    float m = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) { m = fmaxf(m, fabsf(load_plain(src, src_type, i))); }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) { m = fmaxf(m, __shfl_xor(m, off)); }
+    if ((threadIdx.x & 63) == 0) { atomicMax(out, f32_to_bits(m)); }
+}
+
 }    // namespace
+
+int hip_absmax(const void* src, int src_type, unsigned int n, void* d_result)
+{
+    if (src_type != DT_FLOAT && src_type != DT_HALF && src_type != DT_BF16) { return -1; }
+    if (!d_result) { return -1; }
+    const hipError_t err = hipMemsetAsync(d_result, 0, sizeof(float), stream());
+    if (err != hipSuccess)
+    {
+        fprintf(stderr, "absmax clear failed: %s\n", hipGetErrorString(err));
+        return 1;
+    }
+    if (n) { absmax_kernel<<<grid_for(n), kThreads, 0, stream()>>>(src, src_type, n, (unsigned int*)d_result); }
+    return finish("absmax");
+}
 
 int hip_convert(const void* src, int src_type, void* dst, int dst_type, unsigned int n, float scale)
 {

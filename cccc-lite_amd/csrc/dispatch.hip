@@ -39,32 +39,38 @@ bool allow_big_lds(Kernel kernel, size_t bytes)
     return true;
 }
 
-template <int WT, int MT, int R, int U, int WAVES, bool SCALED>
+// One FP8 GEMV launch: PIPE picks the software-pipelined variant, OCC workgroups per CU cap the grid
+// (the kernels walk the row groups with a grid stride).
+template <int WT, int MT, int R, int U, int WAVES, int OCC, bool PIPE, bool SCALED>
 bool launch_gemv8_dot2(const LinearArgs& a)
 {
     const size_t lds = (size_t)MT * ((a.K + 1023) / 1024) * 2048;
-    auto kernel = gemv8_dot2_kernel<WT, MT, R, U, WAVES, SCALED>;
+    auto kernel = PIPE ? gemv8_dot2_pipe_kernel<WT, MT, R, U, WAVES, SCALED, true> : gemv8_dot2_kernel<WT, MT, R, U, WAVES, SCALED>;
     if (!allow_big_lds(kernel, lds)) { return false; }
     const int n_groups = (a.n_out + R - 1) / R;
     const int want = (n_groups + WAVES - 1) / WAVES;
-    const int cap = cu_count() * (lds > 80 * 1024 ? 1 : (16 / WAVES));
+    const int cap = cu_count() * (lds > 80 * 1024 ? 1 : (lds > 40 * 1024 && OCC > 2 ? 2 : OCC));
     kernel<<<want < cap ? want : cap, WAVES * 64, lds, stream()>>>(a);
     return true;
 }
 
+// Shapes were tuned on MI355X with rotating weight buffers (no cache reuse): small weights want
+// every row in flight at once (one row per wave, pipelined), mid-size ones two rows per wave,
+// very tall ones (lm_head) one row per wave again with more waves per workgroup.
 template <int WT, int MT, bool SCALED>
 bool pick_gemv8_dot2(const LinearArgs& a)
 {
-    // rows per CU decides how much each wave must keep in flight
+    const long long bytes = (long long)a.n_out * a.K;
     const long long rows_per_cu = a.n_out / cu_count();
-    if (a.K <= 4096)
+    if (MT <= 2)
     {
-        if (rows_per_cu >= 64) { return launch_gemv8_dot2<WT, MT, (MT > 2 ? 2 : 4), 4, 4, SCALED>(a); }
-        if (rows_per_cu >= 16) { return launch_gemv8_dot2<WT, MT, 2, 4, 4, SCALED>(a); }
-        return launch_gemv8_dot2<WT, MT, 1, 4, 4, SCALED>(a);
+        if (bytes <= (8LL << 20)) { return launch_gemv8_dot2<WT, MT, 1, 4, 8, 2, true, SCALED>(a); }
+        if (rows_per_cu >= 128) { return launch_gemv8_dot2<WT, MT, 1, 4, 8, 2, false, SCALED>(a); }
+        if (a.K > 8192) { return launch_gemv8_dot2<WT, MT, 2, 4, 8, 2, false, SCALED>(a); }
+        return launch_gemv8_dot2<WT, MT, 2, 4, 4, 4, false, SCALED>(a);
     }
-    if (rows_per_cu >= 32) { return launch_gemv8_dot2<WT, MT, 2, 4, 4, SCALED>(a); }
-    return launch_gemv8_dot2<WT, MT, 1, 4, 4, SCALED>(a);
+    if (rows_per_cu >= 128) { return launch_gemv8_dot2<WT, MT, 2, 4, 4, 4, false, SCALED>(a); }
+    return launch_gemv8_dot2<WT, MT, 1, 4, 16, 1, false, SCALED>(a);
 }
 
 template <int WT, bool SCALED>
@@ -84,8 +90,7 @@ template <int WT, bool SCALED>
 bool gemv8_mfma(const LinearArgs& a)
 {
     const int cus = cu_count();
-    if (a.n_out >= cus * 64 * 4) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
-    else if (a.n_out >= cus * 32 * 2) { gemv8_mfma_kernel<WT, 2, 2, 4, SCALED><<<(a.n_out + 31) / 32, 256, 0, stream()>>>(a); }
+    if (a.n_out >= cus * 32) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
     else { gemv8_mfma_kernel<WT, 1, 2, 8, SCALED><<<(a.n_out + 15) / 16, 512, 0, stream()>>>(a); }
     return true;
 }

@@ -190,6 +190,129 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs
 }
 
 // ------------------------------------------------------------------------------------------
+// FP8 GEMV, dot2 + DPP reduction, software pipelined.  Same decomposition as gemv8_dot2_kernel, but
+// the (row group, k trip) pairs a wave walks are flattened into one sequence and the 128-bit loads
+// of the next pair are issued before the current pair is multiplied, so every wave always has
+// U * R KiB in flight -- including across the activation staging barrier at kernel start.
+//   NT      non-temporal weight loads
+
+template <bool NT>
+__device__ __forceinline__ u32x4 load_w128(const uint8_t* p)
+{
+    return NT ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+}
+
+template <int WT, int MT, int R, int U, int WAVES, bool SCALED, bool NT>
+__global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_pipe_kernel(const LinearArgs a)
+{
+    extern __shared__ u32x4 xs[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_steps = (a.K + 1023) / 1024;
+    const int trips = (n_steps + U - 1) / U;
+    const int n_groups = (a.n_out + R - 1) / R;
+    const int last_row = a.n_out - 1;
+    const int g0 = blockIdx.x * WAVES + wave;
+    const int g_stride = gridDim.x * WAVES;
+    const int my_groups = g0 < n_groups ? (n_groups - g0 + g_stride - 1) / g_stride : 0;
+    const int total = my_groups * trips;
+
+    auto issue = [&](int it, u32x4 (&w)[U][R]) {
+        const int gi = it / trips;
+        const int s0 = (it - gi * trips) * U;
+        const int g = g0 + gi * g_stride;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+        {
+            const int row = min(g * R + r, last_row);
+            const uint8_t* base = a.W + (long long)row * a.ldw + lane * 16;
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                const int k = (s0 + u) * 1024 + lane * 16;
+                w[u][r] = u32x4{ 0u, 0u, 0u, 0u };
+                if (k < a.K) { w[u][r] = load_w128<NT>(base + (s0 + u) * 1024); }
+            }
+        }
+    };
+
+    float acc[R][MT];
+    auto compute = [&](int it, const u32x4 (&w)[U][R]) {
+        const int gi = it / trips;
+        const int trip = it - gi * trips;
+        const int s0 = trip * U;
+        if (trip == 0)
+        {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < MT; t++) { acc[r][t] = 0.0f; }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            if (s0 + u < n_steps)
+            {
+                u32x4 x[MT][2];
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                {
+                    x[t][0] = xs[(((s0 + u) * MT + t) * 2 + 0) * 64 + lane];
+                    x[t][1] = xs[(((s0 + u) * MT + t) * 2 + 1) * 64 + lane];
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                {
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                    {
+                        bf16x2 p01, p23;
+                        fp8x4_to_bf16<WT, SCALED>(w[u][r][d], a.w_scale, p01, p23);
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+                        {
+                            acc[r][t] = dot2_bf16(p01, x[t][d >> 1][(d & 1) * 2 + 0], acc[r][t]);
+                            acc[r][t] = dot2_bf16(p23, x[t][d >> 1][(d & 1) * 2 + 1], acc[r][t]);
+                        }
+                    }
+                }
+            }
+        }
+        if (trip == trips - 1)
+        {
+            const int g = g0 + gi * g_stride;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+            {
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                {
+                    const float sum = wave_sum(acc[r][t]);
+                    const int row = g * R + r;
+                    if (lane == 0 && row < a.n_out)
+                    {
+                        uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)row * a.y_stride_out;
+                        *y = finish_output(sum, a.alpha, a.beta, y);
+                    }
+                }
+            }
+        }
+    };
+
+    u32x4 wa[U][R], wb[U][R];
+    if (total > 0) { issue(0, wa); }
+    stage_activations<MT, 2>(a, xs, n_steps, WAVES * 64);
+    __syncthreads();
+    for (int it = 0; it < total; it += 2)
+    {
+        if (it + 1 < total) { issue(it + 1, wb); }
+        compute(it, wa);
+        if (it + 2 < total) { issue(it + 2, wa); }
+        if (it + 1 < total) { compute(it + 1, wb); }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // FP4 block-scale GEMV, dot2 + DPP reduction.  One 128-bit load = 32 nibbles = 32 consecutive
 // elements of one row = 32 / BLOCK blocks (BLOCK = 16 or 32); the block scales of a k-step are
 // 64 * 32 / BLOCK consecutive bytes of the scale array.

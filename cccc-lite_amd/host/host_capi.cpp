@@ -1,0 +1,151 @@
+// Plain-C window onto the host mirror so that tests and the benchmark (Python, ctypes) drive the
+// same Matrix::mulBatched path a cccc graph would, plus a timing loop that runs a chain of linears
+// from native code (Python call overhead would otherwise dominate microsecond kernels).
+#include "Matrix.h"
+#include "../../include/cccc_hip_quant.h"
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <vector>
+
+using namespace cccc;
+
+extern "C" {
+
+int cccc_host_init(int device) { return GpuControl::select(device) ? 0 : 1; }
+
+void* cccc_matrix_create(int w, int h, int c, int n, int dtype)
+{
+    if (!GpuControl::getCurrentGpu()) { GpuControl::select(0); }
+    return new Matrix(w, h, c, n, (DataType)dtype);
+}
+
+void cccc_matrix_destroy(void* m) { delete (Matrix*)m; }
+
+void* cccc_matrix_data(void* m) { return ((Matrix*)m)->data(); }
+
+int cccc_matrix_upload(void* m, const void* host, size_t bytes) { return ((Matrix*)m)->copyFromHost(host, bytes); }
+
+int cccc_matrix_download(void* m, void* host, size_t bytes) { return ((Matrix*)m)->copyToHost(host, bytes); }
+
+int cccc_matrix_load_quantized(void* m, const void* host, long long n_bytes, float scale, int dtype)
+{
+    ((Matrix*)m)->loadQuantizedDirect((const uint8_t*)host, n_bytes, scale, (DataType)dtype);
+    return 0;
+}
+
+int cccc_matrix_set_block_scale(void* m, const void* host, long long n_scales)
+{
+    ((Matrix*)m)->setBlockScaleFromHost(host, n_scales);
+    return ((Matrix*)m)->getBlockScaleData() ? 0 : 1;
+}
+
+int cccc_matrix_quantize(void* m, int dtype)
+{
+    ((Matrix*)m)->quantizeWeights((DataType)dtype);
+    return 0;
+}
+
+int cccc_matrix_dtype(void* m) { return (int)((Matrix*)m)->getDataType(); }
+
+float cccc_matrix_quant_scale(void* m) { return ((Matrix*)m)->getQuantScale(); }
+
+const void* cccc_matrix_block_scale_data(void* m) { return ((Matrix*)m)->getBlockScaleData(); }
+
+long long cccc_matrix_get_block_scale(void* m, void* host, long long capacity)
+{
+    Matrix* mat = (Matrix*)m;
+    if (!mat->getBlockScaleData()) { return 0; }
+    const long long count = mat->getBlockScaleCount();
+    if (count > capacity) { return -count; }
+    mat->getBlockScaleToHost(host);
+    return count;
+}
+
+int cccc_matrix_mul(void* A, void* B, void* R, float a, float r, int ta, int tb)
+{
+    return Matrix::mul(*(Matrix*)A, *(Matrix*)B, *(Matrix*)R, a, r, (MatrixTransType)ta, (MatrixTransType)tb);
+}
+
+int cccc_matrix_mul_batched(void* A, void* B, void* R, int ta, int tb, float a, float r)
+{
+    return Matrix::mulBatched(*(Matrix*)A, *(Matrix*)B, *(Matrix*)R, (MatrixTransType)ta, (MatrixTransType)tb, a, r);
+}
+
+unsigned long long cccc_gpu_allocated_bytes(void)
+{
+    GpuControl* g = GpuControl::getCurrentGpu();
+    return g ? (unsigned long long)g->allocatedBytes() : 0ull;
+}
+
+// Runs `steps` timed passes over a chain of n_ops linears  R[i] = W[i]^T X[i]  (Matrix::mulBatched
+// with TRANS / NO_TRANS, as the LLM graph calls it) after `warmup` untimed passes.  use_graph != 0
+// replays one captured hipGraph per pass instead of issuing the launches one by one.  Events are
+// recorded on the stream the kernels run on.  Returns elapsed milliseconds for all timed passes, or
+// a negative value on error.
+double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int steps, int warmup, int use_graph)
+{
+    auto one_pass = [&]() -> int {
+        int status = 0;
+        for (int i = 0; i < n_ops; i++)
+        {
+            const int rc = Matrix::mulBatched(*(Matrix*)W[i], *(Matrix*)X[i], *(Matrix*)R[i], MATRIX_TRANS, MATRIX_NO_TRANS, 1.0f, 0.0f);
+            if (rc != 0) { status = rc; }
+        }
+        return status;
+    };
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    double result = -1.0;
+    hip_quant_set_sync(0);
+    for (int i = 0; i < warmup; i++) { if (one_pass() != 0) { return -2.0; } }
+    if (hipDeviceSynchronize() != hipSuccess) { return -3.0; }
+    if (use_graph)
+    {
+        if (hipStreamCreate(&stream) != hipSuccess) { return -4.0; }
+        hip_quant_set_stream(stream);
+        bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) == hipSuccess;
+        if (ok) { ok = one_pass() == 0; }
+        ok = (hipStreamEndCapture(stream, &graph) == hipSuccess) && ok;
+        hip_quant_set_stream(nullptr);
+        if (ok) { ok = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess; }
+        if (ok) { ok = hipGraphLaunch(exec, stream) == hipSuccess && hipStreamSynchronize(stream) == hipSuccess; }
+        if (ok)
+        {
+            (void)hipEventRecord(e0, stream);
+            for (int s = 0; s < steps; s++) { (void)hipGraphLaunch(exec, stream); }
+            (void)hipEventRecord(e1, stream);
+            ok = hipEventSynchronize(e1) == hipSuccess;
+        }
+        if (ok)
+        {
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            result = ms;
+        }
+        if (exec) { (void)hipGraphExecDestroy(exec); }
+        if (graph) { (void)hipGraphDestroy(graph); }
+        (void)hipStreamDestroy(stream);
+    }
+    else
+    {
+        (void)hipEventRecord(e0, nullptr);
+        bool ok = true;
+        for (int s = 0; s < steps; s++) { ok = (one_pass() == 0) && ok; }
+        (void)hipEventRecord(e1, nullptr);
+        ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
+        if (ok)
+        {
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            result = ms;
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return result;
+}
+
+}    // extern "C"

@@ -67,6 +67,13 @@ C_EXPORT int hip_float_to_fp4_blockscale(const void* src, void* dst_nibbles, voi
                                          unsigned int n_elems, unsigned int block_size);
 
 /*
+ * Largest |x| of `n` elements (float, half or bf16) written as one float to device memory at
+ * `d_result`.  Stands in for the cuBLAS iamax + 4-byte copy that Matrix::quantizeWeights uses to
+ * derive the per-tensor FP8 scale (cccc/Matrix.cpp:338-343).  NaNs are ignored.
+ */
+C_EXPORT int hip_absmax(const void* src, int src_type, unsigned int n, void* d_result);
+
+/*
  * Unified quantized GEMM, column-major:  C[M x N] = alpha * op(A)[M x K] * op(B)[K x N] + beta * C.
  * Carries the arguments of the reference's unified dispatcher Cublas::gemm
  * (cccc/cublas_real.h:875-880) plus the FP4 block size that the reference hard-codes as 16
