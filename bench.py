@@ -164,7 +164,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode_linears", choices=["decode_linears", "gemv", "prefill"])
+    ap.add_argument("--workload", default="decode_linears", choices=["decode_linears", "gemv", "prefill", "copy"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--no-graph", action="store_true")
@@ -181,6 +181,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "copy":
+        # counter calibration: a plain device copy kernel of known size (reads and writes 256 MiB per launch)
+        n = 256 << 20
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launches": args.steps}))
+        return
     ws = Workspace(pkg, torch)
     use_graph = not args.no_graph
     extra = {}
