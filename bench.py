@@ -29,6 +29,9 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+# HBM bytes per launch of the gate/up-shaped GEMV (K=4096, N=12288, M=1) from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99983 and 1.0)
+GEMV_GATE_UP_TRAFFIC_BYTES = 50503552
 
 FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
 
@@ -243,7 +246,8 @@ def main():
     else:
         achieved = gemv_bytes(K, N, M) / dom_us * 1e-3
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    "traffic": GEMV_GATE_UP_TRAFFIC_BYTES if (K, N, M) == (4096, 12288, 1) else None,
                     "kernel": "gemv8_dot2_kernel", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
                     "bytes_per_launch": gemv_bytes(K, N, M)}
 
