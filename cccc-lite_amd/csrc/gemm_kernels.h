@@ -4,10 +4,12 @@
 // (cccc/cublas_real.h:943-964): the weight value entering a product is bf16(decode(w) * scale).
 //
 // Tiling: a 256-thread workgroup (4 waves, 2 x 2) owns BM output features x BN tokens and walks K
-// in steps of 64.  LDS holds one X tile [BN][64] and one dequantised W tile [BM][64], rows of 128
-// bytes whose 16-byte chunks are XOR-swizzled with (row / 2) % 8 so that the 128-bit fragment
-// reads of 16 consecutive rows hit 16 distinct bank groups.  The next k-tile is fetched from
-// global memory into registers while the current one is multiplied.
+// in steps of BK (64 or 128).  LDS holds one X tile [BN][BK] and one dequantised W tile [BM][BK];
+// the 16-byte chunks of a row are XOR-swizzled so that the 128-bit fragment reads of 16 consecutive
+// rows hit 16 distinct bank groups.  The next k-tile is fetched from global memory into registers
+// while the current one is multiplied.  With XCD = true, workgroup ids that are congruent mod 8
+// (they land on the same XCD) walk the token tiles of one weight tile, so a weight tile is pulled
+// from HBM once per XCD and shared through that XCD's L2.
 //   A operand (rows)    = tokens,          lane (r = lane % 32, h = lane / 32) holds k = 8 h .. 8 h + 7
 //   B operand (columns) = output features, same k split
 //   D: lane holds column lane % 32; register v is row 8 (v / 4) + 4 (lane / 32) + v % 4
@@ -19,7 +21,10 @@
 namespace ccq
 {
 
-__device__ __forceinline__ int swizzled_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+// LDS rows of CPR 16-byte chunks: 8 chunks (128-byte rows, two rows per 256-byte bank sweep) or
+// 16 chunks (256-byte rows, every row starts at bank 0)
+template <int CPR>
+__device__ __forceinline__ int swizzled_chunk_n(int row, int chunk) { return CPR == 16 ? (chunk ^ (row & 15)) : (chunk ^ ((row >> 1) & 7)); }
 
 // 16 FP8 codes -> 16 BF16 (two 16-byte LDS chunks)
 template <int WT, bool SCALED>
@@ -89,10 +94,9 @@ __device__ __forceinline__ u32x4 dequant8_fp4(uint32_t w, float scale)
 
 // WT: DT_E5M2 / DT_E4M3 / DT_FP4.  BLOCK: FP4 block length (16 / 32), unused for FP8.
 // Requires K % 16 == 0 (FP8) or K % 32 == 0 (FP4), and the alignment rules of the GEMV kernels.
-template <int WT, int BLOCK, int BM, int BN, bool SCALED>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
+template <int WT, int BLOCK, int BM, int BN, bool SCALED, int BK = 64, bool XCD = false>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, const int n_tiles, const int m_tiles)
 {
-    constexpr int BK = 64;
     constexpr int WM = BM / 2;          // output features per wave
     constexpr int WN = BN / 2;          // tokens per wave
     constexpr int TM = WM / 32;         // MFMA tiles along output features
@@ -101,18 +105,33 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
     constexpr int W_CHUNK_K = FP4 ? 32 : 16;                // elements per 16-byte global chunk
     constexpr int W_CHUNKS = BM * (BK / W_CHUNK_K);         // per k-tile
     constexpr int W_PER_THREAD = (W_CHUNKS + 255) / 256;
-    constexpr int X_PER_THREAD = BN * 8 / 256;
+    constexpr int X_PER_THREAD = BN * (BK / 8) / 256;
 
-    __shared__ u32x4 xs[BN * 8];
-    __shared__ u32x4 ws[BM * 8];
+    constexpr int CPR = BK / 8;                              // 16-byte BF16 chunks per LDS row
+    __shared__ u32x4 xs[BN * CPR];
+    __shared__ u32x4 ws[BM * CPR];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wave_m = wave & 1;
     const int wave_n = wave >> 1;
-    const int out_base = blockIdx.x * BM;
-    const int tok_base = blockIdx.y * BN;
+    int n_tile, m_tile;
+    if (XCD)
+    {
+        // workgroups whose ids are congruent mod 8 share an XCD: let them walk the token tiles of one weight tile
+        const int seq = blockIdx.x >> 3;
+        n_tile = (blockIdx.x & 7) + 8 * (seq / m_tiles);
+        m_tile = seq % m_tiles;
+        if (n_tile >= n_tiles) { return; }
+    }
+    else
+    {
+        n_tile = blockIdx.x % n_tiles;
+        m_tile = blockIdx.x / n_tiles;
+    }
+    const int out_base = n_tile * BM;
+    const int tok_base = m_tile * BN;
 
     f32x16 acc[TN][TM];
 #pragma unroll
@@ -152,8 +171,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
         for (int i = 0; i < X_PER_THREAD; i++)
         {
             const int q = tid + i * 256;
-            const int row_in_tile = q >> 3;
-            const int chunk = q & 7;
+            const int row_in_tile = q / CPR;
+            const int chunk = q % CPR;
             const int k = k0 + chunk * 8;
             xreg[i] = u32x4{ 0u, 0u, 0u, 0u };
             if (k < a.K)
@@ -180,15 +199,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
 #pragma unroll
                     for (int d = 0; d < 4; d++)
                     {
-                        ws[row * 8 + swizzled_chunk(row, part * 4 + d)] = dequant8_fp4(wreg[i][d], d < 2 ? s0 : s1);
+                        ws[row * CPR + swizzled_chunk_n<CPR>(row, part * 4 + d)] = dequant8_fp4(wreg[i][d], d < 2 ? s0 : s1);
                     }
                 }
                 else
                 {
                     u32x4 lo, hi;
                     dequant16_fp8<WT, SCALED>(wreg[i], a.w_scale, lo, hi);
-                    ws[row * 8 + swizzled_chunk(row, part * 2)] = lo;
-                    ws[row * 8 + swizzled_chunk(row, part * 2 + 1)] = hi;
+                    ws[row * CPR + swizzled_chunk_n<CPR>(row, part * 2)] = lo;
+                    ws[row * CPR + swizzled_chunk_n<CPR>(row, part * 2 + 1)] = hi;
                 }
             }
         }
@@ -196,8 +215,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
         for (int i = 0; i < X_PER_THREAD; i++)
         {
             const int q = tid + i * 256;
-            const int row = q >> 3;
-            xs[row * 8 + swizzled_chunk(row, q & 7)] = xreg[i];
+            const int row = q / CPR;
+            xs[row * CPR + swizzled_chunk_n<CPR>(row, q % CPR)] = xreg[i];
         }
     };
 
@@ -218,13 +237,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
             for (int tn = 0; tn < TN; tn++)
             {
                 const int row = wave_n * WN + tn * 32 + r32;
-                xf[tn] = __builtin_bit_cast(bf16x8, xs[row * 8 + swizzled_chunk(row, ks * 2 + h)]);
+                xf[tn] = __builtin_bit_cast(bf16x8, xs[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
             }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
             {
                 const int row = wave_m * WM + tm * 32 + r32;
-                wf[tm] = __builtin_bit_cast(bf16x8, ws[row * 8 + swizzled_chunk(row, ks * 2 + h)]);
+                wf[tm] = __builtin_bit_cast(bf16x8, ws[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
             }
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
@@ -255,20 +274,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a)
     }
 }
 
-template <int WT, int BLOCK, int BM, int BN>
+template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false>
 void launch_gemm_mfma(const LinearArgs& a)
 {
-    const dim3 grid((a.n_out + BM - 1) / BM, (a.tokens + BN - 1) / BN);
-    if (WT != DT_FP4 && a.w_scale != 1.0f) { gemm_mfma_kernel<WT, BLOCK, BM, BN, true><<<grid, 256, 0, stream()>>>(a); }
-    else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false><<<grid, 256, 0, stream()>>>(a); }
+    const int n_tiles = (a.n_out + BM - 1) / BM;
+    const int m_tiles = (a.tokens + BN - 1) / BN;
+    const int grid = XCD ? 8 * m_tiles * ((n_tiles + 7) / 8) : n_tiles * m_tiles;
+    if (WT != DT_FP4 && a.w_scale != 1.0f) { gemm_mfma_kernel<WT, BLOCK, BM, BN, true, BK, XCD><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+    else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false, BK, XCD><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
 }
 
+// Tile choice (tuned on MI355X): 128 x 128 tiles with the XCD-aware order when they give every CU at
+// least two workgroups (k step 128 for long K, where it halves the barriers per FLOP), otherwise
+// 128 x 64 tiles to put more workgroups on the machine.
 template <int WT, int BLOCK>
 bool gemm_mfma(const LinearArgs& a)
 {
     const long long tiles_big = (long long)((a.n_out + 127) / 128) * ((a.tokens + 127) / 128);
-    if (tiles_big >= 2LL * cu_count()) { launch_gemm_mfma<WT, BLOCK, 128, 128>(a); }
-    else { launch_gemm_mfma<WT, BLOCK, 128, 64>(a); }
+    if (tiles_big >= 2LL * cu_count())
+    {
+        if (a.K >= 8192) { launch_gemm_mfma<WT, BLOCK, 128, 128, 128, true>(a); }
+        else { launch_gemm_mfma<WT, BLOCK, 128, 128, 64, true>(a); }
+    }
+    else { launch_gemm_mfma<WT, BLOCK, 128, 64, 64, false>(a); }
     return true;
 }
 
