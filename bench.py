@@ -54,6 +54,7 @@ class Workspace:
         self.dev = torch.device("cuda:0")
         self.gen = torch.Generator(device=self.dev).manual_seed(1234)
         self.keep = []
+        self.repack = False
 
     def weight_e5m2(self, n_out, K):
         t = self.torch
@@ -64,6 +65,8 @@ class Workspace:
             w = (t.randn(r, K, device=self.dev, generator=self.gen) * 0.02).to(t.bfloat16).to(t.float8_e5m2)
             assert self.lib.convert(w.data_ptr(), E5M2, m.data_ptr + r0 * K, E5M2, r * K, 1.0) == 0
             t.cuda.synchronize()
+        if self.repack:
+            m.prepare_tiled()        # what Matrix::loadQuantizedDirect does after uploading file bytes
         return m
 
     def activation(self, tokens, K):
@@ -173,6 +176,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
@@ -195,6 +199,7 @@ def main():
         print(json.dumps({"workload": "copy", "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launches": args.steps}))
         return
     ws = Workspace(pkg, torch)
+    ws.repack = not args.no_repack
     use_graph = not args.no_graph
     extra = {}
 

@@ -26,6 +26,9 @@ EXPORTS = (
     "hip_float_to_fp4_blockscale",
     "hip_absmax",
     "hip_quant_gemm",
+    "hip_quant_tiled_size",
+    "hip_quant_weight_prepare",
+    "hip_quant_weight_release",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
     "hip_quant_last_kernel",
@@ -63,6 +66,12 @@ class QuantLibrary:
                                      vp, i32, i32, f32,
                                      f32, vp, i32, i32, f32,
                                      vp, vp, u32]
+        L.hip_quant_tiled_size.restype = ctypes.c_ulonglong
+        L.hip_quant_tiled_size.argtypes = [i32, i32, i32]
+        L.hip_quant_weight_prepare.restype = i32
+        L.hip_quant_weight_prepare.argtypes = [vp, i32, i32, i32, i32, vp]
+        L.hip_quant_weight_release.restype = i32
+        L.hip_quant_weight_release.argtypes = [vp]
         L.hip_quant_set_sync.restype = i32
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32
@@ -90,6 +99,15 @@ class QuantLibrary:
         return self.c.hip_quant_gemm(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
                                      B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale,
                                      blk_scA, blk_scB, block_size)
+
+    def tiled_size(self, w_type, n_out, K) -> int:
+        return int(self.c.hip_quant_tiled_size(w_type, n_out, K))
+
+    def weight_prepare(self, W, w_type, n_out, K, ldw, dst_tiled) -> int:
+        return self.c.hip_quant_weight_prepare(W, w_type, n_out, K, ldw, dst_tiled)
+
+    def weight_release(self, W) -> int:
+        return self.c.hip_quant_weight_release(W)
 
     def set_sync(self, enabled: bool) -> int:
         return self.c.hip_quant_set_sync(1 if enabled else 0)

@@ -11,6 +11,10 @@
 #include "gemm_kernels.h"
 #include "runtime.h"
 #include <cstdio>
+#include <mutex>
+#include <shared_mutex>
+#include <unordered_map>
+#include <unordered_set>
 
 using namespace ccq;
 
@@ -22,20 +26,22 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 constexpr int kMaxLds = 160 * 1024;
 
-// Raises a kernel's dynamic LDS limit once; returns false if the runtime refuses.
+// Raises a kernel's dynamic LDS limit the first time it is needed; returns false if the runtime refuses.
 template <typename Kernel>
 bool allow_big_lds(Kernel kernel, size_t bytes)
 {
     if (bytes <= 64 * 1024) { return true; }
     if (bytes > (size_t)kMaxLds) { return false; }
-    static thread_local Kernel done_for = nullptr;
-    if (done_for == kernel) { return true; }
+    static std::mutex mutex;
+    static std::unordered_set<const void*> raised;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (raised.count((const void*)kernel)) { return true; }
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds) != hipSuccess)
     {
         (void)hipGetLastError();
         return false;
     }
-    done_for = kernel;
+    raised.insert((const void*)kernel);
     return true;
 }
 
@@ -93,6 +99,67 @@ bool gemv8_mfma(const LinearArgs& a)
     if (a.n_out >= cus * 32) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
     else { gemv8_mfma_kernel<WT, 1, 2, 8, SCALED><<<(a.n_out + 15) / 16, 512, 0, stream()>>>(a); }
     return true;
+}
+
+// ---- load-time repacked weights: caller's weight pointer -> tiled copy
+struct TiledWeight
+{
+    const uint8_t* tiled;
+    int type, n_out, K;
+    long long ldw;
+};
+std::shared_mutex g_tiled_mutex;
+std::unordered_map<const void*, TiledWeight> g_tiled;
+
+const uint8_t* find_tiled(const LinearArgs& a, int type)
+{
+    std::shared_lock<std::shared_mutex> lock(g_tiled_mutex);
+    if (g_tiled.empty()) { return nullptr; }
+    const auto it = g_tiled.find(a.W);
+    if (it == g_tiled.end()) { return nullptr; }
+    const TiledWeight& t = it->second;
+    return (t.type == type && t.n_out == a.n_out && t.K == a.K && t.ldw == a.ldw) ? t.tiled : nullptr;
+}
+
+// Matrix-core GEMV with the activations in LDS.  S (waves per row tile) is picked from how many tiles
+// a CU gets.  Returns false when the activations (tokens x K) do not fit 128 KiB of LDS: the caller
+// falls back.
+template <int WT, int TP, int S, bool SCALED, bool TILED>
+bool launch_gemv8_mfma_lds(const LinearArgs& a)
+{
+    auto kernel = gemv8_mfma_lds_kernel<WT, TP, S, 8, SCALED, TILED>;
+    const int per_block = 128 * TP;
+    const int max_blocks = (128 * 1024) / per_block;
+    const int k_blocks = (a.K + 63) / 64;
+    const int kc_blocks = k_blocks < max_blocks ? ((k_blocks + S - 1) / S) * S : (max_blocks / S) * S;
+    const size_t lds = (size_t)kc_blocks * per_block + 8192;
+    const int n_tiles = (a.n_out + 15) / 16;
+    const int groups = 8 / S;
+    const int want = (n_tiles + groups - 1) / groups;
+    const int cap = cu_count();
+    const int grid = want < cap ? want : cap;
+    if (kc_blocks < k_blocks) { return false; }    // K does not fit one LDS chunk: leave it to the row-major kernels
+    if (!allow_big_lds(kernel, lds)) { return false; }
+    kernel<<<grid, 512, lds, stream()>>>(a, kc_blocks * 64);
+    return true;
+}
+
+template <int WT, int TP, bool SCALED, bool TILED>
+bool pick_gemv8_mfma_lds(const LinearArgs& a)
+{
+    const int tiles_per_cu = ((a.n_out + 15) / 16) / cu_count();
+    if (tiles_per_cu >= 16) { return launch_gemv8_mfma_lds<WT, TP, 1, SCALED, TILED>(a); }
+    return launch_gemv8_mfma_lds<WT, TP, 8, SCALED, TILED>(a);
+}
+
+template <int WT, bool SCALED>
+bool gemv8_mfma_tiled(const LinearArgs& a, const uint8_t* tiled)
+{
+    LinearArgs t = a;
+    t.W = tiled;
+    if (a.tokens <= 4) { return pick_gemv8_mfma_lds<WT, 4, SCALED, true>(t); }
+    if (a.tokens <= 8) { return pick_gemv8_mfma_lds<WT, 8, SCALED, true>(t); }
+    return pick_gemv8_mfma_lds<WT, 16, SCALED, true>(t);
 }
 
 template <int MT, int BLOCK>
@@ -247,7 +314,19 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         {
             const bool ok = x_ok && K % 16 == 0 && a.ldw % 16 == 0 && aligned16(a.W);
             const bool scaled = a.w_scale != 1.0f;
-            if (ok && a.tokens <= 4)
+            // Measured on MI355X: the tiled matrix-core kernel wins for 5..16 tokens on tall weights (lm_head: 5.0 TB/s
+            // against 3.6); up to 4 tokens the dot2 family is faster everywhere, and on weights with only a few row
+            // tiles per CU the 128 KiB activation staging per workgroup costs more than the contiguous loads gain.
+            if (ok && a.tokens >= 5 && a.tokens <= 16 && ((a.n_out + 15) / 16) / cu_count() >= 16)
+            {
+                if (const uint8_t* tiled = find_tiled(a, g.w_type))
+                {
+                    if (g.w_type == DT_E5M2) { launched = scaled ? gemv8_mfma_tiled<DT_E5M2, true>(a, tiled) : gemv8_mfma_tiled<DT_E5M2, false>(a, tiled); }
+                    else { launched = scaled ? gemv8_mfma_tiled<DT_E4M3, true>(a, tiled) : gemv8_mfma_tiled<DT_E4M3, false>(a, tiled); }
+                    if (launched) { note_kernel("gemv_mfma_tiled"); }
+                }
+            }
+            if (ok && !launched && a.tokens <= 4)
             {
                 if (g.w_type == DT_E5M2) { launched = scaled ? gemv8_dot2<DT_E5M2, true>(a) : gemv8_dot2<DT_E5M2, false>(a); }
                 else { launched = scaled ? gemv8_dot2<DT_E4M3, true>(a) : gemv8_dot2<DT_E4M3, false>(a); }
@@ -273,4 +352,33 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         note_kernel("generic");
     }
     return finish("quant_gemm");
+}
+
+unsigned long long hip_quant_tiled_size(int type, int n_out, int K)
+{
+    if ((type != DT_E4M3 && type != DT_E5M2) || n_out <= 0 || K <= 0) { return 0ull; }
+    return (unsigned long long)((n_out + 15) / 16) * (unsigned long long)((K + 63) / 64) * 1024ull;
+}
+
+int hip_quant_weight_prepare(const void* W, int type, int n_out, int K, int ldw, void* dst_tiled)
+{
+    if ((type != DT_E4M3 && type != DT_E5M2) || !W || !dst_tiled || n_out <= 0 || K <= 0) { return -1; }
+    if (K % 16 != 0 || ldw % 16 != 0 || ldw < K || !aligned16(W) || !aligned16(dst_tiled)) { return -1; }
+    const long long n_chunks = (long long)((n_out + 15) / 16) * ((K + 63) / 64) * 64;
+    long long blocks = (n_chunks + 255) / 256;
+    const long long cap = (long long)cu_count() * 16;
+    if (blocks > cap) { blocks = cap; }
+    repack_tiled_kernel<<<(unsigned)blocks, 256, 0, stream()>>>((const uint8_t*)W, (uint8_t*)dst_tiled, n_out, K, ldw);
+    const int rc = finish("weight_prepare");
+    if (rc != 0) { return rc; }
+    std::unique_lock<std::shared_mutex> lock(g_tiled_mutex);
+    g_tiled[W] = TiledWeight{ (const uint8_t*)dst_tiled, type, n_out, K, (long long)ldw };
+    return 0;
+}
+
+int hip_quant_weight_release(const void* W)
+{
+    std::unique_lock<std::shared_mutex> lock(g_tiled_mutex);
+    g_tiled.erase(W);
+    return 0;
 }

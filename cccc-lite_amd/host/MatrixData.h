@@ -20,6 +20,10 @@ struct MatrixData
     int64_t block_scale_count_ = 0;
     static constexpr unsigned int fp4_block_size_ = 16;
     float input_scale_ = 0.0f;
+    // Load-time repacked (tiled) copy of an FP8 weight for the matrix-core GEMV; owned here, registered
+    // with the kernel library under the key data_.  No counterpart in the reference.
+    void* tiled_data_ = nullptr;
+    static inline bool repack_weights = true;
 
     MatrixData() = default;
     ~MatrixData() { release(); }
@@ -34,6 +38,10 @@ struct MatrixData
     // (Re)allocates when the byte size grows or `force` is set; contents are not kept.
     void* resize(int64_t size, DataType data_type, bool force = false);
     void release();
+
+    // Builds / drops the tiled copy for a [n_out][K] FP8 weight stored in data_.
+    void prepareTiled(int n_out, int K);
+    void releaseTiled();
 
     void setBlockScaleFromHost(const void* src, int64_t n_scales);
     void getBlockScaleToHost(void* dst) const;

@@ -106,6 +106,7 @@ int Rocblas::gemm(MatrixTransType TransA, MatrixTransType TransB, int M, int N, 
 
 void* MatrixData::resize(int64_t size, DataType data_type, bool force)
 {
+    releaseTiled();
     const size_t want = (size_t)size * getDataTypeSize(data_type);
     if (force || want > sizeInByte() || !data_)
     {
@@ -118,8 +119,33 @@ void* MatrixData::resize(int64_t size, DataType data_type, bool force)
     return data_;
 }
 
+void MatrixData::prepareTiled(int n_out, int K)
+{
+    releaseTiled();
+    if (!repack_weights || !gpu_ || !data_ || (data_type_ != FP8_E4M3 && data_type_ != FP8_E5M2)) { return; }
+    const unsigned long long bytes = hip_quant_tiled_size((int)data_type_, n_out, K);
+    if (bytes == 0 || gpu_->malloc(&tiled_data_, (size_t)bytes) != 0) { tiled_data_ = nullptr; return; }
+    if (hip_quant_weight_prepare(data_, (int)data_type_, n_out, K, K, tiled_data_) != 0)
+    {
+        gpu_->free(tiled_data_);
+        tiled_data_ = nullptr;
+    }
+}
+
+void MatrixData::releaseTiled()
+{
+    if (tiled_data_)
+    {
+        hip_quant_weight_release(data_);
+        (void)hipDeviceSynchronize();
+        if (gpu_) { gpu_->free(tiled_data_); }
+        tiled_data_ = nullptr;
+    }
+}
+
 void MatrixData::release()
 {
+    releaseTiled();
     if (gpu_)
     {
         if (data_) { gpu_->free(data_); }
@@ -203,6 +229,8 @@ void Matrix::loadQuantizedDirect(const uint8_t* host_data, int64_t n, float scal
     GpuControl::copyHostToDevice(shared_data_->data_, host_data, (size_t)n);
     shared_data_->quant_scale_ = scale;
     data_ = shared_data_->data_;
+    // a [K x n_out] linear weight (one batch): keep an MI355X-friendly tiled copy next to the file bytes
+    if (number_ == 1 && channel_ == 1 && (int64_t)width_ * height_ == n) { shared_data_->prepareTiled(height_, width_); }
 }
 
 void Matrix::quantizeWeights(DataType target_dt)
@@ -244,6 +272,7 @@ void Matrix::quantizeWeights(DataType target_dt)
     }
     (void)hipDeviceSynchronize();    // float_buf is freed on return
     data_ = shared_data_->data_;
+    if (target_dt != FP4_E2M1 && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); }
 }
 
 // The operand extents a column-major GEMM will touch, checked against what the tensors hold before

@@ -45,6 +45,17 @@ int cccc_matrix_quantize(void* m, int dtype)
     return 0;
 }
 
+// 0 / 1: build tiled copies of FP8 linear weights when they are loaded or quantized (default 1)
+void cccc_host_set_repack(int enabled) { MatrixData::repack_weights = enabled != 0; }
+
+// (re)builds the tiled copy of an FP8 weight matrix whose bytes were written straight into its storage
+int cccc_matrix_prepare_tiled(void* m)
+{
+    Matrix* mat = (Matrix*)m;
+    mat->prepareTiled();
+    return mat->hasTiled() ? 0 : 1;
+}
+
 int cccc_matrix_dtype(void* m) { return (int)((Matrix*)m)->getDataType(); }
 
 float cccc_matrix_quant_scale(void* m) { return ((Matrix*)m)->getQuantScale(); }

@@ -28,6 +28,8 @@ class HostLibrary:
         L.cccc_matrix_load_quantized.restype = i32; L.cccc_matrix_load_quantized.argtypes = [vp, vp, i64, f32, i32]
         L.cccc_matrix_set_block_scale.restype = i32; L.cccc_matrix_set_block_scale.argtypes = [vp, vp, i64]
         L.cccc_matrix_quantize.restype = i32; L.cccc_matrix_quantize.argtypes = [vp, i32]
+        L.cccc_host_set_repack.restype = None; L.cccc_host_set_repack.argtypes = [i32]
+        L.cccc_matrix_prepare_tiled.restype = i32; L.cccc_matrix_prepare_tiled.argtypes = [vp]
         L.cccc_matrix_dtype.restype = i32; L.cccc_matrix_dtype.argtypes = [vp]
         L.cccc_matrix_quant_scale.restype = f32; L.cccc_matrix_quant_scale.argtypes = [vp]
         L.cccc_matrix_block_scale_data.restype = vp; L.cccc_matrix_block_scale_data.argtypes = [vp]
@@ -42,6 +44,9 @@ class HostLibrary:
     def init(self, device: int = 0) -> None:
         if self.c.cccc_host_init(device) != 0:
             raise RuntimeError("cccc_host_init failed")
+
+    def set_repack(self, enabled: bool) -> None:
+        self.c.cccc_host_set_repack(1 if enabled else 0)
 
     def matrix(self, w, h, c, n, dtype) -> "HostMatrix":
         return HostMatrix(self, self.c.cccc_matrix_create(w, h, c, n, dtype))
@@ -100,6 +105,9 @@ class HostMatrix:
         if n > 0:
             assert self.lib.c.cccc_matrix_get_block_scale(self.handle, out.ctypes.data, n) == n
         return out
+
+    def prepare_tiled(self) -> bool:
+        return self.lib.c.cccc_matrix_prepare_tiled(self.handle) == 0
 
     def quantize(self, dtype: int) -> None:
         self.lib.c.cccc_matrix_quantize(self.handle, dtype)

@@ -94,6 +94,21 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
                             const void* blk_scA, const void* blk_scB, unsigned int block_size);
 
 /*
+ * Optional load-time repack (no counterpart in the reference; the on-disk format and the caller's
+ * weight buffer are left untouched).  hip_quant_weight_prepare writes an MI355X-friendly tiled copy
+ * of an FP8 weight W ([n_out][ldw], K contiguous, as loadQuantizedDirect uploads it) into `dst_tiled`
+ * -- caller-owned device memory of hip_quant_tiled_size(...) bytes -- and remembers it under the key
+ * `W`.  Later hip_quant_gemm calls whose weight pointer, type and shape match may use the tiled copy
+ * (today: 5..16 tokens on tall weights such as lm_head), where the matrix-core GEMV wants the 16 rows x
+ * 64 codes of one load to be contiguous.
+ * Results are identical with and without it.  hip_quant_weight_release forgets the key (before the
+ * caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (FP4, K % 16 != 0, ...).
+ */
+C_EXPORT unsigned long long hip_quant_tiled_size(int type, int n_out, int K);
+C_EXPORT int hip_quant_weight_prepare(const void* W, int type, int n_out, int K, int ldw, void* dst_tiled);
+C_EXPORT int hip_quant_weight_release(const void* W);
+
+/*
  * Library controls (no counterpart in the reference, which always uses the null stream and always
  * synchronises: cccc-hip/hip_functions.cpp:32-42).
  *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch (parity/debug)

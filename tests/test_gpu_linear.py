@@ -314,3 +314,75 @@ def test_full_size_prefill_gemm_sampled(gpu, pkg, oracle):
         rows = np.random.default_rng(tokens).choice(n_out, size=192, replace=False)
         want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2), X)
         check_rows(bf16_f64(oracle, y[:, rows]), want, f"gemm {tokens}x{n_out}x{K}")
+
+
+# ------------------------------------------------------------------------------------------ load-time repack
+
+def tiled_reference(W, n_out, K):
+    """NumPy construction of the tiled layout: KiB (t, b) holds at lane l = i + 16 g the 16 codes
+    W[16 t + i][64 b + 16 g ..]; rows / codes beyond the matrix are zero."""
+    n_tiles, kb = (n_out + 15) // 16, (K + 63) // 64
+    pad = np.zeros((n_tiles * 16, kb * 64), dtype=np.uint8)
+    pad[:n_out, :K] = W
+    t = pad.reshape(n_tiles, 16, kb, 4, 16)            # [t][i][b][g][16]
+    return np.ascontiguousarray(t.transpose(0, 2, 3, 1, 4)).ravel()   # [t][b][g][i][16]
+
+
+@pytest.mark.parametrize("n_out,K", [(64, 128), (100, 2064), (4096, 4096)])
+def test_weight_prepare_builds_the_tiled_layout(gpu, pkg, oracle, n_out, K):
+    torch, dev, lib = gpu
+    W = np.random.default_rng(5).integers(0, 256, size=(n_out, K), dtype=np.uint8)
+    wd = to_dev(torch, dev, W)
+    size = lib.tiled_size(oracle.E5M2, n_out, K)
+    assert size == ((n_out + 15) // 16) * ((K + 63) // 64) * 1024
+    td = torch.full((size + 64,), 0xAA, dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, K, K, td.data_ptr()) == 0
+    got = td.cpu().numpy()
+    assert np.array_equal(got[:size], tiled_reference(W, n_out, K)) and np.all(got[size:] == 0xAA)
+    assert lib.weight_release(wd.data_ptr()) == 0
+    # refused: FP4, K not a multiple of 16, null pointers
+    assert lib.tiled_size(oracle.FP4, n_out, K) == 0
+    assert lib.weight_prepare(wd.data_ptr(), oracle.FP4, n_out, K, K, td.data_ptr()) == -1
+    assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, 24, 24, td.data_ptr()) == -1
+    assert lib.weight_prepare(None, oracle.E5M2, n_out, K, K, td.data_ptr()) == -1
+
+
+@pytest.mark.parametrize("tokens", [5, 8, 9, 16])
+@pytest.mark.parametrize("n_out,K", [(65536, 512), (65530, 272), (70000, 16), (151936, 1024)])
+def test_prepared_weights_give_the_same_gemv(gpu, pkg, oracle, tokens, n_out, K):
+    torch, dev, lib = gpu
+    seed = pkg.synth.seed_for(2, 200 + n_out % 91 + tokens)
+    W = pkg.synth.weights_e5m2(seed, n_out, K)
+    X = pkg.synth.activations(seed, tokens, K)
+    wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+    y0 = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+    assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y0.data_ptr(), n_out, tokens, K) == 0
+    plain_kernel = lib.last_kernel()
+    td = torch.zeros(lib.tiled_size(oracle.E5M2, n_out, K), dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, K, K, td.data_ptr()) == 0
+    try:
+        y1 = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y1.data_ptr(), n_out, tokens, K) == 0
+        assert lib.last_kernel() == "gemv_mfma_tiled" and plain_kernel != "gemv_mfma_tiled"
+        # a scaled call and one token (dot2 family) on the same registered weight
+        y2 = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y2.data_ptr(), n_out, tokens, K, inv_scale=0.37) == 0
+        y3 = torch.zeros(4 * n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y3.data_ptr(), n_out, 4, K) == 0
+        assert lib.last_kernel() == "gemv_dot2"
+    finally:
+        assert lib.weight_release(wd.data_ptr()) == 0
+    out = from_dev(y1, np.uint16)
+    assert not out[tokens * n_out:].any()
+    want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X)
+    got = out[: tokens * n_out].reshape(tokens, n_out)
+    check_rows(bf16_f64(oracle, got), want, f"tiled {n_out}x{K} M={tokens}")
+    check_bf16_close(got, want, "tiled", slack_ulp=1.0, abs_floor=2e-5)
+    # the plain path computed the same thing (summation order may differ by an ulp)
+    plain = from_dev(y0, np.uint16).reshape(tokens, n_out)
+    assert np.abs(bf16_f64(oracle, plain) - bf16_f64(oracle, got)).max() <= 2.0 ** -7 * np.abs(want).max()
+    want_s = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K, 0.37), X)
+    check_rows(bf16_f64(oracle, from_dev(y2, np.uint16).reshape(tokens, n_out)), want_s, "tiled scaled")
+    # after release the same call goes back to the plain kernels
+    assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y0.data_ptr(), n_out, tokens, K) == 0
+    assert lib.last_kernel() == plain_kernel
