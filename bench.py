@@ -132,6 +132,38 @@ def shape_sweep(ws, by_shape, token_counts, use_graph):
     return out
 
 
+LLAMA_SHAPES = [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (4096, 128256)]     # (K, N)
+
+
+def fp4_bytes(K, N, M, block):
+    return K * N // 2 + K * N // block + 2 * M * K + 2 * M * N
+
+
+def fp4_sweep(ws):
+    """Llama-3.1-8B-shaped FP4 block-scale GEMVs at M=1, block 16 (the reference's format) and 32, weights
+    rotating over at least 512 MiB of distinct buffers."""
+    t = ws.torch
+    out = []
+    for (K, N) in LLAMA_SHAPES:
+        for block in (16, 32):
+            per = K * N // 2 + K * N // block
+            n_w = max(2, min(48, (768 << 20) // per))
+            nib = [t.randint(0, 256, (N, K // 2), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
+            sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
+            X, Y = ws.activation(1, K), ws.output(1, N)
+            iters = max(20, min(400, (4 << 30) // per))
+            ms = ws.host.bench_fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr,
+                                         N, 1, K, block, iters, 5)
+            if ms < 0:
+                raise RuntimeError(f"fp4 chain failed: {ms}")
+            us = ms * 1000.0 / iters
+            gbs = fp4_bytes(K, N, 1, block) / us * 1e-3
+            out.append({"K": K, "N": N, "M": 1, "block": block, "us": round(us, 2), "GBps": round(gbs, 1),
+                        "frac": round(gbs / HBM_PEAK_GBS, 4), "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(per * n_w / 2 ** 20)})
+            del nib, sc
+    return out
+
+
 def cpu_baseline(pkg, threads):
     """The reference CPU route on one transformer layer's seven linears at M=1 (bounded sample)."""
     import numpy as np
@@ -224,6 +256,7 @@ def main():
         dom_us = dom_ms * 1000.0 / (10 * len(dom_ops))
         if not args.no_sweep:
             extra["sweep"] = shape_sweep(ws, by_shape, (1, 4, 16), False)
+            extra["fp4_sweep"] = fp4_sweep(ws)
     else:
         K, N = (int(v) for v in args.shape.split(","))
         M = args.tokens if args.workload == "gemv" else max(args.tokens, 512)

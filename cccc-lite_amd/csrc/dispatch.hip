@@ -162,28 +162,27 @@ bool gemv8_mfma_tiled(const LinearArgs& a, const uint8_t* tiled)
     return pick_gemv8_mfma_lds<WT, 16, SCALED, true>(t);
 }
 
-template <int MT, int BLOCK>
+template <int MT, int R, int U, int WAVES, int OCC, int BLOCK>
 bool launch_gemv4_dot2(const LinearArgs& a)
 {
     const size_t lds = (size_t)MT * ((a.K + 2047) / 2048) * 4096;
-    const long long rows_per_cu = a.n_out / cu_count();
-    if (rows_per_cu >= 32)
-    {
-        auto kernel = gemv4_dot2_kernel<MT, 2, 2, 4, BLOCK>;
-        if (!allow_big_lds(kernel, lds)) { return false; }
-        const int want = ((a.n_out + 1) / 2 + 3) / 4;
-        const int cap = cu_count() * (lds > 80 * 1024 ? 1 : 4);
-        kernel<<<want < cap ? want : cap, 256, lds, stream()>>>(a);
-    }
-    else
-    {
-        auto kernel = gemv4_dot2_kernel<MT, 1, 2, 4, BLOCK>;
-        if (!allow_big_lds(kernel, lds)) { return false; }
-        const int want = (a.n_out + 3) / 4;
-        const int cap = cu_count() * (lds > 80 * 1024 ? 1 : 4);
-        kernel<<<want < cap ? want : cap, 256, lds, stream()>>>(a);
-    }
+    auto kernel = gemv4_dot2_kernel<MT, R, U, WAVES, BLOCK>;
+    if (!allow_big_lds(kernel, lds)) { return false; }
+    const int want = ((a.n_out + R - 1) / R + WAVES - 1) / WAVES;
+    const int cap = cu_count() * (lds > 80 * 1024 ? 1 : (lds > 40 * 1024 && OCC > 2 ? 2 : OCC));
+    kernel<<<want < cap ? want : cap, WAVES * 64, lds, stream()>>>(a);
     return true;
+}
+
+// Tuned on MI355X (block 16, one token) with rotating weight buffers.
+template <int MT, int BLOCK>
+bool pick_gemv4_dot2(const LinearArgs& a)
+{
+    const long long bytes = (long long)a.n_out * a.K / 2;
+    if (bytes <= (8LL << 20)) { return launch_gemv4_dot2<MT, 1, 4, 8, 2, BLOCK>(a); }
+    if (a.K > 8192) { return launch_gemv4_dot2<MT, 2, 4, 8, 2, BLOCK>(a); }
+    if (a.n_out / cu_count() >= 128) { return launch_gemv4_dot2<MT, 2, 2, 4, 4, BLOCK>(a); }
+    return launch_gemv4_dot2<MT, 2, 4, 4, 4, BLOCK>(a);
 }
 
 template <int BLOCK>
@@ -191,10 +190,10 @@ bool gemv4_dot2(const LinearArgs& a)
 {
     switch (a.tokens)
     {
-    case 1: return launch_gemv4_dot2<1, BLOCK>(a);
-    case 2: return launch_gemv4_dot2<2, BLOCK>(a);
-    case 3: return launch_gemv4_dot2<3, BLOCK>(a);
-    case 4: return launch_gemv4_dot2<4, BLOCK>(a);
+    case 1: return pick_gemv4_dot2<1, BLOCK>(a);
+    case 2: return pick_gemv4_dot2<2, BLOCK>(a);
+    case 3: return pick_gemv4_dot2<3, BLOCK>(a);
+    case 4: return pick_gemv4_dot2<4, BLOCK>(a);
     default: return false;
     }
 }

@@ -159,4 +159,34 @@ double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int step
     return result;
 }
 
+// Times `iters` back-to-back FP4 block-scale linears  Y = W[i % n_w]^T X  issued straight through
+// hip_quant_gemm (the host mirror always passes the reference's block size 16; this loop lets the
+// benchmark also measure block 32).  Returns elapsed milliseconds or a negative value on error.
+double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n_out, int tokens, int K,
+                            unsigned int block, int iters, int warmup)
+{
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    hip_quant_set_sync(0);
+    int status = 0;
+    for (int i = 0; i < warmup + iters; i++)
+    {
+        if (i == warmup) { (void)hipEventRecord(e0, nullptr); }
+        const int rc = hip_quant_gemm(1, 0, n_out, tokens, K, 1.0f, W[i % n_w], (int)FP4_E2M1, K, 1.0f, X, (int)BFLOAT16, K, 1.0f,
+                                      0.0f, Y, (int)BFLOAT16, n_out, 0.0f, S[i % n_w], nullptr, block);
+        if (rc != 0) { status = rc; }
+    }
+    (void)hipEventRecord(e1, nullptr);
+    double result = -2.0;
+    if (hipEventSynchronize(e1) == hipSuccess && status == 0)
+    {
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        result = ms;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return result;
+}
+
 }    // extern "C"

@@ -39,6 +39,8 @@ class HostLibrary:
         L.cccc_gpu_allocated_bytes.restype = ctypes.c_ulonglong; L.cccc_gpu_allocated_bytes.argtypes = []
         L.cccc_bench_linear_chain.restype = ctypes.c_double
         L.cccc_bench_linear_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), i32, i32, i32]
+        L.cccc_bench_fp4_chain.restype = ctypes.c_double
+        L.cccc_bench_fp4_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_uint, i32, i32]
         self.c = L
 
     def init(self, device: int = 0) -> None:
@@ -55,6 +57,12 @@ class HostLibrary:
         n = len(W)
         arr = lambda ms: (ctypes.c_void_p * n)(*[m.handle for m in ms])
         return float(self.c.cccc_bench_linear_chain(n, arr(W), arr(X), arr(R), steps, warmup, 1 if use_graph else 0))
+
+
+    def bench_fp4_chain(self, W_ptrs, S_ptrs, X_ptr, Y_ptr, n_out, tokens, K, block, iters, warmup) -> float:
+        n = len(W_ptrs)
+        return float(self.c.cccc_bench_fp4_chain(n, (ctypes.c_void_p * n)(*W_ptrs), (ctypes.c_void_p * n)(*S_ptrs), X_ptr, Y_ptr,
+                                                 n_out, tokens, K, block, iters, warmup))
 
 
 class HostMatrix:
