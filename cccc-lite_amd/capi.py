@@ -20,6 +20,24 @@ class DataType:
 
 NO_TRANS, TRANS = 0, 1
 
+
+class FusedLinear(ctypes.Structure):
+    """struct hip_fused_linear of include/cccc_hip_quant.h."""
+    _fields_ = [("w_type", ctypes.c_int), ("K", ctypes.c_int), ("n_segments", ctypes.c_int), ("pair", ctypes.c_int),
+                ("W", ctypes.c_void_p * 3), ("n_out", ctypes.c_int * 3), ("w_scale", ctypes.c_float * 3),
+                ("Y", ctypes.c_void_p * 3), ("X", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p),
+                ("norm_eps", ctypes.c_float), ("residual", ctypes.c_void_p)]
+
+
+def make_fused_linear(w_type, K, W, n_out, Y, X, scales=None, norm_weight=None, norm_eps=1e-6, residual=None, pair=False) -> FusedLinear:
+    d = FusedLinear()
+    d.w_type, d.K, d.n_segments, d.pair = w_type, K, len(W), 1 if pair else 0
+    for s in range(len(W)):
+        d.W[s], d.n_out[s], d.Y[s] = W[s], n_out[s], Y[s]
+        d.w_scale[s] = scales[s] if scales else 1.0
+    d.X, d.norm_weight, d.norm_eps, d.residual = X, norm_weight, norm_eps, residual
+    return d
+
 EXPORTS = (
     "hip_convert",
     "hip_fp4_blockscale_to_bf16",
@@ -29,6 +47,14 @@ EXPORTS = (
     "hip_quant_tiled_size",
     "hip_quant_weight_prepare",
     "hip_quant_weight_release",
+    "hip_quant_linear_fused",
+    "hip_rms_norm_fwd",
+    "hip_rope_fwd",
+    "hip_embed_fwd",
+    "hip_embed_token_bf16",
+    "hip_qk_norm_rope_kv_bf16",
+    "hip_attention_decode_bf16",
+    "hip_argmax_bf16",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
     "hip_quant_last_kernel",
@@ -72,6 +98,22 @@ class QuantLibrary:
         L.hip_quant_weight_prepare.argtypes = [vp, i32, i32, i32, i32, vp]
         L.hip_quant_weight_release.restype = i32
         L.hip_quant_weight_release.argtypes = [vp]
+        L.hip_quant_linear_fused.restype = i32
+        L.hip_quant_linear_fused.argtypes = [ctypes.POINTER(FusedLinear)]
+        L.hip_rms_norm_fwd.restype = i32
+        L.hip_rms_norm_fwd.argtypes = [i32, vp, vp, vp, vp, u32, u32, f32]
+        L.hip_rope_fwd.restype = i32
+        L.hip_rope_fwd.argtypes = [i32, vp, vp, vp, vp, u32, u32, u32, u32]
+        L.hip_embed_fwd.restype = i32
+        L.hip_embed_fwd.argtypes = [i32, vp, vp, vp, i32, i32, i32]
+        L.hip_embed_token_bf16.restype = i32
+        L.hip_embed_token_bf16.argtypes = [vp, vp, vp, i32, i32]
+        L.hip_qk_norm_rope_kv_bf16.restype = i32
+        L.hip_qk_norm_rope_kv_bf16.argtypes = [vp] * 10 + [i32, i32, i32, i32, vp, f32]
+        L.hip_attention_decode_bf16.restype = i32
+        L.hip_attention_decode_bf16.argtypes = [vp] * 6 + [i32, i32, i32, i32, vp, i32]
+        L.hip_argmax_bf16.restype = i32
+        L.hip_argmax_bf16.argtypes = [vp, u32, vp, vp]
         L.hip_quant_set_sync.restype = i32
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32
@@ -108,6 +150,9 @@ class QuantLibrary:
 
     def weight_release(self, W) -> int:
         return self.c.hip_quant_weight_release(W)
+
+    def quant_linear_fused(self, desc: FusedLinear) -> int:
+        return self.c.hip_quant_linear_fused(ctypes.byref(desc))
 
     def set_sync(self, enabled: bool) -> int:
         return self.c.hip_quant_set_sync(1 if enabled else 0)

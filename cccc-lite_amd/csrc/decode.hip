@@ -1,0 +1,175 @@
+// C-ABI entry points of the decode-step neighbours (kernels in decode_kernels.h).
+#include "../../include/cccc_hip_quant.h"
+#include "decode_kernels.h"
+#include "runtime.h"
+#include <cstdio>
+
+using namespace ccq;
+
+namespace
+{
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <int WT, bool SCALED>
+int launch_fused(const FusedLinearArgs& a, int n_groups)
+{
+    const size_t lds = (size_t)((a.K + 1023) / 1024) * 2048;
+    if (lds > 64 * 1024) { return -1; }
+    const int cus = cu_count();
+    // long rows (K > 8192) and very tall weights want 8-wave workgroups, as the plain GEMV dispatch found
+    if (a.K > 8192 || n_groups >= cus * 64)
+    {
+        const int want = (n_groups + 7) / 8;
+        gemv8_fused_kernel<WT, 4, 8, SCALED><<<want < cus * 2 ? want : cus * 2, 512, lds, stream()>>>(a);
+    }
+    else
+    {
+        const int want = (n_groups + 3) / 4;
+        gemv8_fused_kernel<WT, 4, 4, SCALED><<<want < cus * 4 ? want : cus * 4, 256, lds, stream()>>>(a);
+    }
+    return finish("quant_linear_fused");
+}
+
+}    // namespace
+
+int hip_quant_linear_fused(const hip_fused_linear* d)
+{
+    if (!d || (d->w_type != DT_E4M3 && d->w_type != DT_E5M2)) { return -1; }
+    if (d->K <= 0 || d->K % 16 != 0 || d->n_segments < 1 || d->n_segments > 3 || !d->X || !aligned16(d->X)) { return -1; }
+    if (d->pair && d->n_segments != 2) { return -1; }
+    if (d->residual && !d->pair && d->n_segments != 1) { return -1; }
+    if (d->norm_weight && !aligned16(d->norm_weight)) { return -1; }
+    FusedLinearArgs a{};
+    bool scaled = false;
+    int n_groups = 0;
+    for (int s = 0; s < d->n_segments; s++)
+    {
+        if (!d->W[s] || !aligned16(d->W[s]) || d->n_out[s] <= 0) { return -1; }
+        if (!d->pair && !d->Y[s]) { return -1; }
+        a.W[s] = (const uint8_t*)d->W[s];
+        a.Y[s] = (uint16_t*)d->Y[s];
+        a.n_out[s] = d->n_out[s];
+        a.w_scale[s] = d->w_scale[s];
+        scaled = scaled || d->w_scale[s] != 1.0f;
+        n_groups += (d->n_out[s] + 1) / 2;
+    }
+    if (d->pair)
+    {
+        if (d->n_out[1] != d->n_out[0] || !d->Y[0]) { return -1; }
+        n_groups = d->n_out[0];
+    }
+    a.n_segments = d->n_segments;
+    a.pair = d->pair ? 1 : 0;
+    a.K = d->K;
+    a.X = (const uint16_t*)d->X;
+    a.norm_w = (const uint16_t*)d->norm_weight;
+    a.norm_eps = d->norm_eps;
+    a.residual = (const uint16_t*)d->residual;
+    note_kernel("gemv_fused");
+    if (d->w_type == DT_E5M2) { return scaled ? launch_fused<DT_E5M2, true>(a, n_groups) : launch_fused<DT_E5M2, false>(a, n_groups); }
+    return scaled ? launch_fused<DT_E4M3, true>(a, n_groups) : launch_fused<DT_E4M3, false>(a, n_groups);
+}
+
+int hip_rms_norm_fwd(int type, void* X, void* Y, void* scale, void* invstd_out, unsigned int outer, unsigned int inner, float epsilon)
+{
+    if (type != DT_BF16)
+    {
+        fprintf(stderr, "hip_rms_norm_fwd: unsupported type=%d\n", type);
+        return 1;
+    }
+    if (outer == 0 || inner == 0) { return 0; }
+    rms_norm_bf16_kernel<<<outer, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)scale, (float*)invstd_out, inner, epsilon);
+    return finish("rms_norm_fwd_bf16");
+}
+
+int hip_rope_fwd(int type, const void* X, void* Y, const void* cos_tab, const void* sin_tab, unsigned int D, unsigned int T, unsigned int B, unsigned int pos_offset)
+{
+    if (D % 2 != 0)
+    {
+        fprintf(stderr, "hip_rope_fwd: D must be even (D=%u)\n", D);
+        return 1;
+    }
+    if (type != DT_BF16)
+    {
+        fprintf(stderr, "hip_rope_fwd: unsupported type=%d\n", type);
+        return 1;
+    }
+    const unsigned total = (D / 2) * T * B;
+    if (total == 0) { return 0; }
+    rope_bf16_kernel<<<(total + 255) / 256, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, D, T, B, pos_offset);
+    return finish("rope_fwd_bf16");
+}
+
+int hip_embed_fwd(int type, const void* ids, const void* W, void* Y, int D, int T, int B)
+{
+    if (type != DT_BF16 || D <= 0 || D % 8 != 0)
+    {
+        fprintf(stderr, "hip_embed_fwd: unsupported type=%d or D=%d\n", type, D);
+        return 1;
+    }
+    if (T * B <= 0) { return 0; }
+    embed_bf16_kernel<<<dim3(1, T * B), 256, 0, stream()>>>((const float*)ids, nullptr, (const uint16_t*)W, (uint16_t*)Y, D, 0x7FFFFFFF);
+    return finish("embed_fwd_bf16");
+}
+
+int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows)
+{
+    if (!d_token || !W || !y || D <= 0 || D % 8 != 0 || n_rows <= 0) { return -1; }
+    embed_bf16_kernel<<<dim3(1, 1), 256, 0, stream()>>>(nullptr, (const int*)d_token, (const uint16_t*)W, (uint16_t*)y, D, n_rows);
+    return finish("embed_token_bf16");
+}
+
+int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v, const void* q_norm_w, const void* k_norm_w,
+                             const void* cos_tab, const void* sin_tab, void* q_out, void* k_cache, void* v_cache,
+                             int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
+{
+    if (head_dim != 128 || n_q_heads <= 0 || n_kv_heads <= 0 || t_kv <= 0 || !d_pos) { return -1; }
+    qk_norm_rope_kv_kernel<<<n_q_heads + 2 * n_kv_heads, 64, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v,
+                                                                           (const uint16_t*)q_norm_w, (const uint16_t*)k_norm_w,
+                                                                           (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,
+                                                                           (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache,
+                                                                           n_q_heads, n_kv_heads, t_kv, (const int*)d_pos, epsilon);
+    return finish("qk_norm_rope_kv");
+}
+
+int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* y, void* scores_ws, void* partial_ws,
+                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, int n_splits)
+{
+    if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || n_splits <= 0 || !d_pos) { return -1; }
+    const int group = n_q_heads / n_kv_heads;
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    const dim3 grid_s((t_kv + 63) / 64, n_kv_heads), grid_p(n_splits, n_kv_heads);
+    const uint16_t* qp = (const uint16_t*)q;
+    const uint16_t* kc = (const uint16_t*)k_cache;
+    const uint16_t* vc = (const uint16_t*)v_cache;
+    uint16_t* sw = (uint16_t*)scores_ws;
+    float* pw = (float*)partial_ws;
+    const int* pos = (const int*)d_pos;
+    switch (group)
+    {
+    case 1:
+        attn_scores_kernel<1><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
+        attn_pv_kernel<1><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
+        break;
+    case 2:
+        attn_scores_kernel<2><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
+        attn_pv_kernel<2><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
+        break;
+    case 4:
+        attn_scores_kernel<4><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
+        attn_pv_kernel<4><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
+        break;
+    default: return -1;
+    }
+    const int n = n_q_heads * head_dim;
+    sum_partials_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(pw, (uint16_t*)y, n_splits, n);
+    return finish("attention_decode");
+}
+
+int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos)
+{
+    if (!x || !d_index || n == 0) { return -1; }
+    argmax_bf16_kernel<<<1, 1024, 0, stream()>>>((const uint16_t*)x, n, (int*)d_index, (int*)d_pos);
+    return finish("argmax_bf16");
+}

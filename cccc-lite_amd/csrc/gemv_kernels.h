@@ -802,7 +802,7 @@ __global__ __launch_bounds__(512) void gemv8_mfma_lds_kernel(const LinearArgs a,
 // Builds the tiled copy of an FP8 weight [n_out][ldw]: for row tile t (16 rows) and k block b (64
 // codes) the KiB at (t * ceil(K / 64) + b) * 1024 holds, at lane l = i + 16 g, the 16 codes
 // W[16 t + i][64 b + 16 g ..].  Rows beyond n_out and codes beyond K are zero.
-__global__ __launch_bounds__(256) void repack_tiled_kernel(const uint8_t* __restrict__ W, uint8_t* __restrict__ dst, int n_out, int K, long long ldw)
+static __global__ __launch_bounds__(256) void repack_tiled_kernel(const uint8_t* __restrict__ W, uint8_t* __restrict__ dst, int n_out, int K, long long ldw)
 {
     const int blocks_per_row = (K + 63) / 64;
     const long long n_chunks = (long long)((n_out + 15) / 16) * blocks_per_row * 64;
@@ -836,7 +836,7 @@ struct GenericArgs
     float w_scale, alpha, beta;
 };
 
-__global__ __launch_bounds__(256) void generic_linear_kernel(const GenericArgs a)
+static __global__ __launch_bounds__(256) void generic_linear_kernel(const GenericArgs a)
 {
     const long long total = (long long)a.n_out * a.tokens;
     for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256)

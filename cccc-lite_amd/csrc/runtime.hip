@@ -46,8 +46,7 @@ int cu_count()
 
 int hip_quant_set_sync(int enabled)
 {
-    ccq::g_sync.store(enabled ? 1 : 0, std::memory_order_relaxed);
-    return 0;
+    return ccq::g_sync.exchange(enabled ? 1 : 0, std::memory_order_relaxed);
 }
 
 int hip_quant_set_stream(void* s)

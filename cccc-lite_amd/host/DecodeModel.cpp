@@ -1,0 +1,284 @@
+#include "DecodeModel.h"
+#include "../../include/cccc_hip_quant.h"
+#include <hip/hip_runtime.h>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+namespace cccc
+{
+
+static std::unique_ptr<Matrix> make(int w, int h, DataType dt, GpuControl* gpu) { return std::make_unique<Matrix>(w, h, 1, 1, dt, gpu); }
+
+static void zero(Matrix& m, size_t bytes) { (void)hipMemset(m.data(), 0, bytes); }
+
+DecodeModel::DecodeModel(const DecodeConfig& cfg, GpuControl* gpu) : cfg_(cfg), gpu_(gpu)
+{
+    gpu_->setAsCurrent();
+    const int q_out = cfg.n_q * cfg.head_dim, kv_out = cfg.n_kv * cfg.head_dim;
+    layers_.resize(cfg.layers);
+    for (auto& L : layers_)
+    {
+        // linears are allocated as 1-byte tensors and re-typed by loadQuantizedDirect; (W, H) = (in, out)
+        L.rms_attn = make(cfg.hidden, 1, BFLOAT16, gpu);
+        L.wq = make(cfg.hidden, q_out, FP8_E5M2, gpu);
+        L.wk = make(cfg.hidden, kv_out, FP8_E5M2, gpu);
+        L.wv = make(cfg.hidden, kv_out, FP8_E5M2, gpu);
+        L.q_norm = make(cfg.head_dim, 1, BFLOAT16, gpu);
+        L.k_norm = make(cfg.head_dim, 1, BFLOAT16, gpu);
+        L.wo = make(q_out, cfg.hidden, FP8_E5M2, gpu);
+        L.rms_ffn = make(cfg.hidden, 1, BFLOAT16, gpu);
+        L.w_gate = make(cfg.hidden, cfg.inter, FP8_E5M2, gpu);
+        L.w_up = make(cfg.hidden, cfg.inter, FP8_E5M2, gpu);
+        L.w_down = make(cfg.inter, cfg.hidden, FP8_E5M2, gpu);
+        k_cache_.push_back(std::make_unique<Matrix>(cfg.head_dim, cfg.t_kv, 1, cfg.n_kv, BFLOAT16, gpu));
+        v_cache_.push_back(std::make_unique<Matrix>(cfg.head_dim, cfg.t_kv, 1, cfg.n_kv, BFLOAT16, gpu));
+        const size_t cache_bytes = (size_t)cfg.head_dim * cfg.t_kv * cfg.n_kv * 2;
+        zero(*k_cache_.back(), cache_bytes);
+        zero(*v_cache_.back(), cache_bytes);
+    }
+    emb_ = make(cfg.hidden, cfg.vocab, BFLOAT16, gpu);
+    rms_final_ = make(cfg.hidden, 1, BFLOAT16, gpu);
+    lm_head_ = make(cfg.hidden, cfg.vocab, FP8_E5M2, gpu);
+    logits_ = make(cfg.vocab, 1, BFLOAT16, gpu);
+    x_ = make(cfg.hidden, 1, BFLOAT16, gpu);
+    r1_ = make(cfg.hidden, 1, BFLOAT16, gpu);
+    q_ = make(q_out, 1, BFLOAT16, gpu);
+    k_ = make(kv_out, 1, BFLOAT16, gpu);
+    v_ = make(kv_out, 1, BFLOAT16, gpu);
+    q_rot_ = make(q_out, 1, BFLOAT16, gpu);
+    att_ = make(q_out, 1, BFLOAT16, gpu);
+    gated_ = make(cfg.inter, 1, BFLOAT16, gpu);
+    scores_ = make(cfg.t_kv, cfg.n_q, BFLOAT16, gpu);
+    partial_ = make(q_out, n_splits_, FLOAT, gpu);
+
+    // RoPE tables as the reference's graph builds them (cccc/NetCifa.cpp:431-475): float math on the host,
+    // stored to BF16 by truncation (cccc/types.h:43-48)
+    const int half = cfg.head_dim / 2;
+    std::vector<uint16_t> cos_h((size_t)cfg.t_kv * half), sin_h(cos_h.size());
+    for (int t = 0; t < cfg.t_kv; t++)
+    {
+        for (int d = 0; d < half; d++)
+        {
+            const float angle = t * std::pow(cfg.theta, -2.0f * d / cfg.head_dim);
+            const float c = (float)std::cos(angle), s = (float)std::sin(angle);
+            uint32_t cu, su;
+            std::memcpy(&cu, &c, 4);
+            std::memcpy(&su, &s, 4);
+            cos_h[(size_t)t * half + d] = (uint16_t)(cu >> 16);
+            sin_h[(size_t)t * half + d] = (uint16_t)(su >> 16);
+        }
+    }
+    cos_ = make(half, cfg.t_kv, BFLOAT16, gpu);
+    sin_ = make(half, cfg.t_kv, BFLOAT16, gpu);
+    cos_->copyFromHost(cos_h.data(), cos_h.size() * 2);
+    sin_->copyFromHost(sin_h.data(), sin_h.size() * 2);
+
+    void* p = nullptr;
+    gpu_->malloc(&p, 2 * sizeof(int));
+    d_state_ = (int*)p;
+    (void)hipMemset(d_state_, 0, 2 * sizeof(int));
+}
+
+DecodeModel::~DecodeModel()
+{
+    if (d_state_) { gpu_->free(d_state_); }
+}
+
+Matrix* DecodeModel::tensor(int layer, int which)
+{
+    if (which >= EMB)
+    {
+        return which == EMB ? emb_.get() : which == RMS_FINAL ? rms_final_.get() : which == LM_HEAD ? lm_head_.get() : nullptr;
+    }
+    if (layer < 0 || layer >= cfg_.layers) { return nullptr; }
+    Layer& L = layers_[layer];
+    Matrix* table[] = { L.rms_attn.get(), L.wq.get(), L.wk.get(), L.wv.get(), L.q_norm.get(), L.k_norm.get(), L.wo.get(),
+                        L.rms_ffn.get(), L.w_gate.get(), L.w_up.get(), L.w_down.get() };
+    return (which >= 0 && which <= W_DOWN) ? table[which] : nullptr;
+}
+
+int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale)
+{
+    Matrix* m = tensor(layer, which);
+    if (!m) { return -1; }
+    if (Rocblas::isQuantized(dt))
+    {
+        if ((int64_t)bytes != m->getDataSize()) { return -1; }
+        m->setAllowRepack(false);    // one token per step: the tiled copy (5..16 tokens) would never be read
+        m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
+        return 0;
+    }
+    return m->copyFromHost(host, bytes);
+}
+
+size_t DecodeModel::weightBytes() const
+{
+    const size_t q_out = (size_t)cfg_.n_q * cfg_.head_dim, kv_out = (size_t)cfg_.n_kv * cfg_.head_dim;
+    const size_t per_layer = (size_t)cfg_.hidden * (q_out + 2 * kv_out) + q_out * cfg_.hidden + 3 * (size_t)cfg_.hidden * cfg_.inter;
+    return per_layer * cfg_.layers + (size_t)cfg_.hidden * cfg_.vocab;
+}
+
+int DecodeModel::reset(int token, int pos)
+{
+    const int state[2] = { token, pos };
+    return GpuControl::copyHostToDevice(d_state_, state, sizeof(state));
+}
+
+int DecodeModel::currentToken()
+{
+    int t = -1;
+    GpuControl::copyDeviceToHost(&t, d_state_, sizeof(int));
+    return t;
+}
+
+int DecodeModel::currentPos()
+{
+    int p = -1;
+    GpuControl::copyDeviceToHost(&p, d_state_ + 1, sizeof(int));
+    return p;
+}
+
+static hip_fused_linear linear_desc(const Matrix& W, int n_out, int K, const void* x, void* y)
+{
+    hip_fused_linear d{};
+    d.w_type = (int)W.getDataType();
+    d.K = K;
+    d.n_segments = 1;
+    d.W[0] = W.data();
+    d.n_out[0] = n_out;
+    d.w_scale[0] = W.getQuantScale();
+    d.Y[0] = y;
+    d.X = x;
+    return d;
+}
+
+int DecodeModel::step()
+{
+    const DecodeConfig& c = cfg_;
+    const int q_out = c.n_q * c.head_dim, kv_out = c.n_kv * c.head_dim;
+    const int* d_token = d_state_;
+    const int* d_pos = d_state_ + 1;
+    int rc = hip_embed_token_bf16(d_token, emb_->data(), x_->data(), c.hidden, c.vocab);
+    for (int li = 0; li < c.layers && rc == 0; li++)
+    {
+        Layer& L = layers_[li];
+        // 1. q, k, v = W_{q,k,v} rmsnorm(x): one launch, three weight segments
+        hip_fused_linear qkv = linear_desc(*L.wq, q_out, c.hidden, x_->data(), q_->data());
+        qkv.n_segments = 3;
+        qkv.W[1] = L.wk->data(); qkv.n_out[1] = kv_out; qkv.w_scale[1] = L.wk->getQuantScale(); qkv.Y[1] = k_->data();
+        qkv.W[2] = L.wv->data(); qkv.n_out[2] = kv_out; qkv.w_scale[2] = L.wv->getQuantScale(); qkv.Y[2] = v_->data();
+        qkv.norm_weight = L.rms_attn->data();
+        qkv.norm_eps = c.eps;
+        rc = hip_quant_linear_fused(&qkv);
+        // 2. per-head q/k norm, RoPE, KV append
+        if (rc == 0)
+        {
+            rc = hip_qk_norm_rope_kv_bf16(q_->data(), k_->data(), v_->data(), L.q_norm->data(), L.k_norm->data(), cos_->data(), sin_->data(),
+                                          q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
+        }
+        // 3. attention over the cache (three launches)
+        if (rc == 0)
+        {
+            rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), scores_->data(),
+                                           partial_->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, n_splits_);
+        }
+        // 4. r1 = x + W_o att
+        if (rc == 0)
+        {
+            hip_fused_linear o = linear_desc(*L.wo, c.hidden, q_out, att_->data(), r1_->data());
+            o.residual = x_->data();
+            rc = hip_quant_linear_fused(&o);
+        }
+        // 5. gated = silu(W_gate n) * (W_up n), n = rmsnorm(r1)
+        if (rc == 0)
+        {
+            hip_fused_linear gu = linear_desc(*L.w_gate, c.inter, c.hidden, r1_->data(), gated_->data());
+            gu.n_segments = 2;
+            gu.pair = 1;
+            gu.W[1] = L.w_up->data(); gu.n_out[1] = c.inter; gu.w_scale[1] = L.w_up->getQuantScale();
+            gu.norm_weight = L.rms_ffn->data();
+            gu.norm_eps = c.eps;
+            rc = hip_quant_linear_fused(&gu);
+        }
+        // 6. x = r1 + W_down gated
+        if (rc == 0)
+        {
+            hip_fused_linear dn = linear_desc(*L.w_down, c.hidden, c.inter, gated_->data(), x_->data());
+            dn.residual = r1_->data();
+            rc = hip_quant_linear_fused(&dn);
+        }
+    }
+    if (rc == 0)
+    {
+        hip_fused_linear head = linear_desc(*lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
+        head.norm_weight = rms_final_->data();
+        head.norm_eps = c.eps;
+        rc = hip_quant_linear_fused(&head);
+    }
+    if (rc == 0) { rc = hip_argmax_bf16(logits_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1); }
+    return rc;
+}
+
+double DecodeModel::run(int n_steps, int use_graph)
+{
+    if (n_steps <= 0 || currentPos() < 0 || currentPos() + n_steps > cfg_.t_kv) { return -2.0; }    // would run past the KV cache
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    double result = -1.0;
+    const int sync_before = hip_quant_set_sync(0);
+    if (use_graph)
+    {
+        hipStream_t stream = nullptr;
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        if (hipStreamCreate(&stream) != hipSuccess)
+        {
+            hip_quant_set_sync(sync_before);
+            return -4.0;
+        }
+        (void)hipDeviceSynchronize();
+        hip_quant_set_stream(stream);
+        bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) == hipSuccess;
+        if (ok) { ok = step() == 0; }
+        ok = (hipStreamEndCapture(stream, &graph) == hipSuccess) && ok;
+        hip_quant_set_stream(nullptr);
+        if (ok) { ok = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess; }
+        if (ok)
+        {
+            (void)hipEventRecord(e0, stream);
+            for (int s = 0; s < n_steps; s++) { ok = (hipGraphLaunch(exec, stream) == hipSuccess) && ok; }
+            (void)hipEventRecord(e1, stream);
+            ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
+        }
+        if (ok)
+        {
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            result = ms;
+        }
+        if (exec) { (void)hipGraphExecDestroy(exec); }
+        if (graph) { (void)hipGraphDestroy(graph); }
+        (void)hipStreamDestroy(stream);
+    }
+    else
+    {
+        bool ok = true;
+        (void)hipEventRecord(e0, nullptr);
+        for (int s = 0; s < n_steps; s++) { ok = (step() == 0) && ok; }
+        (void)hipEventRecord(e1, nullptr);
+        ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
+        if (ok)
+        {
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            result = ms;
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    hip_quant_set_sync(sync_before);
+    return result;
+}
+
+}    // namespace cccc

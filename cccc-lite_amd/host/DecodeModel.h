@@ -1,0 +1,66 @@
+// Batch-1 decode step of a Qwen3-style transformer with weight-only quantized linears, driven from
+// the host mirror: what the reference does per token through MainProcess::testExternalData ->
+// Net::inference -> MatrixOp::forward (cccc/MainProcess.cpp:1171-1239, cccc/Net.cpp:1748-1792,
+// cccc/MatrixOp.cpp:12-26) for the graph of scripts/convert_weights.py:488-692, collapsed into
+// nine launches per layer.  Token id and position live in device memory, so a step is a fixed
+// launch sequence that can be replayed as one hipGraph.
+#pragma once
+#include "Matrix.h"
+#include <memory>
+#include <vector>
+
+namespace cccc
+{
+
+struct DecodeConfig
+{
+    int layers, hidden, n_q, n_kv, head_dim, inter, vocab, t_kv;
+    float theta, eps;
+};
+
+class DecodeModel
+{
+public:
+    enum Tensor
+    {
+        RMS_ATTN = 0, WQ, WK, WV, Q_NORM, K_NORM, WO, RMS_FFN, W_GATE, W_UP, W_DOWN,    // per layer
+        EMB = 100, RMS_FINAL, LM_HEAD                                                    // global (layer ignored)
+    };
+
+    DecodeModel(const DecodeConfig& cfg, GpuControl* gpu);
+    ~DecodeModel();
+
+    const DecodeConfig& config() const { return cfg_; }
+    Matrix* tensor(int layer, int which);
+
+    // Uploads file bytes: FP8 codes for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
+    int setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale);
+
+    int reset(int token, int pos);          // sets the device-side token / position (KV caches are kept)
+    int step();                             // enqueues one decode step; the next token replaces the current one
+    // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
+    double run(int n_steps, int use_graph);
+    int currentToken();                     // blocking 4-byte read
+    int currentPos();
+    Matrix& logits() { return *logits_; }
+    Matrix& kCache(int layer) { return *k_cache_[layer]; }
+    Matrix& vCache(int layer) { return *v_cache_[layer]; }
+    Matrix& cosTable() { return *cos_; }
+    size_t weightBytes() const;
+
+private:
+    struct Layer
+    {
+        std::unique_ptr<Matrix> rms_attn, wq, wk, wv, q_norm, k_norm, wo, rms_ffn, w_gate, w_up, w_down;
+    };
+    DecodeConfig cfg_;
+    GpuControl* gpu_;
+    std::vector<Layer> layers_;
+    std::unique_ptr<Matrix> emb_, rms_final_, lm_head_, logits_, cos_, sin_;
+    std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
+    std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, scores_, partial_;
+    int* d_state_ = nullptr;    // [0] token, [1] position
+    int n_splits_ = 32;
+};
+
+}    // namespace cccc

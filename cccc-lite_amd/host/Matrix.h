@@ -37,6 +37,7 @@ public:
     void getBlockScaleToHost(void* dst) const { shared_data_->getBlockScaleToHost(dst); }
     static unsigned int fp4BlockSize() { return MatrixData::fp4_block_size_; }
     void prepareTiled() { if (shared_data_ && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); } }
+    void setAllowRepack(bool allow) { if (shared_data_) { shared_data_->allow_repack_ = allow; } }
     bool hasTiled() const { return shared_data_ && shared_data_->tiled_data_ != nullptr; }
     float getInputScale() const { return shared_data_ ? shared_data_->input_scale_ : 0.0f; }
 

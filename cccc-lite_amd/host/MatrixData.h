@@ -23,7 +23,8 @@ struct MatrixData
     // Load-time repacked (tiled) copy of an FP8 weight for the matrix-core GEMV; owned here, registered
     // with the kernel library under the key data_.  No counterpart in the reference.
     void* tiled_data_ = nullptr;
-    static inline bool repack_weights = true;
+    static inline bool repack_weights = true;    // global switch
+    bool allow_repack_ = true;                    // per storage (a batch-1 decode model never needs the copy)
 
     MatrixData() = default;
     ~MatrixData() { release(); }

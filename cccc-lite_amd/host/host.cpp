@@ -122,7 +122,7 @@ void* MatrixData::resize(int64_t size, DataType data_type, bool force)
 void MatrixData::prepareTiled(int n_out, int K)
 {
     releaseTiled();
-    if (!repack_weights || !gpu_ || !data_ || (data_type_ != FP8_E4M3 && data_type_ != FP8_E5M2)) { return; }
+    if (!repack_weights || !allow_repack_ || !gpu_ || !data_ || (data_type_ != FP8_E4M3 && data_type_ != FP8_E5M2)) { return; }
     const unsigned long long bytes = hip_quant_tiled_size((int)data_type_, n_out, K);
     if (bytes == 0 || gpu_->malloc(&tiled_data_, (size_t)bytes) != 0) { tiled_data_ = nullptr; return; }
     if (hip_quant_weight_prepare(data_, (int)data_type_, n_out, K, K, tiled_data_) != 0)

@@ -1,6 +1,7 @@
 // Plain-C window onto the host mirror so that tests and the benchmark (Python, ctypes) drive the
 // same Matrix::mulBatched path a cccc graph would, plus a timing loop that runs a chain of linears
 // from native code (Python call overhead would otherwise dominate microsecond kernels).
+#include "DecodeModel.h"
 #include "Matrix.h"
 #include "../../include/cccc_hip_quant.h"
 #include <hip/hip_runtime.h>
@@ -188,5 +189,62 @@ double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n
     (void)hipEventDestroy(e1);
     return result;
 }
+
+// ---- decode model
+
+void* cccc_decode_create(int layers, int hidden, int n_q, int n_kv, int head_dim, int inter, int vocab, int t_kv, float theta, float eps)
+{
+    if (!GpuControl::getCurrentGpu()) { GpuControl::select(0); }
+    if (head_dim != 128 || hidden % 16 != 0 || inter % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) { return nullptr; }
+    const DecodeConfig cfg{ layers, hidden, n_q, n_kv, head_dim, inter, vocab, t_kv, theta, eps };
+    return new DecodeModel(cfg, GpuControl::getCurrentGpu());
+}
+
+void cccc_decode_destroy(void* m) { delete (DecodeModel*)m; }
+
+int cccc_decode_set_tensor(void* m, int layer, int which, const void* host, unsigned long long bytes, int dtype, float scale)
+{
+    return ((DecodeModel*)m)->setTensor(layer, which, host, (size_t)bytes, (DataType)dtype, scale);
+}
+
+void* cccc_decode_tensor_data(void* m, int layer, int which)
+{
+    Matrix* t = ((DecodeModel*)m)->tensor(layer, which);
+    return t ? t->data() : nullptr;
+}
+
+int cccc_decode_tensor_prepare(void* m, int layer, int which)
+{
+    Matrix* t = ((DecodeModel*)m)->tensor(layer, which);
+    if (!t) { return -1; }
+    t->prepareTiled();
+    return t->hasTiled() ? 0 : 1;
+}
+
+int cccc_decode_reset(void* m, int token, int pos) { return ((DecodeModel*)m)->reset(token, pos); }
+
+int cccc_decode_step(void* m)
+{
+    const int rc = ((DecodeModel*)m)->step();
+    return (hipDeviceSynchronize() == hipSuccess) ? rc : 1;
+}
+
+double cccc_decode_run(void* m, int n_steps, int use_graph) { return ((DecodeModel*)m)->run(n_steps, use_graph); }
+
+int cccc_decode_token(void* m) { return ((DecodeModel*)m)->currentToken(); }
+
+int cccc_decode_pos(void* m) { return ((DecodeModel*)m)->currentPos(); }
+
+int cccc_decode_logits(void* m, void* host, unsigned long long bytes) { return ((DecodeModel*)m)->logits().copyToHost(host, (size_t)bytes); }
+
+int cccc_decode_kv(void* m, int layer, int is_v, void* host, unsigned long long bytes)
+{
+    DecodeModel* d = (DecodeModel*)m;
+    return (is_v ? d->vCache(layer) : d->kCache(layer)).copyToHost(host, (size_t)bytes);
+}
+
+int cccc_decode_cos_table(void* m, void* host, unsigned long long bytes) { return ((DecodeModel*)m)->cosTable().copyToHost(host, (size_t)bytes); }
+
+unsigned long long cccc_decode_weight_bytes(void* m) { return (unsigned long long)((DecodeModel*)m)->weightBytes(); }
 
 }    // extern "C"

@@ -41,6 +41,20 @@ class HostLibrary:
         L.cccc_bench_linear_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), i32, i32, i32]
         L.cccc_bench_fp4_chain.restype = ctypes.c_double
         L.cccc_bench_fp4_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_uint, i32, i32]
+        u64 = ctypes.c_ulonglong
+        L.cccc_decode_create.restype = vp; L.cccc_decode_create.argtypes = [i32] * 8 + [f32, f32]
+        L.cccc_decode_destroy.restype = None; L.cccc_decode_destroy.argtypes = [vp]
+        L.cccc_decode_set_tensor.restype = i32; L.cccc_decode_set_tensor.argtypes = [vp, i32, i32, vp, u64, i32, f32]
+        L.cccc_decode_tensor_data.restype = vp; L.cccc_decode_tensor_data.argtypes = [vp, i32, i32]
+        L.cccc_decode_reset.restype = i32; L.cccc_decode_reset.argtypes = [vp, i32, i32]
+        L.cccc_decode_step.restype = i32; L.cccc_decode_step.argtypes = [vp]
+        L.cccc_decode_run.restype = ctypes.c_double; L.cccc_decode_run.argtypes = [vp, i32, i32]
+        L.cccc_decode_token.restype = i32; L.cccc_decode_token.argtypes = [vp]
+        L.cccc_decode_pos.restype = i32; L.cccc_decode_pos.argtypes = [vp]
+        L.cccc_decode_logits.restype = i32; L.cccc_decode_logits.argtypes = [vp, vp, u64]
+        L.cccc_decode_kv.restype = i32; L.cccc_decode_kv.argtypes = [vp, i32, i32, vp, u64]
+        L.cccc_decode_cos_table.restype = i32; L.cccc_decode_cos_table.argtypes = [vp, vp, u64]
+        L.cccc_decode_weight_bytes.restype = u64; L.cccc_decode_weight_bytes.argtypes = [vp]
         self.c = L
 
     def init(self, device: int = 0) -> None:
@@ -137,3 +151,88 @@ def host() -> HostLibrary:
     if _host is None:
         _host = HostLibrary()
     return _host
+
+
+# tensor ids of DecodeModel::Tensor
+LAYER_TENSORS = {"rms_attn": 0, "wq": 1, "wk": 2, "wv": 3, "q_norm": 4, "k_norm": 5, "wo": 6, "rms_ffn": 7,
+                 "w_gate": 8, "w_up": 9, "w_down": 10}
+GLOBAL_TENSORS = {"emb": 100, "rms_final": 101, "lm_head": 102}
+QUANTIZED = {"wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "lm_head"}
+
+
+class DecodeModel:
+    """The C++ DecodeModel (host/DecodeModel.h): a Qwen3-style batch-1 decode step on the fused kernels."""
+
+    def __init__(self, lib: HostLibrary, layers, hidden, n_q, n_kv, head_dim, inter, vocab, t_kv, theta=1e6, eps=1e-6):
+        self.lib = lib
+        self.cfg = dict(layers=layers, hidden=hidden, n_q=n_q, n_kv=n_kv, head_dim=head_dim, inter=inter, vocab=vocab, t_kv=t_kv)
+        self.handle = lib.c.cccc_decode_create(layers, hidden, n_q, n_kv, head_dim, inter, vocab, t_kv, theta, eps)
+        if not self.handle:
+            raise ValueError("unsupported decode configuration")
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            self.lib.c.cccc_decode_destroy(self.handle)
+            self.handle = None
+
+    def set_tensor(self, layer: int, name: str, a: np.ndarray, dtype: int, scale: float = 1.0) -> None:
+        which = LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))
+        a = np.ascontiguousarray(a)
+        rc = self.lib.c.cccc_decode_set_tensor(self.handle, layer, which, a.ctypes.data, a.nbytes, dtype, scale)
+        if rc != 0:
+            raise ValueError(f"set_tensor({layer}, {name}) failed: {rc}")
+
+    def tensor_ptr(self, layer: int, name: str) -> int:
+        return self.lib.c.cccc_decode_tensor_data(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name)))
+
+    def load(self, model: dict, fp8_dtype: int = 5) -> None:
+        """model: the dict layout of oracle.decode_oracle.make_model (uint8 codes / uint16 bf16 bits)."""
+        for name in GLOBAL_TENSORS:
+            self.set_tensor(0, name, model[name], fp8_dtype if name in QUANTIZED else 3)
+        for li, L in enumerate(model["layers"]):
+            for name in LAYER_TENSORS:
+                self.set_tensor(li, name, L[name], fp8_dtype if name in QUANTIZED else 3)
+
+    def reset(self, token: int, pos: int) -> None:
+        assert self.lib.c.cccc_decode_reset(self.handle, token, pos) == 0
+
+    def step(self) -> int:
+        rc = self.lib.c.cccc_decode_step(self.handle)
+        if rc != 0:
+            raise RuntimeError(f"decode step failed: {rc}")
+        return self.token
+
+    def run(self, n_steps: int, use_graph: bool) -> float:
+        ms = float(self.lib.c.cccc_decode_run(self.handle, n_steps, 1 if use_graph else 0))
+        if ms < 0:
+            raise RuntimeError(f"decode run failed: {ms}")
+        return ms
+
+    @property
+    def token(self) -> int:
+        return self.lib.c.cccc_decode_token(self.handle)
+
+    @property
+    def pos(self) -> int:
+        return self.lib.c.cccc_decode_pos(self.handle)
+
+    def logits(self) -> np.ndarray:
+        out = np.empty(self.cfg["vocab"], dtype=np.uint16)
+        assert self.lib.c.cccc_decode_logits(self.handle, out.ctypes.data, out.nbytes) == 0
+        return out
+
+    def kv(self, layer: int, is_v: bool) -> np.ndarray:
+        c = self.cfg
+        out = np.empty((c["n_kv"], c["t_kv"], c["head_dim"]), dtype=np.uint16)
+        assert self.lib.c.cccc_decode_kv(self.handle, layer, 1 if is_v else 0, out.ctypes.data, out.nbytes) == 0
+        return out
+
+    def cos_table(self) -> np.ndarray:
+        c = self.cfg
+        out = np.empty((c["t_kv"], c["head_dim"] // 2), dtype=np.uint16)
+        assert self.lib.c.cccc_decode_cos_table(self.handle, out.ctypes.data, out.nbytes) == 0
+        return out
+
+    @property
+    def weight_bytes(self) -> int:
+        return int(self.lib.c.cccc_decode_weight_bytes(self.handle))

@@ -108,10 +108,76 @@ C_EXPORT unsigned long long hip_quant_tiled_size(int type, int n_out, int K);
 C_EXPORT int hip_quant_weight_prepare(const void* W, int type, int n_out, int K, int ldw, void* dst_tiled);
 C_EXPORT int hip_quant_weight_release(const void* W);
 
+/* ------------------------------------------------------------------------------------------------
+ * Decode-step neighbours of the linear (BF16 activations, one new token).
+ *
+ * hip_rms_norm_fwd, hip_rope_fwd and hip_embed_fwd keep the reference's signatures
+ * (cccc-hip/hip_functions.h:79-80, :91-94, :112-113) and semantics for type 3 (BF16); other types
+ * return 1 with a message, as the reference does for unsupported types.  hip_embed_fwd reads float ids.
+ */
+C_EXPORT int hip_rms_norm_fwd(int type, void* X, void* Y, void* scale, void* invstd_out,
+                              unsigned int outer, unsigned int inner, float epsilon);
+C_EXPORT int hip_rope_fwd(int type, const void* X, void* Y, const void* cos_tab, const void* sin_tab,
+                          unsigned int D, unsigned int T, unsigned int B, unsigned int pos_offset);
+C_EXPORT int hip_embed_fwd(int type, const void* ids, const void* W, void* Y, int D, int T, int B);
+
+/*
+ * Fused pieces of a Qwen3-style decode step (no single counterpart in the reference, which runs the
+ * graph op by op: scripts/convert_weights.py:488-692, cccc/MatrixOp.cpp:104-280).  Each keeps the
+ * rounding points of the ops it replaces: every intermediate the reference stores as a BF16 tensor
+ * is rounded to BF16 here too.  The step position and the current token id live in device memory
+ * (`d_pos`, `d_token`: one int32 each) so that a step is a fixed launch sequence.
+ */
+
+/* y_s = W_s * [rmsnorm](x) for 1..3 FP8 weights sharing x (q/k/v), or the SwiGLU pair
+ * y = bf16(silu(W[0] x) * (W[1] x)) with silu(g) = bf16(g * bf16(sigmoid g)); optional residual
+ * y = bf16(y + residual) on W[0]'s output.  Weights are [n_out][K], K contiguous, K % 16 == 0. */
+typedef struct hip_fused_linear
+{
+    int w_type;              /* 4 (FP8_E4M3) or 5 (FP8_E5M2) */
+    int K;
+    int n_segments;          /* 1..3; 2 when pair != 0 */
+    int pair;                /* 1: SwiGLU pair of W[0] (gate) and W[1] (up), both n_out[0] rows, into Y[0] */
+    const void* W[3];
+    int n_out[3];
+    float w_scale[3];        /* per-tensor dequant multipliers (1.0f when absent) */
+    void* Y[3];              /* bf16 [n_out[s]] */
+    const void* X;           /* bf16 [K] */
+    const void* norm_weight; /* bf16 [K] or NULL */
+    float norm_eps;
+    const void* residual;    /* bf16 [n_out[0]] or NULL */
+} hip_fused_linear;
+C_EXPORT int hip_quant_linear_fused(const hip_fused_linear* desc);
+
+/* Per-head RMSNorm of q and k, RoPE at row *d_pos of the tables, append of k and v to the caches
+ * (layout [kv_head][t_kv][128], the reference's (128, T_kv, 1, Hkv) cache).  head_dim is 128. */
+C_EXPORT int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v,
+                                      const void* q_norm_w, const void* k_norm_w,
+                                      const void* cos_tab, const void* sin_tab,
+                                      void* q_out, void* k_cache, void* v_cache,
+                                      int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                      const void* d_pos, float epsilon);
+
+/* GQA attention of one query token over cache rows 0..*d_pos: scores rounded to BF16, FP32 softmax,
+ * BF16 probabilities, y = bf16(V p).  Workspaces (caller-owned): scores_ws bf16 [n_q_heads][t_kv],
+ * partial_ws float [n_splits][n_q_heads][128].  n_q_heads / n_kv_heads must be 1, 2 or 4. */
+C_EXPORT int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* y,
+                                       void* scores_ws, void* partial_ws,
+                                       int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                       const void* d_pos, int n_splits);
+
+/* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
+C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);
+
+/* Arg-max of n BF16 values (lowest index on ties) into *d_index (int32, device); when d_pos is not
+ * NULL, *d_pos is incremented afterwards (the step counter of a decode loop). */
+C_EXPORT int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos);
+
 /*
  * Library controls (no counterpart in the reference, which always uses the null stream and always
  * synchronises: cccc-hip/hip_functions.cpp:32-42).
- *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch (parity/debug)
+ *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch (parity/debug);
+ *                             returns the previous setting
  *   hip_quant_set_stream(s) : enqueue on hipStream_t `s` (NULL = null stream)
  *   hip_quant_last_kernel() : name of the kernel family the last hip_quant_gemm call dispatched to
  *                             ("gemv_dot2", "gemv_mfma", "gemm_mfma", "generic", ...)

@@ -479,3 +479,20 @@ void orc_encode_e5m2_rne_bulk(const float* src, uint8_t* dst, size_t n)
 {
     for (size_t i = 0; i < n; i++) dst[i] = orc_float_to_e5m2_rne(src[i]);
 }
+
+/* ------------------------------------------------------------------ decode-step helpers */
+
+/* RoPE tables as the reference's graph builds them on the host (cccc/NetCifa.cpp:431-475): float32
+ * angle = t * powf(base, -2.0f * d / d_head), cosf / sinf, stored to BF16 by TRUNCATION (the host
+ * bfloat16(float) constructor drops the low 16 bits, cccc/types.h:43-48).  Layout [T][d_head / 2]. */
+void orc_rope_tables(int T, int d_head, float base, uint16_t* cos_out, uint16_t* sin_out)
+{
+    const int half = d_head / 2;
+    for (int t = 0; t < T; t++) {
+        for (int d = 0; d < half; d++) {
+            float angle = (float)t * powf(base, -2.0f * (float)d / (float)d_head);
+            cos_out[(size_t)t * half + d] = (uint16_t)(f32_bits(cosf(angle)) >> 16);
+            sin_out[(size_t)t * half + d] = (uint16_t)(f32_bits(sinf(angle)) >> 16);
+        }
+    }
+}

@@ -1,0 +1,230 @@
+"""Decode-step neighbours and the fused step against the CPU oracle (oracle/decode_oracle.py),
+through the C-ABI and the C++ DecodeModel."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import from_dev, to_dev
+
+pytestmark = pytest.mark.gpu
+
+BF16, E4M3, E5M2 = 3, 4, 5
+
+
+@pytest.fixture(scope="module")
+def dec():
+    from oracle import decode_oracle
+    return decode_oracle
+
+
+def ulp_close(got_bits, want_vals, ulps=1.0, floor=1e-6):
+    got = (got_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    want = np.asarray(want_vals, dtype=np.float64)
+    tol = ulps * np.maximum(np.abs(want), 2.0 ** -120) * 2.0 ** -8 + floor
+    return np.abs(got - want) <= tol
+
+
+def test_rms_norm_and_rope_match_the_oracle(gpu, oracle, dec):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(0)
+    for outer, inner in ((1, 4096), (40, 128), (3, 1000)):
+        x = oracle.f32_to_bf16((rng.standard_normal((outer, inner)) * 3).astype(np.float32))
+        w = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(inner)).astype(np.float32))
+        xd, wd = to_dev(torch, dev, x), to_dev(torch, dev, w)
+        yd = torch.zeros(outer * inner, dtype=torch.int16, device=dev)
+        inv = torch.zeros(outer, dtype=torch.float32, device=dev)
+        assert lib.c.hip_rms_norm_fwd(BF16, ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(yd.data_ptr()), ctypes.c_void_p(wd.data_ptr()),
+                                      ctypes.c_void_p(inv.data_ptr()), outer, inner, ctypes.c_float(1e-6)) == 0
+        want = dec.rms_norm(dec.f(x), dec.f(w), 1e-6)
+        got = from_dev(yd, np.uint16).reshape(outer, inner)
+        ok = ulp_close(got, want)
+        assert ok.all()
+        assert (got == oracle.f32_to_bf16(want)).mean() > 0.99          # bit-identical except rare rsqrt rounding flips
+        ms = (dec.f(x).astype(np.float64) ** 2).mean(axis=1)
+        assert np.allclose(inv.cpu().numpy(), 1 / np.sqrt(ms + 1e-6), rtol=1e-5)
+    assert lib.c.hip_rms_norm_fwd(0, None, None, None, None, 1, 16, ctypes.c_float(1e-6)) == 1
+    cfg = dec.DecodeConfig(t_kv=64)
+    cos, sin = dec.rope_tables(cfg)
+    x = oracle.f32_to_bf16(rng.standard_normal((6, 128)).astype(np.float32))
+    xd, cd, sd = to_dev(torch, dev, x), to_dev(torch, dev, cos), to_dev(torch, dev, sin)
+    for pos in (0, 1, 37, 63):
+        yd = torch.zeros(6 * 128, dtype=torch.int16, device=dev)
+        assert lib.c.hip_rope_fwd(BF16, ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(yd.data_ptr()), ctypes.c_void_p(cd.data_ptr()),
+                                  ctypes.c_void_p(sd.data_ptr()), 128, 1, 6, pos) == 0
+        want = dec.rope(dec.f(x), dec.f(cos[pos]), dec.f(sin[pos]))
+        assert ulp_close(from_dev(yd, np.uint16).reshape(6, 128), want).all(), pos
+    assert lib.c.hip_rope_fwd(BF16, None, None, None, None, 127, 1, 1, 0) == 1
+
+
+def fused_desc(pkg, **kw):
+    lib = pkg.library()
+    d = pkg.capi.FusedLinear()
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_fused_linear_variants(gpu, pkg, oracle, dec):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(1)
+    K, n0, n1, n2 = 2048, 512, 128, 130
+    x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+    nw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    Ws = [oracle.encode_e5m2_rne((rng.standard_normal((n, K)) * 0.02).astype(np.float32)) for n in (n0, n1, n2)]
+    Wd = [oracle.dequant_fp8_to_bf16(W, oracle.E5M2).reshape(W.shape) for W in Ws]
+    xd, nwd = to_dev(torch, dev, x), to_dev(torch, dev, nw)
+    wds = [to_dev(torch, dev, W) for W in Ws]
+    xn = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6)
+
+    def run(desc, outs):
+        assert lib.quant_linear_fused(desc) == 0
+        assert lib.last_kernel() == "gemv_fused"
+        return [from_dev(o_, np.uint16) for o_ in outs]
+
+    # (1) norm + three segments
+    ys = [torch.zeros(n + 8, dtype=torch.int16, device=dev) for n in (n0, n1, n2)]
+    d = pkg.capi.make_fused_linear(E5M2, K, [w.data_ptr() for w in wds], [n0, n1, n2], [y.data_ptr() for y in ys], xd.data_ptr(),
+                                   norm_weight=nwd.data_ptr(), norm_eps=1e-6)
+    outs = run(d, ys)
+    for s, n in enumerate((n0, n1, n2)):
+        assert not outs[s][n:].any()
+        want = dec.linear(Wd[s], xn)
+        assert ulp_close(outs[s][:n], want, ulps=1.0, floor=2e-5).all(), s
+    # (2) plain single segment with residual and a per-tensor scale
+    res = oracle.f32_to_bf16(rng.standard_normal(n0).astype(np.float32))
+    rd = to_dev(torch, dev, res)
+    y = torch.zeros(n0, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(E5M2, K, [wds[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr(), scales=[0.5], residual=rd.data_ptr())
+    out, = run(d, [y])
+    lin = dec.linear(oracle.dequant_fp8_to_bf16(Ws[0], oracle.E5M2, 0.5).reshape(n0, K), dec.f(x))
+    assert ulp_close(out, dec.r(lin + dec.f(res)), ulps=1.0, floor=2e-5).all()
+    # (3) SwiGLU pair with norm: gate = W0, up = another n0-row weight
+    Wu = oracle.encode_e5m2_rne((rng.standard_normal((n0, K)) * 0.02).astype(np.float32))
+    wud = to_dev(torch, dev, Wu)
+    y = torch.zeros(n0, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(E5M2, K, [wds[0].data_ptr(), wud.data_ptr()], [n0, n0], [y.data_ptr(), None], xd.data_ptr(),
+                                   norm_weight=nwd.data_ptr(), norm_eps=1e-6, pair=True)
+    out, = run(d, [y])
+    gate = dec.linear(Wd[0], xn)
+    up = dec.linear(oracle.dequant_fp8_to_bf16(Wu, oracle.E5M2).reshape(n0, K), xn)
+    want = dec.silu_mul(gate, up)
+    # the product of two rounded factors moves by up to ~2 ulp when a factor flips by one
+    assert ulp_close(out, want, ulps=3.0, floor=1e-4).all()
+    assert (out == oracle.f32_to_bf16(want)).mean() > 0.97
+    # rejected descriptors
+    bad = pkg.capi.make_fused_linear(E5M2, 24, [wds[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr())
+    assert lib.quant_linear_fused(bad) == -1
+    bad = pkg.capi.make_fused_linear(6, K, [wds[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr())
+    assert lib.quant_linear_fused(bad) == -1
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(4, 2), (8, 2), (2, 2)])
+def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(2)
+    t_kv = 200
+    q = oracle.f32_to_bf16(rng.standard_normal((n_q, 128)).astype(np.float32))
+    kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    qd, kd, vd = to_dev(torch, dev, q), to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+    n_splits = 8
+    scores = torch.zeros(n_q * t_kv, dtype=torch.int16, device=dev)
+    partial = torch.zeros(n_splits * n_q * 128, dtype=torch.float32, device=dev)
+    for pos in (0, 1, 63, 64, 130, 199):
+        pd = torch.tensor([pos], dtype=torch.int32, device=dev)
+        y = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        rc = lib.c.hip_attention_decode_bf16(ctypes.c_void_p(qd.data_ptr()), ctypes.c_void_p(kd.data_ptr()), ctypes.c_void_p(vd.data_ptr()),
+                                             ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(scores.data_ptr()), ctypes.c_void_p(partial.data_ptr()),
+                                             n_q, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr()), n_splits)
+        assert rc == 0
+        want = dec.attention(dec.f(q), dec.f(kc), dec.f(vc), pos, n_q, n_kv)
+        got = from_dev(y, np.uint16).reshape(n_q, 128)
+        assert ulp_close(got, want, ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), pos
+        # the BF16 scores themselves (pass 1) are the reference's rounding point
+        s = dec.f(from_dev(scores, np.uint16).reshape(n_q, t_kv)[:, :pos + 1])
+        for h in range(n_q):
+            ref = dec.r(np.float32(1 / np.sqrt(np.float32(128))) * (dec.f(kc)[h // (n_q // n_kv), :pos + 1].astype(np.float64) @ dec.f(q)[h].astype(np.float64)).astype(np.float32))
+            assert ulp_close(oracle.f32_to_bf16(s[h]), ref, ulps=1.0, floor=1e-5).all()
+
+
+def test_argmax_and_embed(gpu, oracle):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(3)
+    x = oracle.f32_to_bf16(rng.standard_normal(151936).astype(np.float32))
+    x[[777, 90000]] = 0x4120                                   # two equal maxima (10.0): the lower index wins
+    xd = to_dev(torch, dev, x)
+    st = torch.tensor([0, 41], dtype=torch.int32, device=dev)
+    assert lib.c.hip_argmax_bf16(ctypes.c_void_p(xd.data_ptr()), 151936, ctypes.c_void_p(st.data_ptr()), ctypes.c_void_p(st.data_ptr() + 4)) == 0
+    assert st.cpu().tolist() == [777, 42]
+    W = oracle.f32_to_bf16(rng.standard_normal((50, 256)).astype(np.float32))
+    wd = to_dev(torch, dev, W)
+    y = torch.zeros(256, dtype=torch.int16, device=dev)
+    tok = torch.tensor([17], dtype=torch.int32, device=dev)
+    assert lib.c.hip_embed_token_bf16(ctypes.c_void_p(tok.data_ptr()), ctypes.c_void_p(wd.data_ptr()), ctypes.c_void_p(y.data_ptr()), 256, 50) == 0
+    assert np.array_equal(from_dev(y, np.uint16), W[17])
+    ids = torch.tensor([3.0, 49.0], dtype=torch.float32, device=dev)
+    y2 = torch.zeros(2 * 256, dtype=torch.int16, device=dev)
+    assert lib.c.hip_embed_fwd(BF16, ctypes.c_void_p(ids.data_ptr()), ctypes.c_void_p(wd.data_ptr()), ctypes.c_void_p(y2.data_ptr()), 256, 2, 1) == 0
+    assert np.array_equal(from_dev(y2, np.uint16).reshape(2, 256), W[[3, 49]])
+
+
+@pytest.fixture(scope="module")
+def small_model(gpu, pkg, dec):
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=64)
+    weights = dec.make_model(cfg, 11)
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    model.load(weights)
+    return cfg, weights, model
+
+
+def test_rope_tables_of_the_host_model(small_model, dec):
+    cfg, _, model = small_model
+    cos, _ = dec.rope_tables(cfg)
+    assert np.array_equal(model.cos_table(), cos)
+
+
+def test_decode_steps_follow_the_oracle(small_model, oracle, dec):
+    cfg, weights, model = small_model
+    orc = dec.DecodeOracle(cfg, weights)
+    token = 5
+    agree = 0
+    for pos in range(12):
+        model.reset(token, pos)
+        got_token = model.step()
+        assert model.pos == pos + 1
+        want_logits, want_token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        err = np.linalg.norm(got - want_logits) / np.linalg.norm(want_logits)
+        assert err < 1e-2, (pos, err)
+        assert np.abs(got - want_logits).max() <= 2e-2 * np.abs(want_logits).max()
+        # the caches hold the rotated keys / raw values of this position
+        for li in range(cfg.layers):
+            assert ulp_close(model.kv(li, False)[:, pos], orc.k[li, :, pos], ulps=2.0, floor=2e-3).all()
+            assert ulp_close(model.kv(li, True)[:, pos], orc.v[li, :, pos], ulps=2.0, floor=2e-3).all()
+        # greedy token: identical unless the oracle's top two logits are within the error
+        top2 = np.sort(want_logits)[-2:]
+        if top2[1] - top2[0] > 2 * np.abs(got - want_logits).max():
+            assert got_token == want_token, pos
+            agree += 1
+        token = want_token
+    assert agree >= 8
+
+
+def test_graph_replay_equals_eager_steps(small_model, dec):
+    cfg, _, model = small_model
+    model.reset(3, 0)
+    eager = []
+    for _ in range(10):
+        eager.append(model.step())
+    logits_eager = model.logits().copy()
+    model.reset(3, 0)
+    assert model.run(10, True) > 0                       # one captured step replayed ten times
+    assert model.pos == 10
+    assert model.token == eager[-1]
+    assert np.array_equal(model.logits(), logits_eager)
+    model.reset(3, 0)
+    assert model.run(10, False) > 0
+    assert model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
