@@ -1,19 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X weight-only quantized linear path (one GPU).
 
-A step is one pass of the hot path over one batch of synthetic input.  Default workload: the
-linear layers of one Qwen3-8B W8A16 decode token at batch 1 -- 36 layers x (q, k, v, o, gate, up,
-down) + lm_head = 253 FP8_E5M2 GEMVs over 7,568,097,280 bytes of distinct, HBM-resident weights --
-issued through the C++ host mirror's Matrix::mulBatched exactly as cccc's graph issues them.
-`value` = algorithmic bytes (K*N + 2*M*K + 2*M*N per GEMV) / elapsed.
+A step is one pass of the hot path over one batch of synthetic input.  Default workload
+(`decode_step`): one greedy batch-1 decode step of a random-init Qwen3-8B-shaped W8A16 model -- 36
+layers, FP8_E5M2 linears, BF16 activations and KV cache holding 4096 positions -- run by the C++
+DecodeModel on the fused kernels; `value` = tokens per second.  The same line then carries the GEMV
+half of the metric: the 253 linears of one token issued through Matrix::mulBatched exactly as
+cccc's graph issues them (`quant_gemv`), the per-shape sweep over M in {1, 4, 16} (`sweep`) and the
+FP4 block-scale sweep (`fp4_sweep`); GB/s figures are algorithmic bytes (K*N + 2*M*K + 2*M*N per
+GEMV) / elapsed.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_linears|gemv|prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_linears|gemv|prefill]
                     [--shape K,N] [--tokens M] [--no-graph] [--no-cpu] [--no-sweep]
 
-Prints ONE JSON line.  `roofline` is measured live on the dominant kernel (the gate/up-shaped
-GEMV, K=4096 N=12288) with HIP events on the stream it runs on; `cpu_baseline` times the CPU
-restatement of the reference's CPU route (scalar dequant of the whole weight + cblas_sgemm) on a
-bounded sample.
+Prints ONE JSON line.  `roofline` is measured live on the dominant kernel (the fused RMSNorm +
+gate/up SwiGLU GEMV for decode_step, the gate/up-shaped GEMV K=4096 N=12288 for decode_linears)
+with HIP events on the stream it runs on; `cpu_baseline` times the CPU restatement of the
+reference's CPU route (scalar dequant of the whole weight + cblas_sgemm) on a bounded sample.
 """
 from __future__ import annotations
 
@@ -32,6 +35,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM bytes per launch of the gate/up-shaped GEMV (K=4096, N=12288, M=1) from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99983 and 1.0)
 GEMV_GATE_UP_TRAFFIC_BYTES = 50503552
+# the same two counters for one launch of the fused RMSNorm + gate/up SwiGLU GEMV (two 4096 x 12288 weights); None until measured
+GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = None
 
 FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
 
@@ -105,6 +110,58 @@ def build_decode_model(ws: Workspace, tokens: int):
         add(c["inter"], c["hidden"], x_i, y[c["q_out"]])          # down
     add(c["hidden"], c["vocab"], x_h, y[c["vocab"]])              # lm_head
     return ops, by_shape
+
+
+DECODE_CTX = 4096
+
+
+def build_decode_step(ws: Workspace, ctx: int):
+    """The full random-init Qwen3-8B W8A16 model of the C++ DecodeModel, tensors generated on the GPU:
+    FP8_E5M2 linears from N(0, 0.02) (bf16, then round to nearest), norms near 1, BF16 embedding and
+    a KV cache already holding `ctx` positions of N(0, 1) keys and values."""
+    t, c = ws.torch, QWEN3_8B
+    model = ws.pkg.host_api.DecodeModel(ws.host, c["layers"], c["hidden"], 32, 8, 128, c["inter"], c["vocab"], ctx)
+
+    def fill_fp8(ptr, n_out, K):
+        rows = max(1, min(n_out, (1 << 27) // K))
+        for r0 in range(0, n_out, rows):
+            r = min(rows, n_out - r0)
+            w = (t.randn(r, K, device=ws.dev, generator=ws.gen) * 0.02).to(t.bfloat16).to(t.float8_e5m2)
+            assert ws.lib.convert(w.data_ptr(), E5M2, ptr + r0 * K, E5M2, r * K, 1.0) == 0
+            t.cuda.synchronize()
+
+    def fill_bf16(ptr, n, mean, std):
+        step = 1 << 26
+        for i0 in range(0, n, step):
+            m = min(step, n - i0)
+            v = (t.randn(m, device=ws.dev, generator=ws.gen) * std + mean).to(t.bfloat16)
+            assert ws.lib.convert(v.data_ptr(), BF16, ptr + i0 * 2, BF16, m * 2, 1.0) == 0
+            t.cuda.synchronize()
+
+    shapes = {"wq": (c["q_out"], c["hidden"]), "wk": (c["kv_out"], c["hidden"]), "wv": (c["kv_out"], c["hidden"]),
+              "wo": (c["hidden"], c["q_out"]), "w_gate": (c["inter"], c["hidden"]), "w_up": (c["inter"], c["hidden"]),
+              "w_down": (c["hidden"], c["inter"])}
+    for li in range(c["layers"]):
+        for name, (n_out, K) in shapes.items():
+            fill_fp8(model.tensor_ptr(li, name), n_out, K)
+        for name, n in (("rms_attn", c["hidden"]), ("rms_ffn", c["hidden"]), ("q_norm", 128), ("k_norm", 128)):
+            fill_bf16(model.tensor_ptr(li, name), n, 1.0, 0.1)
+        for is_v in (False, True):
+            fill_bf16(model.kv_ptr(li, is_v), 8 * ctx * 128, 0.0, 1.0)
+    fill_fp8(model.tensor_ptr(0, "lm_head"), c["vocab"], c["hidden"])
+    fill_bf16(model.tensor_ptr(0, "rms_final"), c["hidden"], 1.0, 0.1)
+    fill_bf16(model.tensor_ptr(0, "emb"), c["vocab"] * c["hidden"], 0.0, 1.0)
+    return model
+
+
+def decode_step_bytes(ctx_mean: float) -> int:
+    """Bytes one decode step must move: every linear weight once, the keys and values of the positions
+    attended to, the embedding row, the norm weights and the logits."""
+    c = QWEN3_8B
+    weights = c["layers"] * (c["hidden"] * (c["q_out"] + 2 * c["kv_out"]) + c["q_out"] * c["hidden"] + 3 * c["hidden"] * c["inter"]) + c["hidden"] * c["vocab"]
+    kv = int(c["layers"] * 2 * c["kv_out"] * 2 * ctx_mean)
+    small = c["layers"] * 2 * (2 * c["hidden"] + 128) + 2 * c["hidden"] * 2 + c["vocab"] * 2
+    return weights + kv + small
 
 
 def time_chain(ws, ops, steps, warmup, use_graph):
@@ -202,7 +259,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode_linears", choices=["decode_linears", "gemv", "prefill", "copy"])
+    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--no-graph", action="store_true")
@@ -235,7 +292,50 @@ def main():
     use_graph = not args.no_graph
     extra = {}
 
-    if args.workload == "decode_linears":
+    metric, unit = "quant GEMV HBM GB/s (Qwen3-8B W8A16 decode linears, bs=1)", "GB/s"
+    if args.workload == "decode_step":
+        # full decode step: tokens / s at context DECODE_CTX; then the GEMV half of the metric on the
+        # same shapes through Matrix::mulBatched (decode linears chain and the per-shape sweep)
+        if args.steps + args.warmup > DECODE_CTX:
+            sys.exit("bench.py: --steps + --warmup must not exceed the context length")
+        model = build_decode_step(ws, DECODE_CTX)
+        start = DECODE_CTX - args.steps - args.warmup
+        torch.cuda.synchronize()
+        model.reset(1, start)
+        if args.warmup:
+            model.run(args.warmup, use_graph)
+        ms = model.run(args.steps, use_graph)
+        assert model.pos == DECODE_CTX
+        model.reset(1, start + args.warmup)
+        ms_other = model.run(args.steps, not use_graph)
+        ms_step = ms / args.steps
+        value = 1000.0 / ms_step
+        metric, unit = "decode tok/s Qwen3-8B W8A16 bs=1", "tok/s"
+        step_bytes = decode_step_bytes(DECODE_CTX - (args.steps - 1) / 2.0)
+        extra["launch_mode"] = "hipGraph" if use_graph else "stream"
+        extra["ms_per_step_" + ("stream" if use_graph else "hipGraph")] = round(ms_other / args.steps, 4)
+        extra["bytes_per_token"] = step_bytes
+        extra["decode_step_GBps"] = round(step_bytes / ms_step * 1e-6, 1)
+        extra["decode_step_frac_of_hbm_bound"] = round(step_bytes / ms_step * 1e-6 / HBM_PEAK_GBS, 4)
+        extra["launches_per_step"] = 9 * QWEN3_8B["layers"] + 4
+        extra["last_token"] = model.token
+        workload = ("full random-init Qwen3-8B W8A16 decode step, batch 1, greedy: 36 layers, hidden 4096, 32 q / 8 kv heads x 128, qk RMSNorm, "
+                    f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions")
+        # dominant kernel: the fused RMSNorm + gate/up SwiGLU launch (two 4096 x 12288 weights), timed over the 36 layers' distinct weights
+        K, N, M = 4096, 2 * 12288, 1
+        dom_us = model.bench_gate_up(10)
+        dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
+        if not args.no_sweep:
+            del model
+            torch.cuda.empty_cache()
+            ops, by_shape = build_decode_model(ws, 1)
+            lin_bytes = sum(gemv_bytes(k, n, 1) for *_, k, n in ops)
+            lin_ms = time_chain(ws, ops, args.steps, args.warmup, use_graph) / args.steps
+            extra["quant_gemv"] = {"workload": "the 253 FP8_E5M2 linears of one decode token through Matrix::mulBatched", "ms_per_step": round(lin_ms, 4),
+                                   "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
+            extra["sweep"] = shape_sweep(ws, by_shape, (1, 4, 16), False)
+            extra["fp4_sweep"] = fp4_sweep(ws)
+    elif args.workload == "decode_linears":
         ops, by_shape = build_decode_model(ws, 1)
         step_bytes = sum(gemv_bytes(K, N, 1) for *_, K, N in ops)
         torch.cuda.synchronize()
@@ -274,8 +374,14 @@ def main():
         extra["launch_mode"] = "stream"
         workload = f"{args.workload} K={K} N={N} M={M} over {n_w} distinct FP8_E5M2 weights"
 
-    assert ws.lib.linear(ops[0][0].data_ptr, E5M2, ops[0][1].data_ptr, ops[0][2].data_ptr, ops[0][4], M if args.workload != "decode_linears" else 1, ops[0][3]) == 0
-    if args.workload == "prefill":
+    if args.workload != "decode_step":
+        assert ws.lib.linear(ops[0][0].data_ptr, E5M2, ops[0][1].data_ptr, ops[0][2].data_ptr, ops[0][4], M if args.workload != "decode_linears" else 1, ops[0][3]) == 0
+    if args.workload == "decode_step":
+        achieved = dom_bytes / dom_us * 1e-3
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    "traffic": GEMV_FUSED_GATE_UP_TRAFFIC_BYTES, "kernel": "gemv8_fused_kernel (RMSNorm + gate/up SwiGLU pair)",
+                    "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3), "bytes_per_launch": dom_bytes}
+    elif args.workload == "prefill":
         flops = 2.0 * M * K * N
         achieved = flops / dom_us * 1e-6
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -290,13 +396,14 @@ def main():
                     "bytes_per_launch": gemv_bytes(K, N, M)}
 
     line = {
-        "metric": "quant GEMV HBM GB/s (Qwen3-8B W8A16 decode linears, bs=1)" if args.workload != "prefill" else "W8A16 prefill GEMM algorithmic GB/s",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": metric if args.workload != "prefill" else "W8A16 prefill GEMM algorithmic GB/s",
+        "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
     }
+    if unit == "GB/s":
+        line["frac_of_hbm_peak"] = round(value / HBM_PEAK_GBS, 4)
     if not args.no_cpu:
         threads = min(16, len(os.sched_getaffinity(0)))
         line["cpu_baseline"] = cpu_baseline(pkg, threads)

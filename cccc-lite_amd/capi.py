@@ -54,6 +54,8 @@ EXPORTS = (
     "hip_embed_token_bf16",
     "hip_qk_norm_rope_kv_bf16",
     "hip_attention_decode_bf16",
+    "hip_attention_decode_workspace_bytes",
+    "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
@@ -111,9 +113,13 @@ class QuantLibrary:
         L.hip_qk_norm_rope_kv_bf16.restype = i32
         L.hip_qk_norm_rope_kv_bf16.argtypes = [vp] * 10 + [i32, i32, i32, i32, vp, f32]
         L.hip_attention_decode_bf16.restype = i32
-        L.hip_attention_decode_bf16.argtypes = [vp] * 6 + [i32, i32, i32, i32, vp, i32]
+        L.hip_attention_decode_bf16.argtypes = [vp] * 5 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp]
+        L.hip_attention_decode_workspace_bytes.restype = ctypes.c_ulonglong
+        L.hip_attention_decode_workspace_bytes.argtypes = [i32, i32, i32]
+        L.hip_argmax_workspace_bytes.restype = ctypes.c_ulonglong
+        L.hip_argmax_workspace_bytes.argtypes = [u32]
         L.hip_argmax_bf16.restype = i32
-        L.hip_argmax_bf16.argtypes = [vp, u32, vp, vp]
+        L.hip_argmax_bf16.argtypes = [vp, u32, vp, vp, vp]
         L.hip_quant_set_sync.restype = i32
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32

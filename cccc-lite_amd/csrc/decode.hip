@@ -133,43 +133,79 @@ int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v, const 
     return finish("qk_norm_rope_kv");
 }
 
-int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* y, void* scores_ws, void* partial_ws,
-                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, int n_splits)
+namespace
 {
-    if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || n_splits <= 0 || !d_pos) { return -1; }
-    const int group = n_q_heads / n_kv_heads;
-    const float scale = 1.0f / sqrtf((float)head_dim);
-    const dim3 grid_s((t_kv + 63) / 64, n_kv_heads), grid_p(n_splits, n_kv_heads);
+
+struct AttentionWorkspace
+{
+    size_t scores, stats, partial, total;
+    int n_blocks;
+};
+
+AttentionWorkspace attention_workspace(int n_q_heads, int t_kv)
+{
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    AttentionWorkspace w{};
+    w.n_blocks = (t_kv + ATT_KEYS - 1) / ATT_KEYS;
+    w.scores = 0;
+    w.stats = up(w.scores + (size_t)n_q_heads * t_kv * 2);
+    w.partial = up(w.stats + (size_t)n_q_heads * w.n_blocks * sizeof(float2));
+    w.total = up(w.partial + (size_t)w.n_blocks * n_q_heads * 128 * sizeof(float));
+    return w;
+}
+
+template <int G>
+void launch_attention(const uint16_t* q, const uint16_t* kc, const uint16_t* vc, uint16_t* y, char* ws, const AttentionWorkspace& w,
+                      int n_q_heads, int n_kv_heads, int t_kv, const int* pos)
+{
+    const dim3 grid(w.n_blocks, n_kv_heads);
+    uint16_t* scores = (uint16_t*)(ws + w.scores);
+    float2* stats = (float2*)(ws + w.stats);
+    float* partial = (float*)(ws + w.partial);
+    attn_scores_kernel<G><<<grid, 256, 0, stream()>>>(q, kc, scores, stats, t_kv, w.n_blocks, pos, 1.0f / sqrtf(128.0f));
+    attn_pv_kernel<G><<<grid, 256, 0, stream()>>>(scores, stats, vc, partial, t_kv, w.n_blocks, pos, n_q_heads);
+    const int n_out = n_q_heads * 128;
+    attn_combine_kernel<<<(n_out + 63) / 64, 256, 0, stream()>>>(partial, y, n_out, t_kv, pos);
+}
+
+}    // namespace
+
+unsigned long long hip_attention_decode_workspace_bytes(int n_q_heads, int n_kv_heads, int t_kv)
+{
+    if (n_q_heads <= 0 || n_kv_heads <= 0 || t_kv <= 0) { return 0; }
+    return attention_workspace(n_q_heads, t_kv).total;
+}
+
+int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* y, void* workspace, unsigned long long workspace_bytes,
+                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos)
+{
+    if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || !d_pos) { return -1; }
+    if (!q || !k_cache || !v_cache || !y || !workspace || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace)) { return -1; }
+    const AttentionWorkspace w = attention_workspace(n_q_heads, t_kv);
+    if (workspace_bytes < w.total) { return -1; }
     const uint16_t* qp = (const uint16_t*)q;
     const uint16_t* kc = (const uint16_t*)k_cache;
     const uint16_t* vc = (const uint16_t*)v_cache;
-    uint16_t* sw = (uint16_t*)scores_ws;
-    float* pw = (float*)partial_ws;
     const int* pos = (const int*)d_pos;
-    switch (group)
+    switch (n_q_heads / n_kv_heads)
     {
-    case 1:
-        attn_scores_kernel<1><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
-        attn_pv_kernel<1><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
-        break;
-    case 2:
-        attn_scores_kernel<2><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
-        attn_pv_kernel<2><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
-        break;
-    case 4:
-        attn_scores_kernel<4><<<grid_s, 256, 0, stream()>>>(qp, kc, sw, t_kv, pos, scale);
-        attn_pv_kernel<4><<<grid_p, 256, 0, stream()>>>(sw, vc, pw, t_kv, pos, n_splits, n_q_heads);
-        break;
+    case 1: launch_attention<1>(qp, kc, vc, (uint16_t*)y, (char*)workspace, w, n_q_heads, n_kv_heads, t_kv, pos); break;
+    case 2: launch_attention<2>(qp, kc, vc, (uint16_t*)y, (char*)workspace, w, n_q_heads, n_kv_heads, t_kv, pos); break;
+    case 4: launch_attention<4>(qp, kc, vc, (uint16_t*)y, (char*)workspace, w, n_q_heads, n_kv_heads, t_kv, pos); break;
     default: return -1;
     }
-    const int n = n_q_heads * head_dim;
-    sum_partials_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(pw, (uint16_t*)y, n_splits, n);
     return finish("attention_decode");
 }
 
-int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos)
+unsigned long long hip_argmax_workspace_bytes(unsigned int n) { return (unsigned long long)((n + ARGMAX_PER_BLOCK - 1) / ARGMAX_PER_BLOCK) * 8; }
+
+int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos, void* workspace)
 {
-    if (!x || !d_index || n == 0) { return -1; }
-    argmax_bf16_kernel<<<1, 1024, 0, stream()>>>((const uint16_t*)x, n, (int*)d_index, (int*)d_pos);
+    if (!x || !d_index || !workspace || n == 0) { return -1; }
+    const unsigned blocks = (n + ARGMAX_PER_BLOCK - 1) / ARGMAX_PER_BLOCK;
+    float* cand_v = (float*)workspace;
+    unsigned* cand_i = (unsigned*)workspace + blocks;
+    argmax_blocks_kernel<<<blocks, 256, 0, stream()>>>((const uint16_t*)x, n, cand_v, cand_i);
+    argmax_pick_kernel<<<1, 256, 0, stream()>>>(cand_v, cand_i, blocks, (int*)d_index, (int*)d_pos);
     return finish("argmax_bf16");
 }

@@ -103,95 +103,146 @@ __device__ __forceinline__ void stage_decode_activation(const FusedLinearArgs& a
     __syncthreads();
 }
 
+// One wave owns a group of two rows at a time and walks its groups in batches of U KiB per row.  The
+// weights of the next batch are requested before the current one is consumed, and those of the very
+// first batch before the activation is staged, so the norm prologue and every reduction overlap loads.
+struct FusedRows
+{
+    const uint8_t *w0, *w1;
+    float s0, s1;
+    int seg, row0, row1;
+};
+
 template <int WT, int U, int WAVES, bool SCALED>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLinearArgs a)
 {
     extern __shared__ u32x4 xs[];
     __shared__ float red[WAVES];
-    stage_decode_activation<WAVES * 64>(a, xs, red);
-
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_steps = (a.K + 1023) / 1024;
+    const int batches = (n_steps + U - 1) / U;
     // row groups of two: in pair mode (gate row i, up row i); otherwise two consecutive rows of one segment
     const int g0 = a.pair ? a.n_out[0] : (a.n_out[0] + 1) / 2;
     const int g1 = (a.pair || a.n_segments < 2) ? g0 : g0 + (a.n_out[1] + 1) / 2;
     const int n_groups = (a.pair || a.n_segments < 3) ? g1 : g1 + (a.n_out[2] + 1) / 2;
+    const int stride = gridDim.x * WAVES;
 
-    for (int g = blockIdx.x * WAVES + wave; g < n_groups; g += gridDim.x * WAVES)
-    {
-        int seg = 0, row0, row1;
-        if (a.pair) { row0 = row1 = g; }
+    auto locate = [&](int g) {
+        FusedRows r;
+        r.seg = 0;
+        if (a.pair) { r.row0 = r.row1 = g; }
         else
         {
             int local = g;
-            if (g >= g1) { seg = 2; local = g - g1; }
-            else if (g >= g0) { seg = 1; local = g - g0; }
-            row0 = local * 2;
-            row1 = min(local * 2 + 1, a.n_out[seg] - 1);
+            if (g >= g1) { r.seg = 2; local = g - g1; }
+            else if (g >= g0) { r.seg = 1; local = g - g0; }
+            r.row0 = local * 2;
+            r.row1 = min(local * 2 + 1, a.n_out[r.seg] - 1);
         }
-        const uint8_t* w0 = a.W[a.pair ? 0 : seg] + (long long)row0 * a.K + lane * 16;
-        const uint8_t* w1 = a.W[a.pair ? 1 : seg] + (long long)row1 * a.K + lane * 16;
-        const float s0 = a.w_scale[a.pair ? 0 : seg], s1 = a.w_scale[a.pair ? 1 : seg];
-        float acc0 = 0.0f, acc1 = 0.0f;
-        for (int st0 = 0; st0 < n_steps; st0 += U)
-        {
-            u32x4 wa[U], wb[U];
+        const int sa = a.pair ? 0 : r.seg, sb = a.pair ? 1 : r.seg;
+        r.w0 = a.W[sa] + (long long)r.row0 * a.K;
+        r.w1 = a.W[sb] + (long long)r.row1 * a.K;
+        r.s0 = a.w_scale[sa];
+        r.s1 = a.w_scale[sb];
+        return r;
+    };
+    auto request = [&](const FusedRows& r, int st0, u32x4* wa, u32x4* wb) {
 #pragma unroll
-            for (int u = 0; u < U; u++)
+        for (int u = 0; u < U; u++)
+        {
+            wa[u] = wb[u] = u32x4{ 0u, 0u, 0u, 0u };
+            const int k = (st0 + u) * 1024 + lane * 16;
+            if (k < a.K)
             {
-                wa[u] = wb[u] = u32x4{ 0u, 0u, 0u, 0u };
-                if ((st0 + u) * 1024 + lane * 16 < a.K)
+                wa[u] = __builtin_nontemporal_load((const u32x4*)(r.w0 + k));
+                wb[u] = __builtin_nontemporal_load((const u32x4*)(r.w1 + k));
+            }
+        }
+    };
+
+    int g = blockIdx.x * WAVES + wave, batch = 0;
+    FusedRows cur{}, nxt{};
+    u32x4 wa[U], wb[U], na[U], nb[U];
+    if (g < n_groups)
+    {
+        cur = locate(g);
+        request(cur, 0, wa, wb);
+    }
+    stage_decode_activation<WAVES * 64>(a, xs, red);
+
+    float acc0 = 0.0f, acc1 = 0.0f;
+    while (g < n_groups)
+    {
+        int ng = g, nbatch = batch + 1;
+        if (nbatch == batches)
+        {
+            ng = g + stride;
+            nbatch = 0;
+        }
+        if (ng < n_groups)
+        {
+            nxt = nbatch == 0 ? locate(ng) : cur;
+            request(nxt, nbatch * U, na, nb);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int st = batch * U + u;
+            if (st < n_steps)
+            {
+                const u32x4 x0 = xs[(st * 2 + 0) * 64 + lane];
+                const u32x4 x1 = xs[(st * 2 + 1) * 64 + lane];
+#pragma unroll
+                for (int d = 0; d < 4; d++)
                 {
-                    wa[u] = __builtin_nontemporal_load((const u32x4*)(w0 + (st0 + u) * 1024));
-                    wb[u] = __builtin_nontemporal_load((const u32x4*)(w1 + (st0 + u) * 1024));
+                    const u32x4& xv = (d < 2) ? x0 : x1;
+                    bf16x2 p01, p23;
+                    fp8x4_to_bf16<WT, SCALED>(wa[u][d], cur.s0, p01, p23);
+                    acc0 = dot2_bf16(p01, xv[(d & 1) * 2 + 0], acc0);
+                    acc0 = dot2_bf16(p23, xv[(d & 1) * 2 + 1], acc0);
+                    fp8x4_to_bf16<WT, SCALED>(wb[u][d], cur.s1, p01, p23);
+                    acc1 = dot2_bf16(p01, xv[(d & 1) * 2 + 0], acc1);
+                    acc1 = dot2_bf16(p23, xv[(d & 1) * 2 + 1], acc1);
                 }
             }
-#pragma unroll
-            for (int u = 0; u < U; u++)
+        }
+        if (batch == batches - 1)
+        {
+            const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
+            acc0 = acc1 = 0.0f;
+            if (lane == 0)
             {
-                if (st0 + u < n_steps)
+                if (a.pair)
                 {
-                    const u32x4 x0 = xs[((st0 + u) * 2 + 0) * 64 + lane];
-                    const u32x4 x1 = xs[((st0 + u) * 2 + 1) * 64 + lane];
-#pragma unroll
-                    for (int d = 0; d < 4; d++)
+                    const float gate = bf16_round(t0), up = bf16_round(t1);
+                    const float sig = bf16_round(1.0f / (1.0f + expf(-gate)));
+                    const float silu = bf16_round(gate * sig);
+                    float out = bf16_round(silu * up);
+                    if (a.residual) { out = bf16_round(out + bf16_bits_to_f32(a.residual[g])); }
+                    a.Y[0][g] = (uint16_t)f32_to_bf16_bits(out);
+                }
+                else
+                {
+                    float o0 = bf16_round(t0), o1 = bf16_round(t1);
+                    if (a.residual && cur.seg == 0)
                     {
-                        const u32x4& xv = (d < 2) ? x0 : x1;
-                        bf16x2 p01, p23;
-                        fp8x4_to_bf16<WT, SCALED>(wa[u][d], s0, p01, p23);
-                        acc0 = dot2_bf16(p01, xv[(d & 1) * 2 + 0], acc0);
-                        acc0 = dot2_bf16(p23, xv[(d & 1) * 2 + 1], acc0);
-                        fp8x4_to_bf16<WT, SCALED>(wb[u][d], s1, p01, p23);
-                        acc1 = dot2_bf16(p01, xv[(d & 1) * 2 + 0], acc1);
-                        acc1 = dot2_bf16(p23, xv[(d & 1) * 2 + 1], acc1);
+                        o0 = bf16_round(o0 + bf16_bits_to_f32(a.residual[cur.row0]));
+                        o1 = bf16_round(o1 + bf16_bits_to_f32(a.residual[cur.row1]));
                     }
+                    a.Y[cur.seg][cur.row0] = (uint16_t)f32_to_bf16_bits(o0);
+                    if (cur.row1 != cur.row0) { a.Y[cur.seg][cur.row1] = (uint16_t)f32_to_bf16_bits(o1); }
                 }
             }
         }
-        const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
-        if (lane == 0)
+        g = ng;
+        batch = nbatch;
+        cur = nxt;
+#pragma unroll
+        for (int u = 0; u < U; u++)
         {
-            if (a.pair)
-            {
-                const float gate = bf16_round(t0), up = bf16_round(t1);
-                const float sig = bf16_round(1.0f / (1.0f + expf(-gate)));
-                const float silu = bf16_round(gate * sig);
-                float out = bf16_round(silu * up);
-                if (a.residual) { out = bf16_round(out + bf16_bits_to_f32(a.residual[g])); }
-                a.Y[0][g] = (uint16_t)f32_to_bf16_bits(out);
-            }
-            else
-            {
-                float o0 = bf16_round(t0), o1 = bf16_round(t1);
-                if (a.residual && seg == 0)
-                {
-                    o0 = bf16_round(o0 + bf16_bits_to_f32(a.residual[row0]));
-                    o1 = bf16_round(o1 + bf16_bits_to_f32(a.residual[row1]));
-                }
-                a.Y[seg][row0] = (uint16_t)f32_to_bf16_bits(o0);
-                if (row1 != row0) { a.Y[seg][row1] = (uint16_t)f32_to_bf16_bits(o1); }
-            }
+            wa[u] = na[u];
+            wb[u] = nb[u];
         }
     }
 }
@@ -289,43 +340,60 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_kernel(const uint16
 }
 
 // ------------------------------------------------------------------------------------------
-// GQA decode attention, head_dim 128, group of G = n_q / n_kv query heads per KV head.
-// Pass 1: scores[qh][t] = bf16(scale * k_t . q_qh) for t <= pos.  16 lanes share a key (8 dims each),
-// a wave covers 4 keys per 1 KiB load; a workgroup covers 64 keys of one KV head.
+// GQA decode attention, head_dim 128, group of G = n_q / n_kv query heads per KV head, two launches
+// over blocks of ATT_KEYS cache positions (grid = (blocks, kv heads); blocks past *d_pos exit at once).
+// 16 lanes share a cache row (8 dims each), a wave covers 4 rows per 1 KiB load, a workgroup 16, and
+// every thread issues its 8 row loads before the first use.
+constexpr int ATT_KEYS = 128;
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) { v = fmaxf(v, __shfl_xor(v, off)); }
+    return v;
+}
+
+__device__ __forceinline__ void unpack8_bf16(const u32x4& raw, float* f)
+{
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        f[2 * d] = bf16_bits_to_f32(raw[d] & 0xFFFFu);
+        f[2 * d + 1] = bf16_bits_to_f32(raw[d] >> 16);
+    }
+}
+
+// Launch 1: scores[qh][t] = bf16(scale * k_t . q_qh) for t <= pos, and per block and query head the
+// softmax statistics of its scores: stats[qh][block] = (max, sum of expf(s - max)).
 template <int G>
 __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, uint16_t* __restrict__ scores,
-                                                         int t_kv, const int* __restrict__ d_pos, float scale)
+                                                         float2* __restrict__ stats, int t_kv, int n_blocks, const int* __restrict__ d_pos, float scale)
 {
-    const int kvh = blockIdx.y;
+    __shared__ float s_lds[G][ATT_KEYS];
+    const int kvh = blockIdx.y, blk = blockIdx.x;
     const int n_keys = min(max(*d_pos, 0), t_kv - 1) + 1;
+    const int t0 = blk * ATT_KEYS;
+    if (t0 >= n_keys) { return; }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15;              // which 8 dims
     const int key_in_wave = lane >> 4;
+    u32x4 raw[8];
+#pragma unroll
+    for (int it = 0; it < 8; it++)
+    {
+        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end repeat the last one and are discarded below
+        raw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+    }
     float qv[G][8];
 #pragma unroll
-    for (int gq = 0; gq < G; gq++)
-    {
-        const u32x4 raw = *(const u32x4*)(q + (size_t)(kvh * G + gq) * 128 + sub * 8);
+    for (int gq = 0; gq < G; gq++) { unpack8_bf16(*(const u32x4*)(q + (size_t)(kvh * G + gq) * 128 + sub * 8), qv[gq]); }
 #pragma unroll
-        for (int d = 0; d < 4; d++)
-        {
-            qv[gq][2 * d] = bf16_bits_to_f32(raw[d] & 0xFFFFu);
-            qv[gq][2 * d + 1] = bf16_bits_to_f32(raw[d] >> 16);
-        }
-    }
-#pragma unroll
-    for (int it = 0; it < 4; it++)
+    for (int it = 0; it < 8; it++)
     {
-        const int t = blockIdx.x * 64 + wave * 16 + it * 4 + key_in_wave;
-        u32x4 raw = { 0u, 0u, 0u, 0u };
-        if (t < n_keys) { raw = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8); }
+        const int kl = it * 16 + wave * 4 + key_in_wave;
+        const int t = t0 + kl;
         float kf[8];
-#pragma unroll
-        for (int d = 0; d < 4; d++)
-        {
-            kf[2 * d] = bf16_bits_to_f32(raw[d] & 0xFFFFu);
-            kf[2 * d + 1] = bf16_bits_to_f32(raw[d] >> 16);
-        }
+        unpack8_bf16(raw[it], kf);
 #pragma unroll
         for (int gq = 0; gq < G; gq++)
         {
@@ -336,68 +404,89 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __rest
             dot += dpp_f32<0x4E>(dot);
             dot += dpp_f32<0x141>(dot);
             dot += dpp_f32<0x140>(dot);     // every lane of the 16-lane row holds the key's dot product
-            if (sub == 0 && t < n_keys) { scores[(size_t)(kvh * G + gq) * t_kv + t] = (uint16_t)f32_to_bf16_bits(scale * dot); }
+            if (sub == 0)
+            {
+                const uint32_t bits = f32_to_bf16_bits(scale * dot);
+                if (t < n_keys) { scores[(size_t)(kvh * G + gq) * t_kv + t] = (uint16_t)bits; }
+                s_lds[gq][kl] = t < n_keys ? bf16_bits_to_f32(bits) : -INFINITY;
+            }
         }
+    }
+    __syncthreads();
+    if (wave < G)
+    {
+        const float v0 = s_lds[wave][lane], v1 = s_lds[wave][lane + 64];
+        const float m = wave_max(fmaxf(v0, v1));            // finite: the block holds at least one valid key
+        const float l = wave_sum(expf(v0 - m) + expf(v1 - m));
+        if (lane == 0) { stats[(size_t)(kvh * G + wave) * n_blocks + blk] = make_float2(m, l); }
     }
 }
 
-// Pass 2: softmax statistics over all scores of each query head (recomputed by every workgroup: the
-// row is at most a few KiB), probabilities p_t = bf16(expf(s_t - max) * (1 / sum)), partial outputs
-// over this workgroup's slice of timesteps: partial[split][qh][128] (FP32).  A workgroup reads its
-// V slice once for all G query heads.
+// Launch 2: softmax over the whole row from the block statistics, probabilities
+// p_t = bf16(expf(s_t - max) * (1 / sum)), this block's partial outputs partial[block][qh][128] (FP32).
+// (Letting the last block to arrive add the partials needs a device-scope fence per workgroup, which
+// writes back the L2 of every XCD: measured 17 us per launch against 3 us for launch 3.)
 template <int G>
-__global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict__ scores, const uint16_t* __restrict__ v_cache, float* __restrict__ partial,
-                                                     int t_kv, const int* __restrict__ d_pos, int n_splits, int n_q)
+__global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict__ scores, const float2* __restrict__ stats, const uint16_t* __restrict__ v_cache,
+                                                     float* __restrict__ partial, int t_kv, int n_blocks, const int* __restrict__ d_pos, int n_q)
 {
-    __shared__ float red[4];
     __shared__ float acc_lds[16][G][128];   // [key slot in workgroup][head][dim]
-    const int kvh = blockIdx.y, split = blockIdx.x;
+    __shared__ float p_lds[G][ATT_KEYS];
+    __shared__ float row_max[G], row_inv[G];
+    const int kvh = blockIdx.y, blk = blockIdx.x;
     const int n_keys = min(max(*d_pos, 0), t_kv - 1) + 1;
+    const int t0 = blk * ATT_KEYS;
+    if (t0 >= n_keys) { return; }
+    const int n_active = (n_keys + ATT_KEYS - 1) / ATT_KEYS;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15, key_in_wave = lane >> 4;
-
-    float maxv[G], inv_sum[G];
+    u32x4 raw[8];
 #pragma unroll
-    for (int gq = 0; gq < G; gq++)
+    for (int it = 0; it < 8; it++)
     {
-        const uint16_t* s = scores + (size_t)(kvh * G + gq) * t_kv;
-        float m = -3.0e38f;
-        for (int t = threadIdx.x; t < n_keys; t += 256) { m = fmaxf(m, bf16_bits_to_f32(s[t])); }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) { m = fmaxf(m, __shfl_xor(m, off)); }
-        if (lane == 0) { red[wave] = m; }
-        __syncthreads();
-        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-        __syncthreads();
-        float sum = 0.0f;
-        for (int t = threadIdx.x; t < n_keys; t += 256) { sum += expf(bf16_bits_to_f32(s[t]) - m); }
-        sum = block_sum<256>(sum, red);
-        maxv[gq] = m;
-        inv_sum[gq] = sum > 0.0f ? 1.0f / sum : 0.0f;
+        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end get probability 0 below
+        raw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
     }
-
-    const int per_split = (n_keys + n_splits - 1) / n_splits;
-    const int t_lo = split * per_split, t_hi = min(t_lo + per_split, n_keys);
+    if (wave < G)
+    {
+        const float2* st = stats + (size_t)(kvh * G + wave) * n_blocks;
+        float m = -INFINITY;
+        for (int i = lane; i < n_active; i += 64) { m = fmaxf(m, st[i].x); }
+        m = wave_max(m);
+        float l = 0.0f;
+        for (int i = lane; i < n_active; i += 64) { l += st[i].y * expf(st[i].x - m); }
+        l = wave_sum(l);
+        if (lane == 0)
+        {
+            row_max[wave] = m;
+            row_inv[wave] = l > 0.0f ? 1.0f / l : 0.0f;
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * ATT_KEYS; idx += 256)
+    {
+        const int gq = idx / ATT_KEYS, kl = idx % ATT_KEYS;
+        const int t = t0 + kl;
+        float p = 0.0f;
+        if (t < n_keys) { p = bf16_round(expf(bf16_bits_to_f32(scores[(size_t)(kvh * G + gq) * t_kv + t]) - row_max[gq]) * row_inv[gq]); }
+        p_lds[gq][kl] = p;
+    }
+    __syncthreads();
     float acc[G][8];
 #pragma unroll
     for (int gq = 0; gq < G; gq++)
 #pragma unroll
         for (int d = 0; d < 8; d++) { acc[gq][d] = 0.0f; }
-    for (int t = t_lo + wave * 4 + key_in_wave; t < t_hi; t += 16)
-    {
-        const u32x4 raw = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
-        float vf[8];
 #pragma unroll
-        for (int d = 0; d < 4; d++)
-        {
-            vf[2 * d] = bf16_bits_to_f32(raw[d] & 0xFFFFu);
-            vf[2 * d + 1] = bf16_bits_to_f32(raw[d] >> 16);
-        }
+    for (int it = 0; it < 8; it++)
+    {
+        const int kl = it * 16 + wave * 4 + key_in_wave;
+        float vf[8];
+        unpack8_bf16(raw[it], vf);
 #pragma unroll
         for (int gq = 0; gq < G; gq++)
         {
-            const float s = bf16_bits_to_f32(scores[(size_t)(kvh * G + gq) * t_kv + t]);
-            const float p = bf16_round(expf(s - maxv[gq]) * inv_sum[gq]);
+            const float p = p_lds[gq][kl];
 #pragma unroll
             for (int d = 0; d < 8; d++) { acc[gq][d] = fmaf(p, vf[d], acc[gq][d]); }
         }
@@ -414,47 +503,99 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict
         float total = 0.0f;
 #pragma unroll
         for (int sl = 0; sl < 16; sl++) { total += acc_lds[sl][gq][d]; }
-        partial[((size_t)split * n_q + kvh * G + gq) * 128 + d] = total;
+        partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d] = total;
     }
 }
 
-// y[i] = bf16(sum_s partial[s][i])
-static __global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y, int n_splits, int n)
+// Launch 3: y[o] = bf16(sum over the active blocks of partial[block][o]), in a fixed order: 64 outputs
+// per workgroup, wave w adds blocks w, w + 4, ... and the four sums are added in wave order.
+static __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y, int n_out, int t_kv,
+                                                          const int* __restrict__ d_pos)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) { return; }
+    __shared__ float part[4][64];
+    const int n_keys = min(max(*d_pos, 0), t_kv - 1) + 1;
+    const int n_active = (n_keys + ATT_KEYS - 1) / ATT_KEYS;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + lane;
     float total = 0.0f;
-    for (int s = 0; s < n_splits; s++) { total += partial[(size_t)s * n + i]; }
-    y[i] = (uint16_t)f32_to_bf16_bits(total);
+    if (o < n_out)
+    {
+        int s = wave;
+        for (; s + 12 < n_active; s += 16)
+        {
+            const float a0 = partial[(size_t)s * n_out + o], a1 = partial[(size_t)(s + 4) * n_out + o];
+            const float a2 = partial[(size_t)(s + 8) * n_out + o], a3 = partial[(size_t)(s + 12) * n_out + o];
+            total = (((total + a0) + a1) + a2) + a3;
+        }
+        for (; s < n_active; s += 4) { total += partial[(size_t)s * n_out + o]; }
+    }
+    part[wave][lane] = total;
+    __syncthreads();
+    if (wave == 0 && o < n_out) { y[o] = (uint16_t)f32_to_bf16_bits(((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]); }
 }
 
-// Index of the largest BF16 value (lowest index on ties) into *d_index; also advances *d_pos when given.
-static __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __restrict__ x, unsigned n, int* __restrict__ d_index, int* __restrict__ d_pos)
+// Arg-max of BF16 values, lowest index on ties, in two launches: per-block candidates, then the pick.
+__device__ __forceinline__ bool better(float v, unsigned i, float bv, unsigned bi) { return v > bv || (v == bv && i < bi); }
+
+template <int THREADS>
+__device__ __forceinline__ void block_argmax(float& bv, unsigned& bi, float* best_v, unsigned* best_i)
 {
-    __shared__ float best_v[16];
-    __shared__ unsigned best_i[16];
-    float bv = -3.4e38f;
-    unsigned bi = 0xFFFFFFFFu;
-    for (unsigned i = threadIdx.x; i < n; i += 1024)
-    {
-        const float v = bf16_bits_to_f32(x[i]);
-        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
-    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1)
     {
         const float ov = __shfl_xor(bv, off);
         const unsigned oi = __shfl_xor(bi, off);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
     }
     if ((threadIdx.x & 63) == 0) { best_v[threadIdx.x >> 6] = bv; best_i[threadIdx.x >> 6] = bi; }
     __syncthreads();
     if (threadIdx.x == 0)
     {
-        for (int w = 1; w < 16; w++)
+        for (int w = 1; w < THREADS / 64; w++)
         {
-            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+            if (better(best_v[w], best_i[w], bv, bi)) { bv = best_v[w]; bi = best_i[w]; }
         }
+    }
+}
+
+constexpr int ARGMAX_PER_BLOCK = 2048;    // 256 threads x 8 values
+
+static __global__ __launch_bounds__(256) void argmax_blocks_kernel(const uint16_t* __restrict__ x, unsigned n, float* __restrict__ cand_v, unsigned* __restrict__ cand_i)
+{
+    __shared__ float best_v[4];
+    __shared__ unsigned best_i[4];
+    float bv = -INFINITY;
+    unsigned bi = 0xFFFFFFFFu;
+    const unsigned base = blockIdx.x * ARGMAX_PER_BLOCK;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+    {
+        const unsigned i = base + j * 256 + threadIdx.x;
+        if (i < n)
+        {
+            const float v = bf16_bits_to_f32(x[i]);
+            if (better(v, i, bv, bi)) { bv = v; bi = i; }
+        }
+    }
+    block_argmax<256>(bv, bi, best_v, best_i);
+    if (threadIdx.x == 0) { cand_v[blockIdx.x] = bv; cand_i[blockIdx.x] = bi; }
+}
+
+// Picks among the block candidates into *d_index; also advances *d_pos when given.
+static __global__ __launch_bounds__(256) void argmax_pick_kernel(const float* __restrict__ cand_v, const unsigned* __restrict__ cand_i, unsigned n_cand,
+                                                         int* __restrict__ d_index, int* __restrict__ d_pos)
+{
+    __shared__ float best_v[4];
+    __shared__ unsigned best_i[4];
+    float bv = -INFINITY;
+    unsigned bi = 0xFFFFFFFFu;
+    for (unsigned c = threadIdx.x; c < n_cand; c += 256)
+    {
+        if (better(cand_v[c], cand_i[c], bv, bi)) { bv = cand_v[c]; bi = cand_i[c]; }
+    }
+    block_argmax<256>(bv, bi, best_v, best_i);
+    if (threadIdx.x == 0)
+    {
         *d_index = (int)(bi == 0xFFFFFFFFu ? 0u : bi);
         if (d_pos) { *d_pos += 1; }
     }

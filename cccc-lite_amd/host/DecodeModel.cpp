@@ -49,8 +49,9 @@ DecodeModel::DecodeModel(const DecodeConfig& cfg, GpuControl* gpu) : cfg_(cfg), 
     q_rot_ = make(q_out, 1, BFLOAT16, gpu);
     att_ = make(q_out, 1, BFLOAT16, gpu);
     gated_ = make(cfg.inter, 1, BFLOAT16, gpu);
-    scores_ = make(cfg.t_kv, cfg.n_q, BFLOAT16, gpu);
-    partial_ = make(q_out, n_splits_, FLOAT, gpu);
+    attn_ws_bytes_ = hip_attention_decode_workspace_bytes(cfg.n_q, cfg.n_kv, cfg.t_kv);
+    attn_ws_ = make((int)((attn_ws_bytes_ + 3) / 4), 1, FLOAT, gpu);
+    argmax_ws_ = make((int)((hip_argmax_workspace_bytes((unsigned)cfg.vocab) + 3) / 4), 1, FLOAT, gpu);
 
     // RoPE tables as the reference's graph builds them (cccc/NetCifa.cpp:431-475): float math on the host,
     // stored to BF16 by truncation (cccc/types.h:43-48)
@@ -180,8 +181,8 @@ int DecodeModel::step()
         // 3. attention over the cache (three launches)
         if (rc == 0)
         {
-            rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), scores_->data(),
-                                           partial_->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, n_splits_);
+            rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(),
+                                           attn_ws_bytes_, c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos);
         }
         // 4. r1 = x + W_o att
         if (rc == 0)
@@ -216,8 +217,39 @@ int DecodeModel::step()
         head.norm_eps = c.eps;
         rc = hip_quant_linear_fused(&head);
     }
-    if (rc == 0) { rc = hip_argmax_bf16(logits_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1); }
+    if (rc == 0) { rc = hip_argmax_bf16(logits_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1, argmax_ws_->data()); }
     return rc;
+}
+
+double DecodeModel::benchGateUp(int reps)
+{
+    if (reps <= 0 || layers_.empty()) { return -2.0; }
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    const int sync_before = hip_quant_set_sync(0);
+    bool ok = true;
+    for (int rep = -1; rep < reps; rep++)    // pass -1 is the warm-up
+    {
+        if (rep == 0) { (void)hipEventRecord(e0, nullptr); }
+        for (auto& L : layers_)
+        {
+            hip_fused_linear gu = linear_desc(*L.w_gate, cfg_.inter, cfg_.hidden, r1_->data(), gated_->data());
+            gu.n_segments = 2;
+            gu.pair = 1;
+            gu.W[1] = L.w_up->data(); gu.n_out[1] = cfg_.inter; gu.w_scale[1] = L.w_up->getQuantScale();
+            gu.norm_weight = L.rms_ffn->data();
+            gu.norm_eps = cfg_.eps;
+            ok = (hip_quant_linear_fused(&gu) == 0) && ok;
+        }
+    }
+    (void)hipEventRecord(e1, nullptr);
+    ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
+    float ms = 0;
+    if (ok) { (void)hipEventElapsedTime(&ms, e0, e1); }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    hip_quant_set_sync(sync_before);
+    return ok ? (double)ms * 1000.0 / ((double)reps * layers_.size()) : -3.0;
 }
 
 double DecodeModel::run(int n_steps, int use_graph)

@@ -40,6 +40,9 @@ public:
     int step();                             // enqueues one decode step; the next token replaces the current one
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
     double run(int n_steps, int use_graph);
+    // Times `reps` passes over every layer's fused gate/up launch (norm + SwiGLU pair, distinct weights per
+    // layer) with events on the launch stream; returns the average microseconds per launch or < 0.
+    double benchGateUp(int reps);
     int currentToken();                     // blocking 4-byte read
     int currentPos();
     Matrix& logits() { return *logits_; }
@@ -58,9 +61,9 @@ private:
     std::vector<Layer> layers_;
     std::unique_ptr<Matrix> emb_, rms_final_, lm_head_, logits_, cos_, sin_;
     std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
-    std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, scores_, partial_;
+    std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, attn_ws_, argmax_ws_;
+    unsigned long long attn_ws_bytes_ = 0;
     int* d_state_ = nullptr;    // [0] token, [1] position
-    int n_splits_ = 32;
 };
 
 }    // namespace cccc

@@ -243,6 +243,15 @@ int cccc_decode_kv(void* m, int layer, int is_v, void* host, unsigned long long 
     return (is_v ? d->vCache(layer) : d->kCache(layer)).copyToHost(host, (size_t)bytes);
 }
 
+void* cccc_decode_kv_data(void* m, int layer, int is_v)
+{
+    DecodeModel* d = (DecodeModel*)m;
+    if (layer < 0 || layer >= d->config().layers) { return nullptr; }
+    return (is_v ? d->vCache(layer) : d->kCache(layer)).data();
+}
+
+double cccc_decode_bench_gate_up(void* m, int reps) { return ((DecodeModel*)m)->benchGateUp(reps); }
+
 int cccc_decode_cos_table(void* m, void* host, unsigned long long bytes) { return ((DecodeModel*)m)->cosTable().copyToHost(host, (size_t)bytes); }
 
 unsigned long long cccc_decode_weight_bytes(void* m) { return (unsigned long long)((DecodeModel*)m)->weightBytes(); }

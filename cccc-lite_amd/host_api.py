@@ -55,6 +55,8 @@ class HostLibrary:
         L.cccc_decode_kv.restype = i32; L.cccc_decode_kv.argtypes = [vp, i32, i32, vp, u64]
         L.cccc_decode_cos_table.restype = i32; L.cccc_decode_cos_table.argtypes = [vp, vp, u64]
         L.cccc_decode_weight_bytes.restype = u64; L.cccc_decode_weight_bytes.argtypes = [vp]
+        L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
+        L.cccc_decode_bench_gate_up.restype = ctypes.c_double; L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
         self.c = L
 
     def init(self, device: int = 0) -> None:
@@ -232,6 +234,16 @@ class DecodeModel:
         out = np.empty((c["t_kv"], c["head_dim"] // 2), dtype=np.uint16)
         assert self.lib.c.cccc_decode_cos_table(self.handle, out.ctypes.data, out.nbytes) == 0
         return out
+
+    def kv_ptr(self, layer: int, is_v: bool) -> int:
+        return self.lib.c.cccc_decode_kv_data(self.handle, layer, 1 if is_v else 0)
+
+    def bench_gate_up(self, reps: int) -> float:
+        """Average microseconds per fused gate/up launch over all layers' distinct weights."""
+        us = float(self.lib.c.cccc_decode_bench_gate_up(self.handle, reps))
+        if us < 0:
+            raise RuntimeError(f"gate/up timing failed: {us}")
+        return us
 
     @property
     def weight_bytes(self) -> int:

@@ -159,19 +159,24 @@ C_EXPORT int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* 
                                       const void* d_pos, float epsilon);
 
 /* GQA attention of one query token over cache rows 0..*d_pos: scores rounded to BF16, FP32 softmax,
- * BF16 probabilities, y = bf16(V p).  Workspaces (caller-owned): scores_ws bf16 [n_q_heads][t_kv],
- * partial_ws float [n_splits][n_q_heads][128].  n_q_heads / n_kv_heads must be 1, 2 or 4. */
+ * BF16 probabilities, y = bf16(V p).  Three launches over blocks of 128 cache rows; the caller owns the
+ * workspace (16-byte aligned, hip_attention_decode_workspace_bytes(...) bytes; its content between
+ * calls does not matter).  n_q_heads / n_kv_heads must be 1, 2 or 4; calls sharing one workspace
+ * must be ordered on the stream. */
+C_EXPORT unsigned long long hip_attention_decode_workspace_bytes(int n_q_heads, int n_kv_heads, int t_kv);
 C_EXPORT int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* y,
-                                       void* scores_ws, void* partial_ws,
+                                       void* workspace, unsigned long long workspace_bytes,
                                        int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
-                                       const void* d_pos, int n_splits);
+                                       const void* d_pos);
 
 /* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
 C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);
 
 /* Arg-max of n BF16 values (lowest index on ties) into *d_index (int32, device); when d_pos is not
- * NULL, *d_pos is incremented afterwards (the step counter of a decode loop). */
-C_EXPORT int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos);
+ * NULL, *d_pos is incremented afterwards (the step counter of a decode loop).  `workspace`:
+ * hip_argmax_workspace_bytes(n) bytes of device memory for the per-block candidates. */
+C_EXPORT unsigned long long hip_argmax_workspace_bytes(unsigned int n);
+C_EXPORT int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos, void* workspace);
 
 /*
  * Library controls (no counterpart in the reference, which always uses the null stream and always

@@ -119,33 +119,38 @@ def test_fused_linear_variants(gpu, pkg, oracle, dec):
     assert lib.quant_linear_fused(bad) == -1
 
 
-@pytest.mark.parametrize("n_q,n_kv", [(4, 2), (8, 2), (2, 2)])
-def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv):
+@pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 200), (2, 2, 200), (8, 2, 1024)])
+def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv, t_kv):
     torch, dev, lib = gpu
     rng = np.random.default_rng(2)
-    t_kv = 200
     q = oracle.f32_to_bf16(rng.standard_normal((n_q, 128)).astype(np.float32))
     kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
     vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
     qd, kd, vd = to_dev(torch, dev, q), to_dev(torch, dev, kc), to_dev(torch, dev, vc)
-    n_splits = 8
-    scores = torch.zeros(n_q * t_kv, dtype=torch.int16, device=dev)
-    partial = torch.zeros(n_splits * n_q * 128, dtype=torch.float32, device=dev)
-    for pos in (0, 1, 63, 64, 130, 199):
+    ws_bytes = lib.c.hip_attention_decode_workspace_bytes(n_q, n_kv, t_kv)
+    assert ws_bytes >= n_q * t_kv * 2 and ws_bytes % 256 == 0
+    ws = torch.full((ws_bytes,), 0x5A, dtype=torch.uint8, device=dev)       # content between calls must not matter
+    positions = (0, 1, 63, 64, 127, 128, 130, 199) if t_kv == 200 else (511, 1000, 1023)
+    for pos in positions:
         pd = torch.tensor([pos], dtype=torch.int32, device=dev)
         y = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
         rc = lib.c.hip_attention_decode_bf16(ctypes.c_void_p(qd.data_ptr()), ctypes.c_void_p(kd.data_ptr()), ctypes.c_void_p(vd.data_ptr()),
-                                             ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(scores.data_ptr()), ctypes.c_void_p(partial.data_ptr()),
-                                             n_q, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr()), n_splits)
+                                             ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(ws.data_ptr()), ws_bytes,
+                                             n_q, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr()))
         assert rc == 0
         want = dec.attention(dec.f(q), dec.f(kc), dec.f(vc), pos, n_q, n_kv)
         got = from_dev(y, np.uint16).reshape(n_q, 128)
         assert ulp_close(got, want, ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), pos
-        # the BF16 scores themselves (pass 1) are the reference's rounding point
-        s = dec.f(from_dev(scores, np.uint16).reshape(n_q, t_kv)[:, :pos + 1])
+        # the BF16 scores themselves (launch 1, first n_q * t_kv BF16 values of the workspace) are the reference's rounding point
+        s = ws[:n_q * t_kv * 2].cpu().numpy().view(np.uint16).reshape(n_q, t_kv)[:, :pos + 1]
         for h in range(n_q):
-            ref = dec.r(np.float32(1 / np.sqrt(np.float32(128))) * (dec.f(kc)[h // (n_q // n_kv), :pos + 1].astype(np.float64) @ dec.f(q)[h].astype(np.float64)).astype(np.float32))
-            assert ulp_close(oracle.f32_to_bf16(s[h]), ref, ulps=1.0, floor=1e-5).all()
+            exact = dec.f(kc)[h // (n_q // n_kv), :pos + 1].astype(np.float64) @ dec.f(q)[h].astype(np.float64)
+            ref = dec.r(np.float32(1 / np.sqrt(np.float32(128))) * exact.astype(np.float32))
+            assert ulp_close(s[h], ref, ulps=1.0, floor=1e-5).all()
+    # too small a workspace and an unsupported head grouping are refused
+    args = [ctypes.c_void_p(t.data_ptr()) for t in (qd, kd, vd, y, ws)]
+    assert lib.c.hip_attention_decode_bf16(*args, ws_bytes - 256, n_q, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr())) == -1
+    assert lib.c.hip_attention_decode_bf16(*args, ws_bytes, 3 * n_kv, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr())) == -1
 
 
 def test_argmax_and_embed(gpu, oracle):
@@ -155,8 +160,16 @@ def test_argmax_and_embed(gpu, oracle):
     x[[777, 90000]] = 0x4120                                   # two equal maxima (10.0): the lower index wins
     xd = to_dev(torch, dev, x)
     st = torch.tensor([0, 41], dtype=torch.int32, device=dev)
-    assert lib.c.hip_argmax_bf16(ctypes.c_void_p(xd.data_ptr()), 151936, ctypes.c_void_p(st.data_ptr()), ctypes.c_void_p(st.data_ptr() + 4)) == 0
+    aws = torch.zeros(lib.c.hip_argmax_workspace_bytes(151936), dtype=torch.uint8, device=dev)
+    assert lib.c.hip_argmax_bf16(ctypes.c_void_p(xd.data_ptr()), 151936, ctypes.c_void_p(st.data_ptr()), ctypes.c_void_p(st.data_ptr() + 4),
+                                 ctypes.c_void_p(aws.data_ptr())) == 0
     assert st.cpu().tolist() == [777, 42]
+    for n, hot in ((1, 0), (2049, 2048), (5000, 4999)):                       # block boundaries, last element
+        x2 = np.full(n, 0xBF80, dtype=np.uint16)
+        x2[hot] = 0x3F80
+        assert lib.c.hip_argmax_bf16(ctypes.c_void_p(to_dev(torch, dev, x2).data_ptr()), n, ctypes.c_void_p(st.data_ptr()), None,
+                                     ctypes.c_void_p(aws.data_ptr())) == 0
+        assert st.cpu().tolist() == [hot, 42]
     W = oracle.f32_to_bf16(rng.standard_normal((50, 256)).astype(np.float32))
     wd = to_dev(torch, dev, W)
     y = torch.zeros(256, dtype=torch.int16, device=dev)
