@@ -52,52 +52,106 @@ struct FusedLinearArgs
     const uint16_t* residual;  // bf16 [n_out[0]] or nullptr (single segment / pair only)
 };
 
-// Stages the activation vector into LDS in the [step][half][lane] layout of the dot2 kernels,
-// applying RMSNorm on the way when asked.  `red` holds THREADS / 64 floats.
+// Staging of the activation vector into LDS in the [step][half][lane] layout of the dot2 kernels,
+// with RMSNorm on the way when asked, in two parts so that the caller can put its first weight
+// requests between them: vector-memory loads complete in issue order, so a wait for the activation
+// would otherwise also wait for every weight request issued before it.  The first PRE 16-byte
+// chunks of each thread travel in registers; longer vectors take the slower loop in finish().
+constexpr int STAGE_PRE = 4;
+
+struct StagedActivation
+{
+    u32x4 x[STAGE_PRE], w[STAGE_PRE];
+};
+
+__device__ __forceinline__ int stage_slot(int c)
+{
+    const int step = c >> 7, in_step = c & 127;
+    return (step * 2 + (in_step & 1)) * 64 + (in_step >> 1);
+}
+
 template <int THREADS>
-__device__ __forceinline__ void stage_decode_activation(const FusedLinearArgs& a, u32x4* xs, float* red)
+__device__ __forceinline__ void stage_issue(const FusedLinearArgs& a, StagedActivation& r)
+{
+#pragma unroll
+    for (int j = 0; j < STAGE_PRE; j++)
+    {
+        const int c = threadIdx.x + j * THREADS;
+        r.x[j] = r.w[j] = u32x4{ 0u, 0u, 0u, 0u };
+        if (c * 8 < a.K)
+        {
+            r.x[j] = *(const u32x4*)(a.X + c * 8);
+            if (a.norm_w) { r.w[j] = *(const u32x4*)(a.norm_w + c * 8); }
+        }
+    }
+}
+
+__device__ __forceinline__ float sumsq8(const u32x4& v)
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu), hi = bf16_bits_to_f32(v[d] >> 16);
+        s += lo * lo + hi * hi;
+    }
+    return s;
+}
+
+__device__ __forceinline__ u32x4 normed8(const u32x4& v, const u32x4& w, float invstd)
+{
+    u32x4 out;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu) * invstd * bf16_bits_to_f32(w[d] & 0xFFFFu);
+        const float hi = bf16_bits_to_f32(v[d] >> 16) * invstd * bf16_bits_to_f32(w[d] >> 16);
+        out[d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    }
+    return out;
+}
+
+// `red` holds THREADS / 64 floats.  Ends with a barrier: xs is complete for every thread.
+template <int THREADS>
+__device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const StagedActivation& r, u32x4* xs, float* red)
 {
     const int n_steps = (a.K + 1023) / 1024;
     const int n_chunks = n_steps * 128;                      // 16-byte chunks incl. zero padding
     float sumsq = 0.0f;
-    for (int c = threadIdx.x; c < n_chunks; c += THREADS)
+    if (a.norm_w)
+    {
+#pragma unroll
+        for (int j = 0; j < STAGE_PRE; j++) { sumsq += sumsq8(r.x[j]); }
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < STAGE_PRE; j++)
+        {
+            const int c = threadIdx.x + j * THREADS;
+            if (c < n_chunks) { xs[stage_slot(c)] = r.x[j]; }
+        }
+    }
+    for (int c = threadIdx.x + STAGE_PRE * THREADS; c < n_chunks; c += THREADS)
     {
         u32x4 v = { 0u, 0u, 0u, 0u };
         if (c * 8 < a.K) { v = *(const u32x4*)(a.X + c * 8); }
-        if (a.norm_w)
-        {
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-            {
-                const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu), hi = bf16_bits_to_f32(v[d] >> 16);
-                sumsq += lo * lo + hi * hi;
-            }
-        }
-        const int step = c >> 7, in_step = c & 127;
-        xs[(step * 2 + (in_step & 1)) * 64 + (in_step >> 1)] = v;
+        if (a.norm_w) { sumsq += sumsq8(v); }
+        xs[stage_slot(c)] = v;
     }
     if (a.norm_w)
     {
-        const float total = block_sum<THREADS>(sumsq, red);   // includes the barrier that publishes xs
+        const float total = block_sum<THREADS>(sumsq, red);   // its barrier also publishes the raw tail chunks
         const float invstd = rsqrtf(total / (float)a.K + a.norm_eps);
-        for (int c = threadIdx.x; c < n_chunks; c += THREADS)
-        {
-            if (c * 8 < a.K)
-            {
-                const int step = c >> 7, in_step = c & 127;
-                const int slot = (step * 2 + (in_step & 1)) * 64 + (in_step >> 1);
-                const u32x4 v = xs[slot];
-                const u32x4 w = *(const u32x4*)(a.norm_w + c * 8);
-                u32x4 out;
 #pragma unroll
-                for (int d = 0; d < 4; d++)
-                {
-                    const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu) * invstd * bf16_bits_to_f32(w[d] & 0xFFFFu);
-                    const float hi = bf16_bits_to_f32(v[d] >> 16) * invstd * bf16_bits_to_f32(w[d] >> 16);
-                    out[d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
-                }
-                xs[slot] = out;
-            }
+        for (int j = 0; j < STAGE_PRE; j++)
+        {
+            const int c = threadIdx.x + j * THREADS;
+            if (c < n_chunks) { xs[stage_slot(c)] = normed8(r.x[j], r.w[j], invstd); }    // padding chunks are zero
+        }
+        for (int c = threadIdx.x + STAGE_PRE * THREADS; c < n_chunks; c += THREADS)
+        {
+            if (c * 8 < a.K) { xs[stage_slot(c)] = normed8(xs[stage_slot(c)], *(const u32x4*)(a.norm_w + c * 8), invstd); }
         }
     }
     __syncthreads();
@@ -164,12 +218,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
     int g = blockIdx.x * WAVES + wave, batch = 0;
     FusedRows cur{}, nxt{};
     u32x4 wa[U], wb[U], na[U], nb[U];
+    StagedActivation staged;
+    stage_issue<WAVES * 64>(a, staged);
     if (g < n_groups)
     {
         cur = locate(g);
         request(cur, 0, wa, wb);
     }
-    stage_decode_activation<WAVES * 64>(a, xs, red);
+    stage_finish<WAVES * 64>(a, staged, xs, red);
 
     float acc0 = 0.0f, acc1 = 0.0f;
     while (g < n_groups)

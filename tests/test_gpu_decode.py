@@ -119,6 +119,29 @@ def test_fused_linear_variants(gpu, pkg, oracle, dec):
     assert lib.quant_linear_fused(bad) == -1
 
 
+@pytest.mark.parametrize("K,n_out", [(1520, 37), (16400, 64), (8192, 33), (8208, 16)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_fused_linear_ragged_lengths(gpu, pkg, oracle, dec, K, n_out, norm):
+    """Row lengths that are not a multiple of 1 KiB, longer than the register-staged part of the
+    activation, and odd row counts."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(K + n_out)
+    x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+    nw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    W = oracle.encode_e5m2_rne((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32))
+    res = oracle.f32_to_bf16(rng.standard_normal(n_out).astype(np.float32))
+    xd, nwd, wd, rd = (to_dev(torch, dev, v) for v in (x, nw, W, res))
+    y = torch.zeros(n_out + 8, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(E5M2, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(),
+                                   norm_weight=nwd.data_ptr() if norm else None, norm_eps=1e-6, residual=rd.data_ptr())
+    assert lib.quant_linear_fused(d) == 0
+    out = from_dev(y, np.uint16)
+    assert not out[n_out:].any()
+    xin = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6) if norm else dec.f(x)
+    lin = dec.linear(oracle.dequant_fp8_to_bf16(W, oracle.E5M2).reshape(n_out, K), xin)
+    assert ulp_close(out[:n_out], dec.r(lin + dec.f(res)), ulps=1.0, floor=1e-4).all()
+
+
 @pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 200), (2, 2, 200), (8, 2, 1024)])
 def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv, t_kv):
     torch, dev, lib = gpu
