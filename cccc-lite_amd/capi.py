@@ -55,6 +55,7 @@ EXPORTS = (
     "hip_qk_norm_rope_kv_bf16",
     "hip_attention_decode_bf16",
     "hip_attention_decode_workspace_bytes",
+    "hip_attention_decode_fused_bf16",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_quant_set_sync",
@@ -114,6 +115,8 @@ class QuantLibrary:
         L.hip_qk_norm_rope_kv_bf16.argtypes = [vp] * 10 + [i32, i32, i32, i32, vp, f32]
         L.hip_attention_decode_bf16.restype = i32
         L.hip_attention_decode_bf16.argtypes = [vp] * 5 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp]
+        L.hip_attention_decode_fused_bf16.restype = i32
+        L.hip_attention_decode_fused_bf16.argtypes = [vp] * 11 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp, f32]
         L.hip_attention_decode_workspace_bytes.restype = ctypes.c_ulonglong
         L.hip_attention_decode_workspace_bytes.argtypes = [i32, i32, i32]
         L.hip_argmax_workspace_bytes.restype = ctypes.c_ulonglong

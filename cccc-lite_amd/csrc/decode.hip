@@ -197,6 +197,39 @@ int hip_attention_decode_bf16(const void* q, const void* k_cache, const void* v_
     return finish("attention_decode");
 }
 
+int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v, const void* q_norm_w, const void* k_norm_w,
+                                    const void* cos_tab, const void* sin_tab, void* k_cache, void* v_cache, void* y,
+                                    void* workspace, unsigned long long workspace_bytes,
+                                    int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
+{
+    if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || !d_pos) { return -1; }
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_tab || !sin_tab || !k_cache || !v_cache || !y || !workspace) { return -1; }
+    if (!aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace)) { return -1; }
+    const AttentionWorkspace w = attention_workspace(n_q_heads, t_kv);
+    if (workspace_bytes < w.total || w.n_blocks > ATT_MAX_BLOCKS) { return -1; }
+    const dim3 grid(w.n_blocks, n_kv_heads);
+    float2* stats = (float2*)((char*)workspace + w.stats);
+    float* partial = (float*)((char*)workspace + w.partial);
+    const float scale = 1.0f / sqrtf(128.0f);
+    const int* pos = (const int*)d_pos;
+#define CCQ_ATTN_FUSED(G)                                                                                                                    \
+    attn_fused_kernel<G><<<grid, 256, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_norm_w, \
+                                                     (const uint16_t*)k_norm_w, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,        \
+                                                     (uint16_t*)k_cache, (uint16_t*)v_cache, stats, partial, t_kv, w.n_blocks, pos,        \
+                                                     n_q_heads, epsilon, scale)
+    switch (n_q_heads / n_kv_heads)
+    {
+    case 1: CCQ_ATTN_FUSED(1); break;
+    case 2: CCQ_ATTN_FUSED(2); break;
+    case 4: CCQ_ATTN_FUSED(4); break;
+    default: return -1;
+    }
+#undef CCQ_ATTN_FUSED
+    const int n_out = n_q_heads * 128;
+    attn_rescale_combine_kernel<<<n_out / 64, 256, 0, stream()>>>(partial, stats, (uint16_t*)y, n_out, t_kv, w.n_blocks, pos);
+    return finish("attention_decode_fused");
+}
+
 unsigned long long hip_argmax_workspace_bytes(unsigned int n) { return (unsigned long long)((n + ARGMAX_PER_BLOCK - 1) / ARGMAX_PER_BLOCK) * 8; }
 
 int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos, void* workspace)

@@ -590,6 +590,223 @@ static __global__ __launch_bounds__(256) void attn_combine_kernel(const float* _
     if (wave == 0 && o < n_out) { y[o] = (uint16_t)f32_to_bf16_bits(((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]); }
 }
 
+// ------------------------------------------------------------------------------------------
+// The same attention in two launches, with the q/k RMSNorm, RoPE and cache append folded in.
+// Differences from the three-launch form above: the softmax of a block is taken against the block's
+// own maximum and rescaled when the blocks are combined (the usual split-softmax identity), so the
+// probabilities stay FP32 instead of being rounded to BF16 before they meet V.  Scores are still
+// rounded to BF16.  Output differences against the three-launch form stay within about one BF16 ulp.
+//
+// Launch 1, grid (blocks, kv heads): raw q [n_q][128], k, v [n_kv][128] of the new token;
+//   waves 0..G-1 normalise and rotate the G query heads of this KV head; the block holding row *d_pos
+//   also normalises / rotates k, appends k and v to the caches, and uses them from LDS;
+//   stats[qh][block] = (max, sum expf(s - max)), partial[block][qh][128] = sum expf(s_t - max) v_t.
+__device__ __forceinline__ void norm_rope_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
+                                               const uint16_t* __restrict__ sin_row, float eps, int lane, float& out_l, float& out_r)
+{
+    const float xl = bf16_bits_to_f32(src[lane]), xr = bf16_bits_to_f32(src[lane + 64]);
+    const float c = bf16_bits_to_f32(cos_row[lane]), sn = bf16_bits_to_f32(sin_row[lane]);
+    const float wl = bf16_bits_to_f32(nw[lane]), wr = bf16_bits_to_f32(nw[lane + 64]);
+    const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
+    const float nl = bf16_round(xl * invstd * wl), nr = bf16_round(xr * invstd * wr);
+    out_l = bf16_round(nl * c - nr * sn);
+    out_r = bf16_round(nr * c + nl * sn);
+}
+
+template <int G>
+__global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                                                        const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
+                                                        const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab,
+                                                        uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+                                                        float2* __restrict__ stats, float* __restrict__ partial,
+                                                        int t_kv, int n_blocks, const int* __restrict__ d_pos, int n_q, float eps, float scale)
+{
+    __shared__ float acc_lds[16][G][128];   // [key slot in workgroup][head][dim]
+    __shared__ float s_lds[G][ATT_KEYS];    // scores, then expf(s - block max)
+    __shared__ float q_lds[G][128];
+    __shared__ float k_new[128], v_new[128];
+    const int kvh = blockIdx.y, blk = blockIdx.x;
+    const int pos = *d_pos;
+    if (pos < 0 || pos >= t_kv) { return; }         // a position outside the cache: nothing to append, nothing to attend
+    const int n_keys = pos + 1;
+    const int t0 = blk * ATT_KEYS;
+    if (t0 >= n_keys) { return; }
+    const bool has_new = pos < t0 + ATT_KEYS;       // this block holds the row being appended
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane & 15, key_in_wave = lane >> 4;
+    u32x4 kraw[8], vraw[8];
+#pragma unroll
+    for (int it = 0; it < 8; it++)
+    {
+        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end, and row pos itself, are replaced or discarded below
+        kraw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+        vraw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+    }
+    const uint16_t* cos_row = cos_tab + (size_t)pos * 64;
+    const uint16_t* sin_row = sin_tab + (size_t)pos * 64;
+    if (wave < G)
+    {
+        float l, r;
+        norm_rope_head(q + (size_t)(kvh * G + wave) * 128, q_norm_w, cos_row, sin_row, eps, lane, l, r);
+        q_lds[wave][lane] = l;
+        q_lds[wave][lane + 64] = r;
+    }
+    if (has_new && wave == 3)
+    {
+        float l, r;
+        norm_rope_head(k + (size_t)kvh * 128, k_norm_w, cos_row, sin_row, eps, lane, l, r);
+        k_new[lane] = l;
+        k_new[lane + 64] = r;
+        uint16_t* dst = k_cache + ((size_t)kvh * t_kv + pos) * 128;
+        dst[lane] = (uint16_t)f32_to_bf16_bits(l);
+        dst[lane + 64] = (uint16_t)f32_to_bf16_bits(r);
+    }
+    if (has_new && wave == 2)
+    {
+        const uint16_t a = v[(size_t)kvh * 128 + lane], b = v[(size_t)kvh * 128 + lane + 64];
+        v_new[lane] = bf16_bits_to_f32(a);
+        v_new[lane + 64] = bf16_bits_to_f32(b);
+        uint16_t* dst = v_cache + ((size_t)kvh * t_kv + pos) * 128;
+        dst[lane] = a;
+        dst[lane + 64] = b;
+    }
+    __syncthreads();
+    float qv[G][8];
+#pragma unroll
+    for (int gq = 0; gq < G; gq++)
+#pragma unroll
+        for (int d = 0; d < 8; d++) { qv[gq][d] = q_lds[gq][sub * 8 + d]; }
+#pragma unroll
+    for (int it = 0; it < 8; it++)
+    {
+        const int kl = it * 16 + wave * 4 + key_in_wave;
+        const int t = t0 + kl;
+        float kf[8];
+        unpack8_bf16(kraw[it], kf);
+        if (t == pos)
+        {
+#pragma unroll
+            for (int d = 0; d < 8; d++) { kf[d] = k_new[sub * 8 + d]; }
+        }
+#pragma unroll
+        for (int gq = 0; gq < G; gq++)
+        {
+            float dot = 0.0f;
+#pragma unroll
+            for (int d = 0; d < 8; d++) { dot = fmaf(kf[d], qv[gq][d], dot); }
+            dot += dpp_f32<0xB1>(dot);
+            dot += dpp_f32<0x4E>(dot);
+            dot += dpp_f32<0x141>(dot);
+            dot += dpp_f32<0x140>(dot);
+            if (sub == 0) { s_lds[gq][kl] = t < n_keys ? bf16_round(scale * dot) : -INFINITY; }
+        }
+    }
+    __syncthreads();
+    if (wave < G)
+    {
+        const float v0 = s_lds[wave][lane], v1 = s_lds[wave][lane + 64];
+        const float m = wave_max(fmaxf(v0, v1));            // finite: the block holds at least one valid key
+        const float e0 = expf(v0 - m), e1 = expf(v1 - m);
+        const float l = wave_sum(e0 + e1);
+        s_lds[wave][lane] = e0;
+        s_lds[wave][lane + 64] = e1;
+        if (lane == 0) { stats[(size_t)(kvh * G + wave) * n_blocks + blk] = make_float2(m, l); }
+    }
+    __syncthreads();
+    float acc[G][8];
+#pragma unroll
+    for (int gq = 0; gq < G; gq++)
+#pragma unroll
+        for (int d = 0; d < 8; d++) { acc[gq][d] = 0.0f; }
+#pragma unroll
+    for (int it = 0; it < 8; it++)
+    {
+        const int kl = it * 16 + wave * 4 + key_in_wave;
+        float vf[8];
+        unpack8_bf16(vraw[it], vf);
+        if (t0 + kl == pos)
+        {
+#pragma unroll
+            for (int d = 0; d < 8; d++) { vf[d] = v_new[sub * 8 + d]; }
+        }
+#pragma unroll
+        for (int gq = 0; gq < G; gq++)
+        {
+            const float p = s_lds[gq][kl];                  // 0 for rows past the end
+#pragma unroll
+            for (int d = 0; d < 8; d++) { acc[gq][d] = fmaf(p, vf[d], acc[gq][d]); }
+        }
+    }
+    const int slot = wave * 4 + key_in_wave;
+#pragma unroll
+    for (int gq = 0; gq < G; gq++)
+#pragma unroll
+        for (int d = 0; d < 8; d++) { acc_lds[slot][gq][sub * 8 + d] = acc[gq][d]; }
+    __syncthreads();
+    for (int o = threadIdx.x; o < G * 128; o += 256)
+    {
+        const int gq = o >> 7, d = o & 127;
+        float total = 0.0f;
+#pragma unroll
+        for (int sl = 0; sl < 16; sl++) { total += acc_lds[sl][gq][d]; }
+        partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d] = total;
+    }
+}
+
+// Launch 2: y[qh][d] = bf16(sum_b w_b partial[b][qh][d]), w_b = expf(max_b - max) / sum_b' l_b' expf(max_b' - max),
+// in a fixed order.  64 outputs (half a head) per workgroup; n_blocks <= ATT_MAX_BLOCKS.
+constexpr int ATT_MAX_BLOCKS = 1024;
+
+static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const float* __restrict__ partial, const float2* __restrict__ stats, uint16_t* __restrict__ y,
+                                                                  int n_out, int t_kv, int n_blocks, const int* __restrict__ d_pos)
+{
+    __shared__ float w_lds[ATT_MAX_BLOCKS];
+    __shared__ float red[4];
+    __shared__ float part[4][64];
+    const int pos = *d_pos;
+    if (pos < 0 || pos >= t_kv) { return; }
+    const int n_active = pos / ATT_KEYS + 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int qh = (blockIdx.x * 64) >> 7;
+    const float2* st = stats + (size_t)qh * n_blocks;
+    float m = -INFINITY;
+    for (int b = threadIdx.x; b < n_active; b += 256) { m = fmaxf(m, st[b].x); }
+    m = wave_max(m);
+    if (lane == 0) { red[wave] = m; }
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float l = 0.0f;
+    for (int b = threadIdx.x; b < n_active; b += 256)
+    {
+        const float2 sb = st[b];
+        const float e = expf(sb.x - m);
+        w_lds[b] = e;
+        l += sb.y * e;
+    }
+    l = block_sum<256>(l, red);                     // its barrier publishes w_lds
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const int o = blockIdx.x * 64 + lane;
+    float total = 0.0f;
+    if (o < n_out)
+    {
+        int b = wave;
+        for (; b + 12 < n_active; b += 16)
+        {
+            const float a0 = partial[(size_t)b * n_out + o], a1 = partial[(size_t)(b + 4) * n_out + o];
+            const float a2 = partial[(size_t)(b + 8) * n_out + o], a3 = partial[(size_t)(b + 12) * n_out + o];
+            total = fmaf(a0, w_lds[b], total);
+            total = fmaf(a1, w_lds[b + 4], total);
+            total = fmaf(a2, w_lds[b + 8], total);
+            total = fmaf(a3, w_lds[b + 12], total);
+        }
+        for (; b < n_active; b += 4) { total = fmaf(partial[(size_t)b * n_out + o], w_lds[b], total); }
+    }
+    part[wave][lane] = total;
+    __syncthreads();
+    if (wave == 0 && o < n_out) { y[o] = (uint16_t)f32_to_bf16_bits((((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]) * inv); }
+}
+
 // Arg-max of BF16 values, lowest index on ties, in two launches: per-block candidates, then the pick.
 __device__ __forceinline__ bool better(float v, unsigned i, float bv, unsigned bi) { return v > bv || (v == bv && i < bi); }
 

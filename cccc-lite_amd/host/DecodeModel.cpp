@@ -172,17 +172,22 @@ int DecodeModel::step()
         qkv.norm_weight = L.rms_attn->data();
         qkv.norm_eps = c.eps;
         rc = hip_quant_linear_fused(&qkv);
-        // 2. per-head q/k norm, RoPE, KV append
-        if (rc == 0)
+        // 2-3. per-head q/k norm, RoPE, KV append and attention over the cache
+        if (rc == 0 && !exact_attention_)
+        {
+            rc = hip_attention_decode_fused_bf16(q_->data(), k_->data(), v_->data(), L.q_norm->data(), L.k_norm->data(), cos_->data(), sin_->data(),
+                                                 k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(), attn_ws_bytes_,
+                                                 c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
+        }
+        else if (rc == 0)
         {
             rc = hip_qk_norm_rope_kv_bf16(q_->data(), k_->data(), v_->data(), L.q_norm->data(), L.k_norm->data(), cos_->data(), sin_->data(),
                                           q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
-        }
-        // 3. attention over the cache (three launches)
-        if (rc == 0)
-        {
-            rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(),
-                                           attn_ws_bytes_, c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos);
+            if (rc == 0)
+            {
+                rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(),
+                                               attn_ws_bytes_, c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos);
+            }
         }
         // 4. r1 = x + W_o att
         if (rc == 0)

@@ -2,7 +2,7 @@
 // the host mirror: what the reference does per token through MainProcess::testExternalData ->
 // Net::inference -> MatrixOp::forward (cccc/MainProcess.cpp:1171-1239, cccc/Net.cpp:1748-1792,
 // cccc/MatrixOp.cpp:12-26) for the graph of scripts/convert_weights.py:488-692, collapsed into
-// nine launches per layer.  Token id and position live in device memory, so a step is a fixed
+// six launches per layer.  Token id and position live in device memory, so a step is a fixed
 // launch sequence that can be replayed as one hipGraph.
 #pragma once
 #include "Matrix.h"
@@ -36,6 +36,9 @@ public:
     // Uploads file bytes: FP8 codes for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
     int setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale);
 
+    // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
+    // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).
+    void setExactAttention(bool exact) { exact_attention_ = exact; }
     int reset(int token, int pos);          // sets the device-side token / position (KV caches are kept)
     int step();                             // enqueues one decode step; the next token replaces the current one
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
@@ -63,6 +66,7 @@ private:
     std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
     std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, attn_ws_, argmax_ws_;
     unsigned long long attn_ws_bytes_ = 0;
+    bool exact_attention_ = false;
     int* d_state_ = nullptr;    // [0] token, [1] position
 };
 

@@ -221,6 +221,8 @@ int cccc_decode_tensor_prepare(void* m, int layer, int which)
     return t->hasTiled() ? 0 : 1;
 }
 
+void cccc_decode_set_exact_attention(void* m, int exact) { ((DecodeModel*)m)->setExactAttention(exact != 0); }
+
 int cccc_decode_reset(void* m, int token, int pos) { return ((DecodeModel*)m)->reset(token, pos); }
 
 int cccc_decode_step(void* m)

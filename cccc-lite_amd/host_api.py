@@ -55,6 +55,7 @@ class HostLibrary:
         L.cccc_decode_kv.restype = i32; L.cccc_decode_kv.argtypes = [vp, i32, i32, vp, u64]
         L.cccc_decode_cos_table.restype = i32; L.cccc_decode_cos_table.argtypes = [vp, vp, u64]
         L.cccc_decode_weight_bytes.restype = u64; L.cccc_decode_weight_bytes.argtypes = [vp]
+        L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         L.cccc_decode_bench_gate_up.restype = ctypes.c_double; L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
         self.c = L
@@ -194,6 +195,11 @@ class DecodeModel:
         for li, L in enumerate(model["layers"]):
             for name in LAYER_TENSORS:
                 self.set_tensor(li, name, L[name], fp8_dtype if name in QUANTIZED else 3)
+
+    def set_exact_attention(self, exact: bool) -> None:
+        """True: separate norm / RoPE / append launch and BF16 probabilities (the reference's rounding
+        points); False (default): the two-launch attention with FP32 probabilities."""
+        self.lib.c.cccc_decode_set_exact_attention(self.handle, 1 if exact else 0)
 
     def reset(self, token: int, pos: int) -> None:
         assert self.lib.c.cccc_decode_reset(self.handle, token, pos) == 0

@@ -169,6 +169,19 @@ C_EXPORT int hip_attention_decode_bf16(const void* q, const void* k_cache, const
                                        int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
                                        const void* d_pos);
 
+/* The q/k RMSNorm, RoPE, cache append and attention of one new token in two launches: q, k, v are the
+ * raw projections ([n_q_heads][128], [n_kv_heads][128]); row *d_pos of both caches is written.  Same
+ * workspace as above.  Scores are rounded to BF16 as in the reference; the softmax probabilities stay
+ * FP32 (the reference rounds them to BF16 before the product with V), so outputs can differ from
+ * hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 by about one BF16 ulp.  t_kv <= 131072. */
+C_EXPORT int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
+                                             const void* q_norm_w, const void* k_norm_w,
+                                             const void* cos_tab, const void* sin_tab,
+                                             void* k_cache, void* v_cache, void* y,
+                                             void* workspace, unsigned long long workspace_bytes,
+                                             int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                             const void* d_pos, float epsilon);
+
 /* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
 C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);
 
