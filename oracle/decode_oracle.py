@@ -17,11 +17,15 @@ its HIP library runs (paths relative to the reference tree):
 Every intermediate tensor is BF16; math inside an op is float32 (sums in float64, then float32,
 which only removes accumulation-order noise).
 
-Pinning: the formulas are textbook (RMSNorm, half-rotate RoPE, softmax attention, SwiGLU); the tests
-check them against closed forms (a constant vector normalises to +-w, RoPE preserves pair norms and
-is the identity at position 0, a one-hot softmax, SiLU(0) = 0) and against an independent float64
-torch implementation of the same step without intermediate rounding (agreement within BF16 noise).
-The reference holds no test vectors for these ops -- PARITY UNPINNED by the reference.
+Pinning: (1) on the GPU, tests/test_gpu_ref_hip.py runs the reference's own HIP kernels
+(oracle/_ref/libref_hip.so, compiled from cccc-hip/hip_functions.cpp where it lies) for RMSNorm, RoPE,
+causal mask, softmax, sigmoid / mul / add and the whole attention sequence of MatrixEx.cpp:3018-3104
+(with BF16 GEMMs) and compares them with the functions below: identical, or one BF16 ulp apart where
+the summation order or the device's expf differ; (2) on the CPU, tests/test_oracle_decode.py checks
+closed forms (a constant vector normalises to +-w, RoPE preserves pair norms and is the identity at
+position 0, a one-hot softmax, SiLU(0) = 0) and an independent float64 torch implementation of the
+same step without intermediate rounding (agreement within BF16 noise).  The reference holds no
+golden vectors for these ops.
 """
 from __future__ import annotations
 
@@ -102,6 +106,13 @@ def silu_mul(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     return r(r(gate * sig) * up)
 
 
+def softmax(scores: np.ndarray) -> np.ndarray:
+    """One row: bf16(expf(x - max) * (1 / sum)), cccc-hip/hip_functions.cpp:776-804 with a = 1, r = 0."""
+    e = np.exp(scores - scores.max(), dtype=np.float32)
+    inv = np.float32(1.0) / np.float32(e.astype(np.float64).sum())
+    return r(e * inv)
+
+
 def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, pos: int, n_q: int, n_kv: int) -> np.ndarray:
     """q [n_q, d]; caches [n_kv, t_kv, d] (float32 BF16 values).  Returns [n_q, d]."""
     d = q.shape[-1]
@@ -112,10 +123,7 @@ def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, pos: int,
         kv = h // (n_q // n_kv)
         scores = r(scale * (k_cache[kv].astype(np.float64) @ q[h].astype(np.float64)).astype(np.float32))
         scores[np.arange(t_kv) > pos] = r(np.float32(-1e9))
-        m = scores.max()
-        e = np.exp(scores - m, dtype=np.float32)
-        inv = np.float32(1.0) / np.float32(e.astype(np.float64).sum())
-        p = r(e * inv)
+        p = softmax(scores)
         out[h] = r((p.astype(np.float64) @ v_cache[kv].astype(np.float64)).astype(np.float32))
     return out
 
