@@ -164,6 +164,124 @@ def decode_step_bytes(ctx_mean: float) -> int:
     return weights + kv + small
 
 
+def gpu_baselines(ws: Workspace, ctx: int, steps_ref: int = 3, steps_torch: int = 10):
+    """Two same-GPU baselines of the decode step on a BF16 copy of the model shape (random init):
+    (1) reference HIP style: the reference's own HIP kernels (oracle/_ref/libref_hip.so, compiled from
+        cccc-hip/hip_functions.cpp) for embedding, RMSNorm, RoPE, causal mask, softmax, sigmoid / mul /
+        add, each followed by the device synchronisation that library does, one launch per graph op as in
+        scripts/convert_weights.py:488-692, K / V tiled to the query heads, BF16 weights (that build has
+        no FP8), GEMMs by torch.matmul (rocBLAS / hipBLASLt, what its Rocblas wrapper calls), driven from
+        Python;  (2) plain PyTorch BF16 eager (rms_norm, matmul, scaled_dot_product_attention), no syncs.
+    Returns a dict, or None when the reference library was not built."""
+    import ctypes
+    from oracle import ref_hip
+    t, c = ws.torch, QWEN3_8B
+    R = ref_hip.lib()
+    dev, bf = ws.dev, t.bfloat16
+    H, NQ, NKV, D, I, V = c["hidden"], 32, 8, 128, c["inter"], c["vocab"]
+
+    def w(n_out, k):
+        return (t.randn(n_out, k, device=dev, generator=ws.gen) * 0.02).to(bf)
+
+    layers = [dict(wq=w(NQ * D, H), wk=w(NKV * D, H), wv=w(NKV * D, H), wo=w(H, NQ * D), wg=w(I, H), wu=w(I, H), wd=w(H, I),
+                   n1=t.ones(H, device=dev, dtype=bf), n2=t.ones(H, device=dev, dtype=bf), qn=t.ones(D, device=dev, dtype=bf), kn=t.ones(D, device=dev, dtype=bf),
+                   kc=t.randn(NKV, ctx, D, device=dev, generator=ws.gen).to(bf), vc=t.randn(NKV, ctx, D, device=dev, generator=ws.gen).to(bf))
+              for _ in range(c["layers"])]
+    emb = t.randn(V, H, device=dev, generator=ws.gen).to(bf)
+    lm, nf = w(V, H), t.ones(H, device=dev, dtype=bf)
+    inv_freq = 1.0 / (1e6 ** (t.arange(0, D, 2, device=dev, dtype=t.float32) / D))
+    ang = t.arange(ctx, device=dev, dtype=t.float32)[:, None] * inv_freq[None, :]
+    cos, sin = ang.cos().to(bf).contiguous(), ang.sin().to(bf).contiguous()
+    scale = 1.0 / 128.0 ** 0.5
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    f32 = ctypes.c_float
+    out = {}
+
+    if R is not None:
+        kt, vt = t.empty(NQ, ctx, D, device=dev, dtype=bf), t.empty(NQ, ctx, D, device=dev, dtype=bf)
+
+        def rms(x, wgt, outer, inner):
+            y = t.empty_like(x)
+            assert R.hip_rms_norm_fwd(3, p(x), p(y), p(wgt), None, outer, inner, f32(1e-6)) == 0
+            return y
+
+        def ref_step(token, pos):
+            ids = t.tensor([float(token)], device=dev)
+            x = t.empty(H, device=dev, dtype=bf)
+            assert R.hip_embed_fwd(3, p(ids), p(emb), p(x), H, 1, 1) == 0
+            for L in layers:
+                xn = rms(x, L["n1"], 1, H)
+                q, k, v = L["wq"] @ xn, L["wk"] @ xn, L["wv"] @ xn
+                qn, kn = rms(q, L["qn"], NQ, D), rms(k, L["kn"], NKV, D)
+                qr, kr = t.empty_like(qn), t.empty_like(kn)
+                assert R.hip_rope_fwd(3, p(qn), p(qr), p(cos), p(sin), D, 1, NQ, pos) == 0
+                assert R.hip_rope_fwd(3, p(kn), p(kr), p(cos), p(sin), D, 1, NKV, pos) == 0
+                L["kc"][:, pos] = kr.view(NKV, D)
+                L["vc"][:, pos] = v.view(NKV, D)
+                kt.view(NKV, NQ // NKV, ctx, D).copy_(L["kc"][:, None])           # GQA by tiling K and V to the query heads
+                vt.view(NKV, NQ // NKV, ctx, D).copy_(L["vc"][:, None])
+                scores = (t.bmm(kt, qr.view(NQ, D, 1)) * scale).view(NQ, ctx)
+                assert R.hip_causal_mask(3, p(scores), 1, ctx, NQ, pos) == 0
+                assert R.hip_softmax_bf16(p(scores), p(scores), ctx, NQ, f32(1.0), f32(0.0)) == 0
+                att = t.bmm(scores.view(NQ, 1, ctx), vt).view(NQ * D)
+                o = L["wo"] @ att
+                r1 = t.empty_like(x)
+                assert R.hip_add(3, p(x), p(o), p(r1), H, f32(1.0), f32(1.0)) == 0
+                rn = rms(r1, L["n2"], 1, H)
+                g, u = L["wg"] @ rn, L["wu"] @ rn
+                sg, si, ga = t.empty_like(g), t.empty_like(g), t.empty_like(g)
+                assert R.hip_sigmoid_bf16(p(sg), p(g), I, f32(1.0), f32(0.0)) == 0
+                assert R.hip_mul(3, p(g), p(sg), p(si), I, f32(1.0), f32(0.0)) == 0
+                assert R.hip_mul(3, p(si), p(u), p(ga), I, f32(1.0), f32(0.0)) == 0
+                dn = L["wd"] @ ga
+                x = t.empty_like(r1)
+                assert R.hip_add(3, p(r1), p(dn), p(x), H, f32(1.0), f32(1.0)) == 0
+            logits = lm @ rms(x, nf, 1, H)
+            return int(logits.argmax())
+
+        tok = ref_step(1, ctx - steps_ref - 1)
+        t.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps_ref):
+            tok = ref_step(tok, ctx - steps_ref + i)
+        t.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps_ref
+        out["reference_hip_style"] = {"tok_s": round(1e3 / ms, 2), "ms_per_step": round(ms, 3), "steps": steps_ref, "weights": "bf16",
+                                      "what": "reference's own HIP kernels (norm, rope, mask, softmax, silu, add; each syncs the device) + rocBLAS/hipBLASLt GEMMs via torch.matmul, one launch per graph op, driven from Python"}
+        del kt, vt
+
+    F = t.nn.functional
+
+    def torch_step(token, pos):
+        x = emb[token]
+        for L in layers:
+            xn = F.rms_norm(x, (H,), L["n1"], 1e-6)
+            q, k, v = (L["wq"] @ xn).view(NQ, D), (L["wk"] @ xn).view(NKV, D), L["wv"] @ xn
+            q, k = F.rms_norm(q, (D,), L["qn"], 1e-6), F.rms_norm(k, (D,), L["kn"], 1e-6)
+            cs, sn = cos[pos], sin[pos]
+            q = t.cat([q[:, :64] * cs - q[:, 64:] * sn, q[:, 64:] * cs + q[:, :64] * sn], dim=1)
+            k = t.cat([k[:, :64] * cs - k[:, 64:] * sn, k[:, 64:] * cs + k[:, :64] * sn], dim=1)
+            L["kc"][:, pos] = k
+            L["vc"][:, pos] = v.view(NKV, D)
+            att = F.scaled_dot_product_attention(q.view(1, NQ, 1, D), L["kc"][None, :, :pos + 1], L["vc"][None, :, :pos + 1], enable_gqa=True).view(NQ * D)
+            r1 = x + L["wo"] @ att
+            rn = F.rms_norm(r1, (H,), L["n2"], 1e-6)
+            x = r1 + L["wd"] @ (F.silu(L["wg"] @ rn) * (L["wu"] @ rn))
+        return (lm @ F.rms_norm(x, (H,), nf, 1e-6)).argmax()
+
+    with t.no_grad():
+        tok = torch_step(1, ctx - steps_torch - 1)
+        t.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps_torch):
+            tok = torch_step(tok, ctx - steps_torch + i)
+        t.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps_torch
+    out["torch_bf16_eager"] = {"tok_s": round(1e3 / ms, 2), "ms_per_step": round(ms, 3), "steps": steps_torch, "weights": "bf16",
+                               "what": "PyTorch-ROCm eager BF16 (rms_norm, matmul, scaled_dot_product_attention), no device syncs inside a step"}
+    return out
+
+
 def time_chain(ws, ops, steps, warmup, use_graph):
     ms = ws.host.bench_linear_chain([o[0] for o in ops], [o[1] for o in ops], [o[2] for o in ops], steps, warmup, use_graph)
     if ms < 0:
@@ -265,6 +383,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-baselines", action="store_true", help="skip the same-GPU BF16 baselines of the decode step")
     ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -317,7 +436,7 @@ def main():
         extra["bytes_per_token"] = step_bytes
         extra["decode_step_GBps"] = round(step_bytes / ms_step * 1e-6, 1)
         extra["decode_step_frac_of_hbm_bound"] = round(step_bytes / ms_step * 1e-6 / HBM_PEAK_GBS, 4)
-        extra["launches_per_step"] = 9 * QWEN3_8B["layers"] + 4
+        extra["launches_per_step"] = 6 * QWEN3_8B["layers"] + 4
         extra["last_token"] = model.token
         workload = ("full random-init Qwen3-8B W8A16 decode step, batch 1, greedy: 36 layers, hidden 4096, 32 q / 8 kv heads x 128, qk RMSNorm, "
                     f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions")
@@ -325,9 +444,14 @@ def main():
         K, N, M = 4096, 2 * 12288, 1
         dom_us = model.bench_gate_up(10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
-        if not args.no_sweep:
-            del model
+        del model
+        torch.cuda.empty_cache()
+        if not args.no_baselines:
+            extra["gpu_baselines"] = gpu_baselines(ws, DECODE_CTX)
+            for b in extra["gpu_baselines"].values():
+                b["speedup_of_this_build"] = round(value / b["tok_s"], 2)
             torch.cuda.empty_cache()
+        if not args.no_sweep:
             ops, by_shape = build_decode_model(ws, 1)
             lin_bytes = sum(gemv_bytes(k, n, 1) for *_, k, n in ops)
             lin_ms = time_chain(ws, ops, args.steps, args.warmup, use_graph) / args.steps

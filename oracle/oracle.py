@@ -27,7 +27,7 @@ def build(force: bool = False) -> None:
     if force or not (HERE / "liboracle.so").exists():
         subprocess.run(["make", "-C", str(HERE), "-B", "liboracle.so"], check=True, capture_output=True)
     if Path(os.environ.get("CCCC_REFERENCE", "/root/reference")).joinpath("cccc/types.h").exists():
-        if force or not (HERE / "_ref" / "libref_types.so").exists():
+        if force or not (HERE / "_ref" / "libref_types.so").exists() or not (HERE / "_ref" / "libref_hip.so").exists():
             subprocess.run(["make", "-C", str(HERE), "ref"], check=True, capture_output=True)
 
 
