@@ -113,6 +113,73 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     return m->copyFromHost(host, bytes);
 }
 
+int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, std::string* failed)
+{
+    gpu_->setAsCurrent();
+    auto fail = [&](const std::string& name, int code) {
+        if (failed) { *failed = name; }
+        return code;
+    };
+    // norms and the embedding: BF16 tensors
+    auto load_plain = [&](Matrix& m, const std::string& name) -> int {
+        const auto wk = file.resolve(name);
+        if (!wk.valid()) { return fail(name, -1); }
+        if (wk.is_quant) { return fail(name, -3); }
+        const std::vector<int> dim = { m.getWidth(), m.getHeight(), m.getChannel(), m.getNumber() };
+        Matrix tmp(dim, BFLOAT16, gpu_);
+        if (file.loadNamed(tmp, name) != 0) { return fail(name, -2); }
+        if (tmp.getDataType() == FLOAT || tmp.getDataType() == HALF)      // the file's type was kept: round to BF16 on the device
+        {
+            Matrix bf(dim, BFLOAT16, gpu_);
+            if (hip_convert(tmp.data(), (int)tmp.getDataType(), bf.data(), (int)BFLOAT16, (unsigned)tmp.getDataSize(), 1.0f) != 0) { return fail(name, -3); }
+            (void)hipDeviceSynchronize();
+            tmp = bf;
+        }
+        if (tmp.getDataType() != BFLOAT16) { return fail(name, -3); }
+        m = tmp;
+        return 0;
+    };
+    auto load_linear = [&](Matrix& m, const std::string& name) -> int {
+        const auto wk = file.resolve(name);
+        if (!wk.valid()) { return fail(name, -1); }
+        if (wk.is_quant)
+        {
+            if (wk.dt == FP4_E2M1) { return fail(name, -3); }
+            m.setAllowRepack(false);
+            return file.loadNamed(m, name) == 0 ? 0 : fail(name, -2);
+        }
+        Matrix tmp(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
+        tmp.setAllowRepack(false);
+        if (file.loadNamed(tmp, name) != 0) { return fail(name, -2); }
+        if (tmp.getDataType() == FLOAT)
+        {
+            Matrix bf(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
+            bf.setAllowRepack(false);
+            if (hip_convert(tmp.data(), (int)FLOAT, bf.data(), (int)BFLOAT16, (unsigned)tmp.getDataSize(), 1.0f) != 0) { return fail(name, -3); }
+            (void)hipDeviceSynchronize();
+            tmp = bf;
+        }
+        tmp.quantizeWeights(quantize_to);
+        if (tmp.getDataType() != FP8_E4M3 && tmp.getDataType() != FP8_E5M2) { return fail(name, -3); }
+        m = tmp;
+        return 0;
+    };
+    int rc = load_plain(*emb_, "W_emb");
+    if (rc == 0) { rc = load_plain(*rms_final_, "W_rms_final"); }
+    if (rc == 0) { rc = load_linear(*lm_head_, file.resolve("W_lm_head").valid() ? "W_lm_head" : "W_emb"); }
+    for (int i = 0; i < cfg_.layers && rc == 0; i++)
+    {
+        Layer& L = layers_[i];
+        const std::string n = std::to_string(i);
+        const std::pair<Matrix*, const char*> plain[] = { { L.rms_attn.get(), "W_rms_attn_" }, { L.q_norm.get(), "W_qnorm_" }, { L.k_norm.get(), "W_knorm_" }, { L.rms_ffn.get(), "W_rms_ffn_" } };
+        const std::pair<Matrix*, const char*> linear[] = { { L.wq.get(), "W_q_" }, { L.wk.get(), "W_k_" }, { L.wv.get(), "W_v_" }, { L.wo.get(), "W_o_" },
+                                                          { L.w_gate.get(), "W_gate_" }, { L.w_up.get(), "W_up_" }, { L.w_down.get(), "W_down_" } };
+        for (auto& [m, prefix] : plain) { if (rc == 0) { rc = load_plain(*m, prefix + n); } }
+        for (auto& [m, prefix] : linear) { if (rc == 0) { rc = load_linear(*m, prefix + n); } }
+    }
+    return rc;
+}
+
 size_t DecodeModel::weightBytes() const
 {
     const size_t q_out = (size_t)cfg_.n_q * cfg_.head_dim, kv_out = (size_t)cfg_.n_kv * cfg_.head_dim;

@@ -6,6 +6,8 @@
 // launch sequence that can be replayed as one hipGraph.
 #pragma once
 #include "Matrix.h"
+#include "WeightFile.h"
+#include <string>
 #include <memory>
 #include <vector>
 
@@ -35,6 +37,14 @@ public:
 
     // Uploads file bytes: FP8 codes for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
     int setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale);
+
+    // Loads every tensor from a converted model file by the converter's names (scripts/convert_weights.py:142-166):
+    // W_emb, W_rms_final, W_lm_head (W_emb when absent: tied), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
+    // W_qnorm_<i>, W_knorm_<i>, W_rms_ffn_<i>, W_gate_<i>, W_up_<i>, W_down_<i>.  FP8 linears are taken as stored;
+    // linears stored as BF16 / HALF / FLOAT are quantized on load to `quantize_to` with a per-tensor absmax scale
+    // (the reference's weight_data_type route, cccc/Matrix.cpp:301-355).  0 ok; otherwise `failed` names the tensor:
+    // -1 missing, -2 wrong size, -3 a type the fused decode kernels do not take (FP4, or too small to quantize).
+    int loadNamedWeights(const WeightFile& file, DataType quantize_to = FP8_E5M2, std::string* failed = nullptr);
 
     // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
     // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).

@@ -40,6 +40,9 @@ public:
     void setAllowRepack(bool allow) { if (shared_data_) { shared_data_->allow_repack_ = allow; } }
     bool hasTiled() const { return shared_data_ && shared_data_->tiled_data_ != nullptr; }
     float getInputScale() const { return shared_data_ ? shared_data_->input_scale_ : 0.0f; }
+    void setInputScale(float s) { if (shared_data_) { shared_data_->input_scale_ = s; } }
+    // Re-allocates the storage for the same dims with another element type (contents are not kept).
+    void retype(DataType dt);
 
     // Raw byte transfers between host memory and this tensor's storage.
     int copyFromHost(const void* src, size_t bytes);

@@ -1,0 +1,79 @@
+// Reader of cccc's weight container ("CFG_BIN INI") and the named-weight loading rules on top of it.
+//
+// Container, as scripts/convert_weights.py:54-83 writes it (the reading side lives in the reference's
+// un-vendored mlcc library, INIReaderBin):
+//     bytes 0..31   "CFG_BIN INI" padded with zeros
+//     bytes 32..39  little-endian uint64: length L of the index text
+//     L bytes       ASCII lines  "<key> = <offset>,<length>\n"   (offsets relative to the data area)
+//     rest          data area
+// Keys of a model file: "weight_<dtype>_<name>" with dtype in {fp8_e4m3, fp8e4m3, fp8, bf16, bfloat16,
+// float, half, fp8_e5m2, fp4_e2m1} (cccc/Net.cpp:238-248), the legacy "weight_<name>" (FP8_E4M3),
+// "scale_<name>" / "input_scale_<name>" (one float32), "blockscale_<name>" (FP4: one E4M3 byte per
+// 16 elements, or legacy float32 per block).  Loading follows Net::loadNamedWeights
+// (cccc/Net.cpp:1324-1527).  The file is memory-mapped, never read whole.
+#pragma once
+#include "Matrix.h"
+#include <string>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+namespace cccc
+{
+
+// Host-side scalar conversions the loader needs, exposed for tests.
+uint8_t floatToE4m3Truncated(float f);
+uint16_t halfBitsToBf16Truncated(uint16_t h);
+
+class WeightFile
+{
+public:
+    WeightFile() = default;
+    ~WeightFile();
+    WeightFile(const WeightFile&) = delete;
+    WeightFile& operator=(const WeightFile&) = delete;
+
+    // 0 ok; -1 cannot open / map; -2 not a CFG_BIN INI file; -3 malformed index; -4 an entry lies outside the file
+    int parseFile(const std::string& filename);
+    void close();
+
+    bool has_value(const std::string& key) const { return index_.count(key) != 0; }
+    // Bytes of an entry ({nullptr, 0} when absent); valid while the file is open.
+    std::pair<const uint8_t*, size_t> get_value(const std::string& key) const;
+    const std::vector<std::string>& keys() const { return order_; }
+    float loadFloat(const std::string& key, float default_val = 0.0f) const;
+
+    struct WeightKey
+    {
+        std::string source;    // weight name
+        std::string key;       // key of its bytes in the file
+        DataType dt = CURRENT;
+        bool is_quant = false;
+        bool valid() const { return !source.empty(); }
+    };
+    // Typed quantized key first, then the legacy "weight_<name>" (FP8_E4M3), then a typed plain key
+    // (cccc/Net.cpp:1376-1396).
+    WeightKey resolve(const std::string& name) const;
+
+    // Loads the weight `name` into m (cccc/Net.cpp:1429-1518): quantized bytes through
+    // loadQuantizedDirect with scale_<name>, FP4 block scales (E4M3 bytes or legacy float32; surplus
+    // bytes beyond elements / 16 are ignored), plain weights copied as they are (HALF converted to
+    // BF16 by truncation when m is BF16; otherwise m takes the file's dtype).
+    // 0 loaded; 1 not in the file; -1 byte count does not fit the tensor.
+    int loadNamed(Matrix& m, const std::string& name) const;
+
+private:
+    struct Entry
+    {
+        uint64_t offset, length;
+    };
+    int fd_ = -1;
+    const uint8_t* map_ = nullptr;
+    size_t map_bytes_ = 0;
+    const uint8_t* data_ = nullptr;    // start of the data area
+    size_t data_bytes_ = 0;
+    std::unordered_map<std::string, Entry> index_;
+    std::vector<std::string> order_;
+};
+
+}    // namespace cccc

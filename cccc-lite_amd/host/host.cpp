@@ -221,11 +221,21 @@ int Matrix::copyToHost(void* dst, size_t bytes) const
     return GpuControl::copyDeviceToHost(dst, data_, bytes);
 }
 
+void Matrix::retype(DataType dt)
+{
+    if (!shared_data_ || !gpu()) { return; }
+    gpu()->setAsCurrent();
+    const int64_t n = dt == FP4_E2M1 ? (getDataSize() + 1) / 2 : getDataSize();
+    shared_data_->resize(n, dt, true);
+    data_ = shared_data_->data_;
+}
+
 void Matrix::loadQuantizedDirect(const uint8_t* host_data, int64_t n, float scale, DataType fp8_dt)
 {
     if (!gpu()) { return; }
     gpu()->setAsCurrent();
-    if (getDataType() != fp8_dt) { shared_data_->resize(n, fp8_dt, true); }
+    // a storage of another type, or one too small for the upload, is replaced
+    if (getDataType() != fp8_dt || (size_t)n > shared_data_->sizeInByte()) { shared_data_->resize(n, fp8_dt, true); }
     GpuControl::copyHostToDevice(shared_data_->data_, host_data, (size_t)n);
     shared_data_->quant_scale_ = scale;
     data_ = shared_data_->data_;

@@ -2,6 +2,7 @@
 // same Matrix::mulBatched path a cccc graph would, plus a timing loop that runs a chain of linears
 // from native code (Python call overhead would otherwise dominate microsecond kernels).
 #include "DecodeModel.h"
+#include <cstring>
 #include "Matrix.h"
 #include "../../include/cccc_hip_quant.h"
 #include <hip/hip_runtime.h>
@@ -190,6 +191,60 @@ double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n
     return result;
 }
 
+// ---- weight container
+
+void* cccc_weightfile_open(const char* path, int* status)
+{
+    auto* f = new WeightFile();
+    const int rc = f->parseFile(path);
+    if (status) { *status = rc; }
+    if (rc != 0)
+    {
+        delete f;
+        return nullptr;
+    }
+    return f;
+}
+
+void cccc_weightfile_close(void* f) { delete (WeightFile*)f; }
+
+int cccc_weightfile_count(void* f) { return (int)((WeightFile*)f)->keys().size(); }
+
+const char* cccc_weightfile_key(void* f, int i)
+{
+    const auto& keys = ((WeightFile*)f)->keys();
+    return (i >= 0 && i < (int)keys.size()) ? keys[i].c_str() : nullptr;
+}
+
+// Copies up to `capacity` bytes of the entry to dst (dst may be NULL); returns its length, -1 when absent.
+long long cccc_weightfile_get(void* f, const char* key, void* dst, unsigned long long capacity)
+{
+    auto [p, n] = ((WeightFile*)f)->get_value(key);
+    if (!p && !((WeightFile*)f)->has_value(key)) { return -1; }
+    if (dst && n) { std::memcpy(dst, p, n < capacity ? n : (size_t)capacity); }
+    return (long long)n;
+}
+
+// Resolves a weight name: writes the key into key_out (NUL-terminated, truncated to capacity) and returns the
+// dtype, with bit 16 set when the entry is quantized; -1 when the name is not in the file.
+int cccc_weightfile_resolve(void* f, const char* name, char* key_out, int capacity)
+{
+    const auto wk = ((WeightFile*)f)->resolve(name);
+    if (!wk.valid()) { return -1; }
+    if (key_out && capacity > 0)
+    {
+        std::strncpy(key_out, wk.key.c_str(), (size_t)capacity - 1);
+        key_out[capacity - 1] = 0;
+    }
+    return (int)wk.dt | (wk.is_quant ? 0x10000 : 0);
+}
+
+int cccc_weightfile_load_named(void* f, void* m, const char* name) { return ((WeightFile*)f)->loadNamed(*(Matrix*)m, name); }
+
+unsigned char cccc_host_float_to_e4m3(float v) { return floatToE4m3Truncated(v); }
+
+unsigned short cccc_host_half_to_bf16(unsigned short h) { return halfBitsToBf16Truncated(h); }
+
 // ---- decode model
 
 void* cccc_decode_create(int layers, int hidden, int n_q, int n_kv, int head_dim, int inter, int vocab, int t_kv, float theta, float eps)
@@ -219,6 +274,18 @@ int cccc_decode_tensor_prepare(void* m, int layer, int which)
     if (!t) { return -1; }
     t->prepareTiled();
     return t->hasTiled() ? 0 : 1;
+}
+
+int cccc_decode_load_named(void* m, void* f, int quantize_to, char* failed_out, int capacity)
+{
+    std::string failed;
+    const int rc = ((DecodeModel*)m)->loadNamedWeights(*(WeightFile*)f, (DataType)quantize_to, &failed);
+    if (failed_out && capacity > 0)
+    {
+        std::strncpy(failed_out, failed.c_str(), (size_t)capacity - 1);
+        failed_out[capacity - 1] = 0;
+    }
+    return rc;
 }
 
 void cccc_decode_set_exact_attention(void* m, int exact) { ((DecodeModel*)m)->setExactAttention(exact != 0); }

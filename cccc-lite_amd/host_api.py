@@ -55,6 +55,16 @@ class HostLibrary:
         L.cccc_decode_kv.restype = i32; L.cccc_decode_kv.argtypes = [vp, i32, i32, vp, u64]
         L.cccc_decode_cos_table.restype = i32; L.cccc_decode_cos_table.argtypes = [vp, vp, u64]
         L.cccc_decode_weight_bytes.restype = u64; L.cccc_decode_weight_bytes.argtypes = [vp]
+        L.cccc_weightfile_open.restype = vp; L.cccc_weightfile_open.argtypes = [ctypes.c_char_p, ctypes.POINTER(i32)]
+        L.cccc_weightfile_close.restype = None; L.cccc_weightfile_close.argtypes = [vp]
+        L.cccc_weightfile_count.restype = i32; L.cccc_weightfile_count.argtypes = [vp]
+        L.cccc_weightfile_key.restype = ctypes.c_char_p; L.cccc_weightfile_key.argtypes = [vp, i32]
+        L.cccc_weightfile_get.restype = ctypes.c_longlong; L.cccc_weightfile_get.argtypes = [vp, ctypes.c_char_p, vp, u64]
+        L.cccc_weightfile_resolve.restype = i32; L.cccc_weightfile_resolve.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p, i32]
+        L.cccc_weightfile_load_named.restype = i32; L.cccc_weightfile_load_named.argtypes = [vp, vp, ctypes.c_char_p]
+        L.cccc_host_float_to_e4m3.restype = ctypes.c_ubyte; L.cccc_host_float_to_e4m3.argtypes = [f32]
+        L.cccc_host_half_to_bf16.restype = ctypes.c_ushort; L.cccc_host_half_to_bf16.argtypes = [ctypes.c_ushort]
+        L.cccc_decode_load_named.restype = i32; L.cccc_decode_load_named.argtypes = [vp, vp, i32, ctypes.c_char_p, i32]
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         L.cccc_decode_bench_gate_up.restype = ctypes.c_double; L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
@@ -80,6 +90,45 @@ class HostLibrary:
         n = len(W_ptrs)
         return float(self.c.cccc_bench_fp4_chain(n, (ctypes.c_void_p * n)(*W_ptrs), (ctypes.c_void_p * n)(*S_ptrs), X_ptr, Y_ptr,
                                                  n_out, tokens, K, block, iters, warmup))
+
+
+class WeightFile:
+    """host/WeightFile.h: memory-mapped reader of a CFG_BIN INI container (no GPU needed to open or query it)."""
+
+    def __init__(self, lib: HostLibrary, path):
+        self.lib = lib
+        status = ctypes.c_int(0)
+        self.handle = lib.c.cccc_weightfile_open(str(path).encode(), ctypes.byref(status))
+        self.status = status.value
+        if not self.handle:
+            raise OSError(f"cannot read weight file {path}: status {self.status}")
+
+    def close(self) -> None:
+        if getattr(self, "handle", None):
+            self.lib.c.cccc_weightfile_close(self.handle)
+            self.handle = None
+
+    __del__ = close
+
+    def keys(self) -> list[str]:
+        return [self.lib.c.cccc_weightfile_key(self.handle, i).decode() for i in range(self.lib.c.cccc_weightfile_count(self.handle))]
+
+    def get(self, key: str):
+        n = self.lib.c.cccc_weightfile_get(self.handle, key.encode(), None, 0)
+        if n < 0:
+            return None
+        buf = ctypes.create_string_buffer(max(int(n), 1))
+        self.lib.c.cccc_weightfile_get(self.handle, key.encode(), buf, n)
+        return buf.raw[:n]
+
+    def resolve(self, name: str):
+        """(key, dtype, is_quantized) or None."""
+        buf = ctypes.create_string_buffer(256)
+        rc = self.lib.c.cccc_weightfile_resolve(self.handle, name.encode(), buf, 256)
+        return None if rc < 0 else (buf.value.decode(), rc & 0xFFFF, bool(rc & 0x10000))
+
+    def load_named(self, m: "HostMatrix", name: str) -> int:
+        return self.lib.c.cccc_weightfile_load_named(self.handle, m.handle, name.encode())
 
 
 class HostMatrix:
@@ -195,6 +244,13 @@ class DecodeModel:
         for li, L in enumerate(model["layers"]):
             for name in LAYER_TENSORS:
                 self.set_tensor(li, name, L[name], fp8_dtype if name in QUANTIZED else 3)
+
+    def load_named(self, wf: WeightFile, quantize_to: int = 5) -> None:
+        """Every tensor from a converted model file by the converter's names; plain linears are quantized on load."""
+        failed = ctypes.create_string_buffer(128)
+        rc = self.lib.c.cccc_decode_load_named(self.handle, wf.handle, quantize_to, failed, 128)
+        if rc != 0:
+            raise ValueError(f"loading {failed.value.decode()!r} failed: {rc}")
 
     def set_exact_attention(self, exact: bool) -> None:
         """True: separate norm / RoPE / append launch and BF16 probabilities (the reference's rounding
