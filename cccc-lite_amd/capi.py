@@ -174,12 +174,12 @@ class QuantLibrary:
 
     # -- the call the LLM graph makes --------------------------------------------------------
     def linear(self, W, w_type, X, Y, n_out, tokens, K, inv_scale=1.0, blk_sc=None, block_size=16,
-               alpha=1.0, beta=0.0) -> int:
+               alpha=1.0, beta=0.0, act_type=DataType.BFLOAT16) -> int:
         """y[t][o] = sum_k W[o][k] x[t][k], argument layout of Matrix::mulBatched(W, X, Y, TRANS,
         NO_TRANS) for a linear layer (reference cccc/Matrix.cpp:1162-1203): BLAS M = n_out,
         BLAS N = tokens, lda = ldb = K, ldc = n_out."""
         return self.quant_gemm(TRANS, NO_TRANS, n_out, tokens, K, alpha, W, w_type, K, inv_scale,
-                               X, DataType.BFLOAT16, K, 1.0, beta, Y, DataType.BFLOAT16, n_out, 0.0,
+                               X, act_type, K, 1.0, beta, Y, act_type, n_out, 0.0,
                                blk_sc, None, block_size)
 
 

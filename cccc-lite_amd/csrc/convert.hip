@@ -31,13 +31,6 @@ __device__ __forceinline__ float decode8(uint32_t b)
     return SRC == DT_E5M2 ? e5m2_to_f32(b) : e4m3_to_f32(b);
 }
 
-__device__ __forceinline__ uint32_t f32_to_half_bits(float f)
-{
-    const _Float16 h = (_Float16)f;    // v_cvt_f16_f32, round to nearest even
-    // the sign is carried over explicitly so that -0.0 stays -0.0
-    return ((uint32_t)__builtin_bit_cast(uint16_t, h) & 0x7FFFu) | ((f32_to_bits(f) >> 16) & 0x8000u);
-}
-
 template <int DST>
 __device__ __forceinline__ void store_one(void* dst, size_t i, float v)
 {

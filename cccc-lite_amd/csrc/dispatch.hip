@@ -8,6 +8,7 @@
 //     FP4 without block scales): generic
 #include "../../include/cccc_hip_quant.h"
 #include "gemv_kernels.h"
+#include "dispatch_half.h"
 #include "gemm_kernels.h"
 #include "runtime.h"
 #include <cstdio>
@@ -217,14 +218,18 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                    const void* blk_scA, const void* blk_scB, unsigned int block_size)
 {
     const bool aQ = is_quantized(typeA), bQ = is_quantized(typeB);
-    if (aQ == bQ || typeC != DT_BF16) { return -1; }
-    if ((aQ && typeB != DT_BF16) || (bQ && typeA != DT_BF16)) { return -1; }
+    if (aQ == bQ) { return -1; }
+    // the unquantized operand and C share one 16-bit type: BF16 (cccc/cublas_real.h:943-964) or HALF (:921-938, FP8 weights only)
+    const int act_type = aQ ? typeB : typeA;
+    if ((act_type != DT_BF16 && act_type != DT_HALF) || typeC != act_type) { return -1; }
+    if (act_type == DT_HALF && (aQ ? typeA : typeB) == DT_FP4) { return -1; }
     if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1)) { return -1; }
     if (M < 0 || N < 0 || K < 0 || lda <= 0 || ldb <= 0 || ldc <= 0) { return -1; }
     if (M == 0 || N == 0) { return 0; }
     if (!A || !B || !C) { return -1; }
 
     GenericArgs g{};
+    g.act_type = act_type;
     g.K = K;
     g.alpha = alpha;
     g.beta = beta;
@@ -285,7 +290,15 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         a.alpha = alpha;
         a.beta = beta;
         const bool x_ok = aligned16(a.X) && a.ldx % 8 == 0;
-        if (g.w_type == DT_FP4)
+        if (act_type == DT_HALF)
+        {
+            if (x_ok && K % 16 == 0 && a.ldw % 16 == 0 && aligned16(a.W))
+            {
+                note_kernel(half_linear(a, g.w_type));
+                launched = true;
+            }
+        }
+        else if (g.w_type == DT_FP4)
         {
             const bool ok = x_ok && a.blk_sc && (a.block_size == 16 || a.block_size == 32) && K % 32 == 0 && a.ldw % 32 == 0 &&
                             aligned16(a.W) && ((uintptr_t)a.blk_sc & 1u) == 0;

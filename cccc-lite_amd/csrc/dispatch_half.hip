@@ -1,0 +1,61 @@
+#include "dispatch_half.h"
+#include "gemm_kernels.h"
+#include "gemv_kernels.h"
+#include "runtime.h"
+
+namespace ccq
+{
+
+namespace
+{
+
+template <int WT, int MT, int R, int WAVES, int OCC, bool SCALED>
+void launch_half_gemv(const LinearArgs& a)
+{
+    const int n_groups = (a.n_out + R - 1) / R;
+    const int want = (n_groups + WAVES - 1) / WAVES;
+    const int cap = cu_count() * OCC;
+    const size_t lds = (size_t)MT * ((a.K + 1023) / 1024) * 2048;
+    gemv8_dot2_kernel<WT, MT, R, 4, WAVES, SCALED, DT_HALF><<<want < cap ? want : cap, WAVES * 64, lds, stream()>>>(a);
+}
+
+// the two shapes of the BF16 dispatch that matter most: tall weights and long rows take 8-wave workgroups
+template <int WT, int MT, bool SCALED>
+void pick_half_gemv(const LinearArgs& a)
+{
+    if (a.K > 8192 || a.n_out / cu_count() >= 128) { launch_half_gemv<WT, MT, 1, 8, 2, SCALED>(a); }
+    else { launch_half_gemv<WT, MT, 2, 4, 4, SCALED>(a); }
+}
+
+template <int WT, bool SCALED>
+bool half_gemv(const LinearArgs& a)
+{
+    if ((size_t)a.tokens * ((a.K + 1023) / 1024) * 2048 > 64 * 1024) { return false; }
+    switch (a.tokens)
+    {
+    case 1: pick_half_gemv<WT, 1, SCALED>(a); return true;
+    case 2: pick_half_gemv<WT, 2, SCALED>(a); return true;
+    case 3: pick_half_gemv<WT, 3, SCALED>(a); return true;
+    case 4: pick_half_gemv<WT, 4, SCALED>(a); return true;
+    default: return false;
+    }
+}
+
+}    // namespace
+
+const char* half_linear(const LinearArgs& a, int w_type)
+{
+    const bool scaled = a.w_scale != 1.0f;
+    if (a.tokens <= 4)
+    {
+        bool ok;
+        if (w_type == DT_E5M2) { ok = scaled ? half_gemv<DT_E5M2, true>(a) : half_gemv<DT_E5M2, false>(a); }
+        else { ok = scaled ? half_gemv<DT_E4M3, true>(a) : half_gemv<DT_E4M3, false>(a); }
+        if (ok) { return "gemv_dot2_half"; }
+    }
+    if (w_type == DT_E5M2) { gemm_mfma<DT_E5M2, 0, DT_HALF>(a); }
+    else { gemm_mfma<DT_E4M3, 0, DT_HALF>(a); }
+    return "gemm_mfma_half";
+}
+
+}    // namespace ccq

@@ -14,9 +14,11 @@
 //   B operand (columns) = output features, same k split
 //   D: lane holds column lane % 32; register v is row 8 (v / 4) + 4 (lane / 32) + v % 4
 #pragma once
+#include "gemv_kernels.h"
 #include "linear_args.h"
 #include "quant_device.h"
 #include "runtime.h"
+#include <type_traits>
 
 namespace ccq
 {
@@ -27,43 +29,15 @@ template <int CPR>
 __device__ __forceinline__ int swizzled_chunk_n(int row, int chunk) { return CPR == 16 ? (chunk ^ (row & 15)) : (chunk ^ ((row >> 1) & 7)); }
 
 // 16 FP8 codes -> 16 BF16 (two 16-byte LDS chunks)
-template <int WT, bool SCALED>
+template <int WT, bool SCALED, int AT = DT_BF16>
 __device__ __forceinline__ void dequant16_fp8(const u32x4& w, float scale, u32x4& lo, u32x4& hi)
 {
     uint32_t out[8];
 #pragma unroll
     for (int d = 0; d < 4; d++)
     {
-        bf16x2 p, q;
-        if (!SCALED)
-        {
-            if (WT == DT_E5M2)
-            {
-                p = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w[d], 1.0f, false);
-                q = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w[d], 1.0f, true);
-            }
-            else
-            {
-                p = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[d], 1.0f, false);
-                q = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[d], 1.0f, true);
-            }
-        }
-        else
-        {
-            f32x2 a, b;
-            if (WT == DT_E5M2)
-            {
-                a = __builtin_amdgcn_cvt_pk_f32_bf8(w[d], false);
-                b = __builtin_amdgcn_cvt_pk_f32_bf8(w[d], true);
-            }
-            else
-            {
-                a = __builtin_amdgcn_cvt_pk_f32_fp8(w[d], false);
-                b = __builtin_amdgcn_cvt_pk_f32_fp8(w[d], true);
-            }
-            p = bf16x2{ (__bf16)(a.x * scale), (__bf16)(a.y * scale) };
-            q = bf16x2{ (__bf16)(b.x * scale), (__bf16)(b.y * scale) };
-        }
+        typename ActPair<AT>::type p, q;
+        fp8x4_to_pairs<WT, SCALED, AT>(w[d], scale, p, q);
         out[2 * d] = __builtin_bit_cast(uint32_t, p);
         out[2 * d + 1] = __builtin_bit_cast(uint32_t, q);
     }
@@ -94,7 +68,7 @@ __device__ __forceinline__ u32x4 dequant8_fp4(uint32_t w, float scale)
 
 // WT: DT_E5M2 / DT_E4M3 / DT_FP4.  BLOCK: FP4 block length (16 / 32), unused for FP8.
 // Requires K % 16 == 0 (FP8) or K % 32 == 0 (FP4), and the alignment rules of the GEMV kernels.
-template <int WT, int BLOCK, int BM, int BN, bool SCALED, int BK = 64, bool XCD = false>
+template <int WT, int BLOCK, int BM, int BN, bool SCALED, int BK = 64, bool XCD = false, int AT = DT_BF16>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, const int n_tiles, const int m_tiles)
 {
     constexpr int WM = BM / 2;          // output features per wave
@@ -205,7 +179,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
                 else
                 {
                     u32x4 lo, hi;
-                    dequant16_fp8<WT, SCALED>(wreg[i], a.w_scale, lo, hi);
+                    dequant16_fp8<WT, SCALED, AT>(wreg[i], a.w_scale, lo, hi);
                     ws[row * CPR + swizzled_chunk_n<CPR>(row, part * 2)] = lo;
                     ws[row * CPR + swizzled_chunk_n<CPR>(row, part * 2 + 1)] = hi;
                 }
@@ -232,23 +206,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++)
         {
-            bf16x8 xf[TN], wf[TM];
+            typedef typename std::conditional<AT == DT_HALF, f16x8, bf16x8>::type frag_t;
+            frag_t xf[TN], wf[TM];
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
             {
                 const int row = wave_n * WN + tn * 32 + r32;
-                xf[tn] = __builtin_bit_cast(bf16x8, xs[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
+                xf[tn] = __builtin_bit_cast(frag_t, xs[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
             }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
             {
                 const int row = wave_m * WM + tm * 32 + r32;
-                wf[tm] = __builtin_bit_cast(bf16x8, ws[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
+                wf[tm] = __builtin_bit_cast(frag_t, ws[row * CPR + swizzled_chunk_n<CPR>(row, ks * 2 + h)]);
             }
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++) { acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tn], wf[tm], acc[tn][tm], 0, 0, 0); }
+                for (int tm = 0; tm < TM; tm++)
+                {
+                    if constexpr (AT == DT_HALF) { acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[tn], wf[tm], acc[tn][tm], 0, 0, 0); }
+                    else { acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tn], wf[tm], acc[tn][tm], 0, 0, 0); }
+                }
         }
         __syncthreads();
     }
@@ -267,36 +246,36 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
                 if (out < a.n_out && tok < a.tokens)
                 {
                     uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
-                    *y = finish_output(acc[tn][tm][v], a.alpha, a.beta, y);
+                    *y = finish_output_act<AT>(acc[tn][tm][v], a.alpha, a.beta, y);
                 }
             }
         }
     }
 }
 
-template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false>
+template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false, int AT = DT_BF16>
 void launch_gemm_mfma(const LinearArgs& a)
 {
     const int n_tiles = (a.n_out + BM - 1) / BM;
     const int m_tiles = (a.tokens + BN - 1) / BN;
     const int grid = XCD ? 8 * m_tiles * ((n_tiles + 7) / 8) : n_tiles * m_tiles;
-    if (WT != DT_FP4 && a.w_scale != 1.0f) { gemm_mfma_kernel<WT, BLOCK, BM, BN, true, BK, XCD><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
-    else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false, BK, XCD><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+    if (WT != DT_FP4 && a.w_scale != 1.0f) { gemm_mfma_kernel<WT, BLOCK, BM, BN, true, BK, XCD, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+    else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false, BK, XCD, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
 }
 
 // Tile choice (tuned on MI355X): 128 x 128 tiles with the XCD-aware order when they give every CU at
 // least two workgroups (k step 128 for long K, where it halves the barriers per FLOP), otherwise
 // 128 x 64 tiles to put more workgroups on the machine.
-template <int WT, int BLOCK>
+template <int WT, int BLOCK, int AT = DT_BF16>
 bool gemm_mfma(const LinearArgs& a)
 {
     const long long tiles_big = (long long)((a.n_out + 127) / 128) * ((a.tokens + 127) / 128);
     if (tiles_big >= 2LL * cu_count())
     {
-        if (a.K >= 8192) { launch_gemm_mfma<WT, BLOCK, 128, 128, 128, true>(a); }
-        else { launch_gemm_mfma<WT, BLOCK, 128, 128, 64, true>(a); }
+        if (a.K >= 8192) { launch_gemm_mfma<WT, BLOCK, 128, 128, 128, true, AT>(a); }
+        else { launch_gemm_mfma<WT, BLOCK, 128, 128, 64, true, AT>(a); }
     }
-    else { launch_gemm_mfma<WT, BLOCK, 128, 64, 64, false>(a); }
+    else { launch_gemm_mfma<WT, BLOCK, 128, 64, 64, false, AT>(a); }
     return true;
 }
 

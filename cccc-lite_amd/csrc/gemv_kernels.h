@@ -60,6 +60,61 @@ __device__ __forceinline__ float dot2_bf16(bf16x2 a, uint32_t x, float acc)
     return __builtin_amdgcn_fdot2_f32_bf16(a, __builtin_bit_cast(bf16x2, x), acc, false);
 }
 
+// The same two steps for either 16-bit activation type.  HALF: the weight entering a product is
+// half(decode(w) * scale) (cccc/cublas_real.h:921-938); every E5M2 / E4M3 value is a half exactly.
+template <int AT>
+struct ActPair
+{
+    typedef bf16x2 type;
+};
+template <>
+struct ActPair<DT_HALF>
+{
+    typedef f16x2 type;
+};
+
+template <int WT, bool SCALED, int AT>
+__device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, float scale, typename ActPair<AT>::type& p01, typename ActPair<AT>::type& p23)
+{
+    if constexpr (AT == DT_BF16) { fp8x4_to_bf16<WT, SCALED>(w, scale, p01, p23); }
+    else if constexpr (!SCALED)
+    {
+        if (WT == DT_E5M2)
+        {
+            p01 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(w, 1.0f, false);
+            p23 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(w, 1.0f, true);
+        }
+        else
+        {
+            p01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+            p23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+        }
+    }
+    else
+    {
+        f32x2 a, b;
+        if (WT == DT_E5M2)
+        {
+            a = __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+            b = __builtin_amdgcn_cvt_pk_f32_bf8(w, true);
+        }
+        else
+        {
+            a = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+            b = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+        }
+        p01 = f16x2{ (_Float16)(a.x * scale), (_Float16)(a.y * scale) };
+        p23 = f16x2{ (_Float16)(b.x * scale), (_Float16)(b.y * scale) };
+    }
+}
+
+template <int AT>
+__device__ __forceinline__ float dot2_act(typename ActPair<AT>::type a, uint32_t x, float acc)
+{
+    if constexpr (AT == DT_BF16) { return dot2_bf16(a, x, acc); }
+    else { return __builtin_amdgcn_fdot2(a, __builtin_bit_cast(f16x2, x), acc, false); }
+}
+
 // ------------------------------------------------------------------------------------------
 // Activations in LDS.  A "k-step" is the span one wave covers with one 128-bit load per lane:
 // KSTEP elements.  Each lane needs KSTEP/64 consecutive BF16 of every token per step; they are
@@ -97,7 +152,7 @@ __device__ __forceinline__ void stage_activations(const LinearArgs& a, u32x4* xs
 // Requires: K % 16 == 0, ldw % 16 == 0, W 16-byte aligned, ldx % 8 == 0, X 16-byte aligned.
 // Dynamic LDS: MT * ceil(K / 1024) * 2048 bytes.
 
-template <int WT, int MT, int R, int U, int WAVES, bool SCALED>
+template <int WT, int MT, int R, int U, int WAVES, bool SCALED, int AT = DT_BF16>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs a)
 {
     extern __shared__ u32x4 xs[];
@@ -157,13 +212,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs
 #pragma unroll
                         for (int d = 0; d < 4; d++)
                         {
-                            bf16x2 p01, p23;
-                            fp8x4_to_bf16<WT, SCALED>(w[u][r][d], a.w_scale, p01, p23);
+                            typename ActPair<AT>::type p01, p23;
+                            fp8x4_to_pairs<WT, SCALED, AT>(w[u][r][d], a.w_scale, p01, p23);
 #pragma unroll
                             for (int t = 0; t < MT; t++)
                             {
-                                acc[r][t] = dot2_bf16(p01, x[t][d >> 1][(d & 1) * 2 + 0], acc[r][t]);
-                                acc[r][t] = dot2_bf16(p23, x[t][d >> 1][(d & 1) * 2 + 1], acc[r][t]);
+                                acc[r][t] = dot2_act<AT>(p01, x[t][d >> 1][(d & 1) * 2 + 0], acc[r][t]);
+                                acc[r][t] = dot2_act<AT>(p23, x[t][d >> 1][(d & 1) * 2 + 1], acc[r][t]);
                             }
                         }
                     }
@@ -182,7 +237,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs
                 if (lane == 0 && row < a.n_out)
                 {
                     uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)row * a.y_stride_out;
-                    *y = finish_output(total, a.alpha, a.beta, y);
+                    *y = finish_output_act<AT>(total, a.alpha, a.beta, y);
                 }
             }
         }
@@ -832,6 +887,7 @@ struct GenericArgs
     uint16_t* Y;
     long long w_stride_out, w_stride_k, x_stride_tok, x_stride_k, y_stride_tok, y_stride_out;
     int n_out, tokens, K, w_type;
+    int act_type;              // DT_BF16 or DT_HALF: type of X and Y, and the rounding of the dequantised weight
     unsigned block_size;
     float w_scale, alpha, beta;
 };
@@ -858,12 +914,13 @@ static __global__ __launch_bounds__(256) void generic_linear_kernel(const Generi
             {
                 wv = (a.w_type == DT_E5M2 ? e5m2_to_f32(a.W[fi]) : e4m3_to_f32(a.W[fi])) * a.w_scale;
             }
-            const float wq = bf16_bits_to_f32(f32_to_bf16_bits(wv));
-            const float xv = bf16_bits_to_f32(a.X[(long long)t * a.x_stride_tok + (long long)k * a.x_stride_k]);
-            acc = fmaf(wq, xv, acc);
+            const uint32_t xb = a.X[(long long)t * a.x_stride_tok + (long long)k * a.x_stride_k];
+            const bool half = a.act_type == DT_HALF;
+            const float wq = half ? half_bits_to_f32(f32_to_half_bits(wv)) : bf16_bits_to_f32(f32_to_bf16_bits(wv));
+            acc = fmaf(wq, half ? half_bits_to_f32(xb) : bf16_bits_to_f32(xb), acc);
         }
         uint16_t* y = a.Y + (long long)t * a.y_stride_tok + (long long)o * a.y_stride_out;
-        *y = finish_output(acc, a.alpha, a.beta, y);
+        *y = a.act_type == DT_HALF ? finish_output_act<DT_HALF>(acc, a.alpha, a.beta, y) : finish_output(acc, a.alpha, a.beta, y);
     }
 }
 

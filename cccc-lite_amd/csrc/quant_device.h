@@ -28,6 +28,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
@@ -93,6 +95,32 @@ __device__ __forceinline__ uint16_t finish_output(float acc, float alpha, float 
     float r = alpha * acc;
     if (beta != 0.0f) { r += beta * bf16_bits_to_f32(*y); }
     return (uint16_t)f32_to_bf16_bits(r);
+}
+
+// ---- IEEE half (the reference's other 16-bit activation type, cccc/cublas_real.h:921-938)
+
+__device__ __forceinline__ uint32_t f32_to_half_bits(float f)
+{
+    const _Float16 h = (_Float16)f;    // v_cvt_f16_f32, round to nearest even
+    // the sign is carried over explicitly so that -0.0 stays -0.0
+    return ((uint32_t)__builtin_bit_cast(uint16_t, h) & 0x7FFFu) | ((f32_to_bits(f) >> 16) & 0x8000u);
+}
+
+__device__ __forceinline__ float half_bits_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
+
+// 16-bit activation / output element of type AT (DT_BF16 or DT_HALF)
+template <int AT>
+__device__ __forceinline__ float act_bits_to_f32(uint32_t h) { return AT == DT_HALF ? half_bits_to_f32(h) : bf16_bits_to_f32(h); }
+
+template <int AT>
+__device__ __forceinline__ uint32_t f32_to_act_bits(float f) { return AT == DT_HALF ? f32_to_half_bits(f) : f32_to_bf16_bits(f); }
+
+template <int AT>
+__device__ __forceinline__ uint16_t finish_output_act(float acc, float alpha, float beta, const uint16_t* y)
+{
+    float r = alpha * acc;
+    if (beta != 0.0f) { r += beta * act_bits_to_f32<AT>(*y); }
+    return (uint16_t)f32_to_act_bits<AT>(r);
 }
 
 // ---- wave64 reductions (DPP inside a 16-lane row, then across the four rows)

@@ -83,9 +83,11 @@ C_EXPORT int hip_absmax(const void* src, int src_type, unsigned int n, void* d_r
  * BF16, C BF16 -- the W8A16 / FP4 branches cccc/cublas_real.h:943-964 (weight is A) and
  * :1066-1087 (weight is B).  Semantics are the reference's: the weight is dequantised to BF16
  * (times invScale, or times its per-block E4M3 scale when blk_sc is given for FP4), multiplied
- * with FP32 accumulation, alpha/beta applied in FP32, rounded once to BF16.  `act_scale` is
- * accepted and ignored (it only drives the W8A8 route, cccc/cublas_real.h:871-873).
- * Anything else returns -1.
+ * with FP32 accumulation, alpha/beta applied in FP32, rounded once to BF16.  The HALF twin of the
+ * FP8 branches is implemented as well (cccc/cublas_real.h:921-938: FP8 weight, the other operand and
+ * C of type HALF; the weight is dequantised to half, FP32 accumulation, one rounding to half).
+ * `act_scale` is accepted and ignored (it only drives the W8A8 route, cccc/cublas_real.h:871-873).
+ * Anything else (both operands quantized, FP4 with HALF, mixed 16-bit types, other C types) returns -1.
  */
 C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                             const void* A, int typeA, int lda, float invScaleA,

@@ -120,6 +120,25 @@ def dequant_fp8_to_bf16(codes: np.ndarray, dtype: int, inv_scale: float = 1.0) -
     return f32_to_bf16(f)
 
 
+def dequant_fp8_to_half(codes: np.ndarray, dtype: int, inv_scale: float = 1.0) -> np.ndarray:
+    """half_rne(decode(code) * inv_scale) as float16: the workspace of the reference's HALF route
+    (cccc/cublas_real.h:921-938 -> cuda_convert(.., HALF, .., invScaleA)).  NumPy's float32 -> float16
+    cast rounds to nearest even; with inv_scale 1 every FP8 value is a half exactly (E5M2 is the high
+    byte of an IEEE half, which tests/test_oracle_formats.py checks)."""
+    table = decode_table(dtype)
+    with np.errstate(over="ignore", invalid="ignore"):
+        return (table[np.asarray(codes, dtype=np.uint8)] * np.float32(inv_scale)).astype(np.float16)
+
+
+def contract_exact(W: np.ndarray, X: np.ndarray, chunk: int = 8192) -> np.ndarray:
+    """float64 X @ W^T for W [n_out, K] and X [tokens, K] of any float type."""
+    out = np.empty((X.shape[0], W.shape[0]), dtype=np.float64)
+    X64 = X.astype(np.float64)
+    for r0 in range(0, W.shape[0], chunk):
+        out[:, r0:r0 + chunk] = X64 @ W[r0:r0 + chunk].astype(np.float64).T
+    return out
+
+
 def unpack_fp4(nibbles: np.ndarray, n: int) -> np.ndarray:
     """uint8 codes of n elements: low nibble = even element (cccc/types.h:257-261)."""
     b = np.ascontiguousarray(nibbles, dtype=np.uint8).ravel()
