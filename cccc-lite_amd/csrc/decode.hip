@@ -23,6 +23,12 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
         const int want = (n_groups + 7) / 8;
         gemv8_fused_kernel<WT, 4, 8, SCALED><<<want < cus * 2 ? want : cus * 2, 512, lds, stream()>>>(a);
     }
+    else if (a.K <= 4096)
+    {
+        // short rows: two batches of 2 KiB per row pair keep the next request ahead of the multiply (measured 5-10 % faster than one batch of 4)
+        const int want = (n_groups + 3) / 4;
+        gemv8_fused_kernel<WT, 2, 4, SCALED><<<want < cus * 4 ? want : cus * 4, 256, lds, stream()>>>(a);
+    }
     else
     {
         const int want = (n_groups + 3) / 4;
