@@ -383,6 +383,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--sweep-tokens", default="1,4,16", help="token counts of the per-shape GEMV sweep")
     ap.add_argument("--no-baselines", action="store_true", help="skip the same-GPU BF16 baselines of the decode step")
     ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
     args = ap.parse_args()
@@ -457,7 +458,7 @@ def main():
             lin_ms = time_chain(ws, ops, args.steps, args.warmup, use_graph) / args.steps
             extra["quant_gemv"] = {"workload": "the 253 FP8_E5M2 linears of one decode token through Matrix::mulBatched", "ms_per_step": round(lin_ms, 4),
                                    "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
-            extra["sweep"] = shape_sweep(ws, by_shape, (1, 4, 16), False)
+            extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
             extra["fp4_sweep"] = fp4_sweep(ws)
     elif args.workload == "decode_linears":
         ops, by_shape = build_decode_model(ws, 1)
@@ -479,7 +480,7 @@ def main():
         dom_ms = time_chain(ws, dom_ops, 10, 2, False)
         dom_us = dom_ms * 1000.0 / (10 * len(dom_ops))
         if not args.no_sweep:
-            extra["sweep"] = shape_sweep(ws, by_shape, (1, 4, 16), False)
+            extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
             extra["fp4_sweep"] = fp4_sweep(ws)
     else:
         K, N = (int(v) for v in args.shape.split(","))
@@ -516,7 +517,7 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "traffic": GEMV_GATE_UP_TRAFFIC_BYTES if (K, N, M) == (4096, 12288, 1) else None,
-                    "kernel": "gemv8_dot2_kernel", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
+                    "kernel": ws.lib.last_kernel(), "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
                     "bytes_per_launch": gemv_bytes(K, N, M)}
 
     line = {

@@ -12,6 +12,7 @@
 #include "gemm_kernels.h"
 #include "runtime.h"
 #include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <shared_mutex>
 #include <unordered_map>
@@ -102,6 +103,48 @@ bool gemv8_mfma(const LinearArgs& a)
     return true;
 }
 
+// The same kernel on the load-time tiled copy: every load instruction of a wave covers one contiguous
+// KiB and a workgroup walks one contiguous row tile, which streams better than the row-major kernels
+// at every token count (lm_head, one token: 89.8 us against 92.7 for the dot2 kernel; 16 tokens:
+// 100 us against 125 for a variant that kept the activations in LDS).  Configurations tuned on
+// MI355X over the Qwen3-8B shapes with rotating weights.
+template <int WT, int RT, int U, int WAVES, bool SCALED>
+void launch_ksplit_tiled(const LinearArgs& t)
+{
+    gemv8_mfma_kernel<WT, RT, U, WAVES, SCALED, true><<<(t.n_out + 16 * RT - 1) / (16 * RT), WAVES * 64, 0, stream()>>>(t);
+}
+
+template <int WT, bool SCALED>
+bool gemv8_mfma_ksplit_tiled(const LinearArgs& a, const uint8_t* tiled)
+{
+    LinearArgs t = a;
+    t.W = tiled;
+    const int tiles_per_cu = ((a.n_out + 15) / 16) / cu_count();
+    if (tiles_per_cu >= 16)
+    {
+        if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED>(t); }
+        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED>(t); }
+    }
+    else if (tiles_per_cu >= 2)
+    {
+        if (a.tokens <= 2) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 1, 8, SCALED>(t); }
+        else { launch_ksplit_tiled<WT, 4, 1, 8, SCALED>(t); }
+    }
+    else if (a.K > 8192)
+    {
+        if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
+        else { launch_ksplit_tiled<WT, 1, 2, 8, SCALED>(t); }
+    }
+    else
+    {
+        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
+        else { launch_ksplit_tiled<WT, 1, 2, 8, SCALED>(t); }
+    }
+    return true;
+}
+
 // ---- load-time repacked weights: caller's weight pointer -> tiled copy
 struct TiledWeight
 {
@@ -120,47 +163,6 @@ const uint8_t* find_tiled(const LinearArgs& a, int type)
     if (it == g_tiled.end()) { return nullptr; }
     const TiledWeight& t = it->second;
     return (t.type == type && t.n_out == a.n_out && t.K == a.K && t.ldw == a.ldw) ? t.tiled : nullptr;
-}
-
-// Matrix-core GEMV with the activations in LDS.  S (waves per row tile) is picked from how many tiles
-// a CU gets.  Returns false when the activations (tokens x K) do not fit 128 KiB of LDS: the caller
-// falls back.
-template <int WT, int TP, int S, bool SCALED, bool TILED>
-bool launch_gemv8_mfma_lds(const LinearArgs& a)
-{
-    auto kernel = gemv8_mfma_lds_kernel<WT, TP, S, 8, SCALED, TILED>;
-    const int per_block = 128 * TP;
-    const int max_blocks = (128 * 1024) / per_block;
-    const int k_blocks = (a.K + 63) / 64;
-    const int kc_blocks = k_blocks < max_blocks ? ((k_blocks + S - 1) / S) * S : (max_blocks / S) * S;
-    const size_t lds = (size_t)kc_blocks * per_block + 8192;
-    const int n_tiles = (a.n_out + 15) / 16;
-    const int groups = 8 / S;
-    const int want = (n_tiles + groups - 1) / groups;
-    const int cap = cu_count();
-    const int grid = want < cap ? want : cap;
-    if (kc_blocks < k_blocks) { return false; }    // K does not fit one LDS chunk: leave it to the row-major kernels
-    if (!allow_big_lds(kernel, lds)) { return false; }
-    kernel<<<grid, 512, lds, stream()>>>(a, kc_blocks * 64);
-    return true;
-}
-
-template <int WT, int TP, bool SCALED, bool TILED>
-bool pick_gemv8_mfma_lds(const LinearArgs& a)
-{
-    const int tiles_per_cu = ((a.n_out + 15) / 16) / cu_count();
-    if (tiles_per_cu >= 16) { return launch_gemv8_mfma_lds<WT, TP, 1, SCALED, TILED>(a); }
-    return launch_gemv8_mfma_lds<WT, TP, 8, SCALED, TILED>(a);
-}
-
-template <int WT, bool SCALED>
-bool gemv8_mfma_tiled(const LinearArgs& a, const uint8_t* tiled)
-{
-    LinearArgs t = a;
-    t.W = tiled;
-    if (a.tokens <= 4) { return pick_gemv8_mfma_lds<WT, 4, SCALED, true>(t); }
-    if (a.tokens <= 8) { return pick_gemv8_mfma_lds<WT, 8, SCALED, true>(t); }
-    return pick_gemv8_mfma_lds<WT, 16, SCALED, true>(t);
 }
 
 template <int MT, int R, int U, int WAVES, int OCC, int BLOCK>
@@ -326,15 +328,16 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         {
             const bool ok = x_ok && K % 16 == 0 && a.ldw % 16 == 0 && aligned16(a.W);
             const bool scaled = a.w_scale != 1.0f;
-            // Measured on MI355X: the tiled matrix-core kernel wins for 5..16 tokens on tall weights (lm_head: 5.0 TB/s
-            // against 3.6); up to 4 tokens the dot2 family is faster everywhere, and on weights with only a few row
-            // tiles per CU the 128 KiB activation staging per workgroup costs more than the contiguous loads gain.
-            if (ok && a.tokens >= 5 && a.tokens <= 16 && ((a.n_out + 15) / 16) / cu_count() >= 16)
+            // With a tiled copy registered for this weight the matrix-core kernel on that copy is the fastest
+            // choice for every token count up to 16 (3-17 % faster than the dot2 kernels at one and two tokens,
+            // more above), except one or two tokens on weights of a few MiB, where the software-pipelined dot2
+            // kernel starts sooner.
+            if (ok && a.tokens <= 16 && (a.tokens >= 3 || (long long)a.n_out * K >= (8LL << 20)))
             {
                 if (const uint8_t* tiled = find_tiled(a, g.w_type))
                 {
-                    if (g.w_type == DT_E5M2) { launched = scaled ? gemv8_mfma_tiled<DT_E5M2, true>(a, tiled) : gemv8_mfma_tiled<DT_E5M2, false>(a, tiled); }
-                    else { launched = scaled ? gemv8_mfma_tiled<DT_E4M3, true>(a, tiled) : gemv8_mfma_tiled<DT_E4M3, false>(a, tiled); }
+                    if (g.w_type == DT_E5M2) { launched = scaled ? gemv8_mfma_ksplit_tiled<DT_E5M2, true>(a, tiled) : gemv8_mfma_ksplit_tiled<DT_E5M2, false>(a, tiled); }
+                    else { launched = scaled ? gemv8_mfma_ksplit_tiled<DT_E4M3, true>(a, tiled) : gemv8_mfma_ksplit_tiled<DT_E4M3, false>(a, tiled); }
                     if (launched) { note_kernel("gemv_mfma_tiled"); }
                 }
             }

@@ -609,7 +609,9 @@ namespace ccq
 // Requires: K % 16 == 0, ldw % 16 == 0, W 16-byte aligned, ldx % 8 == 0, X 16-byte aligned.
 // Static LDS: WAVES * RT * 1 KiB.
 
-template <int WT, int RT, int U, int WAVES, bool SCALED>
+// TILED = true: a.W is the load-time repacked copy (repack_tiled_kernel), where the 16 rows x 64 codes
+// of one load instruction are one contiguous KiB and consecutive k blocks follow each other.
+template <int WT, int RT, int U, int WAVES, bool SCALED, bool TILED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs a)
 {
     __shared__ float partial[WAVES][RT][64][4];
@@ -622,11 +624,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs
     const int last_row = a.n_out - 1;
 
     const uint8_t* wrow[RT];
+    const int blocks_per_row = (a.K + 63) / 64;
+    const int n_tiles = (a.n_out + 15) / 16;
 #pragma unroll
     for (int rt = 0; rt < RT; rt++)
     {
         const int row = min(row_base + rt * 16 + i, last_row);
-        wrow[rt] = a.W + (long long)row * a.ldw + g * 16;
+        if (TILED) { wrow[rt] = a.W + (long long)min(blockIdx.x * RT + rt, n_tiles - 1) * blocks_per_row * 1024 + lane * 16; }
+        else { wrow[rt] = a.W + (long long)row * a.ldw + g * 16; }
     }
     const bool has_token = i < a.tokens;
     const uint16_t* xrow = a.X + (long long)(has_token ? i : 0) * a.ldx + g * 16;
@@ -649,7 +654,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs
             for (int rt = 0; rt < RT; rt++)
             {
                 w[u][rt] = u32x4{ 0u, 0u, 0u, 0u };
-                if (in_k) { w[u][rt] = __builtin_nontemporal_load((const u32x4*)(wrow[rt] + kb + u * 64)); }
+                if (in_k) { w[u][rt] = __builtin_nontemporal_load((const u32x4*)(wrow[rt] + (TILED ? (long long)(kb + u * 64) * 16 : (long long)(kb + u * 64)))); }
             }
             x[u][0] = x[u][1] = u32x4{ 0u, 0u, 0u, 0u };
             if (in_k && has_token)
@@ -698,158 +703,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs
         {
             uint16_t* y = a.Y + (long long)token * a.y_stride_tok + (long long)row * a.y_stride_out;
             *y = finish_output(total, a.alpha, a.beta, y);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// FP8 GEMV on the matrix cores with the activations resident in LDS (tokens 3..16, large n_out).
-//
-// A 512-thread workgroup (8 waves) stages a K chunk of the activations -- up to 128 KiB -- into LDS
-// once and then walks 16-row weight tiles with a grid stride.  A tile is shared by S waves (S = 1, 2,
-// 4 or 8 parts of the chunk's K range), so 8 / S tiles are in flight per workgroup; with S > 1 the
-// partial 16 x 16 tiles meet in LDS.  Per 64-element block a lane (i = lane % 16, g = lane / 16)
-// loads the 16 codes W[row i][block + 16 g ..] (one 128-bit load) and feeds two MFMAs, exactly as
-// gemv8_mfma_kernel does; the matching activation fragments are two conflict-free ds_read_b128.
-// LDS layout of the chunk: entry (block b, half, g, token j) at ((b * 2 + half) * 4 + g) * TP + j,
-// 16 bytes each, TP = tokens padded to 4 / 8 / 16.
-// K longer than one chunk: the chunks are staged one after another and the accumulators stay in
-// registers, which requires that every wave owns at most one tile (the launcher checks).
-// TILED = true reads the weight from the load-time repacked copy (repack_tiled_kernel): the 16 rows x
-// 64 codes a wave consumes per load instruction are then one contiguous KiB instead of sixteen
-// 64-byte row segments, which is what lets this kernel stream at the speed of the dot2 family.
-// Requires: K % 16 == 0, ldw % 16 == 0, W 16-byte aligned, ldx % 8 == 0, X 16-byte aligned,
-// chunk length a multiple of 64 * S.  Dynamic LDS: (kc / 64) * 8 * TP * 16 + 8 KiB bytes.
-
-template <int WT, int TP, int S, int U, bool SCALED, bool TILED>
-__global__ __launch_bounds__(512) void gemv8_mfma_lds_kernel(const LinearArgs a, const int kc)
-{
-    extern __shared__ u32x4 smem[];
-    constexpr int GROUPS = 8 / S;
-    const int x_entries = (kc / 64) * 8 * TP;
-    u32x4* xs = smem;
-    f32x4* partial = (f32x4*)(smem + x_entries);    // [8 waves][64 lanes]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int i = lane & 15;
-    const int g = lane >> 4;
-    const int group = wave / S;
-    const int part = wave % S;
-    const int n_tiles = (a.n_out + 15) / 16;
-    const int blocks_per_part = (kc / 64) / S;
-    const bool has_token = i < a.tokens;
-    const int blocks_per_row = (a.K + 63) / 64;
-    const int batches = (blocks_per_part + U - 1) / U;
-    const int t_first = blockIdx.x * GROUPS;
-    const int t_stride = gridDim.x * GROUPS;
-    const int n_iters = t_first < n_tiles ? (n_tiles - t_first + t_stride - 1) / t_stride : 0;    // same for all waves
-    const int total = n_iters * batches;
-    const int b_lo = part * blocks_per_part, b_hi = b_lo + blocks_per_part;
-
-    f32x4 acc = { 0.0f, 0.0f, 0.0f, 0.0f };
-    for (int k0 = 0; k0 < a.K; k0 += kc)
-    {
-        if (k0) { __syncthreads(); }    // every wave is done with the previous chunk
-        const int chunks16 = kc / 8;    // 16-byte pieces per token
-        for (int id = tid; id < a.tokens * chunks16; id += 512)
-        {
-            const int token = id / chunks16;
-            const int c = id - token * chunks16;
-            u32x4 v = { 0u, 0u, 0u, 0u };
-            if (k0 + c * 8 < a.K) { v = *(const u32x4*)(a.X + (long long)token * a.ldx + k0 + c * 8); }
-            const int b = c >> 3, q = c & 7;
-            xs[((b * 2 + (q & 1)) * 4 + (q >> 1)) * TP + token] = v;
-        }
-
-        // The (tile, block batch) pairs of this wave form one sequence; the loads of the next pair are
-        // issued before the current one is multiplied, so 2 * U KiB per wave are always in flight.
-        auto issue = [&](int q, u32x4 (&w)[U]) {
-            const int it = q / batches;
-            const int b0 = b_lo + (q - it * batches) * U;
-            const int tile = t_first + it * t_stride + group;
-            const int row = min(tile * 16 + i, a.n_out - 1);
-            // TILED: a.W is the repacked copy, KiB (tile, b) at (tile * blocks_per_row + b) * 1024, lane l's 16
-            // codes at l * 16 inside it; otherwise the row-major weight
-            const uint8_t* wrow = TILED ? a.W + ((long long)min(tile, n_tiles - 1) * blocks_per_row + k0 / 64) * 1024 + lane * 16
-                                        : a.W + (long long)row * a.ldw + k0 + g * 16;
-#pragma unroll
-            for (int u = 0; u < U; u++)
-            {
-                w[u] = u32x4{ 0u, 0u, 0u, 0u };
-                const int b = b0 + u;
-                if (b < b_hi && k0 + b * 64 + g * 16 < a.K) { w[u] = __builtin_nontemporal_load((const u32x4*)(wrow + b * (TILED ? 1024 : 64))); }
-            }
-        };
-        auto compute = [&](int q, const u32x4 (&w)[U]) {
-            const int it = q / batches;
-            const int bb = q - it * batches;
-            const int b0 = b_lo + bb * U;
-            const int tile = t_first + it * t_stride + group;
-            if (bb == 0 && k0 == 0) { acc = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
-#pragma unroll
-            for (int u = 0; u < U; u++)
-            {
-                const int b = b0 + u;
-                if (b < b_hi)
-                {
-#pragma unroll
-                    for (int h = 0; h < 2; h++)
-                    {
-                        u32x4 xv = { 0u, 0u, 0u, 0u };
-                        if (has_token) { xv = xs[((b * 2 + h) * 4 + g) * TP + i]; }
-                        bf16x2 p0, p1, p2, p3;
-                        fp8x4_to_bf16<WT, SCALED>(w[u][2 * h], a.w_scale, p0, p1);
-                        fp8x4_to_bf16<WT, SCALED>(w[u][2 * h + 1], a.w_scale, p2, p3);
-                        const bf16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, __builtin_bit_cast(bf16x8, xv), acc, 0, 0, 0);
-                    }
-                }
-            }
-            if (bb == batches - 1 && k0 + kc >= a.K)
-            {
-                f32x4 total_acc = acc;
-                if (S > 1)
-                {
-                    partial[wave * 64 + lane] = acc;
-                    __syncthreads();
-                    if (part == 0)
-                    {
-#pragma unroll
-                        for (int p = 1; p < S; p++)
-                        {
-                            const f32x4 other = partial[(wave + p) * 64 + lane];
-                            total_acc[0] += other[0]; total_acc[1] += other[1]; total_acc[2] += other[2]; total_acc[3] += other[3];
-                        }
-                    }
-                    __syncthreads();
-                }
-                if (part == 0 && has_token && tile < n_tiles)
-                {
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                    {
-                        const int out = tile * 16 + 4 * g + c;
-                        if (out < a.n_out)
-                        {
-                            uint16_t* y = a.Y + (long long)i * a.y_stride_tok + (long long)out * a.y_stride_out;
-                            *y = finish_output(total_acc[c], a.alpha, a.beta, y);
-                        }
-                    }
-                }
-            }
-        };
-
-        u32x4 wa[U], wb[U];
-        if (total > 0) { issue(0, wa); }
-        __syncthreads();    // the chunk is staged
-        for (int q = 0; q < total; q += 2)
-        {
-            if (q + 1 < total) { issue(q + 1, wb); }
-            compute(q, wa);
-            if (q + 2 < total) { issue(q + 2, wa); }
-            if (q + 1 < total) { compute(q + 1, wb); }
         }
     }
 }

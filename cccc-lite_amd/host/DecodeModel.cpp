@@ -106,7 +106,7 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     if (Rocblas::isQuantized(dt))
     {
         if ((int64_t)bytes != m->getDataSize()) { return -1; }
-        m->setAllowRepack(false);    // one token per step: the tiled copy (5..16 tokens) would never be read
+        m->setAllowRepack(false);    // the fused decode kernels read the row-major bytes: a tiled copy would never be read
         m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
         return 0;
     }

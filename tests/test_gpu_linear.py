@@ -260,7 +260,8 @@ def test_rejected_argument_combinations(gpu, oracle):
     BF, E5 = oracle.BF16, oracle.E5M2
     assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, E5, 16, 1.0, 0.0, p, BF, 16) == -1       # both quantized (W8A8 route)
     assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, BF, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == -1       # nothing quantized
-    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, oracle.HALF, 16, 1.0, 0.0, p, oracle.HALF, 16) == -1
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, oracle.HALF, 16, 1.0, 0.0, p, BF, 16) == -1       # mixed 16-bit types
+    assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, oracle.FP4, 16, 1.0, p, oracle.HALF, 16, 1.0, 0.0, p, oracle.HALF, 16) == -1   # FP4 has no HALF route
     assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, oracle.FLOAT, 16) == -1
     assert lib.quant_gemm(2, 0, 16, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == -1
     assert lib.quant_gemm(1, 0, 0, 1, 16, 1.0, p, E5, 16, 1.0, p, BF, 16, 1.0, 0.0, p, BF, 16) == 0         # empty output
@@ -347,9 +348,11 @@ def test_weight_prepare_builds_the_tiled_layout(gpu, pkg, oracle, n_out, K):
     assert lib.weight_prepare(None, oracle.E5M2, n_out, K, K, td.data_ptr()) == -1
 
 
-@pytest.mark.parametrize("tokens", [5, 8, 9, 16])
-@pytest.mark.parametrize("n_out,K", [(65536, 512), (65530, 272), (70000, 16), (151936, 1024)])
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4, 5, 9, 16])
+@pytest.mark.parametrize("n_out,K", [(300, 528), (4096, 2048), (12288, 1024), (1024, 12288), (65530, 272), (70000, 16), (151936, 1024)])
 def test_prepared_weights_give_the_same_gemv(gpu, pkg, oracle, tokens, n_out, K):
+    """Every launch configuration of the matrix-core kernel on the tiled copy (few / several / many row
+    tiles per CU, short and long rows, ragged row counts and row lengths) against the exact contraction."""
     torch, dev, lib = gpu
     seed = pkg.synth.seed_for(2, 200 + n_out % 91 + tokens)
     W = pkg.synth.weights_e5m2(seed, n_out, K)
@@ -358,18 +361,16 @@ def test_prepared_weights_give_the_same_gemv(gpu, pkg, oracle, tokens, n_out, K)
     y0 = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
     assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y0.data_ptr(), n_out, tokens, K) == 0
     plain_kernel = lib.last_kernel()
+    assert plain_kernel != "gemv_mfma_tiled"
     td = torch.zeros(lib.tiled_size(oracle.E5M2, n_out, K), dtype=torch.uint8, device=dev)
     assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, K, K, td.data_ptr()) == 0
+    uses_tiled = tokens >= 3 or n_out * K >= (8 << 20)          # one or two tokens on a small weight stay on the dot2 kernels
     try:
         y1 = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
         assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y1.data_ptr(), n_out, tokens, K) == 0
-        assert lib.last_kernel() == "gemv_mfma_tiled" and plain_kernel != "gemv_mfma_tiled"
-        # a scaled call and one token (dot2 family) on the same registered weight
+        assert lib.last_kernel() == ("gemv_mfma_tiled" if uses_tiled else plain_kernel)
         y2 = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
         assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y2.data_ptr(), n_out, tokens, K, inv_scale=0.37) == 0
-        y3 = torch.zeros(4 * n_out, dtype=torch.int16, device=dev)
-        assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y3.data_ptr(), n_out, 4, K) == 0
-        assert lib.last_kernel() == "gemv_dot2"
     finally:
         assert lib.weight_release(wd.data_ptr()) == 0
     out = from_dev(y1, np.uint16)
