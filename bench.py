@@ -302,8 +302,76 @@ def shape_sweep(ws, by_shape, token_counts, use_graph):
             us = ms * 1000.0 / (3 * len(ops))
             gbs = gemv_bytes(K, N, M) / us * 1e-3
             assert ws.lib.linear(weights[0].data_ptr, E5M2, X.data_ptr, Y.data_ptr, N, M, K) == 0
-            out.append({"K": K, "N": N, "M": M, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
-                        "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(K * N * len(weights) / 2 ** 20)})
+            row = {"K": K, "N": N, "M": M, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                   "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(K * N * len(weights) / 2 ** 20)}
+            if M == 1:
+                row.update(same_gpu_comparators(ws, weights, K, N, M))
+            out.append(row)
+    return out
+
+
+def same_gpu_comparators(ws, weights, K, N, M, max_ops=24):
+    """The same linear on the same GPU the way the reference's unified GEMM does it (cccc/cublas_real.h:943-964
+    expressed with HIP calls): dequantise the whole weight to a BF16 workspace, then a BF16 GEMM with FP32
+    accumulation (rocBLAS / hipBLASLt through torch), with the device synchronisation the reference's kernel
+    wrappers make after each step -- and the plain BF16 GEMM alone, which is what the reference's HIP build
+    (no FP8 support) would run on BF16 weights.  Microseconds per linear over rotating weights."""
+    t = ws.torch
+    wsb = t.empty(N, K, dtype=t.bfloat16, device=ws.dev)
+    x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
+    ops = weights[:max_ops]
+    out = {}
+    for name, sync in (("ref_style_us", True), ("ref_style_nosync_us", False)):
+        for rep in range(2):                                   # first pass warms up
+            t.cuda.synchronize()
+            t0 = time.perf_counter()
+            for W in ops:
+                assert ws.lib.convert(W.data_ptr, E5M2, wsb.data_ptr(), BF16, N * K, 1.0) == 0
+                if sync:
+                    t.cuda.synchronize()
+                y = x @ wsb.T
+                if sync:
+                    t.cuda.synchronize()
+            t.cuda.synchronize()
+            out[name] = round((time.perf_counter() - t0) * 1e6 / len(ops), 2)
+    n_bf = max(2, min(8, (1 << 30) // (2 * K * N)))
+    bf = [t.randn(N, K, device=ws.dev, generator=ws.gen).to(t.bfloat16) for _ in range(n_bf)]
+    for rep in range(2):
+        t.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(4 * n_bf):
+            y = x @ bf[i % n_bf].T
+        t.cuda.synchronize()
+        out["bf16_gemm_us"] = round((time.perf_counter() - t0) * 1e6 / (4 * n_bf), 2)
+    return out
+
+
+def prefill_cases(ws, by_shape):
+    """BASELINE config 4: W8A16 prefill GEMM, M in {512, 2048} x the two MLP shapes, with the plain BF16 GEMM
+    of the vendor library (torch.matmul) on the same shape beside it."""
+    t = ws.torch
+    out = []
+    for (K, N) in ((4096, 12288), (12288, 4096)):
+        weights = by_shape[(K, N)][:16]
+        bf = [t.randn(N, K, device=ws.dev, generator=ws.gen).to(t.bfloat16) for _ in range(4)]
+        for M in (512, 2048):
+            X, Y = ws.activation(M, K), ws.output(M, N)
+            ops = [(W, X, Y, K, N) for W in weights]
+            ms = time_chain(ws, ops, 3, 1, False)
+            us = ms * 1000.0 / (3 * len(ops))
+            tf = 2.0 * M * K * N / us * 1e-6
+            x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
+            for rep in range(2):
+                t.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(16):
+                    y = x @ bf[i % 4].T
+                t.cuda.synchronize()
+                lib_us = (time.perf_counter() - t0) * 1e6 / 16
+            out.append({"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "kernel": ws.lib.last_kernel(), "vendor_bf16_gemm_us": round(lib_us, 2),
+                        "vendor_bf16_gemm_TFLOPs": round(2.0 * M * K * N / lib_us * 1e-6, 1)})
+        del bf
     return out
 
 
@@ -459,6 +527,7 @@ def main():
             extra["quant_gemv"] = {"workload": "the 253 FP8_E5M2 linears of one decode token through Matrix::mulBatched", "ms_per_step": round(lin_ms, 4),
                                    "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
             extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
+            extra["prefill"] = prefill_cases(ws, by_shape)
             extra["fp4_sweep"] = fp4_sweep(ws)
     elif args.workload == "decode_linears":
         ops, by_shape = build_decode_model(ws, 1)
