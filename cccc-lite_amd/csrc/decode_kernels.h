@@ -399,8 +399,9 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_kernel(const uint16
 // GQA decode attention, head_dim 128, group of G = n_q / n_kv query heads per KV head, two launches
 // over blocks of ATT_KEYS cache positions (grid = (blocks, kv heads); blocks past *d_pos exit at once).
 // 16 lanes share a cache row (8 dims each), a wave covers 4 rows per 1 KiB load, a workgroup 16, and
-// every thread issues its 8 row loads before the first use.
-constexpr int ATT_KEYS = 128;
+// every thread issues its ATT_ITS row loads before the first use.
+constexpr int ATT_KEYS = 64;
+constexpr int ATT_ITS = ATT_KEYS / 16;     // cache rows per thread
 
 __device__ __forceinline__ float wave_max(float v)
 {
@@ -433,9 +434,9 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __rest
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15;              // which 8 dims
     const int key_in_wave = lane >> 4;
-    u32x4 raw[8];
+    u32x4 raw[ATT_ITS];
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end repeat the last one and are discarded below
         raw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
@@ -444,7 +445,7 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __rest
 #pragma unroll
     for (int gq = 0; gq < G; gq++) { unpack8_bf16(*(const u32x4*)(q + (size_t)(kvh * G + gq) * 128 + sub * 8), qv[gq]); }
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int kl = it * 16 + wave * 4 + key_in_wave;
         const int t = t0 + kl;
@@ -471,9 +472,14 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __rest
     __syncthreads();
     if (wave < G)
     {
-        const float v0 = s_lds[wave][lane], v1 = s_lds[wave][lane + 64];
-        const float m = wave_max(fmaxf(v0, v1));            // finite: the block holds at least one valid key
-        const float l = wave_sum(expf(v0 - m) + expf(v1 - m));
+        constexpr int PER_LANE = (ATT_KEYS + 63) / 64;
+        float v[PER_LANE], m = -INFINITY, l = 0.0f;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; j++) { m = fmaxf(m, v[j] = (lane + 64 * j < ATT_KEYS) ? s_lds[wave][lane + 64 * j] : -INFINITY); }
+        m = wave_max(m);                                    // finite: the block holds at least one valid key
+#pragma unroll
+        for (int j = 0; j < PER_LANE; j++) { l += expf(v[j] - m); }
+        l = wave_sum(l);
         if (lane == 0) { stats[(size_t)(kvh * G + wave) * n_blocks + blk] = make_float2(m, l); }
     }
 }
@@ -496,9 +502,9 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict
     const int n_active = (n_keys + ATT_KEYS - 1) / ATT_KEYS;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15, key_in_wave = lane >> 4;
-    u32x4 raw[8];
+    u32x4 raw[ATT_ITS];
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end get probability 0 below
         raw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
@@ -534,7 +540,7 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict
 #pragma unroll
         for (int d = 0; d < 8; d++) { acc[gq][d] = 0.0f; }
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int kl = it * 16 + wave * 4 + key_in_wave;
         float vf[8];
@@ -634,9 +640,9 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     const bool has_new = pos < t0 + ATT_KEYS;       // this block holds the row being appended
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15, key_in_wave = lane >> 4;
-    u32x4 kraw[8], vraw[8];
+    u32x4 kraw[ATT_ITS], vraw[ATT_ITS];
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end, and row pos itself, are replaced or discarded below
         kraw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
@@ -677,7 +683,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 #pragma unroll
         for (int d = 0; d < 8; d++) { qv[gq][d] = q_lds[gq][sub * 8 + d]; }
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int kl = it * 16 + wave * 4 + key_in_wave;
         const int t = t0 + kl;
@@ -704,12 +710,19 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     __syncthreads();
     if (wave < G)
     {
-        const float v0 = s_lds[wave][lane], v1 = s_lds[wave][lane + 64];
-        const float m = wave_max(fmaxf(v0, v1));            // finite: the block holds at least one valid key
-        const float e0 = expf(v0 - m), e1 = expf(v1 - m);
-        const float l = wave_sum(e0 + e1);
-        s_lds[wave][lane] = e0;
-        s_lds[wave][lane + 64] = e1;
+        constexpr int PER_LANE = (ATT_KEYS + 63) / 64;
+        float v[PER_LANE], m = -INFINITY, l = 0.0f;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; j++) { m = fmaxf(m, v[j] = (lane + 64 * j < ATT_KEYS) ? s_lds[wave][lane + 64 * j] : -INFINITY); }
+        m = wave_max(m);                                    // finite: the block holds at least one valid key
+#pragma unroll
+        for (int j = 0; j < PER_LANE; j++)
+        {
+            const float e = expf(v[j] - m);
+            if (lane + 64 * j < ATT_KEYS) { s_lds[wave][lane + 64 * j] = e; }
+            l += e;
+        }
+        l = wave_sum(l);
         if (lane == 0) { stats[(size_t)(kvh * G + wave) * n_blocks + blk] = make_float2(m, l); }
     }
     __syncthreads();
@@ -719,7 +732,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 #pragma unroll
         for (int d = 0; d < 8; d++) { acc[gq][d] = 0.0f; }
 #pragma unroll
-    for (int it = 0; it < 8; it++)
+    for (int it = 0; it < ATT_ITS; it++)
     {
         const int kl = it * 16 + wave * 4 + key_in_wave;
         float vf[8];

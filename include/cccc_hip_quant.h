@@ -161,7 +161,7 @@ C_EXPORT int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* 
                                       const void* d_pos, float epsilon);
 
 /* GQA attention of one query token over cache rows 0..*d_pos: scores rounded to BF16, FP32 softmax,
- * BF16 probabilities, y = bf16(V p).  Three launches over blocks of 128 cache rows; the caller owns the
+ * BF16 probabilities, y = bf16(V p).  Three launches over blocks of 64 cache rows; the caller owns the
  * workspace (16-byte aligned, hip_attention_decode_workspace_bytes(...) bytes; its content between
  * calls does not matter).  n_q_heads / n_kv_heads must be 1, 2 or 4; calls sharing one workspace
  * must be ordered on the stream. */
@@ -175,7 +175,7 @@ C_EXPORT int hip_attention_decode_bf16(const void* q, const void* k_cache, const
  * raw projections ([n_q_heads][128], [n_kv_heads][128]); row *d_pos of both caches is written.  Same
  * workspace as above.  Scores are rounded to BF16 as in the reference; the softmax probabilities stay
  * FP32 (the reference rounds them to BF16 before the product with V), so outputs can differ from
- * hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 by about one BF16 ulp.  t_kv <= 131072. */
+ * hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 by about one BF16 ulp.  t_kv <= 65536. */
 C_EXPORT int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
                                              const void* q_norm_w, const void* k_norm_w,
                                              const void* cos_tab, const void* sin_tab,
