@@ -33,10 +33,10 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM bytes per launch of the gate/up-shaped GEMV (K=4096, N=12288, M=1) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99983 and 1.0)
-GEMV_GATE_UP_TRAFFIC_BYTES = 50503552
+# WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99979 and 1.0)
+GEMV_GATE_UP_TRAFFIC_BYTES = 50451344
 # the same two counters for one launch of the fused RMSNorm + gate/up SwiGLU GEMV (two 4096 x 12288 weights)
-GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = 101031904
+GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = 101012454
 
 FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
 
