@@ -149,6 +149,7 @@ def build_decode_step(ws: Workspace, ctx: int):
         for is_v in (False, True):
             fill_bf16(model.kv_ptr(li, is_v), 8 * ctx * 128, 0.0, 1.0)
     fill_fp8(model.tensor_ptr(0, "lm_head"), c["vocab"], c["hidden"])
+    model.prepare_tiled(0, "lm_head")                  # what loading through set_tensor / load_named does
     fill_bf16(model.tensor_ptr(0, "rms_final"), c["hidden"], 1.0, 0.1)
     fill_bf16(model.tensor_ptr(0, "emb"), c["vocab"] * c["hidden"], 0.0, 1.0)
     return model

@@ -37,6 +37,27 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     return finish("quant_linear_fused");
 }
 
+// Matrix-core variant on the tiled copies.  Configurations from the tuning of gemv8_mfma_kernel at one token.
+template <int WT, int RT, int U, int WAVES, bool SCALED>
+void launch_fused_mfma_cfg(const FusedLinearArgs& a, int n_tiles, size_t lds)
+{
+    if (a.norm_w) { gemv8_fused_mfma_kernel<WT, RT, U, WAVES, SCALED, true><<<(n_tiles + RT - 1) / RT, WAVES * 64, lds, stream()>>>(a); }
+    else { gemv8_fused_mfma_kernel<WT, RT, U, WAVES, SCALED, false><<<(n_tiles + RT - 1) / RT, WAVES * 64, 0, stream()>>>(a); }
+}
+
+template <int WT, bool SCALED>
+int launch_fused_mfma(const FusedLinearArgs& a, int n_tiles)
+{
+    const size_t lds = (size_t)((a.K + 1023) / 1024) * 2048;
+    if (lds > 48 * 1024) { return -1; }
+    const int tiles_per_cu = n_tiles / cu_count();
+    if (tiles_per_cu >= 16) { launch_fused_mfma_cfg<WT, 2, 2, 8, SCALED>(a, n_tiles, lds); }
+    else if (tiles_per_cu >= 2) { launch_fused_mfma_cfg<WT, 1, 1, 8, SCALED>(a, n_tiles, lds); }
+    else if (a.K > 8192) { launch_fused_mfma_cfg<WT, 1, 4, 8, SCALED>(a, n_tiles, lds); }
+    else { launch_fused_mfma_cfg<WT, 1, 2, 16, SCALED>(a, n_tiles, lds); }
+    return finish("quant_linear_fused");
+}
+
 }    // namespace
 
 int hip_quant_linear_fused(const hip_fused_linear* d)
@@ -72,6 +93,30 @@ int hip_quant_linear_fused(const hip_fused_linear* d)
     a.norm_w = (const uint16_t*)d->norm_weight;
     a.norm_eps = d->norm_eps;
     a.residual = (const uint16_t*)d->residual;
+    // every segment has a registered tiled copy (and this is not the SwiGLU pair): matrix-core variant
+    if (!d->pair)
+    {
+        int n_tiles = 0;
+        bool all = true;
+        for (int s = 0; s < d->n_segments && all; s++)
+        {
+            a.T[s] = lookup_tiled(d->W[s], d->w_type, d->n_out[s], d->K, d->K);
+            all = a.T[s] != nullptr;
+            n_tiles += (d->n_out[s] + 15) / 16;
+        }
+        // measured inside the decode step: on tall weights the matrix-core variant wins (lm_head 91 us against 97);
+        // on the per-layer weights it is level with the dot2 kernel without a norm in front (o 5.6 against 5.9 us,
+        // down 11.4 against 11.45) and slower with one (q,k,v 10.5 against 7.3), so those stay on the row-major bytes
+        if (all && n_tiles / cu_count() < 16) { all = false; }
+        if (all)
+        {
+            note_kernel("gemv_fused_mfma");
+            int rc;
+            if (d->w_type == DT_E5M2) { rc = scaled ? launch_fused_mfma<DT_E5M2, true>(a, n_tiles) : launch_fused_mfma<DT_E5M2, false>(a, n_tiles); }
+            else { rc = scaled ? launch_fused_mfma<DT_E4M3, true>(a, n_tiles) : launch_fused_mfma<DT_E4M3, false>(a, n_tiles); }
+            if (rc >= 0) { return rc; }
+        }
+    }
     note_kernel("gemv_fused");
     if (d->w_type == DT_E5M2) { return scaled ? launch_fused<DT_E5M2, true>(a, n_groups) : launch_fused<DT_E5M2, false>(a, n_groups); }
     return scaled ? launch_fused<DT_E4M3, true>(a, n_groups) : launch_fused<DT_E4M3, false>(a, n_groups);

@@ -50,6 +50,7 @@ struct FusedLinearArgs
     const uint16_t* norm_w;    // bf16 [K] or nullptr
     float norm_eps;
     const uint16_t* residual;  // bf16 [n_out[0]] or nullptr (single segment / pair only)
+    const uint8_t* T[3];       // load-time tiled copies of W[s] (matrix-core variant only)
 };
 
 // Staging of the activation vector into LDS in the [step][half][lane] layout of the dot2 kernels,
@@ -300,6 +301,161 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
             wa[u] = na[u];
             wb[u] = nb[u];
         }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// The same fused one-token linear on the matrix cores, reading the load-time tiled copies (T[s]):
+// structure of gemv8_mfma_kernel -- a workgroup owns RT tiles of 16 rows, its waves split K in
+// interleaved spans of 64 * U codes, every load instruction covers one contiguous KiB -- with the
+// activation (normalised on the way when asked) staged once per workgroup in LDS and used as the
+// single live column of the 16-column operand.  Up to three segments; a tile never straddles two
+// segments (every segment's tiled copy is padded to whole tiles).  No SwiGLU pair mode.
+// NORM = false: no RMSNorm in front, and then no staging either -- the lanes of the live column take
+// their activation chunks straight from global memory and the kernel has no prologue at all.
+// Dynamic LDS (NORM only): ceil(K / 1024) * 2048 bytes.
+template <int WT, int RT, int U, int WAVES, bool SCALED, bool NORM>
+__global__ __launch_bounds__(WAVES * 64) void gemv8_fused_mfma_kernel(const FusedLinearArgs a)
+{
+    extern __shared__ u32x4 xs[];
+    __shared__ float red[WAVES];
+    __shared__ float partial[WAVES][RT][16];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15;
+    const int g = lane >> 4;
+    const int blocks_per_row = (a.K + 63) / 64;
+    const int t0 = (a.n_out[0] + 15) / 16;
+    const int t1 = a.n_segments < 2 ? t0 : t0 + (a.n_out[1] + 15) / 16;
+    const int n_tiles = a.n_segments < 3 ? t1 : t1 + (a.n_out[2] + 15) / 16;
+
+    const uint8_t* wtile[RT];
+    float scale[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+    {
+        const int tile = min((int)blockIdx.x * RT + rt, n_tiles - 1);      // a clamped tile is computed and dropped
+        const int seg = tile >= t1 ? 2 : (tile >= t0 ? 1 : 0);
+        const int local = tile - (seg == 2 ? t1 : (seg == 1 ? t0 : 0));
+        wtile[rt] = a.T[seg] + (long long)local * blocks_per_row * 1024 + lane * 16;
+        scale[rt] = a.w_scale[seg];
+    }
+    const int span = 64 * U;
+    // requests the weights of the span at kb and, without a norm, the matching activation chunks of the live column
+    auto request = [&](int kb, u32x4 (*w)[RT], u32x4 (*x)[2]) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const bool in_k = kb + u * 64 + g * 16 < a.K;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+            {
+                w[u][rt] = u32x4{ 0u, 0u, 0u, 0u };
+                if (in_k) { w[u][rt] = __builtin_nontemporal_load((const u32x4*)(wtile[rt] + (long long)(kb + u * 64) * 16)); }
+            }
+            if constexpr (!NORM)
+            {
+                x[u][0] = x[u][1] = u32x4{ 0u, 0u, 0u, 0u };
+                if (in_k && i == 0)
+                {
+                    x[u][0] = *(const u32x4*)(a.X + kb + u * 64 + g * 16);
+                    x[u][1] = *(const u32x4*)(a.X + kb + u * 64 + g * 16 + 8);
+                }
+            }
+        }
+    };
+
+    u32x4 w[U][RT], wn[U][RT], xr[U][2], xn[U][2];
+    int kb = wave * span;
+    if constexpr (NORM)
+    {
+        StagedActivation staged;
+        stage_issue<WAVES * 64>(a, staged);
+        if (kb < a.K) { request(kb, w, xr); }
+        stage_finish<WAVES * 64>(a, staged, xs, red);
+    }
+    else if (kb < a.K) { request(kb, w, xr); }
+
+    f32x4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) { acc[rt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+    while (kb < a.K)
+    {
+        const int nk = kb + WAVES * span;
+        if (nk < a.K) { request(nk, wn, xn); }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            // the activation of block b: codes 64 b + 16 g .. + 16 of lane group g are the 16-byte chunks 8 b + 2 g and + 1
+            const int c = ((kb + u * 64) >> 3) + 2 * g;
+            u32x4 x[2] = { u32x4{ 0u, 0u, 0u, 0u }, u32x4{ 0u, 0u, 0u, 0u } };
+            if constexpr (NORM)
+            {
+                if (i == 0 && kb + u * 64 + g * 16 < a.K)
+                {
+                    x[0] = xs[stage_slot(c)];
+                    x[1] = xs[stage_slot(c + 1)];
+                }
+            }
+            else
+            {
+                x[0] = xr[u][0];
+                x[1] = xr[u][1];
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+            {
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                {
+                    bf16x2 p0, p1, p2, p3;
+                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h], scale[rt], p0, p1);
+                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h + 1], scale[rt], p2, p3);
+                    const bf16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, __builtin_bit_cast(bf16x8, x[h]), acc[rt], 0, 0, 0);
+                }
+            }
+        }
+        kb = nk;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) { w[u][rt] = wn[u][rt]; }
+        if constexpr (!NORM)
+        {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+            {
+                xr[u][0] = xn[u][0];
+                xr[u][1] = xn[u][1];
+            }
+        }
+    }
+
+    // D: lane (i, g) holds token column i, rows 4 g .. 4 g + 3; only column 0 is live
+    if (i == 0)
+    {
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) { partial[wave][rt][4 * g + c] = acc[rt][c]; }
+    }
+    __syncthreads();
+    for (int v = threadIdx.x; v < RT * 16; v += WAVES * 64)
+    {
+        const int rt = v >> 4, r = v & 15;
+        const int tile = (int)blockIdx.x * RT + rt;
+        if (tile >= n_tiles) { continue; }
+        const int seg = tile >= t1 ? 2 : (tile >= t0 ? 1 : 0);
+        const int row = (tile - (seg == 2 ? t1 : (seg == 1 ? t0 : 0))) * 16 + r;
+        if (row >= a.n_out[seg]) { continue; }
+        float total = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; wv++) { total += partial[wv][rt][r]; }
+        float out = bf16_round(total);
+        if (a.residual && seg == 0) { out = bf16_round(out + bf16_bits_to_f32(a.residual[row])); }
+        a.Y[seg][row] = (uint16_t)f32_to_bf16_bits(out);
     }
 }
 

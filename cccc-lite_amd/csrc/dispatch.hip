@@ -155,15 +155,7 @@ struct TiledWeight
 std::shared_mutex g_tiled_mutex;
 std::unordered_map<const void*, TiledWeight> g_tiled;
 
-const uint8_t* find_tiled(const LinearArgs& a, int type)
-{
-    std::shared_lock<std::shared_mutex> lock(g_tiled_mutex);
-    if (g_tiled.empty()) { return nullptr; }
-    const auto it = g_tiled.find(a.W);
-    if (it == g_tiled.end()) { return nullptr; }
-    const TiledWeight& t = it->second;
-    return (t.type == type && t.n_out == a.n_out && t.K == a.K && t.ldw == a.ldw) ? t.tiled : nullptr;
-}
+const uint8_t* find_tiled(const LinearArgs& a, int type) { return ccq::lookup_tiled(a.W, type, a.n_out, a.K, a.ldw); }
 
 template <int MT, int R, int U, int WAVES, int OCC, int BLOCK>
 bool launch_gemv4_dot2(const LinearArgs& a)
@@ -212,6 +204,16 @@ void launch_generic(const GenericArgs& g)
 }
 
 }    // namespace
+
+const unsigned char* ccq::lookup_tiled(const void* W, int type, int n_out, int K, long long ldw)
+{
+    std::shared_lock<std::shared_mutex> lock(g_tiled_mutex);
+    if (g_tiled.empty()) { return nullptr; }
+    const auto it = g_tiled.find(W);
+    if (it == g_tiled.end()) { return nullptr; }
+    const TiledWeight& t = it->second;
+    return (t.type == type && t.n_out == n_out && t.K == K && t.ldw == ldw) ? t.tiled : nullptr;
+}
 
 int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                    const void* A, int typeA, int lda, float invScaleA,

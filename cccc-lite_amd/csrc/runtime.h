@@ -18,4 +18,8 @@ int finish(const char* what);
 // Number of compute units of the current device (cached per device).
 int cu_count();
 
+// The load-time tiled copy registered for the FP8 weight `W` by hip_quant_weight_prepare, or nullptr
+// when there is none or its type / shape / row stride differ (defined with the registry in dispatch.hip).
+const unsigned char* lookup_tiled(const void* W, int type, int n_out, int K, long long ldw);
+
 }    // namespace ccq

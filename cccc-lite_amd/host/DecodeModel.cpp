@@ -106,7 +106,8 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     if (Rocblas::isQuantized(dt))
     {
         if ((int64_t)bytes != m->getDataSize()) { return -1; }
-        m->setAllowRepack(false);    // the fused decode kernels read the row-major bytes: a tiled copy would never be read
+        // only a tall weight (lm_head) is read through its tiled copy by the fused decode kernels
+        m->setAllowRepack(which == LM_HEAD);
         m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
         return 0;
     }
@@ -139,22 +140,22 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         m = tmp;
         return 0;
     };
-    auto load_linear = [&](Matrix& m, const std::string& name) -> int {
+    auto load_linear = [&](Matrix& m, const std::string& name, bool tiled = false) -> int {
         const auto wk = file.resolve(name);
         if (!wk.valid()) { return fail(name, -1); }
         if (wk.is_quant)
         {
             if (wk.dt == FP4_E2M1) { return fail(name, -3); }
-            m.setAllowRepack(false);
+            m.setAllowRepack(tiled);
             return file.loadNamed(m, name) == 0 ? 0 : fail(name, -2);
         }
         Matrix tmp(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
-        tmp.setAllowRepack(false);
+        tmp.setAllowRepack(tiled);
         if (file.loadNamed(tmp, name) != 0) { return fail(name, -2); }
         if (tmp.getDataType() == FLOAT)
         {
             Matrix bf(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
-            bf.setAllowRepack(false);
+            bf.setAllowRepack(tiled);
             if (hip_convert(tmp.data(), (int)FLOAT, bf.data(), (int)BFLOAT16, (unsigned)tmp.getDataSize(), 1.0f) != 0) { return fail(name, -3); }
             (void)hipDeviceSynchronize();
             tmp = bf;
@@ -166,7 +167,7 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
     };
     int rc = load_plain(*emb_, "W_emb");
     if (rc == 0) { rc = load_plain(*rms_final_, "W_rms_final"); }
-    if (rc == 0) { rc = load_linear(*lm_head_, file.resolve("W_lm_head").valid() ? "W_lm_head" : "W_emb"); }
+    if (rc == 0) { rc = load_linear(*lm_head_, file.resolve("W_lm_head").valid() ? "W_lm_head" : "W_emb", true); }
     for (int i = 0; i < cfg_.layers && rc == 0; i++)
     {
         Layer& L = layers_[i];

@@ -24,7 +24,7 @@ struct MatrixData
     // with the kernel library under the key data_.  No counterpart in the reference.
     void* tiled_data_ = nullptr;
     static inline bool repack_weights = true;    // global switch
-    bool allow_repack_ = true;                    // per storage (a batch-1 decode model never needs the copy)
+    bool allow_repack_ = true;                    // per storage (e.g. off for weights only the row-major SwiGLU pair kernel reads)
 
     MatrixData() = default;
     ~MatrixData() { release(); }

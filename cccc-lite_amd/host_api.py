@@ -66,6 +66,7 @@ class HostLibrary:
         L.cccc_host_half_to_bf16.restype = ctypes.c_ushort; L.cccc_host_half_to_bf16.argtypes = [ctypes.c_ushort]
         L.cccc_decode_load_named.restype = i32; L.cccc_decode_load_named.argtypes = [vp, vp, i32, ctypes.c_char_p, i32]
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
+        L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         L.cccc_decode_bench_gate_up.restype = ctypes.c_double; L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
         self.c = L
@@ -236,6 +237,11 @@ class DecodeModel:
 
     def tensor_ptr(self, layer: int, name: str) -> int:
         return self.lib.c.cccc_decode_tensor_data(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name)))
+
+    def prepare_tiled(self, layer: int, name: str) -> bool:
+        """Builds the tiled copy of a linear whose bytes were written through tensor_ptr (set_tensor and
+        load_named do this themselves)."""
+        return self.lib.c.cccc_decode_tensor_prepare(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))) == 0
 
     def load(self, model: dict, fp8_dtype: int = 5) -> None:
         """model: the dict layout of oracle.decode_oracle.make_model (uint8 codes / uint16 bf16 bits)."""

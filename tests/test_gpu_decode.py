@@ -65,7 +65,25 @@ def fused_desc(pkg, **kw):
     return d
 
 
-def test_fused_linear_variants(gpu, pkg, oracle, dec):
+class TiledCopies:
+    """Registers load-time tiled copies for device weights (hip_quant_weight_prepare) and releases them."""
+
+    def __init__(self, torch, dev, lib, weights, w_type, K):
+        self.lib, self.keys, self.bufs = lib, [], []
+        for w in weights:
+            n_out = w.numel() // K
+            t = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
+            assert lib.weight_prepare(w.data_ptr(), w_type, n_out, K, K, t.data_ptr()) == 0
+            self.keys.append(w.data_ptr())
+            self.bufs.append(t)
+
+    def release(self):
+        for k in self.keys:
+            assert self.lib.weight_release(k) == 0
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+def test_fused_linear_variants(gpu, pkg, oracle, dec, tiled):
     torch, dev, lib = gpu
     rng = np.random.default_rng(1)
     K, n0, n1, n2 = 2048, 512, 128, 130
@@ -77,8 +95,13 @@ def test_fused_linear_variants(gpu, pkg, oracle, dec):
     wds = [to_dev(torch, dev, W) for W in Ws]
     xn = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6)
 
-    def run(desc, outs):
+    Wu = oracle.encode_e5m2_rne((rng.standard_normal((n0, K)) * 0.02).astype(np.float32))
+    wud = to_dev(torch, dev, Wu)
+    copies = TiledCopies(torch, dev, lib, wds + [wud], E5M2, K) if tiled else None
+
+    def run(desc, outs, pair=False):
         assert lib.quant_linear_fused(desc) == 0
+        # these weights are not tall: tiled copies or not, they stay on the row-major kernel
         assert lib.last_kernel() == "gemv_fused"
         return [from_dev(o_, np.uint16) for o_ in outs]
 
@@ -100,12 +123,10 @@ def test_fused_linear_variants(gpu, pkg, oracle, dec):
     lin = dec.linear(oracle.dequant_fp8_to_bf16(Ws[0], oracle.E5M2, 0.5).reshape(n0, K), dec.f(x))
     assert ulp_close(out, dec.r(lin + dec.f(res)), ulps=1.0, floor=2e-5).all()
     # (3) SwiGLU pair with norm: gate = W0, up = another n0-row weight
-    Wu = oracle.encode_e5m2_rne((rng.standard_normal((n0, K)) * 0.02).astype(np.float32))
-    wud = to_dev(torch, dev, Wu)
     y = torch.zeros(n0, dtype=torch.int16, device=dev)
     d = pkg.capi.make_fused_linear(E5M2, K, [wds[0].data_ptr(), wud.data_ptr()], [n0, n0], [y.data_ptr(), None], xd.data_ptr(),
                                    norm_weight=nwd.data_ptr(), norm_eps=1e-6, pair=True)
-    out, = run(d, [y])
+    out, = run(d, [y], pair=True)
     gate = dec.linear(Wd[0], xn)
     up = dec.linear(oracle.dequant_fp8_to_bf16(Wu, oracle.E5M2).reshape(n0, K), xn)
     want = dec.silu_mul(gate, up)
@@ -117,11 +138,14 @@ def test_fused_linear_variants(gpu, pkg, oracle, dec):
     assert lib.quant_linear_fused(bad) == -1
     bad = pkg.capi.make_fused_linear(6, K, [wds[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr())
     assert lib.quant_linear_fused(bad) == -1
+    if copies:
+        copies.release()
 
 
-@pytest.mark.parametrize("K,n_out", [(1520, 37), (16400, 64), (8192, 33), (8208, 16)])
+@pytest.mark.parametrize("K,n_out", [(1520, 37), (16400, 64), (8192, 33), (8208, 16), (272, 70000), (1040, 65550), (2064, 65600)])
 @pytest.mark.parametrize("norm", [False, True])
-def test_fused_linear_ragged_lengths(gpu, pkg, oracle, dec, K, n_out, norm):
+@pytest.mark.parametrize("tiled", [False, True])
+def test_fused_linear_ragged_lengths(gpu, pkg, oracle, dec, K, n_out, norm, tiled):
     """Row lengths that are not a multiple of 1 KiB, longer than the register-staged part of the
     activation, and odd row counts."""
     torch, dev, lib = gpu
@@ -134,12 +158,22 @@ def test_fused_linear_ragged_lengths(gpu, pkg, oracle, dec, K, n_out, norm):
     y = torch.zeros(n_out + 8, dtype=torch.int16, device=dev)
     d = pkg.capi.make_fused_linear(E5M2, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(),
                                    norm_weight=nwd.data_ptr() if norm else None, norm_eps=1e-6, residual=rd.data_ptr())
+    copies = TiledCopies(torch, dev, lib, [wd], E5M2, K) if tiled else None
     assert lib.quant_linear_fused(d) == 0
+    assert lib.last_kernel() == ("gemv_fused_mfma" if tiled and n_out >= 65536 else "gemv_fused")      # tall weights only
+    if copies:
+        copies.release()
     out = from_dev(y, np.uint16)
     assert not out[n_out:].any()
     xin = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6) if norm else dec.f(x)
     lin = dec.linear(oracle.dequant_fp8_to_bf16(W, oracle.E5M2).reshape(n_out, K), xin)
-    assert ulp_close(out[:n_out], dec.r(lin + dec.f(res)), ulps=1.0, floor=1e-4).all()
+    # bf16(bf16(lin) + res): a one-ulp flip of lin (summation order) carries into the sum at lin's magnitude, not the sum's
+    want = dec.r(lin + dec.f(res))
+    got = dec.f(out[:n_out]).astype(np.float64)
+    tol = np.maximum(np.maximum(np.abs(lin), np.abs(dec.f(res))), np.abs(want)) * 2.0 ** -7 + 1e-4      # one BF16 spacing of the largest term
+    bad = np.abs(got - want) > tol
+    assert not bad.any(), (int(bad.sum()), float((np.abs(got - want) / tol).max()), np.flatnonzero(bad)[:5], got[bad][:5], want[bad][:5], lin[bad][:5])
+    assert (out[:n_out] == oracle.f32_to_bf16(want)).mean() > 0.98
 
 
 @pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 200), (2, 2, 200), (8, 2, 1024)])
