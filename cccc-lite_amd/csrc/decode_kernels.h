@@ -898,6 +898,11 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 #pragma unroll
             for (int d = 0; d < 8; d++) { vf[d] = v_new[sub * 8 + d]; }
         }
+        if (t0 + kl > pos)                                  // read from the row being appended, which may still hold anything (0 * NaN is NaN)
+        {
+#pragma unroll
+            for (int d = 0; d < 8; d++) { vf[d] = 0.0f; }
+        }
 #pragma unroll
         for (int gq = 0; gq < G; gq++)
         {

@@ -223,6 +223,9 @@ def test_fused_attention_appends_and_attends(gpu, oracle, dec, n_q, n_kv, t_kv):
     kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
     vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
     kd, vd = to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+    # a second pair of caches whose rows were never written: NaN patterns everywhere; it is filled position by position below
+    kn = torch.full((n_kv * t_kv * 128,), -1, dtype=torch.int16, device=dev)
+    vn = torch.full((n_kv * t_kv * 128,), 0x7FC1, dtype=torch.int16, device=dev)
     ws_bytes = lib.c.hip_attention_decode_workspace_bytes(n_q, n_kv, t_kv)
     ws = torch.full((ws_bytes,), 0xA5, dtype=torch.uint8, device=dev)
     consts = [to_dev(torch, dev, a) for a in (qw, kw, cos, sin)]
@@ -252,6 +255,16 @@ def test_fused_attention_appends_and_attends(gpu, oracle, dec, n_q, n_kv, t_kv):
         # two BF16 tensors rounded from slightly different exact values: about 1.6e-3 from the roundings alone
         assert np.linalg.norm(dec.f(got) - want) <= 4e-3 * np.linalg.norm(want)
         k_ref = dec.f(got_k).copy()
+        if pos <= 2:
+            # the same call on the never-written caches (positions 0, 1 in order): rows past the position must not leak into the output
+            y2 = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+            rc = lib.c.hip_attention_decode_fused_bf16(ptr(qd), ptr(knd), ptr(vnd), ptr(consts[0]), ptr(consts[1]), ptr(consts[2]), ptr(consts[3]),
+                                                       ptr(kn), ptr(vn), ptr(y2), ptr(ws), ws_bytes, n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6))
+            assert rc == 0
+            got2 = dec.f(from_dev(y2, np.uint16).reshape(n_q, 128))
+            assert np.isfinite(got2).all()
+            want2 = dec.attention(qr, dec.f(from_dev(kn, np.uint16).reshape(n_kv, t_kv, 128))[:, :pos + 1], dec.f(from_dev(vn, np.uint16).reshape(n_kv, t_kv, 128))[:, :pos + 1], pos, n_q, n_kv)
+            assert ulp_close(from_dev(y2, np.uint16).reshape(n_q, 128), want2, ulps=3.0, floor=4e-3 * np.abs(want2).max()).all()
 
 
 def test_argmax_and_embed(gpu, oracle):
