@@ -176,6 +176,30 @@ def test_fused_linear_ragged_lengths(gpu, pkg, oracle, dec, K, n_out, norm, tile
     assert (out[:n_out] == oracle.f32_to_bf16(want)).mean() > 0.98
 
 
+@pytest.mark.parametrize("n_out,tiled", [(96, False), (66000, False), (66000, True)])
+def test_fused_linear_e4m3_with_a_per_tensor_scale(gpu, pkg, oracle, dec, n_out, tiled):
+    """FP8_E4M3 weights with scale_<name> (the hy-mt2 file layout) through both forms of the fused kernel."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(n_out)
+    K, scale = 1024, 0.0123
+    x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+    nw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    W = oracle.encode_e4m3_rne((rng.standard_normal((n_out, K)) * 0.02 / scale).astype(np.float32))
+    xd, nwd, wd = (to_dev(torch, dev, v) for v in (x, nw, W))
+    y = torch.zeros(n_out, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(E4M3, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(), scales=[scale],
+                                   norm_weight=nwd.data_ptr(), norm_eps=1e-6)
+    copies = TiledCopies(torch, dev, lib, [wd], E4M3, K) if tiled else None
+    assert lib.quant_linear_fused(d) == 0
+    assert lib.last_kernel() == ("gemv_fused_mfma" if tiled else "gemv_fused")
+    if copies:
+        copies.release()
+    want = dec.linear(oracle.dequant_fp8_to_bf16(W, oracle.E4M3, scale).reshape(n_out, K), dec.rms_norm(dec.f(x), dec.f(nw), 1e-6))
+    got = dec.f(from_dev(y, np.uint16))
+    assert np.linalg.norm(got - want) <= 2e-3 * np.linalg.norm(want)
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -7 + 1e-4).all()
+
+
 @pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 200), (2, 2, 200), (8, 2, 1024)])
 def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv, t_kv):
     torch, dev, lib = gpu
