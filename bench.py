@@ -594,7 +594,8 @@ def main():
         achieved = flops / dom_us * 1e-6
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                    "kernel": "gemm_mfma_kernel", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3)}
+                    "kernel": "gemm_mfma_direct_kernel" if ws.lib.last_kernel() == "gemm_mfma_tiled" or (K % 64 == 0 and M >= 48) else "gemm_mfma_kernel",
+                    "weight_layout": "tiled copy" if ws.lib.last_kernel() == "gemm_mfma_tiled" else "row-major", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3)}
     else:
         achieved = gemv_bytes(K, N, M) / dom_us * 1e-3
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -357,9 +357,10 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
             }
             if (ok && !launched)
             {
-                if (g.w_type == DT_E5M2) { launched = gemm_mfma<DT_E5M2, 0>(a); }
-                else { launched = gemm_mfma<DT_E4M3, 0>(a); }
-                if (launched) { note_kernel("gemm_mfma"); }
+                const uint8_t* tiled = find_tiled(a, g.w_type);
+                if (g.w_type == DT_E5M2) { launched = gemm_mfma<DT_E5M2, 0>(a, tiled); }
+                else { launched = gemm_mfma<DT_E4M3, 0>(a, tiled); }
+                if (launched) { note_kernel(tiled ? "gemm_mfma_tiled" : "gemm_mfma"); }
             }
         }
     }

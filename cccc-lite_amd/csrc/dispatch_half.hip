@@ -53,8 +53,9 @@ const char* half_linear(const LinearArgs& a, int w_type)
         else { ok = scaled ? half_gemv<DT_E4M3, true>(a) : half_gemv<DT_E4M3, false>(a); }
         if (ok) { return "gemv_dot2_half"; }
     }
-    if (w_type == DT_E5M2) { gemm_mfma<DT_E5M2, 0, DT_HALF>(a); }
-    else { gemm_mfma<DT_E4M3, 0, DT_HALF>(a); }
+    const uint8_t* tiled = lookup_tiled(a.W, w_type, a.n_out, a.K, a.ldw);
+    if (w_type == DT_E5M2) { gemm_mfma<DT_E5M2, 0, DT_HALF>(a, tiled); }
+    else { gemm_mfma<DT_E4M3, 0, DT_HALF>(a, tiled); }
     return "gemm_mfma_half";
 }
 

@@ -253,6 +253,209 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// FP8 GEMM whose weights never pass through LDS.  A workgroup of four waves owns MB * 16 tokens x
+// 256 output features; wave w owns features 64 w .. 64 w + 63 for all of the tokens.  Each lane
+// loads the 16 weight bytes it will feed to the matrix cores itself -- row (lane % 16) of a 16-row
+// block, bytes 16 (lane / 16) .. + 15 of the 64-byte k-tile -- and converts them in registers: the
+// low 8 bytes are its B operand of the first v_mfma_f32_16x16x32 of the k-tile and the high 8 bytes
+// that of the second.  The contraction does not care in which order k is visited as long as both
+// operands agree, so the token operand is read from LDS with the matching k assignment (chunk
+// 2 (lane / 16) + step of the row).  Only the activations are staged through LDS (one 128-byte row
+// per token and k-tile, XOR-swizzled, two buffers, one barrier per k-tile); per matrix-core
+// instruction the LDS then moves a quarter of the bytes the two-operand kernel above needs.
+//   A operand (rows)    = tokens:   lane (i = lane % 16, g = lane / 16) holds k = 16 g + 8 step .. + 7
+//   B operand (columns) = features: same k
+//   D: lane holds feature lane % 16; register v is token 4 (lane / 16) + v
+template <int WT, bool SCALED, int MB, bool XCD, bool TILED, int AT = DT_BF16>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, const int m_tiles)
+{
+    constexpr int NB = 4;                       // 16-feature blocks per wave
+    constexpr int BTOK = MB * 16;               // tokens per workgroup
+    constexpr int BK = 64, CPR = 8;
+    constexpr int X_PER_THREAD = BTOK * CPR / 256;
+    __shared__ u32x4 xs[2][BTOK * CPR];
+    typedef typename std::conditional<AT == DT_HALF, f16x8, bf16x8>::type frag_t;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int n_tile, m_tile;
+    if (XCD)
+    {
+        const int seq = blockIdx.x >> 3;
+        n_tile = (blockIdx.x & 7) + 8 * (seq / m_tiles);
+        m_tile = seq % m_tiles;
+        if (n_tile >= n_tiles) { return; }
+    }
+    else
+    {
+        n_tile = blockIdx.x % n_tiles;
+        m_tile = blockIdx.x / n_tiles;
+    }
+    const int out_base = n_tile * 256 + wave * 64;
+    const int tok_base = m_tile * BTOK;
+    const int i16 = lane & 15;
+    const int g = lane >> 4;
+    const int n_kt = (a.K + BK - 1) / BK;
+
+    f32x4 acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { acc[mb][nb] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+
+    // Every address in the loop is a wave-uniform base (scalar registers, advanced by scalar adds) plus a
+    // 32-bit per-lane byte offset fixed for the whole kernel; the launcher checks that both operands are
+    // smaller than 4 GiB.
+    // TILED: a.W is the repacked copy (repack_tiled_kernel), where the KiB one load instruction of a wave
+    // takes -- 16 rows x 64 codes -- is contiguous and the next k-tile follows it.
+    long long w_tile_base[NB];
+    uint32_t w_off[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+    {
+        if (TILED)
+        {
+            w_tile_base[nb] = (long long)min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1) * n_kt * 1024;
+            w_off[nb] = lane * 16;
+        }
+        else
+        {
+            w_tile_base[nb] = 0;
+            w_off[nb] = (uint32_t)((long long)min(out_base + nb * 16 + i16, a.n_out - 1) * a.ldw + g * 16);
+        }
+    }
+    uint32_t x_off[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; i++)
+    {
+        const int q = tid + i * 256;
+        x_off[i] = (uint32_t)(((long long)min(tok_base + q / CPR, a.tokens - 1) * a.ldx + (q % CPR) * 8) * 2);
+    }
+    // LDS slots: where this thread stores its activation chunks, and where it reads its A operands
+    int x_store[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; i++)
+    {
+        const int q = tid + i * 256;
+        x_store[i] = (q / CPR) * CPR + swizzled_chunk_n<CPR>(q / CPR, q % CPR);
+    }
+
+    u32x4 wraw_a[NB], wraw_b[NB], xreg[X_PER_THREAD];
+    // K is a multiple of 64 here and the k-tile index of a prefetch is clamped to the last one, so no load
+    // or store in the loop needs a predicate or a branch: the wait counts stay exact
+    auto fetch_x = [&](int kt) {
+        const int k0 = min(kt, n_kt - 1) * BK;
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++) { xreg[i] = *(const u32x4*)((const uint8_t*)a.X + (size_t)k0 * 2 + (size_t)x_off[i]); }
+    };
+    auto fetch_w = [&](int kt, u32x4* wraw) {
+        const int k0 = min(kt, n_kt - 1) * (TILED ? 1024 : BK);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { wraw[nb] = *(const u32x4*)(a.W + w_tile_base[nb] + k0 + (size_t)w_off[nb]); }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++) { xs[buf][x_store[i]] = xreg[i]; }
+    };
+
+    // Order of one k-tile: barrier | request the next weights | first half of the matrix-core work |
+    // store the next activation tile to LDS and request the one after it | second half.  The LDS stores
+    // and the global loads are thus a whole k-tile of work away from the instructions that wait for
+    // them, and nothing but the barrier and the first fragment read stands between two k-tiles.
+    auto k_tile = [&](int kt, u32x4* wcur, u32x4* wnext) {
+        u32x4 wf[2][NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { dequant16_fp8<WT, SCALED, AT>(wcur[nb], a.w_scale, wf[0][nb], wf[1][nb]); }
+        __syncthreads();                                     // tile kt is in xs[kt & 1]; the other buffer is free
+        fetch_w(kt + 1, wnext);
+        const u32x4* xt = xs[kt & 1];
+        // token fragments run AHEAD instructions in front of the matrix-core instructions that use them
+        constexpr int AHEAD = 3, FRAGS = 2 * MB;
+        auto read_frag = [&](int f) {
+            const int row = (f % MB) * 16 + i16;
+            return xt[row * CPR + swizzled_chunk_n<CPR>(row, 2 * g + f / MB)];
+        };
+        u32x4 ring[AHEAD + 1];
+#pragma unroll
+        for (int f = 0; f < AHEAD; f++) { ring[f] = read_frag(f); }
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++)
+        {
+            if (f == FRAGS / 2)
+            {
+                stage((kt + 1) & 1);
+                fetch_x(kt + 2);
+            }
+            if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
+            const frag_t xf = __builtin_bit_cast(frag_t, ring[f % (AHEAD + 1)]);
+            const int s = f / MB, mb = f % MB;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+            {
+                const frag_t w = __builtin_bit_cast(frag_t, wf[s][nb]);
+                if constexpr (AT == DT_HALF) { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf, w, acc[mb][nb], 0, 0, 0); }
+                else { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, w, acc[mb][nb], 0, 0, 0); }
+            }
+        }
+        // pin the order: the scheduler otherwise pulls every read down to just before its first use
+        __builtin_amdgcn_sched_group_barrier(0x020, NB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++)
+        {
+            if (f == FRAGS / 2)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x200, X_PER_THREAD, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, X_PER_THREAD, 0);
+            }
+            if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+            __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
+        }
+    };
+
+    fetch_x(0);
+    fetch_w(0, wraw_a);
+    stage(0);
+    fetch_x(1);
+    for (int kt = 0; kt < n_kt; kt += 2)
+    {
+        k_tile(kt, wraw_a, wraw_b);
+        if (kt + 1 < n_kt) { k_tile(kt + 1, wraw_b, wraw_a); }
+    }
+
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+    {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+        {
+            const int out = out_base + nb * 16 + i16;
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+            {
+                const int tok = tok_base + mb * 16 + 4 * g + v;
+                if (out < a.n_out && tok < a.tokens)
+                {
+                    uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                    *y = finish_output_act<AT>(acc[mb][nb][v], a.alpha, a.beta, y);
+                }
+            }
+        }
+    }
+}
+
+template <int WT, int MB, bool XCD, bool TILED, int AT = DT_BF16>
+void launch_gemm_mfma_direct(const LinearArgs& a)
+{
+    const int n_tiles = (a.n_out + 255) / 256;
+    const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
+    const int grid = XCD ? 8 * m_tiles * ((n_tiles + 7) / 8) : n_tiles * m_tiles;
+    if (a.w_scale != 1.0f) { gemm_mfma_direct_kernel<WT, true, MB, XCD, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+    else { gemm_mfma_direct_kernel<WT, false, MB, XCD, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+}
+
 template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false, int AT = DT_BF16>
 void launch_gemm_mfma(const LinearArgs& a)
 {
@@ -263,12 +466,36 @@ void launch_gemm_mfma(const LinearArgs& a)
     else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false, BK, XCD, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
 }
 
-// Tile choice (tuned on MI355X): 128 x 128 tiles with the XCD-aware order when they give every CU at
-// least two workgroups (k step 128 for long K, where it halves the barriers per FLOP), otherwise
-// 128 x 64 tiles to put more workgroups on the machine.
+// Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
+// kernel that keeps the weights out of LDS -- on the tiled copy of the weight when one is registered
+// (1.10-1.15x the row-major rate: a wave's load is then eight full cache lines instead of sixteen half
+// lines) -- with 128-token tiles above 64 tokens and 64-token tiles below.  Everything else (FP4, ragged
+// K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they give
+// every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
+// otherwise 128 x 64 tiles to put more workgroups on the machine.
 template <int WT, int BLOCK, int AT = DT_BF16>
-bool gemm_mfma(const LinearArgs& a)
+bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr)
 {
+    if constexpr (WT != DT_FP4)
+    {
+        const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
+        if (a.K % 64 == 0 && a.tokens >= 48 && small_offsets)
+        {
+            LinearArgs d = a;
+            if (tiled)
+            {
+                d.W = tiled;
+                if (a.tokens > 64) { launch_gemm_mfma_direct<WT, 8, false, true, AT>(d); }
+                else { launch_gemm_mfma_direct<WT, 4, false, true, AT>(d); }
+            }
+            else
+            {
+                if (a.tokens > 64) { launch_gemm_mfma_direct<WT, 8, false, false, AT>(d); }
+                else { launch_gemm_mfma_direct<WT, 4, false, false, AT>(d); }
+            }
+            return true;
+        }
+    }
     const long long tiles_big = (long long)((a.n_out + 127) / 128) * ((a.tokens + 127) / 128);
     if (tiles_big >= 2LL * cu_count())
     {

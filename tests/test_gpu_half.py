@@ -48,6 +48,34 @@ def test_half_activations(gpu, oracle, w_type, tokens, kernel, scale):
     check_half(out[:tokens * n_out].reshape(tokens, n_out), exact, label=f"{w_type} {tokens} {scale}")
 
 
+@pytest.mark.parametrize("w_type", [E5M2, E4M3])
+@pytest.mark.parametrize("tokens", [64, 200])
+def test_half_gemm_with_weights_kept_out_of_lds(gpu, oracle, w_type, tokens):
+    """K % 64 == 0 and 48 tokens or more: the GEMM that converts weights in registers, row-major and tiled."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + w_type)
+    n_out, K, scale = 328, 1024, 0.37
+    codes, x, exact = make_case(oracle, rng, w_type, n_out, K, tokens, scale)
+    wd, xd = to_dev(torch, dev, codes), to_dev(torch, dev, x.view(np.uint16))
+    td = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
+    outs = []
+    for tiled in (False, True):
+        if tiled:
+            assert lib.weight_prepare(wd.data_ptr(), w_type, n_out, K, K, td.data_ptr()) == 0
+        try:
+            y = torch.zeros(tokens * n_out + 16, dtype=torch.int16, device=dev)
+            assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, inv_scale=scale, act_type=HALF) == 0
+            assert lib.last_kernel() == "gemm_mfma_half"
+        finally:
+            if tiled:
+                assert lib.weight_release(wd.data_ptr()) == 0
+        out = from_dev(y, np.uint16)
+        assert not out[tokens * n_out:].any()
+        outs.append(out[:tokens * n_out].reshape(tokens, n_out))
+        check_half(outs[-1], exact, label=f"{w_type} {tokens} tiled={tiled}")
+    assert np.array_equal(outs[0], outs[1])
+
+
 def test_half_alpha_beta_tall_and_generic(gpu, oracle):
     torch, dev, lib = gpu
     rng = np.random.default_rng(5)

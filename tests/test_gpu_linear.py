@@ -180,6 +180,55 @@ def test_prefill_gemm_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, fmt):
     assert kernel == "gemm_mfma"
 
 
+@pytest.mark.parametrize("tokens", [48, 64, 65, 128, 200, 513])
+@pytest.mark.parametrize("n_out,K", [(256, 64), (1000, 192), (520, 1024), (1536, 2048)])
+@pytest.mark.parametrize("w_type_name", ["e5m2", "e4m3"])
+def test_prefill_gemm_with_weights_kept_out_of_lds(gpu, pkg, oracle, tokens, n_out, K, w_type_name):
+    """FP8 GEMM kernel for K % 64 == 0 and 48 tokens or more (64- and 128-token tiles, ragged token and
+    row counts, one k-tile and many), on the row-major weight and on its tiled copy, with and without a
+    per-tensor scale and with alpha / beta, against the exact contraction."""
+    torch, dev, lib = gpu
+    seed = pkg.synth.seed_for(4, 300 + tokens % 89 + n_out % 13)
+    if w_type_name == "e5m2":
+        w_type, W = oracle.E5M2, pkg.synth.weights_e5m2(seed, n_out, K)
+    else:
+        w_type, W = oracle.E4M3, pkg.synth.weights_e4m3(seed, n_out, K)[0]
+    X = pkg.synth.activations(seed, tokens, K)
+    want = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K), X)
+    want_s = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K, 0.37), X)
+    c0 = pkg.synth.activations(seed + 1, tokens, n_out)
+    wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+    td = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
+
+    def run(label, expect_kernel):
+        y = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), y.data_ptr(), n_out, tokens, K) == 0
+        assert lib.last_kernel() == expect_kernel
+        out = from_dev(y, np.uint16)
+        assert not out[tokens * n_out:].any(), "wrote past the end"
+        got = out[: tokens * n_out].reshape(tokens, n_out)
+        check_rows(bf16_f64(oracle, got), want, f"{label} {w_type_name} {tokens}x{n_out}x{K}")
+        # one BF16 ulp plus the FP32 accumulation noise, which grows with the size of the terms (E4M3 codes reach 448)
+        check_bf16_close(got, want, label, slack_ulp=1.0, abs_floor=max(2e-5, 1e-6 * np.sqrt(K) * np.abs(want).max()))
+        ys = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), ys.data_ptr(), n_out, tokens, K, inv_scale=0.37) == 0
+        check_rows(bf16_f64(oracle, from_dev(ys, np.uint16).reshape(tokens, n_out)), want_s, label + " scaled")
+        yb = to_dev(torch, dev, c0.reshape(-1))
+        assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), yb.data_ptr(), n_out, tokens, K, alpha=0.5, beta=-2.0) == 0
+        want_b = 0.5 * want - 2.0 * bf16_f64(oracle, c0)
+        check_rows(bf16_f64(oracle, from_dev(yb, np.uint16).reshape(tokens, n_out)), want_b, label + " alpha beta")
+        return got
+
+    plain = run("row-major", "gemm_mfma")
+    assert lib.weight_prepare(wd.data_ptr(), w_type, n_out, K, K, td.data_ptr()) == 0
+    try:
+        tiled = run("tiled", "gemm_mfma_tiled")
+    finally:
+        assert lib.weight_release(wd.data_ptr()) == 0
+    # same products, same order of summation: the two layouts agree to the bit
+    assert np.array_equal(plain, tiled)
+
+
 # ------------------------------------------------------------------------------------------ dispatcher
 
 def test_weight_as_B_and_transposed_layouts_match_the_scalar_oracle(gpu, pkg, oracle):
