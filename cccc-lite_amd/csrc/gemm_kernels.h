@@ -264,11 +264,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // 2 (lane / 16) + step of the row).  Only the activations are staged through LDS (one 128-byte row
 // per token and k-tile, XOR-swizzled, two buffers, one barrier per k-tile); per matrix-core
 // instruction the LDS then moves a quarter of the bytes the two-operand kernel above needs.
-//   A operand (rows)    = tokens:   lane (i = lane % 16, g = lane / 16) holds k = 16 g + 8 step .. + 7
-//   B operand (columns) = features: same k
-//   D: lane holds feature lane % 16; register v is token 4 (lane / 16) + v
-template <int WT, bool SCALED, int MB, bool XCD, bool TILED, int AT = DT_BF16>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, const int m_tiles)
+//   A operand (rows)    = features: lane (i = lane % 16, g = lane / 16) holds k = 16 g + 8 step .. + 7
+//   B operand (columns) = tokens:   same k
+//   D: lane holds token lane % 16; register v is feature 4 (lane / 16) + v, so a lane ends with four
+//      consecutive outputs of one token row (one 8-byte store)
+// SPLIT: blockIdx.y selects one of gridDim.y equal ranges of k-tiles; the FP32 partial sums of range s go
+// to partial[s][token][feature] (no alpha / beta) and gemm_splitk_combine_kernel finishes them.  Used when
+// the output has too few tiles to fill the machine.
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, float* __restrict__ partial)
 {
     constexpr int NB = 4;                       // 16-feature blocks per wave
     constexpr int BTOK = MB * 16;               // tokens per workgroup
@@ -280,24 +284,17 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    int n_tile, m_tile;
-    if (XCD)
-    {
-        const int seq = blockIdx.x >> 3;
-        n_tile = (blockIdx.x & 7) + 8 * (seq / m_tiles);
-        m_tile = seq % m_tiles;
-        if (n_tile >= n_tiles) { return; }
-    }
-    else
-    {
-        n_tile = blockIdx.x % n_tiles;
-        m_tile = blockIdx.x / n_tiles;
-    }
+    const int n_tile = blockIdx.x % n_tiles;
+    const int m_tile = blockIdx.x / n_tiles;
     const int out_base = n_tile * 256 + wave * 64;
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
     const int g = lane >> 4;
-    const int n_kt = (a.K + BK - 1) / BK;
+    const int n_kt_total = a.K / BK;
+    const int kt_begin = SPLIT ? (int)((long long)n_kt_total * blockIdx.y / gridDim.y) : 0;
+    const int n_kt = SPLIT ? (int)((long long)n_kt_total * (blockIdx.y + 1) / gridDim.y) - kt_begin : n_kt_total;
+    const uint8_t* const w_begin = a.W + (long long)kt_begin * (TILED ? 1024 : BK);
+    const uint8_t* const x_begin = (const uint8_t*)a.X + (long long)kt_begin * BK * 2;
 
     f32x4 acc[MB][NB];
 #pragma unroll
@@ -317,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     {
         if (TILED)
         {
-            w_tile_base[nb] = (long long)min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1) * n_kt * 1024;
+            w_tile_base[nb] = (long long)min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1) * n_kt_total * 1024;
             w_off[nb] = lane * 16;
         }
         else
@@ -348,12 +345,12 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     auto fetch_x = [&](int kt) {
         const int k0 = min(kt, n_kt - 1) * BK;
 #pragma unroll
-        for (int i = 0; i < X_PER_THREAD; i++) { xreg[i] = *(const u32x4*)((const uint8_t*)a.X + (size_t)k0 * 2 + (size_t)x_off[i]); }
+        for (int i = 0; i < X_PER_THREAD; i++) { xreg[i] = *(const u32x4*)(x_begin + (size_t)k0 * 2 + (size_t)x_off[i]); }
     };
     auto fetch_w = [&](int kt, u32x4* wraw) {
         const int k0 = min(kt, n_kt - 1) * (TILED ? 1024 : BK);
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) { wraw[nb] = *(const u32x4*)(a.W + w_tile_base[nb] + k0 + (size_t)w_off[nb]); }
+        for (int nb = 0; nb < NB; nb++) { wraw[nb] = *(const u32x4*)(w_begin + w_tile_base[nb] + k0 + (size_t)w_off[nb]); }
     };
     auto stage = [&](int buf) {
 #pragma unroll
@@ -395,8 +392,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
             for (int nb = 0; nb < NB; nb++)
             {
                 const frag_t w = __builtin_bit_cast(frag_t, wf[s][nb]);
-                if constexpr (AT == DT_HALF) { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf, w, acc[mb][nb], 0, 0, 0); }
-                else { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, w, acc[mb][nb], 0, 0, 0); }
+                if constexpr (AT == DT_HALF) { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, xf, acc[mb][nb], 0, 0, 0); }
+                else { acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, xf, acc[mb][nb], 0, 0, 0); }
             }
         }
         // pin the order: the scheduler otherwise pulls every read down to just before its first use
@@ -425,35 +422,110 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         if (kt + 1 < n_kt) { k_tile(kt + 1, wraw_b, wraw_a); }
     }
 
+    const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
     {
+        const int tok = tok_base + mb * 16 + i16;
+        if (tok >= a.tokens) { continue; }
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
         {
-            const int out = out_base + nb * 16 + i16;
-#pragma unroll
-            for (int v = 0; v < 4; v++)
+            const int out = out_base + nb * 16 + 4 * g;
+            if (out >= a.n_out) { continue; }
+            const f32x4 r = acc[mb][nb];
+            if constexpr (SPLIT)
             {
-                const int tok = tok_base + mb * 16 + 4 * g + v;
-                if (out < a.n_out && tok < a.tokens)
+                float* p = partial + ((long long)blockIdx.y * a.tokens + tok) * a.n_out + out;
+                if (wide_store && out + 3 < a.n_out) { *(f32x4*)p = r; }
+                else
                 {
-                    uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
-                    *y = finish_output_act<AT>(acc[mb][nb][v], a.alpha, a.beta, y);
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { p[v] = r[v]; }
+                    }
+                }
+            }
+            else
+            {
+                uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                if (wide_store && out + 3 < a.n_out)
+                {
+                    uint16_t old[4] = { 0, 0, 0, 0 };
+                    if (a.beta != 0.0f) { *(uint2*)old = *(const uint2*)y; }
+                    uint16_t o[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) { o[v] = finish_output_act<AT>(r[v], a.alpha, a.beta, &old[v]); }
+                    *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) };
+                }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { y[v * a.y_stride_out] = finish_output_act<AT>(r[v], a.alpha, a.beta, y + v * a.y_stride_out); }
+                    }
                 }
             }
         }
     }
 }
 
-template <int WT, int MB, bool XCD, bool TILED, int AT = DT_BF16>
-void launch_gemm_mfma_direct(const LinearArgs& a)
+// Sums the FP32 partial tiles of a k-split GEMM and applies alpha / beta and the one rounding.  One thread
+// per four consecutive features of a token (n_out is a multiple of 4 on this path).
+template <int AT>
+__global__ __launch_bounds__(256) void gemm_splitk_combine_kernel(const float* __restrict__ partial, const int splits, const LinearArgs a)
+{
+    const long long groups = (long long)a.tokens * (a.n_out / 4);
+    const long long slice = (long long)a.tokens * a.n_out;
+    const bool wide_store = a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0;
+    for (long long q = (long long)blockIdx.x * 256 + threadIdx.x; q < groups; q += (long long)gridDim.x * 256)
+    {
+        const int tok = (int)(q / (a.n_out / 4));
+        const int out = (int)(q % (a.n_out / 4)) * 4;
+        f32x4 r = *(const f32x4*)(partial + q * 4);
+        for (int s = 1; s < splits; s++) { r += *(const f32x4*)(partial + s * slice + q * 4); }
+        uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+        if (wide_store)
+        {
+            uint16_t old[4] = { 0, 0, 0, 0 };
+            if (a.beta != 0.0f) { *(uint2*)old = *(const uint2*)y; }
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) { o[v] = finish_output_act<AT>(r[v], a.alpha, a.beta, &old[v]); }
+            *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) };
+        }
+        else
+        {
+#pragma unroll
+            for (int v = 0; v < 4; v++) { y[v * a.y_stride_out] = finish_output_act<AT>(r[v], a.alpha, a.beta, y + v * a.y_stride_out); }
+        }
+    }
+}
+
+// splits > 1: `partial` holds splits * tokens * n_out floats
+template <int WT, int MB, bool TILED, int AT = DT_BF16>
+void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial = nullptr)
 {
     const int n_tiles = (a.n_out + 255) / 256;
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
-    const int grid = XCD ? 8 * m_tiles * ((n_tiles + 7) / 8) : n_tiles * m_tiles;
-    if (a.w_scale != 1.0f) { gemm_mfma_direct_kernel<WT, true, MB, XCD, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
-    else { gemm_mfma_direct_kernel<WT, false, MB, XCD, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
+    const dim3 grid(n_tiles * m_tiles, splits);
+    const bool scaled = a.w_scale != 1.0f;
+    if (splits > 1)
+    {
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        const long long groups = (long long)a.tokens * (a.n_out / 4);
+        const long long blocks = (groups + 255) / 256;
+        const long long cap = (long long)cu_count() * 16;
+        gemm_splitk_combine_kernel<AT><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
+    }
+    else
+    {
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+        else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+    }
 }
 
 template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false, int AT = DT_BF16>
@@ -469,9 +541,11 @@ void launch_gemm_mfma(const LinearArgs& a)
 // Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
 // kernel that keeps the weights out of LDS -- on the tiled copy of the weight when one is registered
 // (1.10-1.15x the row-major rate: a wave's load is then eight full cache lines instead of sixteen half
-// lines) -- with 128-token tiles above 64 tokens and 64-token tiles below.  Everything else (FP4, ragged
-// K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they give
-// every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
+// lines).  128-token tiles when they give every CU two workgroups; else 64-token tiles when those fill the
+// machine; else the k range is split over workgroups (about one per CU, 16 k-tiles or more each) and a
+// second kernel adds the partial sums -- 2x on 512 tokens x 4096 features x K 12288.  Everything else (FP4,
+// ragged K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they
+// give every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
 // otherwise 128 x 64 tiles to put more workgroups on the machine.
 template <int WT, int BLOCK, int AT = DT_BF16>
 bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr)
@@ -482,16 +556,35 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr)
         if (a.K % 64 == 0 && a.tokens >= 48 && small_offsets)
         {
             LinearArgs d = a;
+            if (tiled) { d.W = tiled; }
+            const int cus = cu_count();
+            const long long n_tiles = (a.n_out + 255) / 256;
+            const long long tiles8 = n_tiles * ((a.tokens + 127) / 128), tiles4 = n_tiles * ((a.tokens + 63) / 64);
+            int mb = 4, splits = 1;
+            float* partial = nullptr;
+            if (a.tokens > 64 && tiles8 >= 2LL * cus) { mb = 8; }
+            else if (tiles4 * 4 < 5LL * cus && a.n_out % 4 == 0)
+            {
+                const long long base = a.tokens > 64 ? tiles8 : tiles4;
+                long long s = (cus + base / 2) / base;
+                if (s > 8) { s = 8; }
+                if (s > a.K / 64 / 16) { s = a.K / 64 / 16; }
+                if (s > 1) { partial = (float*)workspace((size_t)s * a.tokens * a.n_out * sizeof(float)); }
+                if (partial)
+                {
+                    splits = (int)s;
+                    mb = a.tokens > 64 ? 8 : 4;
+                }
+            }
             if (tiled)
             {
-                d.W = tiled;
-                if (a.tokens > 64) { launch_gemm_mfma_direct<WT, 8, false, true, AT>(d); }
-                else { launch_gemm_mfma_direct<WT, 4, false, true, AT>(d); }
+                if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial); }
+                else { launch_gemm_mfma_direct<WT, 4, true, AT>(d, splits, partial); }
             }
             else
             {
-                if (a.tokens > 64) { launch_gemm_mfma_direct<WT, 8, false, false, AT>(d); }
-                else { launch_gemm_mfma_direct<WT, 4, false, false, AT>(d); }
+                if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial); }
+                else { launch_gemm_mfma_direct<WT, 4, false, AT>(d, splits, partial); }
             }
             return true;
         }

@@ -18,6 +18,12 @@ int finish(const char* what);
 // Number of compute units of the current device (cached per device).
 int cu_count();
 
+// Device scratch memory of at least `bytes` for the launches about to be enqueued on `stream()`: one
+// grow-only buffer per (device, stream), kept until the process ends, so kernels enqueued on one stream
+// reuse it in order.  Returns nullptr when it cannot be provided (allocation failure, or the buffer would
+// have to grow while the stream is being captured into a graph); callers then take a path that needs none.
+void* workspace(size_t bytes);
+
 // The load-time tiled copy registered for the FP8 weight `W` by hip_quant_weight_prepare, or nullptr
 // when there is none or its type / shape / row stride differ (defined with the registry in dispatch.hip).
 const unsigned char* lookup_tiled(const void* W, int type, int n_out, int K, long long ldw);

@@ -2,6 +2,9 @@
 #include "../../include/cccc_hip_quant.h"
 #include <atomic>
 #include <cstdio>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace ccq
 {
@@ -40,6 +43,36 @@ int cu_count()
         cached[dev].store(n, std::memory_order_relaxed);
     }
     return n;
+}
+
+void* workspace(size_t bytes)
+{
+    struct Buffer { void* ptr; size_t bytes; };
+    static std::mutex mutex;
+    static std::map<std::pair<int, hipStream_t>, Buffer> buffers;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { return nullptr; }
+    std::lock_guard<std::mutex> lock(mutex);
+    Buffer& b = buffers[{ dev, stream() }];
+    if (b.bytes >= bytes) { return b.ptr; }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream(), &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+    {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    // work already enqueued on the stream may still be using the old buffer
+    if (b.ptr && (hipStreamSynchronize(stream()) != hipSuccess || hipFree(b.ptr) != hipSuccess)) { (void)hipGetLastError(); }
+    b = Buffer{ nullptr, 0 };
+    const size_t want = bytes + bytes / 4;
+    void* p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    b = Buffer{ p, want };
+    return p;
 }
 
 }    // namespace ccq

@@ -181,12 +181,14 @@ def test_prefill_gemm_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, fmt):
 
 
 @pytest.mark.parametrize("tokens", [48, 64, 65, 128, 200, 513])
-@pytest.mark.parametrize("n_out,K", [(256, 64), (1000, 192), (520, 1024), (1536, 2048)])
+@pytest.mark.parametrize("n_out,K", [(256, 64), (1000, 192), (250, 1024), (1536, 2048), (512, 8192)])
 @pytest.mark.parametrize("w_type_name", ["e5m2", "e4m3"])
 def test_prefill_gemm_with_weights_kept_out_of_lds(gpu, pkg, oracle, tokens, n_out, K, w_type_name):
     """FP8 GEMM kernel for K % 64 == 0 and 48 tokens or more (64- and 128-token tiles, ragged token and
     row counts, one k-tile and many), on the row-major weight and on its tiled copy, with and without a
-    per-tensor scale and with alpha / beta, against the exact contraction."""
+    per-tensor scale and with alpha / beta, against the exact contraction.  The two long-K shapes have so
+    few output tiles that the k range is split over workgroups (2 and 8 ranges) and a second kernel adds
+    the partial sums; n_out = 250 is not a multiple of 4 and never splits."""
     torch, dev, lib = gpu
     seed = pkg.synth.seed_for(4, 300 + tokens % 89 + n_out % 13)
     if w_type_name == "e5m2":
