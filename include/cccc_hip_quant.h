@@ -88,6 +88,11 @@ C_EXPORT int hip_absmax(const void* src, int src_type, unsigned int n, void* d_r
  * C of type HALF; the weight is dequantised to half, FP32 accumulation, one rounding to half).
  * `act_scale` is accepted and ignored (it only drives the W8A8 route, cccc/cublas_real.h:871-873).
  * Anything else (both operands quantized, FP4 with HALF, mixed 16-bit types, other C types) returns -1.
+ * Device memory: the one case in which the library allocates is an FP8 GEMM of 48 tokens or more whose
+ * output has too few tiles to fill the GPU; it then splits K over workgroups and keeps FP32 partial sums in a
+ * scratch buffer per (device, stream) that grows on demand and lives until the process ends (at most
+ * 8 * M * N * 4 bytes).  While the stream is being captured into a graph the buffer is never grown: the
+ * call then runs without the split.
  */
 C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                             const void* A, int typeA, int lda, float invScaleA,
