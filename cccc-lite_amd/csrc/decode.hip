@@ -130,6 +130,11 @@ int hip_rms_norm_fwd(int type, void* X, void* Y, void* scale, void* invstd_out, 
         return 1;
     }
     if (outer == 0 || inner == 0) { return 0; }
+    if (!X || !Y || !scale)
+    {
+        fprintf(stderr, "hip_rms_norm_fwd: null pointer\n");
+        return 1;
+    }
     rms_norm_bf16_kernel<<<outer, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)scale, (float*)invstd_out, inner, epsilon);
     return finish("rms_norm_fwd_bf16");
 }
@@ -148,6 +153,11 @@ int hip_rope_fwd(int type, const void* X, void* Y, const void* cos_tab, const vo
     }
     const unsigned total = (D / 2) * T * B;
     if (total == 0) { return 0; }
+    if (!X || !Y || !cos_tab || !sin_tab)
+    {
+        fprintf(stderr, "hip_rope_fwd: null pointer\n");
+        return 1;
+    }
     rope_bf16_kernel<<<(total + 255) / 256, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, D, T, B, pos_offset);
     return finish("rope_fwd_bf16");
 }
@@ -160,6 +170,11 @@ int hip_embed_fwd(int type, const void* ids, const void* W, void* Y, int D, int 
         return 1;
     }
     if (T * B <= 0) { return 0; }
+    if (!ids || !W || !Y)
+    {
+        fprintf(stderr, "hip_embed_fwd: null pointer\n");
+        return 1;
+    }
     embed_bf16_kernel<<<dim3(1, T * B), 256, 0, stream()>>>((const float*)ids, nullptr, (const uint16_t*)W, (uint16_t*)Y, D, 0x7FFFFFFF);
     return finish("embed_fwd_bf16");
 }
@@ -176,6 +191,7 @@ int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v, const 
                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
 {
     if (head_dim != 128 || n_q_heads <= 0 || n_kv_heads <= 0 || t_kv <= 0 || !d_pos) { return -1; }
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_tab || !sin_tab || !q_out || !k_cache || !v_cache) { return -1; }
     qk_norm_rope_kv_kernel<<<n_q_heads + 2 * n_kv_heads, 64, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v,
                                                                            (const uint16_t*)q_norm_w, (const uint16_t*)k_norm_w,
                                                                            (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,

@@ -90,6 +90,31 @@ unsigned long long cccc_gpu_allocated_bytes(void)
     return g ? (unsigned long long)g->allocatedBytes() : 0ull;
 }
 
+namespace
+{
+
+// Two timing events and the library's sync switch (off while timing), both put back on every way out.
+struct TimingScope
+{
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int previous_sync;
+    bool ok;
+    TimingScope() : previous_sync(hip_quant_set_sync(0))
+    {
+        ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+    }
+    ~TimingScope()
+    {
+        if (e0) { (void)hipEventDestroy(e0); }
+        if (e1) { (void)hipEventDestroy(e1); }
+        hip_quant_set_sync(previous_sync);
+    }
+    TimingScope(const TimingScope&) = delete;
+    TimingScope& operator=(const TimingScope&) = delete;
+};
+
+}    // namespace
+
 // Runs `steps` timed passes over a chain of n_ops linears  R[i] = W[i]^T X[i]  (Matrix::mulBatched
 // with TRANS / NO_TRANS, as the LLM graph calls it) after `warmup` untimed passes.  use_graph != 0
 // replays one captured hipGraph per pass instead of issuing the launches one by one.  Events are
@@ -109,10 +134,10 @@ double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int step
     hipStream_t stream = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    TimingScope timing;
+    if (!timing.ok) { return -1.0; }
+    const hipEvent_t e0 = timing.e0, e1 = timing.e1;
     double result = -1.0;
-    hip_quant_set_sync(0);
     for (int i = 0; i < warmup; i++) { if (one_pass() != 0) { return -2.0; } }
     if (hipDeviceSynchronize() != hipSuccess) { return -3.0; }
     if (use_graph)
@@ -156,8 +181,6 @@ double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int step
             result = ms;
         }
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     return result;
 }
 
@@ -167,9 +190,9 @@ double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int step
 double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n_out, int tokens, int K,
                             unsigned int block, int iters, int warmup)
 {
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
-    hip_quant_set_sync(0);
+    TimingScope timing;
+    if (!timing.ok) { return -1.0; }
+    const hipEvent_t e0 = timing.e0, e1 = timing.e1;
     int status = 0;
     for (int i = 0; i < warmup + iters; i++)
     {
@@ -186,8 +209,6 @@ double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n
         (void)hipEventElapsedTime(&ms, e0, e1);
         result = ms;
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     return result;
 }
 
