@@ -353,19 +353,32 @@ def test_full_size_gemv_properties(gpu, pkg, oracle):
 
 
 def test_full_size_prefill_gemm_sampled(gpu, pkg, oracle):
+    """The benchmark's prefill shapes at full size, on the row-major weight and on its tiled copy (the
+    second shape has 64 output tiles, so its k range is split over workgroups): 192 sampled features of
+    every token against the exact contraction, and the two layouts against each other."""
     torch, dev, lib = gpu
-    for tokens, n_out, K in ((512, 12288, 4096), (2048, 4096, 12288)):
+    for tokens, n_out, K in ((512, 12288, 4096), (2048, 4096, 12288), (512, 4096, 12288)):
         g = torch.Generator(device="cpu").manual_seed(tokens + K)
         W = (torch.randn(n_out, K, generator=g) * 0.02).to(torch.bfloat16).to(torch.float8_e5m2).view(torch.uint8).numpy()
         X = pkg.synth.activations(tokens, tokens, K)
         wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+        rows = np.random.default_rng(tokens).choice(n_out, size=192, replace=False)
+        want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2), X)
         yd = torch.zeros(tokens, n_out, dtype=torch.int16, device=dev)
         assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
         assert lib.last_kernel() == "gemm_mfma"
         y = from_dev(yd, np.uint16)
-        rows = np.random.default_rng(tokens).choice(n_out, size=192, replace=False)
-        want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2), X)
         check_rows(bf16_f64(oracle, y[:, rows]), want, f"gemm {tokens}x{n_out}x{K}")
+        td = torch.zeros(lib.tiled_size(oracle.E5M2, n_out, K), dtype=torch.uint8, device=dev)
+        assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, K, K, td.data_ptr()) == 0
+        try:
+            yt = torch.zeros(tokens, n_out, dtype=torch.int16, device=dev)
+            assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), yt.data_ptr(), n_out, tokens, K) == 0
+            assert lib.last_kernel() == "gemm_mfma_tiled"
+        finally:
+            assert lib.weight_release(wd.data_ptr()) == 0
+        assert np.array_equal(from_dev(yt, np.uint16), y), "tiled and row-major weights give different outputs"
+        del wd, xd, yd, yt, td
 
 
 # ------------------------------------------------------------------------------------------ load-time repack
