@@ -931,54 +931,68 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 // in a fixed order.  64 outputs (half a head) per workgroup; n_blocks <= ATT_MAX_BLOCKS.
 constexpr int ATT_MAX_BLOCKS = 1024;
 
+// Every load of the common case is requested before anything is known -- the position, up to four (max, sum)
+// pairs per thread and the partials of the first 64 blocks -- so the launch costs one trip to memory instead of
+// three dependent ones (position -> statistics -> partials).  Blocks past the position hold whatever the
+// workspace held before: they are masked out by select, never multiplied.
 static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const float* __restrict__ partial, const float2* __restrict__ stats, uint16_t* __restrict__ y,
                                                                   int n_out, int t_kv, int n_blocks, const int* __restrict__ d_pos)
 {
     __shared__ float w_lds[ATT_MAX_BLOCKS];
     __shared__ float red[4];
     __shared__ float part[4][64];
-    const int pos = *d_pos;
-    if (pos < 0 || pos >= t_kv) { return; }
-    const int n_active = pos / ATT_KEYS + 1;
+    constexpr int PRE = 16;                              // blocks per wave requested up front (4 waves: 64 blocks)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int qh = (blockIdx.x * 64) >> 7;
+    const int o = min(blockIdx.x * 64 + lane, n_out - 1);
     const float2* st = stats + (size_t)qh * n_blocks;
+
+    const int pos = *d_pos;
+    float2 sb[ATT_MAX_BLOCKS / 256];
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++) { sb[i] = st[min((int)threadIdx.x + i * 256, n_blocks - 1)]; }
+    float pre[PRE];
+#pragma unroll
+    for (int j = 0; j < PRE; j++) { pre[j] = partial[(size_t)min(wave + 4 * j, n_blocks - 1) * n_out + o]; }
+
+    if (pos < 0 || pos >= t_kv) { return; }
+    const int n_active = pos / ATT_KEYS + 1;
     float m = -INFINITY;
-    for (int b = threadIdx.x; b < n_active; b += 256) { m = fmaxf(m, st[b].x); }
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
+    {
+        if ((int)threadIdx.x + i * 256 < n_active) { m = fmaxf(m, sb[i].x); }
+    }
     m = wave_max(m);
     if (lane == 0) { red[wave] = m; }
     __syncthreads();
     m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     __syncthreads();
     float l = 0.0f;
-    for (int b = threadIdx.x; b < n_active; b += 256)
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
     {
-        const float2 sb = st[b];
-        const float e = expf(sb.x - m);
-        w_lds[b] = e;
-        l += sb.y * e;
+        const int b = threadIdx.x + i * 256;
+        if (b < n_active)
+        {
+            const float e = expf(sb[i].x - m);
+            w_lds[b] = e;
+            l += sb[i].y * e;
+        }
     }
     l = block_sum<256>(l, red);                     // its barrier publishes w_lds
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    const int o = blockIdx.x * 64 + lane;
     float total = 0.0f;
-    if (o < n_out)
+#pragma unroll
+    for (int j = 0; j < PRE; j++)
     {
-        int b = wave;
-        for (; b + 12 < n_active; b += 16)
-        {
-            const float a0 = partial[(size_t)b * n_out + o], a1 = partial[(size_t)(b + 4) * n_out + o];
-            const float a2 = partial[(size_t)(b + 8) * n_out + o], a3 = partial[(size_t)(b + 12) * n_out + o];
-            total = fmaf(a0, w_lds[b], total);
-            total = fmaf(a1, w_lds[b + 4], total);
-            total = fmaf(a2, w_lds[b + 8], total);
-            total = fmaf(a3, w_lds[b + 12], total);
-        }
-        for (; b < n_active; b += 4) { total = fmaf(partial[(size_t)b * n_out + o], w_lds[b], total); }
+        const int b = wave + 4 * j;
+        if (b < n_active) { total = fmaf(pre[j], w_lds[b], total); }
     }
+    for (int b = wave + 4 * PRE; b < n_active; b += 4) { total = fmaf(partial[(size_t)b * n_out + o], w_lds[b], total); }
     part[wave][lane] = total;
     __syncthreads();
-    if (wave == 0 && o < n_out) { y[o] = (uint16_t)f32_to_bf16_bits((((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]) * inv); }
+    if (wave == 0 && blockIdx.x * 64 + lane < n_out) { y[o] = (uint16_t)f32_to_bf16_bits((((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]) * inv); }
 }
 
 // Arg-max of BF16 values, lowest index on ties, in two launches: per-block candidates, then the pick.
