@@ -269,6 +269,54 @@ def test_weight_as_B_and_transposed_layouts_match_the_scalar_oracle(gpu, pkg, or
                 assert diff.max() <= 2.0 ** -7 * np.abs(bf16_f64(oracle, want)).max(), (weight_is_a, ta, tb, lib.last_kernel())
 
 
+@pytest.mark.parametrize("case", range(36))
+def test_random_shapes_with_padded_strides(gpu, pkg, oracle, case):
+    """Seeded random FP8 problems in the two LLM layouts (weight as A with TRANS / NO_TRANS, weight as B
+    mirrored) with row strides larger than the rows -- lda, ldb and ldc padded, the padding filled with NaN
+    codes or NaN values -- against the scalar C restatement of the dispatcher; token counts straddle every
+    kernel family (GEMV, matrix-core GEMV, both GEMMs, k-split).  The padding of C must come back untouched."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(1000 + case)
+    tokens = int(rng.choice([1, 2, 3, 5, 9, 16, 17, 40, 48, 63, 64, 65, 100, 129, 200, 260]))
+    n_out = int(rng.choice([16, 40, 64, 250, 256, 300, 512, 1000]))
+    K = int(rng.choice([64, 128, 192, 448, 1024, 2048]) if case % 3 else rng.choice([16, 48, 80, 272, 1040]))
+    if tokens * n_out * K > 6e7:
+        K = 128
+    w_type = oracle.E5M2 if case % 2 else oracle.E4M3
+    pad_w, pad_x, pad_c = int(rng.choice([0, 16, 64])), int(rng.choice([0, 8, 24])), int(rng.choice([0, 4, 5, 12]))
+    ldw, ldx = K + pad_w, K + pad_x
+    scale = float(rng.choice([1.0, 0.37]))
+    alpha, beta = float(rng.choice([1.0, 0.5])), float(rng.choice([0.0, 0.0, -1.5]))
+    enc = oracle.encode_e5m2_rne if w_type == oracle.E5M2 else oracle.encode_e4m3_rne
+    W = np.full((n_out, ldw), 0x7F, dtype=np.uint8)                         # NaN code in both FP8 formats
+    W[:, :K] = enc((rng.standard_normal((n_out, K)) * 0.02 / scale).astype(np.float32))
+    X = np.full((tokens, ldx), 0x7FC0, dtype=np.uint16)                     # BF16 NaN
+    X[:, :K] = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
+    weight_is_a = bool(case % 4 < 2)
+    if weight_is_a:                                                          # C is [tokens][ldc >= n_out]
+        M, N, ldc = n_out, tokens, n_out + pad_c
+        args = lambda a, b: (1, 0, M, N, K, alpha, a, w_type, ldw, scale, b, oracle.BF16, ldx, 1.0, beta)
+        A, B = W, X
+        C0 = oracle.f32_to_bf16(rng.standard_normal((tokens, ldc)).astype(np.float32))
+        rows, cols = tokens, n_out
+    else:                                                                    # C is [n_out][ldc >= tokens]
+        M, N, ldc = tokens, n_out, tokens + pad_c
+        args = lambda a, b: (1, 0, M, N, K, alpha, a, oracle.BF16, ldx, 1.0, b, w_type, ldw, scale, beta)
+        A, B = X, W
+        C0 = oracle.f32_to_bf16(rng.standard_normal((n_out, ldc)).astype(np.float32))
+        rows, cols = n_out, tokens
+    want = C0.copy()
+    assert oracle.quant_gemm(*args(A, B), want, ldc) == 0
+    Ad, Bd, Cd = to_dev(torch, dev, A), to_dev(torch, dev, B), to_dev(torch, dev, C0)
+    assert lib.quant_gemm(*args(Ad.data_ptr(), Bd.data_ptr()), Cd.data_ptr(), oracle.BF16, ldc) == 0
+    kernel = lib.last_kernel()
+    got = from_dev(Cd, np.uint16).reshape(rows, ldc)
+    assert np.array_equal(got[:, cols:], C0[:, cols:]), f"{kernel}: padding of C was written"
+    g, w = bf16_f64(oracle, got[:, :cols]), bf16_f64(oracle, want[:, :cols])
+    assert np.isfinite(g).all(), f"{kernel}: padding leaked into the result"
+    assert np.abs(g - w).max() <= 2.0 ** -7 * np.abs(w).max() + 1e-6, (kernel, tokens, n_out, K, ldw, ldx, ldc, weight_is_a)
+
+
 def test_fp4_weight_as_B_with_block_scales(gpu, pkg, oracle):
     torch, dev, lib = gpu
     n_out, tokens, K = 64, 3, 128
