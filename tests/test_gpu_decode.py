@@ -234,10 +234,11 @@ def test_attention_decode_matches_the_oracle(gpu, oracle, dec, n_q, n_kv, t_kv):
     assert lib.c.hip_attention_decode_bf16(*args, ws_bytes, 3 * n_kv, n_kv, 128, t_kv, ctypes.c_void_p(pd.data_ptr())) == -1
 
 
-@pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 300), (2, 2, 130)])
+@pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 300), (2, 2, 130), (4, 2, 6000)])
 def test_fused_attention_appends_and_attends(gpu, oracle, dec, n_q, n_kv, t_kv):
     """q/k norm + RoPE + cache append + attention in two launches: cache rows as the oracle's, outputs
-    within a few BF16 ulps (the probabilities are not rounded to BF16 on this path)."""
+    within a few BF16 ulps (the probabilities are not rounded to BF16 on this path).  The 6000-row cache has
+    94 blocks, more than the merge kernel requests up front, and its workspace starts out as NaN patterns."""
     torch, dev, lib = gpu
     rng = np.random.default_rng(5)
     cfg = dec.DecodeConfig(n_q=n_q, n_kv=n_kv, t_kv=t_kv)
@@ -251,10 +252,10 @@ def test_fused_attention_appends_and_attends(gpu, oracle, dec, n_q, n_kv, t_kv):
     kn = torch.full((n_kv * t_kv * 128,), -1, dtype=torch.int16, device=dev)
     vn = torch.full((n_kv * t_kv * 128,), 0x7FC1, dtype=torch.int16, device=dev)
     ws_bytes = lib.c.hip_attention_decode_workspace_bytes(n_q, n_kv, t_kv)
-    ws = torch.full((ws_bytes,), 0xA5, dtype=torch.uint8, device=dev)
+    ws = torch.full((ws_bytes,), 0xFF if t_kv > 4096 else 0xA5, dtype=torch.uint8, device=dev)
     consts = [to_dev(torch, dev, a) for a in (qw, kw, cos, sin)]
     k_ref, v_ref = dec.f(kc).copy(), dec.f(vc).copy()
-    for pos in (0, 1, 127, 128, 129, t_kv - 1):
+    for pos in ((0, 4095, 4096, 4160, t_kv - 1) if t_kv > 4096 else (0, 1, 127, 128, 129, t_kv - 1)):
         q = oracle.f32_to_bf16((2 * rng.standard_normal((n_q, 128))).astype(np.float32))
         k = oracle.f32_to_bf16((2 * rng.standard_normal((n_kv, 128))).astype(np.float32))
         v = oracle.f32_to_bf16(rng.standard_normal((n_kv, 128)).astype(np.float32))
