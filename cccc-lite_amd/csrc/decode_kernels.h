@@ -948,6 +948,7 @@ static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const 
     const float2* st = stats + (size_t)qh * n_blocks;
 
     const int pos = *d_pos;
+    const float2 mine = st[min(lane, n_blocks - 1)];    // every wave: block `lane` (used when no more than 64 blocks are live)
     float2 sb[ATT_MAX_BLOCKS / 256];
 #pragma unroll
     for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++) { sb[i] = st[min((int)threadIdx.x + i * 256, n_blocks - 1)]; }
@@ -957,39 +958,56 @@ static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const 
 
     if (pos < 0 || pos >= t_kv) { return; }
     const int n_active = pos / ATT_KEYS + 1;
-    float m = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
+    float total = 0.0f, inv;
+    if (n_active <= 64)
     {
-        if ((int)threadIdx.x + i * 256 < n_active) { m = fmaxf(m, sb[i].x); }
-    }
-    m = wave_max(m);
-    if (lane == 0) { red[wave] = m; }
-    __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    float l = 0.0f;
+        // Up to 64 blocks: every wave holds one block's statistics per lane and works out the weights for
+        // itself (the same reductions in the same order as below, whose other three wave sums are zero), so
+        // nothing is exchanged before the final sum over the four waves.
+        const bool live = lane < n_active;
+        const float m = wave_max(live ? mine.x : -INFINITY);
+        const float e = live ? expf(mine.x - m) : 0.0f;
+        const float l = wave_sum(live ? mine.y * e : 0.0f);
+        inv = l > 0.0f ? 1.0f / l : 0.0f;
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
-    {
-        const int b = threadIdx.x + i * 256;
-        if (b < n_active)
+        for (int j = 0; j < PRE; j++)
         {
-            const float e = expf(sb[i].x - m);
-            w_lds[b] = e;
-            l += sb[i].y * e;
+            const int b = wave + 4 * j;
+            const float w = __shfl(e, b);
+            if (b < n_active) { total = fmaf(pre[j], w, total); }
         }
     }
-    l = block_sum<256>(l, red);                     // its barrier publishes w_lds
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    float total = 0.0f;
-#pragma unroll
-    for (int j = 0; j < PRE; j++)
+    else
     {
-        const int b = wave + 4 * j;
-        if (b < n_active) { total = fmaf(pre[j], w_lds[b], total); }
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
+        {
+            if ((int)threadIdx.x + i * 256 < n_active) { m = fmaxf(m, sb[i].x); }
+        }
+        m = wave_max(m);
+        if (lane == 0) { red[wave] = m; }
+        __syncthreads();
+        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        __syncthreads();
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++)
+        {
+            const int b = threadIdx.x + i * 256;
+            if (b < n_active)
+            {
+                const float e = expf(sb[i].x - m);
+                w_lds[b] = e;
+                l += sb[i].y * e;
+            }
+        }
+        l = block_sum<256>(l, red);                     // its barrier publishes w_lds
+        inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+        for (int j = 0; j < PRE; j++) { total = fmaf(pre[j], w_lds[wave + 4 * j], total); }
+        for (int b = wave + 4 * PRE; b < n_active; b += 4) { total = fmaf(partial[(size_t)b * n_out + o], w_lds[b], total); }
     }
-    for (int b = wave + 4 * PRE; b < n_active; b += 4) { total = fmaf(partial[(size_t)b * n_out + o], w_lds[b], total); }
     part[wave][lane] = total;
     __syncthreads();
     if (wave == 0 && blockIdx.x * 64 + lane < n_out) { y[o] = (uint16_t)f32_to_bf16_bits((((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]) * inv); }
