@@ -142,7 +142,14 @@ __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const Sta
     }
     if (a.norm_w)
     {
-        const float total = block_sum<THREADS>(sumsq, red);   // its barrier also publishes the raw tail chunks
+        // block sum in the order of block_sum(), without its closing barrier: `red` is not written again
+        // before the barrier at the end of this function.  The barrier also publishes the raw tail chunks.
+        sumsq = wave_sum(sumsq);
+        if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = sumsq; }
+        __syncthreads();
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; w++) { total += red[w]; }
         const float invstd = rsqrtf(total / (float)a.K + a.norm_eps);
 #pragma unroll
         for (int j = 0; j < STAGE_PRE; j++)
