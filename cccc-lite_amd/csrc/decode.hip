@@ -17,8 +17,15 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     const size_t lds = (size_t)((a.K + 1023) / 1024) * 2048;
     if (lds > 64 * 1024) { return -1; }
     const int cus = cu_count();
-    // long rows (K > 8192) and very tall weights want 8-wave workgroups, as the plain GEMV dispatch found
-    if (a.K > 8192 || n_groups >= cus * 64)
+    // Configurations chosen by whole-step time of the Qwen3-8B decode (the isolated kernel prefers 8 waves for long rows;
+    // inside the step two 4-wave workgroups per CU are 0.2 us per launch faster).
+    if (a.K > 8192 && n_groups < cus * 64)
+    {
+        const int want = (n_groups + 3) / 4;
+        gemv8_fused_kernel<WT, 4, 4, SCALED><<<want < cus * 2 ? want : cus * 2, 256, lds, stream()>>>(a);
+    }
+    // very tall weights want 8-wave workgroups, as the plain GEMV dispatch found
+    else if (n_groups >= cus * 64)
     {
         const int want = (n_groups + 7) / 8;
         gemv8_fused_kernel<WT, 4, 8, SCALED><<<want < cus * 2 ? want : cus * 2, 512, lds, stream()>>>(a);
