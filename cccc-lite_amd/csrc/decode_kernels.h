@@ -770,16 +770,32 @@ static __global__ __launch_bounds__(256) void attn_combine_kernel(const float* _
 //   waves 0..G-1 normalise and rotate the G query heads of this KV head; the block holding row *d_pos
 //   also normalises / rotates k, appends k and v to the caches, and uses them from LDS;
 //   stats[qh][block] = (max, sum expf(s - max)), partial[block][qh][128] = sum expf(s_t - max) v_t.
-__device__ __forceinline__ void norm_rope_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
-                                               const uint16_t* __restrict__ sin_row, float eps, int lane, float& out_l, float& out_r)
+struct HeadLoads
 {
-    const float xl = bf16_bits_to_f32(src[lane]), xr = bf16_bits_to_f32(src[lane + 64]);
-    const float c = bf16_bits_to_f32(cos_row[lane]), sn = bf16_bits_to_f32(sin_row[lane]);
-    const float wl = bf16_bits_to_f32(nw[lane]), wr = bf16_bits_to_f32(nw[lane + 64]);
+    uint16_t xl, xr, c, sn, wl, wr;       // lane's two elements of the head, its cos / sin, the two norm weights
+};
+
+__device__ __forceinline__ HeadLoads load_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
+                                               const uint16_t* __restrict__ sin_row, int lane)
+{
+    return HeadLoads{ src[lane], src[lane + 64], cos_row[lane], sin_row[lane], nw[lane], nw[lane + 64] };
+}
+
+__device__ __forceinline__ void norm_rope_finish(const HeadLoads& h, float eps, float& out_l, float& out_r)
+{
+    const float xl = bf16_bits_to_f32(h.xl), xr = bf16_bits_to_f32(h.xr);
+    const float c = bf16_bits_to_f32(h.c), sn = bf16_bits_to_f32(h.sn);
+    const float wl = bf16_bits_to_f32(h.wl), wr = bf16_bits_to_f32(h.wr);
     const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
     const float nl = bf16_round(xl * invstd * wl), nr = bf16_round(xr * invstd * wr);
     out_l = bf16_round(nl * c - nr * sn);
     out_r = bf16_round(nr * c + nl * sn);
+}
+
+__device__ __forceinline__ void norm_rope_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
+                                               const uint16_t* __restrict__ sin_row, float eps, int lane, float& out_l, float& out_r)
+{
+    norm_rope_finish(load_head(src, nw, cos_row, sin_row, lane), eps, out_l, out_r);
 }
 
 template <int G>
@@ -803,20 +819,29 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     const bool has_new = pos < t0 + ATT_KEYS;       // this block holds the row being appended
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15, key_in_wave = lane >> 4;
+    const uint16_t* cos_row = cos_tab + (size_t)pos * 64;
+    const uint16_t* sin_row = sin_tab + (size_t)pos * 64;
+    // the query head's few bytes are requested before the cache rows, and the key rows before the value rows:
+    // loads return in the order they were issued
+    HeadLoads hq{};
+    if (wave < G) { hq = load_head(q + (size_t)(kvh * G + wave) * 128, q_norm_w, cos_row, sin_row, lane); }
     u32x4 kraw[ATT_ITS], vraw[ATT_ITS];
 #pragma unroll
     for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end, and row pos itself, are replaced or discarded below
         kraw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+    }
+#pragma unroll
+    for (int it = 0; it < ATT_ITS; it++)
+    {
+        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);
         vraw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
     }
-    const uint16_t* cos_row = cos_tab + (size_t)pos * 64;
-    const uint16_t* sin_row = sin_tab + (size_t)pos * 64;
     if (wave < G)
     {
         float l, r;
-        norm_rope_head(q + (size_t)(kvh * G + wave) * 128, q_norm_w, cos_row, sin_row, eps, lane, l, r);
+        norm_rope_finish(hq, eps, l, r);
         q_lds[wave][lane] = l;
         q_lds[wave][lane + 64] = r;
     }
