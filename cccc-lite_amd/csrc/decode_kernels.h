@@ -808,8 +808,10 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 {
     __shared__ float acc_lds[16][G][128];   // [key slot in workgroup][head][dim]
     __shared__ float s_lds[G][ATT_KEYS];    // scores, then expf(s - block max)
-    __shared__ float q_lds[G][128];
-    __shared__ float k_new[128], v_new[128];
+    static_assert(ATT_KEYS == 64, "the score stage gives each of the four waves one 16-key matrix-core tile");
+    __shared__ __attribute__((aligned(16))) uint16_t q_lds[G][128];     // normalised, rotated query heads (BF16 values)
+    __shared__ __attribute__((aligned(16))) uint16_t k_new[128];
+    __shared__ float v_new[128];
     const int kvh = blockIdx.y, blk = blockIdx.x;
     const int pos = *d_pos;
     if (pos < 0 || pos >= t_kv) { return; }         // a position outside the cache: nothing to append, nothing to attend
@@ -825,12 +827,15 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     // loads return in the order they were issued
     HeadLoads hq{};
     if (wave < G) { hq = load_head(q + (size_t)(kvh * G + wave) * 128, q_norm_w, cos_row, sin_row, lane); }
-    u32x4 kraw[ATT_ITS], vraw[ATT_ITS];
-#pragma unroll
-    for (int it = 0; it < ATT_ITS; it++)
+    // Keys in the layout of the matrix-core row operand: wave w owns keys 16 w .. 16 w + 15 of the block, lane
+    // (i = lane % 16, g = lane / 16) holds dims 32 c + 8 g .. + 7 of key i for c = 0..3.  Values as before: lane
+    // (sub, key_in_wave) holds dims 8 sub .. + 7 of key it * 16 + wave * 4 + key_in_wave.
+    u32x4 kraw[4], vraw[ATT_ITS];
+    const int key_row = wave * 16 + sub;                                         // this lane's key within the block
     {
-        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end, and row pos itself, are replaced or discarded below
-        kraw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+        const int t = min(t0 + key_row, n_keys - 1);                             // rows past the end, and row pos itself, are replaced or discarded below
+#pragma unroll
+        for (int c = 0; c < 4; c++) { kraw[c] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + c * 32 + key_in_wave * 8); }
     }
 #pragma unroll
     for (int it = 0; it < ATT_ITS; it++)
@@ -842,15 +847,15 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     {
         float l, r;
         norm_rope_finish(hq, eps, l, r);
-        q_lds[wave][lane] = l;
-        q_lds[wave][lane + 64] = r;
+        q_lds[wave][lane] = (uint16_t)f32_to_bf16_bits(l);
+        q_lds[wave][lane + 64] = (uint16_t)f32_to_bf16_bits(r);
     }
     if (has_new && wave == 3)
     {
         float l, r;
         norm_rope_head(k + (size_t)kvh * 128, k_norm_w, cos_row, sin_row, eps, lane, l, r);
-        k_new[lane] = l;
-        k_new[lane + 64] = r;
+        k_new[lane] = (uint16_t)f32_to_bf16_bits(l);
+        k_new[lane + 64] = (uint16_t)f32_to_bf16_bits(r);
         uint16_t* dst = k_cache + ((size_t)kvh * t_kv + pos) * 128;
         dst[lane] = (uint16_t)f32_to_bf16_bits(l);
         dst[lane + 64] = (uint16_t)f32_to_bf16_bits(r);
@@ -865,34 +870,27 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
         dst[lane + 64] = b;
     }
     __syncthreads();
-    float qv[G][8];
-#pragma unroll
-    for (int gq = 0; gq < G; gq++)
-#pragma unroll
-        for (int d = 0; d < 8; d++) { qv[gq][d] = q_lds[gq][sub * 8 + d]; }
-#pragma unroll
-    for (int it = 0; it < ATT_ITS; it++)
+    // scores[key][head] = K[16 keys x 128] . q^T[128 x heads]: four v_mfma_f32_16x16x32_bf16 per wave (the products of two
+    // BF16 values are exact in FP32); columns G..15 of the head operand are zero.  D: lane holds head lane % 16, keys 4 g .. 4 g + 3.
     {
-        const int kl = it * 16 + wave * 4 + key_in_wave;
-        const int t = t0 + kl;
-        float kf[8];
-        unpack8_bf16(kraw[it], kf);
-        if (t == pos)
-        {
+        f32x4 sc = { 0.0f, 0.0f, 0.0f, 0.0f };
 #pragma unroll
-            for (int d = 0; d < 8; d++) { kf[d] = k_new[sub * 8 + d]; }
+        for (int c = 0; c < 4; c++)
+        {
+            u32x4 kc = kraw[c];
+            if (t0 + key_row == pos) { kc = *(const u32x4*)&k_new[c * 32 + key_in_wave * 8]; }
+            u32x4 qc = { 0u, 0u, 0u, 0u };
+            if (sub < G) { qc = *(const u32x4*)&q_lds[sub][c * 32 + key_in_wave * 8]; }
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kc), __builtin_bit_cast(bf16x8, qc), sc, 0, 0, 0);
         }
-#pragma unroll
-        for (int gq = 0; gq < G; gq++)
+        if (sub < G)
         {
-            float dot = 0.0f;
 #pragma unroll
-            for (int d = 0; d < 8; d++) { dot = fmaf(kf[d], qv[gq][d], dot); }
-            dot += dpp_f32<0xB1>(dot);
-            dot += dpp_f32<0x4E>(dot);
-            dot += dpp_f32<0x141>(dot);
-            dot += dpp_f32<0x140>(dot);
-            if (sub == 0) { s_lds[gq][kl] = t < n_keys ? bf16_round(scale * dot) : -INFINITY; }
+            for (int v = 0; v < 4; v++)
+            {
+                const int kl = wave * 16 + key_in_wave * 4 + v;
+                s_lds[sub][kl] = t0 + kl < n_keys ? bf16_round(scale * sc[v]) : -INFINITY;
+            }
         }
     }
     __syncthreads();
