@@ -106,8 +106,9 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
  * of an FP8 weight W ([n_out][ldw], K contiguous, as loadQuantizedDirect uploads it) into `dst_tiled`
  * -- caller-owned device memory of hip_quant_tiled_size(...) bytes -- and remembers it under the key
  * `W`.  Later hip_quant_gemm calls whose weight pointer, type and shape match may use the tiled copy
- * (today: up to 16 tokens, except one or two tokens on weights under 8 MiB): the matrix-core GEMV wants
- * the 16 rows x 64 codes of one load instruction to be one contiguous KiB.
+ * (today: up to 16 tokens, except one or two tokens on weights under 8 MiB, and the GEMM of 48 tokens or
+ * more when K is a multiple of 64): the matrix-core kernels want the 16 rows x 64 codes of one load
+ * instruction to be one contiguous KiB.
  * Results agree with the row-major kernels up to the FP32 summation order.  hip_quant_weight_release forgets the key (before the
  * caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (FP4, K % 16 != 0, ...).
  */
