@@ -175,7 +175,10 @@ struct FusedRows
     int seg, row0, row1;
 };
 
-template <int WT, int U, int WAVES, bool SCALED>
+// DIRECT_X (no RMSNorm in front, K a multiple of 1024): the activation is not staged at all -- every lane requests
+// the 32 bytes of x it needs for a step together with the weights of that step (x is a few KiB and stays in
+// the CU's L1), so the kernel has no prologue, no LDS and no barrier.
+template <int WT, int U, int WAVES, bool SCALED, bool DIRECT_X = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLinearArgs a)
 {
     extern __shared__ u32x4 xs[];
@@ -209,7 +212,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         r.s1 = a.w_scale[sb];
         return r;
     };
-    auto request = [&](const FusedRows& r, int st0, u32x4* wa, u32x4* wb) {
+    u32x4 xa[DIRECT_X ? U : 1][2], xn[DIRECT_X ? U : 1][2];      // x of the current / next batch (DIRECT_X)
+    auto request = [&](const FusedRows& r, int st0, u32x4* wa, u32x4* wb, u32x4 (*xq)[2]) {
 #pragma unroll
         for (int u = 0; u < U; u++)
         {
@@ -217,6 +221,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
             const int k = (st0 + u) * 1024 + lane * 16;
             if (k < a.K)
             {
+                if constexpr (DIRECT_X)
+                {
+                    xq[u][0] = *(const u32x4*)(a.X + k);
+                    xq[u][1] = *(const u32x4*)(a.X + k + 8);
+                }
                 wa[u] = __builtin_nontemporal_load((const u32x4*)(r.w0 + k));
                 wb[u] = __builtin_nontemporal_load((const u32x4*)(r.w1 + k));
             }
@@ -227,13 +236,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
     FusedRows cur{}, nxt{};
     u32x4 wa[U], wb[U], na[U], nb[U];
     StagedActivation staged;
-    stage_issue<WAVES * 64>(a, staged);
+    if constexpr (!DIRECT_X) { stage_issue<WAVES * 64>(a, staged); }
     if (g < n_groups)
     {
         cur = locate(g);
-        request(cur, 0, wa, wb);
+        request(cur, 0, wa, wb, xa);
     }
-    stage_finish<WAVES * 64>(a, staged, xs, red);
+    if constexpr (!DIRECT_X) { stage_finish<WAVES * 64>(a, staged, xs, red); }
 
     float acc0 = 0.0f, acc1 = 0.0f;
     while (g < n_groups)
@@ -247,7 +256,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         if (ng < n_groups)
         {
             nxt = nbatch == 0 ? locate(ng) : cur;
-            request(nxt, nbatch * U, na, nb);
+            request(nxt, nbatch * U, na, nb, xn);
         }
 #pragma unroll
         for (int u = 0; u < U; u++)
@@ -255,8 +264,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
             const int st = batch * U + u;
             if (st < n_steps)
             {
-                const u32x4 x0 = xs[(st * 2 + 0) * 64 + lane];
-                const u32x4 x1 = xs[(st * 2 + 1) * 64 + lane];
+                const u32x4 x0 = DIRECT_X ? xa[u][0] : xs[(st * 2 + 0) * 64 + lane];
+                const u32x4 x1 = DIRECT_X ? xa[u][1] : xs[(st * 2 + 1) * 64 + lane];
 #pragma unroll
                 for (int d = 0; d < 4; d++)
                 {
@@ -307,6 +316,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         {
             wa[u] = na[u];
             wb[u] = nb[u];
+            if constexpr (DIRECT_X)
+            {
+                xa[u][0] = xn[u][0];
+                xa[u][1] = xn[u][1];
+            }
         }
     }
 }
