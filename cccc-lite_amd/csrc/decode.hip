@@ -17,14 +17,19 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     const size_t lds = (size_t)((a.K + 1023) / 1024) * 2048;
     if (lds > 64 * 1024) { return -1; }
     const int cus = cu_count();
-    // Configurations chosen by whole-step time of the Qwen3-8B decode (the isolated kernel prefers 8 waves for long rows;
-    // inside the step two 4-wave workgroups per CU are 0.2 us per launch faster).
-    const bool direct_x = !a.norm_w && a.K % 1024 == 0;
-    if (a.K > 8192 && n_groups < cus * 64)
+    // Configurations chosen by whole-step time of the Qwen3-8B decode, which resolves 0.05 us per launch (the kernels
+    // timed alone prefer other settings, e.g. 8 waves for long rows).
+    const int want4 = (n_groups + 3) / 4;
+    if (!a.norm_w && a.K % 1024 == 0 && n_groups < cus * 64)
     {
-        const int want = (n_groups + 3) / 4;
-        if (direct_x) { gemv8_fused_kernel<WT, 4, 4, SCALED, true><<<want < cus * 2 ? want : cus * 2, 256, 0, stream()>>>(a); }
-        else { gemv8_fused_kernel<WT, 4, 4, SCALED><<<want < cus * 2 ? want : cus * 2, 256, lds, stream()>>>(a); }
+        // nothing to normalise: x comes with the weights, no LDS.  Long rows in batches of 2 KiB per row, rows of up to
+        // 4 KiB in one request.
+        if (a.K > 4096) { gemv8_fused_kernel<WT, 2, 4, SCALED, true><<<want4 < cus * 4 ? want4 : cus * 4, 256, 0, stream()>>>(a); }
+        else { gemv8_fused_kernel<WT, 4, 4, SCALED, true><<<want4 < cus * 2 ? want4 : cus * 2, 256, 0, stream()>>>(a); }
+    }
+    else if (a.K > 8192 && n_groups < cus * 64)
+    {
+        gemv8_fused_kernel<WT, 4, 4, SCALED><<<want4 < cus * 2 ? want4 : cus * 2, 256, lds, stream()>>>(a);
     }
     // very tall weights want 8-wave workgroups, as the plain GEMV dispatch found
     else if (n_groups >= cus * 64)
@@ -35,14 +40,11 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     else if (a.K <= 4096)
     {
         // short rows: two batches of 2 KiB per row pair keep the next request ahead of the multiply (measured 5-10 % faster than one batch of 4)
-        const int want = (n_groups + 3) / 4;
-        if (direct_x) { gemv8_fused_kernel<WT, 2, 4, SCALED, true><<<want < cus * 4 ? want : cus * 4, 256, 0, stream()>>>(a); }
-        else { gemv8_fused_kernel<WT, 2, 4, SCALED><<<want < cus * 4 ? want : cus * 4, 256, lds, stream()>>>(a); }
+        gemv8_fused_kernel<WT, 2, 4, SCALED><<<want4 < cus * 4 ? want4 : cus * 4, 256, lds, stream()>>>(a);
     }
     else
     {
-        const int want = (n_groups + 3) / 4;
-        gemv8_fused_kernel<WT, 4, 4, SCALED><<<want < cus * 4 ? want : cus * 4, 256, lds, stream()>>>(a);
+        gemv8_fused_kernel<WT, 4, 4, SCALED><<<want4 < cus * 4 ? want4 : cus * 4, 256, lds, stream()>>>(a);
     }
     return finish("quant_linear_fused");
 }
