@@ -742,7 +742,7 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const uint16_t* __restrict
         float total = 0.0f;
 #pragma unroll
         for (int sl = 0; sl < 16; sl++) { total += acc_lds[sl][gq][d]; }
-        partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d] = total;
+        __builtin_nontemporal_store(total, &partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d]);      // read once, by the merge kernel
     }
 }
 
@@ -968,7 +968,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
         float total = 0.0f;
 #pragma unroll
         for (int sl = 0; sl < 16; sl++) { total += acc_lds[sl][gq][d]; }
-        partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d] = total;
+        __builtin_nontemporal_store(total, &partial[((size_t)blk * n_q + kvh * G + gq) * 128 + d]);      // read once, by the merge kernel
     }
 }
 
@@ -999,7 +999,7 @@ static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const 
     for (int i = 0; i < ATT_MAX_BLOCKS / 256; i++) { sb[i] = st[min((int)threadIdx.x + i * 256, n_blocks - 1)]; }
     float pre[PRE];
 #pragma unroll
-    for (int j = 0; j < PRE; j++) { pre[j] = partial[(size_t)min(wave + 4 * j, n_blocks - 1) * n_out + o]; }
+    for (int j = 0; j < PRE; j++) { pre[j] = __builtin_nontemporal_load(&partial[(size_t)min(wave + 4 * j, n_blocks - 1) * n_out + o]); }
 
     if (pos < 0 || pos >= t_kv) { return; }
     const int n_active = pos / ATT_KEYS + 1;
