@@ -258,7 +258,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // 256 output features; wave w owns features 64 w .. 64 w + 63 for all of the tokens.  Each lane
 // loads the 16 weight bytes it will feed to the matrix cores itself -- row (lane % 16) of a 16-row
 // block, bytes 16 (lane / 16) .. + 15 of the 64-byte k-tile -- and converts them in registers: the
-// low 8 bytes are its B operand of the first v_mfma_f32_16x16x32 of the k-tile and the high 8 bytes
+// low 8 bytes are its row operand of the first v_mfma_f32_16x16x32 of the k-tile and the high 8 bytes
 // that of the second.  The contraction does not care in which order k is visited as long as both
 // operands agree, so the token operand is read from LDS with the matching k assignment (chunk
 // 2 (lane / 16) + step of the row).  Only the activations are staged through LDS (one 128-byte row
