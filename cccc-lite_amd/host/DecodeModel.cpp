@@ -99,6 +99,12 @@ Matrix* DecodeModel::tensor(int layer, int which)
     return (which >= 0 && which <= W_DOWN) ? table[which] : nullptr;
 }
 
+Matrix* DecodeModel::activation(int which)
+{
+    Matrix* table[] = { x_.get(), r1_.get(), q_.get(), k_.get(), v_.get(), att_.get(), gated_.get() };
+    return (which >= 0 && which <= ACT_GATED) ? table[which] : nullptr;
+}
+
 int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale)
 {
     Matrix* m = tensor(layer, which);
@@ -177,6 +183,8 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
                                                           { L.w_gate.get(), "W_gate_" }, { L.w_up.get(), "W_up_" }, { L.w_down.get(), "W_down_" } };
         for (auto& [m, prefix] : plain) { if (rc == 0) { rc = load_plain(*m, prefix + n); } }
         for (auto& [m, prefix] : linear) { if (rc == 0) { rc = load_linear(*m, prefix + n); } }
+        // gate and up are decoded by one launch with one format
+        if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType()) { rc = fail("W_up_" + n, -3); }
     }
     return rc;
 }
@@ -233,13 +241,29 @@ int DecodeModel::step()
     {
         Layer& L = layers_[li];
         // 1. q, k, v = W_{q,k,v} rmsnorm(x): one launch, three weight segments
+        // (a descriptor carries one weight type: projections stored in different FP8 formats go out as three launches)
         hip_fused_linear qkv = linear_desc(*L.wq, q_out, c.hidden, x_->data(), q_->data());
-        qkv.n_segments = 3;
-        qkv.W[1] = L.wk->data(); qkv.n_out[1] = kv_out; qkv.w_scale[1] = L.wk->getQuantScale(); qkv.Y[1] = k_->data();
-        qkv.W[2] = L.wv->data(); qkv.n_out[2] = kv_out; qkv.w_scale[2] = L.wv->getQuantScale(); qkv.Y[2] = v_->data();
         qkv.norm_weight = L.rms_attn->data();
         qkv.norm_eps = c.eps;
-        rc = hip_quant_linear_fused(&qkv);
+        if (L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
+        {
+            qkv.n_segments = 3;
+            qkv.W[1] = L.wk->data(); qkv.n_out[1] = kv_out; qkv.w_scale[1] = L.wk->getQuantScale(); qkv.Y[1] = k_->data();
+            qkv.W[2] = L.wv->data(); qkv.n_out[2] = kv_out; qkv.w_scale[2] = L.wv->getQuantScale(); qkv.Y[2] = v_->data();
+            rc = hip_quant_linear_fused(&qkv);
+        }
+        else
+        {
+            rc = hip_quant_linear_fused(&qkv);
+            for (Matrix* w : { L.wk.get(), L.wv.get() })
+            {
+                if (rc != 0) { break; }
+                hip_fused_linear kv = linear_desc(*w, kv_out, c.hidden, x_->data(), w == L.wk.get() ? k_->data() : v_->data());
+                kv.norm_weight = L.rms_attn->data();
+                kv.norm_eps = c.eps;
+                rc = hip_quant_linear_fused(&kv);
+            }
+        }
         // 2-3. per-head q/k norm, RoPE, KV append and attention over the cache
         if (rc == 0 && !exact_attention_)
         {
@@ -265,6 +289,7 @@ int DecodeModel::step()
             rc = hip_quant_linear_fused(&o);
         }
         // 5. gated = silu(W_gate n) * (W_up n), n = rmsnorm(r1)
+        if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType()) { rc = -1; }    // the SwiGLU pair kernel decodes both with one format
         if (rc == 0)
         {
             hip_fused_linear gu = linear_desc(*L.w_gate, c.inter, c.hidden, r1_->data(), gated_->data());

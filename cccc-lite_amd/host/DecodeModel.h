@@ -32,8 +32,15 @@ public:
     DecodeModel(const DecodeConfig& cfg, GpuControl* gpu);
     ~DecodeModel();
 
+    // Intermediate BF16 vectors of the step in flight (what the last layer that ran left in them)
+    enum Activation
+    {
+        ACT_X = 0, ACT_R1, ACT_Q, ACT_K, ACT_V, ACT_ATT, ACT_GATED
+    };
+
     const DecodeConfig& config() const { return cfg_; }
     Matrix* tensor(int layer, int which);
+    Matrix* activation(int which);
 
     // Uploads file bytes: FP8 codes for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
     int setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale);

@@ -327,6 +327,12 @@ int cccc_decode_pos(void* m) { return ((DecodeModel*)m)->currentPos(); }
 
 int cccc_decode_logits(void* m, void* host, unsigned long long bytes) { return ((DecodeModel*)m)->logits().copyToHost(host, (size_t)bytes); }
 
+int cccc_decode_activation(void* m, int which, void* host, unsigned long long bytes)
+{
+    Matrix* a = ((DecodeModel*)m)->activation(which);
+    return a ? a->copyToHost(host, (size_t)bytes) : -1;
+}
+
 int cccc_decode_kv(void* m, int layer, int is_v, void* host, unsigned long long bytes)
 {
     DecodeModel* d = (DecodeModel*)m;

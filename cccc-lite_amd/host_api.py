@@ -52,6 +52,7 @@ class HostLibrary:
         L.cccc_decode_token.restype = i32; L.cccc_decode_token.argtypes = [vp]
         L.cccc_decode_pos.restype = i32; L.cccc_decode_pos.argtypes = [vp]
         L.cccc_decode_logits.restype = i32; L.cccc_decode_logits.argtypes = [vp, vp, u64]
+        L.cccc_decode_activation.restype = i32; L.cccc_decode_activation.argtypes = [vp, i32, vp, u64]
         L.cccc_decode_kv.restype = i32; L.cccc_decode_kv.argtypes = [vp, i32, i32, vp, u64]
         L.cccc_decode_cos_table.restype = i32; L.cccc_decode_cos_table.argtypes = [vp, vp, u64]
         L.cccc_decode_weight_bytes.restype = u64; L.cccc_decode_weight_bytes.argtypes = [vp]
@@ -289,6 +290,17 @@ class DecodeModel:
     def logits(self) -> np.ndarray:
         out = np.empty(self.cfg["vocab"], dtype=np.uint16)
         assert self.lib.c.cccc_decode_logits(self.handle, out.ctypes.data, out.nbytes) == 0
+        return out
+
+    ACTIVATIONS = {"x": 0, "r1": 1, "q": 2, "k": 3, "v": 4, "att": 5, "gated": 6}
+
+    def activation(self, name: str) -> np.ndarray:
+        """BF16 bits of an intermediate vector as the last layer that ran left it."""
+        c = self.cfg
+        n = {"x": c["hidden"], "r1": c["hidden"], "q": c["n_q"] * c["head_dim"], "k": c["n_kv"] * c["head_dim"],
+             "v": c["n_kv"] * c["head_dim"], "att": c["n_q"] * c["head_dim"], "gated": c["inter"]}[name]
+        out = np.empty(n, dtype=np.uint16)
+        assert self.lib.c.cccc_decode_activation(self.handle, self.ACTIVATIONS[name], out.ctypes.data, out.nbytes) == 0
         return out
 
     def kv(self, layer: int, is_v: bool) -> np.ndarray:

@@ -168,7 +168,11 @@ class DecodeOracle:
             self._deq[key] = o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape)
         return self._deq[key]
 
-    def step(self, token: int, pos: int, trace: dict | None = None):
+    def step(self, token: int, pos: int, trace: dict | None = None, logit_rows=None):
+        """One decode step.  `trace`, when given, receives the intermediate tensors of every layer
+        (keys suffixed with the layer index; layer 0 also under the bare names).  `logit_rows` limits
+        the lm_head to those output rows (a full-size vocabulary is then affordable); the returned
+        token is the arg-max over the rows computed."""
         c = self.cfg
         x = f(self.model["emb"][token])
         for li, L in enumerate(self.model["layers"]):
@@ -186,8 +190,13 @@ class DecodeOracle:
             x = r(r1 + linear(self.deq(li, "w_down"), gated))
             if trace is not None:
                 trace[f"x{li}"] = x.copy()
+                trace.update({f"xn{li}": xn, f"q{li}": q.copy(), f"att{li}": att.copy(), f"r1_{li}": r1, f"gated{li}": gated})
                 if li == 0:
                     trace.update(xn=xn, q=q.copy(), att=att.copy(), r1=r1, gated=gated)
         xf = rms_norm(x, f(self.model["rms_final"]), c.eps)
+        if logit_rows is not None:
+            W = self.model["lm_head"][np.asarray(logit_rows)]
+            logits = linear(o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape), xf)
+            return logits, int(np.asarray(logit_rows)[int(np.argmax(logits))])
         logits = linear(self.deq(None, "lm_head"), xf)
         return logits, int(np.argmax(logits))

@@ -1,0 +1,318 @@
+"""Parity at the benchmark's full sizes, on the kernels the benchmark launches: the tiled matrix-core
+GEMV at the five Qwen3-8B shapes, the FP4 block-scale GEMV at the Llama-3.1-8B shapes, the fused decode
+linears at their Qwen3-8B instantiations and a whole decode step at Qwen3-8B widths with a filled KV
+cache.  Weights are drawn on the GPU (a full-size weight takes seconds to draw on the host); the oracle
+sees the very bytes the kernels read, downloaded for the sampled rows."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import check_bf16_close, check_rows, from_dev, to_dev
+
+pytestmark = pytest.mark.gpu
+
+BF16, E4M3, E5M2, FP4 = 3, 4, 5, 6
+QWEN_SHAPES = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096), (4096, 151936)]      # (K, n_out)
+LLAMA_SHAPES = [(4096, 14336), (14336, 4096), (4096, 128256)]
+
+
+@pytest.fixture(scope="module")
+def dec():
+    from oracle import decode_oracle
+    return decode_oracle
+
+
+def bf16_f64(oracle, bits):
+    return oracle.bf16_to_f32(bits).astype(np.float64)
+
+
+def draw_e5m2(torch, dev, gen, n_out, K):
+    """uint8 E5M2 codes [n_out, K] on the device: N(0, 0.02) -> BF16 -> FP8 (round to nearest)."""
+    out = torch.empty(n_out, K, dtype=torch.uint8, device=dev)
+    rows = max(1, (1 << 27) // K)
+    for r0 in range(0, n_out, rows):
+        r = min(rows, n_out - r0)
+        out[r0:r0 + r] = (torch.randn(r, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16).to(torch.float8_e5m2).view(torch.uint8)
+    return out
+
+
+def draw_bf16(torch, dev, gen, shape, mean=0.0, std=1.0):
+    return (torch.randn(*shape, device=dev, generator=gen) * std + mean).to(torch.bfloat16).view(torch.int16)
+
+
+def host_bits(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+# ------------------------------------------------------------------------------------------ FP8, tiled copy
+
+@pytest.mark.parametrize("K,n_out", QWEN_SHAPES)
+def test_tiled_gemv_at_the_qwen3_8b_shapes(gpu, pkg, oracle, K, n_out):
+    """hip_quant_gemm with the load-time tiled copy registered, 1 / 4 / 16 tokens: sampled rows against the
+    exact contraction, all-ones activations against the row sums of the decoded weight."""
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(K + n_out)
+    wd = draw_e5m2(torch, dev, gen, n_out, K)
+    td = torch.zeros(lib.tiled_size(E5M2, n_out, K), dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare(wd.data_ptr(), E5M2, n_out, K, K, td.data_ptr()) == 0
+    try:
+        rows = np.sort(np.random.default_rng(n_out).choice(n_out, size=257, replace=False))
+        W_rows = wd[torch.from_numpy(rows).to(dev)].cpu().numpy()
+        Wd_rows = oracle.dequant_fp8_to_bf16(W_rows, oracle.E5M2).reshape(W_rows.shape)
+        for tokens in (1, 4, 16):
+            X = pkg.synth.activations(n_out + tokens, tokens, K)
+            xd = to_dev(torch, dev, X)
+            yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+            assert lib.linear(wd.data_ptr(), E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
+            small = tokens <= 2 and n_out * K < (8 << 20)               # one or two tokens on a few MiB stay on the pipelined dot2 kernel
+            assert lib.last_kernel() == ("gemv_dot2" if small else "gemv_mfma_tiled")
+            out = from_dev(yd, np.uint16)
+            assert not out[tokens * n_out:].any(), "wrote past the end"
+            y = out[:tokens * n_out].reshape(tokens, n_out)
+            want = oracle.linear_exact(Wd_rows, X)
+            check_rows(bf16_f64(oracle, y[:, rows]), want, f"tiled {n_out}x{K} M={tokens}")
+            check_bf16_close(y[:, rows], want, "tiled", slack_ulp=1.0, abs_floor=2e-5)
+        ones = np.full((1, K), 0x3F80, dtype=np.uint16)
+        yd = torch.zeros(n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(wd.data_ptr(), E5M2, to_dev(torch, dev, ones).data_ptr(), yd.data_ptr(), n_out, 1, K) == 0
+        sums = oracle.decode_table(oracle.E5M2).astype(np.float64)[W_rows].sum(axis=1)
+        got = bf16_f64(oracle, from_dev(yd, np.uint16))[rows]
+        assert np.all(np.abs(got - sums) <= 2.0 ** -8 * np.abs(sums) + 1e-5)
+    finally:
+        assert lib.weight_release(wd.data_ptr()) == 0
+
+
+# ------------------------------------------------------------------------------------------ FP4
+
+FP4_BOUNDS = (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0)
+
+
+def pack_fp4_on_device(torch, w, block):
+    """The converter's packing (absmax / 6 -> E4M3 by round to nearest, codes from the unrounded 6 / absmax,
+    boundaries to the lower code, low nibble = even element) on a float32 device tensor [n_out, K]; the
+    test below checks it against the host packer on a slab before trusting it."""
+    n_out, K = w.shape
+    b = w.reshape(-1, block)
+    amax = b.abs().amax(dim=1)
+    live = amax > 1e-10
+    one = torch.ones_like(amax)
+    scales = torch.where(live, amax / 6.0, one)
+    fwd = torch.where(live, 6.0 / amax, one)
+    scaled = (b * fwd[:, None]).reshape(-1)
+    bounds = torch.tensor(FP4_BOUNDS, dtype=torch.float32, device=w.device)
+    code = torch.bucketize(scaled.abs(), bounds, right=False).to(torch.uint8) | ((scaled < 0).to(torch.uint8) << 3)
+    nib = (code[0::2] | (code[1::2] << 4)).reshape(n_out, K // 2)
+    sc = scales.to(torch.float8_e4m3fn).view(torch.uint8).reshape(n_out, K // block)
+    return nib, sc
+
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("K,n_out", LLAMA_SHAPES)
+def test_fp4_gemv_at_the_llama_8b_shapes(gpu, pkg, oracle, K, n_out, block):
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(K + n_out + block)
+    nib = torch.empty(n_out, K // 2, dtype=torch.uint8, device=dev)
+    sc = torch.empty(n_out, K // block, dtype=torch.uint8, device=dev)
+    slab = max(1, (1 << 26) // K)
+    for r0 in range(0, n_out, slab):
+        r = min(slab, n_out - r0)
+        w = (torch.randn(r, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16).to(torch.float32)
+        nib[r0:r0 + r], sc[r0:r0 + r] = pack_fp4_on_device(torch, w, block)
+        if r0 == 0:
+            want_nib, want_sc = pkg.synth.pack_fp4_blockscale(w[:64].cpu().numpy(), block)
+            assert np.array_equal(nib[:64].cpu().numpy().ravel(), want_nib) and np.array_equal(sc[:64].cpu().numpy().ravel(), want_sc)
+    rows = np.sort(np.random.default_rng(n_out + block).choice(n_out, size=257, replace=False))
+    ridx = torch.from_numpy(rows).to(dev)
+    nib_rows, sc_rows = nib[ridx].cpu().numpy(), sc[ridx].cpu().numpy()
+    Wd_rows = oracle.dequant_weight(nib_rows, oracle.FP4, len(rows), K, blk_sc=sc_rows, block=block)
+    for tokens in (1, 4):
+        X = pkg.synth.activations(n_out + tokens, tokens, K)
+        xd = to_dev(torch, dev, X)
+        yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+        assert lib.linear(nib.data_ptr(), FP4, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, blk_sc=sc.data_ptr(), block_size=block) == 0
+        kernel = lib.last_kernel()
+        assert kernel.startswith("gemv")
+        out = from_dev(yd, np.uint16)
+        assert not out[tokens * n_out:].any(), "wrote past the end"
+        y = out[:tokens * n_out].reshape(tokens, n_out)
+        want = oracle.linear_exact(Wd_rows, X)
+        check_rows(bf16_f64(oracle, y[:, rows]), want, f"{kernel} fp4 {n_out}x{K} M={tokens} block {block}")
+        check_bf16_close(y[:, rows], want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    ones = np.full((1, K), 0x3F80, dtype=np.uint16)
+    yd = torch.zeros(n_out, dtype=torch.int16, device=dev)
+    assert lib.linear(nib.data_ptr(), FP4, to_dev(torch, dev, ones).data_ptr(), yd.data_ptr(), n_out, 1, K, blk_sc=sc.data_ptr(), block_size=block) == 0
+    sums = bf16_f64(oracle, Wd_rows).sum(axis=1)
+    got = bf16_f64(oracle, from_dev(yd, np.uint16))[rows]
+    assert np.all(np.abs(got - sums) <= 2.0 ** -8 * np.abs(sums) + 1e-5)
+
+
+# ------------------------------------------------------------------------------------------ fused decode linears
+
+def ulp_close(got_bits, want_vals, ulps=1.0, floor=1e-6):
+    got = (got_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    want = np.asarray(want_vals, dtype=np.float64)
+    return np.abs(got - want) <= ulps * np.maximum(np.abs(want), 2.0 ** -120) * 2.0 ** -8 + floor
+
+
+@pytest.mark.parametrize("case", ["o", "down", "qkv", "gate_up", "lm_head"])
+def test_fused_linears_at_their_qwen3_8b_instantiations(gpu, pkg, oracle, dec, case):
+    """hip_quant_linear_fused with the arguments DecodeModel::step passes at Qwen3-8B widths: unscaled
+    E5M2 weights, o and down without a norm (activation requested with the weights) and with the residual,
+    q/k/v as three segments behind an RMSNorm, the SwiGLU pair behind an RMSNorm, lm_head behind the final
+    norm on its tiled copy."""
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(len(case) * 7919)
+    K = {"o": 4096, "down": 12288, "qkv": 4096, "gate_up": 4096, "lm_head": 4096}[case]
+    n_outs = {"o": [4096], "down": [4096], "qkv": [4096, 1024, 1024], "gate_up": [12288, 12288], "lm_head": [151936]}[case]
+    norm = case in ("qkv", "gate_up", "lm_head")
+    wds = [draw_e5m2(torch, dev, gen, n, K) for n in n_outs]
+    x_std = 0.3 if case == "down" else 1.0
+    xd = draw_bf16(torch, dev, gen, (K,), std=x_std)
+    nwd = draw_bf16(torch, dev, gen, (K,), mean=1.0, std=0.1)
+    x, nw = dec.f(host_bits(xd)), dec.f(host_bits(nwd))
+    xin = dec.rms_norm(x, nw, 1e-6) if norm else x
+    tiled = None
+    if case == "lm_head":
+        tiled = torch.zeros(lib.tiled_size(E5M2, n_outs[0], K), dtype=torch.uint8, device=dev)
+        assert lib.weight_prepare(wds[0].data_ptr(), E5M2, n_outs[0], K, K, tiled.data_ptr()) == 0
+
+    def sampled(w, n, count=512):
+        rows = np.sort(np.random.default_rng(n).choice(n, size=min(count, n), replace=False))
+        codes = w[torch.from_numpy(rows).to(dev)].cpu().numpy()
+        return rows, dec.linear(oracle.dequant_fp8_to_bf16(codes, oracle.E5M2).reshape(codes.shape), xin)
+
+    try:
+        if case == "gate_up":
+            y = torch.zeros(n_outs[0] + 8, dtype=torch.int16, device=dev)
+            d = pkg.capi.make_fused_linear(E5M2, K, [w.data_ptr() for w in wds], n_outs, [y.data_ptr(), None], xd.data_ptr(),
+                                           norm_weight=nwd.data_ptr(), norm_eps=1e-6, pair=True)
+            assert lib.quant_linear_fused(d) == 0 and lib.last_kernel() == "gemv_fused"
+            out = from_dev(y, np.uint16)
+            assert not out[n_outs[0]:].any()
+            rows, gate = sampled(wds[0], n_outs[0], 1024)
+            _, up = sampled(wds[1], n_outs[0], 1024)
+            want = dec.silu_mul(gate, up)
+            assert ulp_close(out[rows], want, ulps=3.0, floor=1e-4).all()
+            assert (out[rows] == oracle.f32_to_bf16(want)).mean() > 0.97
+            return
+        ys = [torch.zeros(n + 8, dtype=torch.int16, device=dev) for n in n_outs]
+        resd = draw_bf16(torch, dev, gen, (n_outs[0],)) if case in ("o", "down") else None
+        d = pkg.capi.make_fused_linear(E5M2, K, [w.data_ptr() for w in wds], n_outs, [y.data_ptr() for y in ys], xd.data_ptr(),
+                                       norm_weight=nwd.data_ptr() if norm else None, norm_eps=1e-6,
+                                       residual=resd.data_ptr() if resd is not None else None)
+        assert lib.quant_linear_fused(d) == 0
+        assert lib.last_kernel() == ("gemv_fused_mfma" if case == "lm_head" else "gemv_fused")
+        for s, n in enumerate(n_outs):
+            out = from_dev(ys[s], np.uint16)
+            assert not out[n:].any()
+            rows, lin = sampled(wds[s], n)
+            if resd is not None:
+                res = dec.f(host_bits(resd))[rows]
+                want = dec.r(lin + res)
+                tol = np.maximum(np.maximum(np.abs(lin), np.abs(res)), np.abs(want)) * 2.0 ** -7 + 1e-4
+                assert (np.abs(dec.f(out[rows]).astype(np.float64) - want) <= tol).all()
+                assert (out[rows] == oracle.f32_to_bf16(want)).mean() > 0.98
+            else:
+                assert ulp_close(out[rows], lin, ulps=1.0, floor=2e-5).all(), s
+    finally:
+        if tiled is not None:
+            assert lib.weight_release(wds[0].data_ptr()) == 0
+
+
+# ------------------------------------------------------------------------------------------ decode step
+
+@pytest.mark.parametrize("exact_attention", [False, True])
+def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
+    """Two layers of the Qwen3-8B shape (hidden 4096, 32 / 8 heads, intermediate 12288, vocabulary 151936,
+    4096 cache rows) with caches already holding 4090 positions, two steps from position 4090: every launch
+    configuration the benchmark's 36-layer model uses is reached.  The last layer's intermediate vectors, the
+    appended cache rows of both layers and 4096 sampled logits against the CPU oracle on the same bytes."""
+    torch, dev, lib = gpu
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=12288, vocab=151936, t_kv=4096)
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    model.set_exact_attention(exact_attention)
+    gen = torch.Generator(device=dev).manual_seed(8)
+    copy = lambda src, dst, nbytes: lib.convert(src.data_ptr(), BF16, dst, BF16, nbytes, 1.0)      # same type: a byte copy on the device
+
+    weights = {"layers": []}
+    lin_shapes = {"wq": (cfg.q_out, cfg.hidden), "wk": (cfg.kv_out, cfg.hidden), "wv": (cfg.kv_out, cfg.hidden), "wo": (cfg.hidden, cfg.q_out),
+                  "w_gate": (cfg.inter, cfg.hidden), "w_up": (cfg.inter, cfg.hidden), "w_down": (cfg.hidden, cfg.inter)}
+    norm_sizes = {"rms_attn": cfg.hidden, "rms_ffn": cfg.hidden, "q_norm": 128, "k_norm": 128}
+    start = 4090
+    k_host = np.zeros((cfg.layers, cfg.n_kv, cfg.t_kv, 128), dtype=np.float32)
+    v_host = np.zeros_like(k_host)
+    for li in range(cfg.layers):
+        L = {}
+        for name, (n_out, K) in lin_shapes.items():
+            w = draw_e5m2(torch, dev, gen, n_out, K)
+            assert copy(w, model.tensor_ptr(li, name), n_out * K) == 0
+            L[name] = w.cpu().numpy()
+        for name, n in norm_sizes.items():
+            v = draw_bf16(torch, dev, gen, (n,), mean=1.0, std=0.1)
+            assert copy(v, model.tensor_ptr(li, name), n * 2) == 0
+            L[name] = host_bits(v)
+        weights["layers"].append(L)
+        for is_v, dst in ((False, k_host), (True, v_host)):
+            c = draw_bf16(torch, dev, gen, (cfg.n_kv, cfg.t_kv, 128))
+            c[:, start:] = 0x7FC1                                    # rows not written yet hold NaN patterns
+            assert copy(c, model.kv_ptr(li, is_v), c.numel() * 2) == 0
+            dst[li] = dec.f(host_bits(c))
+    lm = draw_e5m2(torch, dev, gen, cfg.vocab, cfg.hidden)
+    assert copy(lm, model.tensor_ptr(0, "lm_head"), cfg.vocab * cfg.hidden) == 0
+    assert model.prepare_tiled(0, "lm_head")
+    fin = draw_bf16(torch, dev, gen, (cfg.hidden,), mean=1.0, std=0.1)
+    assert copy(fin, model.tensor_ptr(0, "rms_final"), cfg.hidden * 2) == 0
+    emb_rows = {}
+    emb = draw_bf16(torch, dev, gen, (cfg.vocab, cfg.hidden))
+    assert copy(emb, model.tensor_ptr(0, "emb"), cfg.vocab * cfg.hidden * 2) == 0
+    torch.cuda.synchronize()
+
+    logit_rows = np.sort(np.random.default_rng(3).choice(cfg.vocab, size=4096, replace=False))
+    lm_rows = lm[torch.from_numpy(logit_rows).to(dev)].cpu().numpy()
+
+    class Rows:
+        """Stands in for a [vocab, hidden] array of which only a few rows were downloaded."""
+
+        def __init__(self, fetch):
+            self.fetch = fetch
+
+        def __getitem__(self, i):
+            return self.fetch(i)
+
+    weights["emb"] = Rows(lambda t: host_bits(emb[int(t)]))
+    weights["rms_final"] = host_bits(fin)
+    weights["lm_head"] = Rows(lambda idx: lm_rows[np.searchsorted(logit_rows, np.asarray(idx))])
+    del emb_rows
+    orc = dec.DecodeOracle(cfg, weights)
+    orc.k[:], orc.v[:] = k_host, v_host
+    orc.k[:, :, start:], orc.v[:, :, start:] = 0.0, 0.0              # the oracle masks them; NaN * 0 would poison its matrix products
+
+    token = 1234
+    for pos in (start, start + 1):
+        model.reset(token, pos)
+        got_token = model.step()
+        assert model.pos == pos + 1
+        trace = {}
+        want_logits, _ = orc.step(token, pos, trace=trace, logit_rows=logit_rows)
+        last = cfg.layers - 1
+        for name, want in (("att", trace[f"att{last}"]), ("r1", trace[f"r1_{last}"]), ("gated", trace[f"gated{last}"]), ("x", trace[f"x{last}"])):
+            got = dec.f(model.activation(name))
+            assert np.isfinite(got).all(), name
+            err = np.linalg.norm(got - want.reshape(-1)) / np.linalg.norm(want)
+            assert err < 1e-2, (pos, name, err)
+        for li in range(cfg.layers):
+            gk, gv = dec.f(model.kv(li, False)[:, pos]), dec.f(model.kv(li, True)[:, pos])
+            tol = 2e-3 if li == 0 else 1e-2                          # layer 0 sees identical inputs
+            assert np.linalg.norm(gk - orc.k[li, :, pos]) <= tol * np.linalg.norm(orc.k[li, :, pos]), (pos, li)
+            assert np.linalg.norm(gv - orc.v[li, :, pos]) <= tol * np.linalg.norm(orc.v[li, :, pos]), (pos, li)
+        logits = model.logits()
+        got = dec.f(logits[logit_rows])
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        assert np.abs(got - want_logits).max() <= 2e-2 * np.abs(want_logits).max()
+        # greedy pick = lowest index of the largest logit the kernel itself produced
+        all_logits = dec.f(logits)
+        assert got_token == int(np.argmax(all_logits))
+        token = got_token

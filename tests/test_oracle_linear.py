@@ -104,6 +104,46 @@ def test_converter_packer_by_hand(oracle, pkg):
     assert oracle.unpack_fp4(kn, 16).tolist()[:10] == [7, 1, 2, 3, 4, 5, 6, 7, 9, 15]
 
 
+def test_on_the_fly_fp4_quantiser_scale_byte_by_hand(oracle):
+    """The scale byte of the on-the-fly quantiser (cccc-cuda/cuda_functions.cu:2896-2923) is absmax / 6
+    through the TRUNCATING E4M3 encoder (:2383-2412), worked out by hand below; the cases marked (*) are
+    the ones where round-to-nearest would give the next byte up."""
+    step = 2.0 ** -9                                              # E4M3 subnormal spacing
+    cases = [
+        # absmax, absmax / 6,           byte
+        (0.0, "scale 1.0 for an all-zero block", 0x38),
+        (6.0, "1.0 = 2^0: e = 7, m = 0", 0x38),
+        (1.5, "0.25 = 2^-2: e = 5, m = 0", 0x28),
+        (10.5, "1.75 = 1.110b: e = 7, m = 6", 0x3E),
+        (11.0, "1.8333 = 1.110101..b: m = 6 (*) nearest is m = 7", 0x3E),
+        (0.021, "0.0035 = 1.79 subnormal steps: 1 (*) nearest is 2", 0x01),
+        (0.06, "0.01 = 5.12 subnormal steps: 5", 0x05),
+        (0.0115, "0.00192 = 0.98 subnormal steps: 0 (*) nearest is 1", 0x00),
+        (6 * 7 * step, "7 subnormal steps exactly", 0x07),
+        (6 * 2.0 ** -6, "smallest normal 2^-6: e = 1, m = 0", 0x08),
+        (6 * 448.0, "largest finite 448: e = 15, m = 6", 0x7E),
+        (6 * 1000.0, "beyond the range: saturates at 448", 0x7E),
+    ]
+    for amax, why, byte in cases:
+        block = np.zeros(16, dtype=np.float32)
+        block[5], block[9] = -amax, amax / 2
+        nib, sc = oracle.quantize_fp4_blockscale_kernel(block, 16)
+        assert sc.tolist() == [byte], (amax, why, hex(int(sc[0])))
+        if amax > 0:
+            # codes come from 6 / absmax: the extreme element is -6 (code 15), half of it 3 (code 5)
+            codes = oracle.unpack_fp4(nib, 16).tolist()
+            assert codes[5] == 15 and codes[9] == 5 and sum(codes) == 20, (amax, codes)
+    # the same bytes through round-to-nearest differ exactly at the marked cases
+    rne = oracle.encode_e4m3_rne(np.array([11.0 / 6, 0.021 / 6, 0.0115 / 6], dtype=np.float32))
+    assert rne.tolist() == [0x3F, 0x02, 0x01]
+    # blocks of 32, two blocks, ragged tail (3 elements in the last block)
+    x = np.zeros(35, dtype=np.float32)
+    x[31], x[34] = 3.0, -0.75
+    nib, sc = oracle.quantize_fp4_blockscale_kernel(x, 32)
+    assert sc.tolist() == [0x30, 0x20] and nib.size == 18              # 0.5 = 2^-1: e = 6; 0.125 = 2^-3: e = 4
+    assert oracle.unpack_fp4(nib, 35).tolist()[31] == 7 and oracle.unpack_fp4(nib, 35).tolist()[34] == 15
+
+
 def test_packers_agree_and_round_trip_is_bounded(oracle, pkg):
     w = pkg.synth.weights_f32(3, 64, 256)
     a = oracle.quantize_fp4_blockscale_converter(w, 16)
