@@ -97,8 +97,10 @@ def pack_fp4_on_device(torch, w, block):
     amax = b.abs().amax(dim=1)
     live = amax > 1e-10
     one = torch.ones_like(amax)
-    scales = torch.where(live, amax / 6.0, one)
-    fwd = torch.where(live, 6.0 / amax, one)
+    # float32 quotients as the host computes them: divided in float64 and rounded once (a float32 division on the
+    # device need not be correctly rounded)
+    scales = torch.where(live, (amax.double() / 6.0).float(), one)
+    fwd = torch.where(live, (6.0 / amax.double()).float(), one)
     scaled = (b * fwd[:, None]).reshape(-1)
     bounds = torch.tensor(FP4_BOUNDS, dtype=torch.float32, device=w.device)
     code = torch.bucketize(scaled.abs(), bounds, right=False).to(torch.uint8) | ((scaled < 0).to(torch.uint8) << 3)
@@ -121,7 +123,9 @@ def test_fp4_gemv_at_the_llama_8b_shapes(gpu, pkg, oracle, K, n_out, block):
         nib[r0:r0 + r], sc[r0:r0 + r] = pack_fp4_on_device(torch, w, block)
         if r0 == 0:
             want_nib, want_sc = pkg.synth.pack_fp4_blockscale(w[:64].cpu().numpy(), block)
-            assert np.array_equal(nib[:64].cpu().numpy().ravel(), want_nib) and np.array_equal(sc[:64].cpu().numpy().ravel(), want_sc)
+            bad_nib = int((nib[:64].cpu().numpy().ravel() != want_nib).sum())
+            bad_sc = int((sc[:64].cpu().numpy().ravel() != want_sc).sum())
+            assert bad_nib == 0 and bad_sc == 0, f"device packer differs from the host packer: {bad_nib} code bytes, {bad_sc} scale bytes"
     rows = np.sort(np.random.default_rng(n_out + block).choice(n_out, size=257, replace=False))
     ridx = torch.from_numpy(rows).to(dev)
     nib_rows, sc_rows = nib[ridx].cpu().numpy(), sc[ridx].cpu().numpy()
