@@ -9,12 +9,14 @@
 namespace ccq
 {
 
-static std::atomic<hipStream_t> g_stream{ nullptr };
-static std::atomic<int> g_sync{ 0 };
+// Per host thread, like the reference's current-device pointer (cccc/GpuControl.cpp:18): one thread
+// capturing its launches into a graph on its own stream does not redirect another thread's work.
+static thread_local hipStream_t g_stream = nullptr;
+static thread_local int g_sync = 0;
 static thread_local const char* g_last_kernel = "";
 
-hipStream_t stream() { return g_stream.load(std::memory_order_relaxed); }
-bool sync_enabled() { return g_sync.load(std::memory_order_relaxed) != 0; }
+hipStream_t stream() { return g_stream; }
+bool sync_enabled() { return g_sync != 0; }
 void note_kernel(const char* name) { g_last_kernel = name; }
 
 int finish(const char* what)
@@ -79,12 +81,14 @@ void* workspace(size_t bytes)
 
 int hip_quant_set_sync(int enabled)
 {
-    return ccq::g_sync.exchange(enabled ? 1 : 0, std::memory_order_relaxed);
+    const int before = ccq::g_sync;
+    ccq::g_sync = enabled ? 1 : 0;
+    return before;
 }
 
 int hip_quant_set_stream(void* s)
 {
-    ccq::g_stream.store((hipStream_t)s, std::memory_order_relaxed);
+    ccq::g_stream = (hipStream_t)s;
     return 0;
 }
 
