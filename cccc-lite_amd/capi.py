@@ -44,6 +44,7 @@ EXPORTS = (
     "hip_float_to_fp4_blockscale",
     "hip_absmax",
     "hip_quant_gemm",
+    "hip_quant_gemm_noalloc",
     "hip_quant_tiled_size",
     "hip_quant_weight_prepare",
     "hip_quant_weight_release",
@@ -95,6 +96,8 @@ class QuantLibrary:
                                      vp, i32, i32, f32,
                                      f32, vp, i32, i32, f32,
                                      vp, vp, u32]
+        L.hip_quant_gemm_noalloc.restype = i32
+        L.hip_quant_gemm_noalloc.argtypes = L.hip_quant_gemm.argtypes
         L.hip_quant_tiled_size.restype = ctypes.c_ulonglong
         L.hip_quant_tiled_size.argtypes = [i32, i32, i32]
         L.hip_quant_weight_prepare.restype = i32
@@ -146,8 +149,9 @@ class QuantLibrary:
 
     def quant_gemm(self, transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
                    B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale=0.0,
-                   blk_scA=None, blk_scB=None, block_size=16) -> int:
-        return self.c.hip_quant_gemm(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
+                   blk_scA=None, blk_scB=None, block_size=16, noalloc=False) -> int:
+        entry = self.c.hip_quant_gemm_noalloc if noalloc else self.c.hip_quant_gemm
+        return entry(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA,
                                      B, typeB, ldb, invScaleB, beta, C, typeC, ldc, act_scale,
                                      blk_scA, blk_scB, block_size)
 
@@ -174,13 +178,13 @@ class QuantLibrary:
 
     # -- the call the LLM graph makes --------------------------------------------------------
     def linear(self, W, w_type, X, Y, n_out, tokens, K, inv_scale=1.0, blk_sc=None, block_size=16,
-               alpha=1.0, beta=0.0, act_type=DataType.BFLOAT16) -> int:
+               alpha=1.0, beta=0.0, act_type=DataType.BFLOAT16, noalloc=False) -> int:
         """y[t][o] = sum_k W[o][k] x[t][k], argument layout of Matrix::mulBatched(W, X, Y, TRANS,
         NO_TRANS) for a linear layer (reference cccc/Matrix.cpp:1162-1203): BLAS M = n_out,
         BLAS N = tokens, lda = ldb = K, ldc = n_out."""
         return self.quant_gemm(TRANS, NO_TRANS, n_out, tokens, K, alpha, W, w_type, K, inv_scale,
                                X, act_type, K, 1.0, beta, Y, act_type, n_out, 0.0,
-                               blk_sc, None, block_size)
+                               blk_sc, None, block_size, noalloc=noalloc)
 
 
 _library = None

@@ -1,9 +1,16 @@
 // hip_quant_gemm: the unified quantized GEMM entry point.  Normalises the BLAS-style arguments of
 // the reference's dispatcher (cccc/cublas_real.h:875-880) into "one quantized linear" and picks a
-// kernel family by token count:
-//     tokens <= 4   gemv_dot2   (FP8 / FP4, dot2 + DPP)
-//     tokens <= 16  gemv_mfma   (FP8), token groups of 4 through gemv_dot2 (FP4)
-//     otherwise     gemm_mfma   (dequant-to-LDS + bf16 MFMA)
+// kernel family:
+//     FP8, tokens <= 16, tiled copy registered     gemv_mfma_tiled (matrix cores over the load-time copy; one or
+//                                                  two tokens on a weight under 8 MiB stay on gemv_dot2)
+//     FP8, tokens <= 4                             gemv_dot2 (dot2 + DPP, software pipelined for small weights)
+//     FP8, tokens 5..16                            gemv_mfma (matrix cores, row-major weight)
+//     FP8, tokens >= 17                            gemm_mfma: weights straight into the matrix-core operands when
+//                                                  tokens >= 48 and K % 64 == 0 (row-major or tiled copy, k split
+//                                                  over workgroups when the output has few tiles), else dequant-to-LDS
+//     FP4 block scales, tokens <= 16               gemv_dot2 in token groups of four
+//     FP4 block scales, tokens >= 17               gemm_mfma (dequant-to-LDS)
+//     HALF activations                             the half instantiations of gemv_dot2 / gemm_mfma
 //     anything the fast kernels cannot take (transposed layouts, odd sizes, misaligned pointers,
 //     FP4 without block scales): generic
 #include "../../include/cccc_hip_quant.h"
@@ -17,6 +24,10 @@
 #include <shared_mutex>
 #include <unordered_map>
 #include <unordered_set>
+
+// Scratch of hip_quant_gemm_noalloc: the FP32 partial sums of a k-split GEMM.  One copy per GPU the library
+// runs on, held until the process ends; every call on a GPU shares it.
+static __device__ __align__(256) unsigned char scratch[HIP_QUANT_NOALLOC_SCRATCH_BYTES];
 
 using namespace ccq;
 
@@ -215,11 +226,43 @@ const unsigned char* ccq::lookup_tiled(const void* W, int type, int n_out, int K
     return (t.type == type && t.n_out == n_out && t.K == K && t.ldw == ldw) ? t.tiled : nullptr;
 }
 
-int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
-                   const void* A, int typeA, int lda, float invScaleA,
-                   const void* B, int typeB, int ldb, float invScaleB,
-                   float beta, void* C, int typeC, int ldc, float /*act_scale*/,
-                   const void* blk_scA, const void* blk_scB, unsigned int block_size)
+namespace
+{
+
+// Device address of `scratch` on the current device (the array's name is only a host-side handle), looked up
+// once per device with that device current.
+float* static_scratch()
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static void* ptr[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!ptr[dev])
+    {
+        void* p = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p)
+        {
+            fprintf(stderr, "hip_quant_gemm_noalloc: hipGetSymbolAddress failed on device %d: %s\n", dev, hipGetErrorString(err));
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    return (float*)ptr[dev];
+}
+
+int quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
+               const void* A, int typeA, int lda, float invScaleA,
+               const void* B, int typeB, int ldb, float invScaleB,
+               float beta, void* C, int typeC, int ldc,
+               const void* blk_scA, const void* blk_scB, unsigned int block_size, SplitScratch* split_scratch)
 {
     const bool aQ = is_quantized(typeA), bQ = is_quantized(typeB);
     if (aQ == bQ) { return -1; }
@@ -298,7 +341,9 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         {
             if (x_ok && K % 16 == 0 && a.ldw % 16 == 0 && aligned16(a.W))
             {
-                note_kernel(half_linear(a, g.w_type));
+                const char* name = half_linear(a, g.w_type, split_scratch);
+                if (!name) { return -2; }
+                note_kernel(name);
                 launched = true;
             }
         }
@@ -358,9 +403,10 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
             if (ok && !launched)
             {
                 const uint8_t* tiled = find_tiled(a, g.w_type);
-                if (g.w_type == DT_E5M2) { launched = gemm_mfma<DT_E5M2, 0>(a, tiled); }
-                else { launched = gemm_mfma<DT_E4M3, 0>(a, tiled); }
-                if (launched) { note_kernel(tiled ? "gemm_mfma_tiled" : "gemm_mfma"); }
+                if (g.w_type == DT_E5M2) { launched = gemm_mfma<DT_E5M2, 0>(a, tiled, split_scratch); }
+                else { launched = gemm_mfma<DT_E4M3, 0>(a, tiled, split_scratch); }
+                if (!launched) { return -2; }                    // only a fixed scratch buffer that is too small ends here
+                note_kernel(tiled ? "gemm_mfma_tiled" : "gemm_mfma");
             }
         }
     }
@@ -370,6 +416,41 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         note_kernel("generic");
     }
     return finish("quant_gemm");
+}
+
+}    // namespace
+
+int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
+                   const void* A, int typeA, int lda, float invScaleA,
+                   const void* B, int typeB, int ldb, float invScaleB,
+                   float beta, void* C, int typeC, int ldc, float /*act_scale*/,
+                   const void* blk_scA, const void* blk_scB, unsigned int block_size)
+{
+    return quant_gemm(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA, B, typeB, ldb, invScaleB, beta, C, typeC, ldc,
+                      blk_scA, blk_scB, block_size, nullptr);
+}
+
+int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K, float alpha,
+                           const void* A, int typeA, int lda, float invScaleA,
+                           const void* B, int typeB, int ldb, float invScaleB,
+                           float beta, void* C, int typeC, int ldc, float /*act_scale*/,
+                           const void* blk_scA, const void* blk_scB, unsigned int block_size)
+{
+    SplitScratch fixed;
+    fixed.strict = true;
+    fixed.fixed = static_scratch();
+    fixed.fixed_bytes = HIP_QUANT_NOALLOC_SCRATCH_BYTES;
+    const int rc = quant_gemm(transA, transB, M, N, K, alpha, A, typeA, lda, invScaleA, B, typeB, ldb, invScaleB, beta, C, typeC, ldc,
+                              blk_scA, blk_scB, block_size, &fixed);
+    if (rc == -2 && !fixed.fixed) { return 1; }      // the symbol lookup failed and said so
+    if (rc == -2)
+    {
+        fprintf(stderr, "hip_quant_gemm_noalloc: this shape splits K over workgroups and needs %zu bytes of partial sums; "
+                        "the static scratch holds %llu (nothing was launched)\n",
+                fixed.refused, (unsigned long long)HIP_QUANT_NOALLOC_SCRATCH_BYTES);
+        return -1;
+    }
+    return rc;
 }
 
 unsigned long long hip_quant_tiled_size(int type, int n_out, int K)

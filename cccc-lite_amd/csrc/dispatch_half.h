@@ -4,8 +4,10 @@
 // K % 16 == 0, ldw % 16 == 0, 16-byte aligned pointers, ldx % 8 == 0); returns the kernel family name.
 #pragma once
 #include "linear_args.h"
+#include "runtime.h"
 
 namespace ccq
 {
-const char* half_linear(const LinearArgs& a, int w_type);
+// `scratch` as in gemm_mfma; returns nullptr when a fixed scratch buffer was too small (nothing launched).
+const char* half_linear(const LinearArgs& a, int w_type, SplitScratch* scratch = nullptr);
 }

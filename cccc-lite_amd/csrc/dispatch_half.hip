@@ -43,7 +43,7 @@ bool half_gemv(const LinearArgs& a)
 
 }    // namespace
 
-const char* half_linear(const LinearArgs& a, int w_type)
+const char* half_linear(const LinearArgs& a, int w_type, SplitScratch* scratch)
 {
     const bool scaled = a.w_scale != 1.0f;
     if (a.tokens <= 4)
@@ -54,9 +54,8 @@ const char* half_linear(const LinearArgs& a, int w_type)
         if (ok) { return "gemv_dot2_half"; }
     }
     const uint8_t* tiled = lookup_tiled(a.W, w_type, a.n_out, a.K, a.ldw);
-    if (w_type == DT_E5M2) { gemm_mfma<DT_E5M2, 0, DT_HALF>(a, tiled); }
-    else { gemm_mfma<DT_E4M3, 0, DT_HALF>(a, tiled); }
-    return "gemm_mfma_half";
+    const bool launched = w_type == DT_E5M2 ? gemm_mfma<DT_E5M2, 0, DT_HALF>(a, tiled, scratch) : gemm_mfma<DT_E4M3, 0, DT_HALF>(a, tiled, scratch);
+    return launched ? "gemm_mfma_half" : nullptr;
 }
 
 }    // namespace ccq

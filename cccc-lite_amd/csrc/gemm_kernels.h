@@ -547,8 +547,10 @@ void launch_gemm_mfma(const LinearArgs& a)
 // ragged K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they
 // give every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
 // otherwise 128 x 64 tiles to put more workgroups on the machine.
+// `scratch`: see SplitScratch; nullptr = the stream's grow-on-demand workspace.  Returns false (nothing launched)
+// only when a fixed scratch buffer is too small for the k-split this shape takes.
 template <int WT, int BLOCK, int AT = DT_BF16>
-bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr)
+bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch* scratch = nullptr)
 {
     if constexpr (WT != DT_FP4)
     {
@@ -569,7 +571,17 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr)
                 long long s = (cus + base / 2) / base;
                 if (s > 8) { s = 8; }
                 if (s > a.K / 64 / 16) { s = a.K / 64 / 16; }
-                if (s > 1) { partial = (float*)workspace((size_t)s * a.tokens * a.n_out * sizeof(float)); }
+                const size_t need = (size_t)s * a.tokens * a.n_out * sizeof(float);
+                if (s > 1 && scratch && scratch->strict)
+                {
+                    if (!scratch->fixed || need > scratch->fixed_bytes)
+                    {
+                        scratch->refused = need;
+                        return false;
+                    }
+                    partial = scratch->fixed;
+                }
+                else if (s > 1) { partial = (float*)workspace(need); }
                 if (partial)
                 {
                     splits = (int)s;

@@ -24,6 +24,18 @@ int cu_count();
 // have to grow while the stream is being captured into a graph); callers then take a path that needs none.
 void* workspace(size_t bytes);
 
+// Where a k-split GEMM keeps its FP32 partial sums.  Default (no SplitScratch, or strict == false): workspace()
+// above.  strict: the fixed buffer and nothing else, so nothing is ever allocated -- a request beyond
+// fixed_bytes (or with no buffer at all) is recorded in `refused` and the caller reports an error instead of
+// launching.
+struct SplitScratch
+{
+    bool strict = false;
+    float* fixed = nullptr;
+    size_t fixed_bytes = 0;
+    size_t refused = 0;
+};
+
 // The load-time tiled copy registered for the FP8 weight `W` by hip_quant_weight_prepare, or nullptr
 // when there is none or its type / shape / row stride differ (defined with the registry in dispatch.hip).
 const unsigned char* lookup_tiled(const void* W, int type, int n_out, int K, long long ldw);

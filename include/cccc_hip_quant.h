@@ -101,6 +101,26 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
                             const void* blk_scA, const void* blk_scB, unsigned int block_size);
 
 /*
+ * hip_quant_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
+ * kernels and results as hip_quant_gemm; the only difference is where the k-split GEMM keeps its FP32
+ * partial sums: in a static device array of HIP_QUANT_NOALLOC_SCRATCH_BYTES inside the library (one per
+ * GPU the library runs on, held until the process ends) instead of a buffer grown on demand.  The call
+ * never allocates or frees device memory.  A shape whose k-split needs more than that (splits * M * N * 4
+ * bytes, splits <= 8; only FP8 GEMMs of 48 tokens or more with few output tiles split at all) returns -1
+ * with a message on stderr and launches nothing; 32 MiB covers 512 tokens x 4096 features.
+ * Every call on a GPU shares the one array: calls that overlap on one GPU (two streams, two host
+ * threads) race on it and must be ordered by the caller.  Nothing in it needs clearing between calls:
+ * each call overwrites every partial sum it later reads.
+ */
+#define HIP_QUANT_NOALLOC_SCRATCH_BYTES (32u << 20)
+C_EXPORT int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K, float alpha,
+                                    const void* A, int typeA, int lda, float invScaleA,
+                                    const void* B, int typeB, int ldb, float invScaleB,
+                                    float beta, void* C, int typeC, int ldc, float act_scale,
+                                    const void* blk_scA, const void* blk_scB, unsigned int block_size);
+
+/*
  * Optional load-time repack (no counterpart in the reference; the on-disk format and the caller's
  * weight buffer are left untouched).  hip_quant_weight_prepare writes an MI355X-friendly tiled copy
  * of an FP8 weight W ([n_out][ldw], K contiguous, as loadQuantizedDirect uploads it) into `dst_tiled`
@@ -202,9 +222,11 @@ C_EXPORT int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void*
 /*
  * Library controls (no counterpart in the reference, which always uses the null stream and always
  * synchronises: cccc-hip/hip_functions.cpp:32-42).
- *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch (parity/debug);
- *                             returns the previous setting
- *   hip_quant_set_stream(s) : enqueue on hipStream_t `s` (NULL = null stream)
+ * Both switches are per host thread, like the reference's current-device pointer (cccc/GpuControl.cpp:18);
+ * the library is meant to be driven by one host thread per device, as the reference drives its own.
+ *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch of this thread
+ *                             (parity/debug); returns the previous setting
+ *   hip_quant_set_stream(s) : this thread's launches go to hipStream_t `s` (NULL = null stream)
  *   hip_quant_last_kernel() : name of the kernel family the last hip_quant_gemm call dispatched to
  *                             ("gemv_dot2", "gemv_mfma", "gemm_mfma", "generic", ...)
  */
