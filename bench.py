@@ -38,6 +38,9 @@ GEMV_GATE_UP_TRAFFIC_BYTES = 50451344
 # the same two counters for one launch of the fused RMSNorm + gate/up SwiGLU GEMV (two 4096 x 12288 weights)
 GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = 101012454
 
+# `roofline.traffic` is a constant from a counter run, not measured by this script (rocprofv3 --pmc needs a run of its own)
+TRAFFIC_SOURCE = "constant copied from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/"
+
 FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
 
 QWEN3_8B = dict(layers=36, hidden=4096, q_out=4096, kv_out=1024, inter=12288, vocab=151936)
@@ -48,6 +51,43 @@ def gemv_bytes(K, N, M):
     return K * N + 2 * M * K + 2 * M * N
 
 
+class BenchLibrary:
+    """libcccc_bench.so: the timing loops (host/bench_capi.cpp), native so that Python call overhead stays out
+    of microsecond kernels.  Only this script loads it."""
+
+    def __init__(self, pkg_dir: Path):
+        import ctypes
+        path = pkg_dir / "libcccc_bench.so"
+        if not path.exists():
+            raise FileNotFoundError(f"{path} is missing: build it with `make -C {pkg_dir}`")
+        L = ctypes.CDLL(str(path))
+        vp, i32 = ctypes.c_void_p, ctypes.c_int
+        L.cccc_bench_linear_chain.restype = ctypes.c_double
+        L.cccc_bench_linear_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), i32, i32, i32]
+        L.cccc_bench_fp4_chain.restype = ctypes.c_double
+        L.cccc_bench_fp4_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_uint, i32, i32]
+        L.cccc_decode_bench_gate_up.restype = ctypes.c_double
+        L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
+        self.c, self.ctypes = L, ctypes
+
+    def linear_chain(self, W, X, R, steps, warmup, use_graph) -> float:
+        n = len(W)
+        arr = lambda ms: (self.ctypes.c_void_p * n)(*[m.handle for m in ms])
+        return float(self.c.cccc_bench_linear_chain(n, arr(W), arr(X), arr(R), steps, warmup, 1 if use_graph else 0))
+
+    def fp4_chain(self, W_ptrs, S_ptrs, X_ptr, Y_ptr, n_out, tokens, K, block, iters, warmup) -> float:
+        n = len(W_ptrs)
+        vp = self.ctypes.c_void_p
+        return float(self.c.cccc_bench_fp4_chain(n, (vp * n)(*W_ptrs), (vp * n)(*S_ptrs), X_ptr, Y_ptr, n_out, tokens, K, block, iters, warmup))
+
+    def gate_up_us(self, model, reps: int) -> float:
+        """Average microseconds per fused gate/up launch over all layers' distinct weights."""
+        us = float(self.c.cccc_decode_bench_gate_up(model.handle, reps))
+        if us < 0:
+            raise RuntimeError(f"gate/up timing failed: {us}")
+        return us
+
+
 class Workspace:
     """Weights, activations and outputs of the benchmark as host-mirror matrices on cuda:0."""
 
@@ -56,6 +96,7 @@ class Workspace:
         self.lib = pkg.library()
         self.host = pkg.host_api.host()
         self.host.init(0)
+        self.bench = BenchLibrary(ROOT / "cccc-lite_amd")
         self.dev = torch.device("cuda:0")
         self.gen = torch.Generator(device=self.dev).manual_seed(1234)
         self.keep = []
@@ -284,7 +325,7 @@ def gpu_baselines(ws: Workspace, ctx: int, steps_ref: int = 3, steps_torch: int 
 
 
 def time_chain(ws, ops, steps, warmup, use_graph):
-    ms = ws.host.bench_linear_chain([o[0] for o in ops], [o[1] for o in ops], [o[2] for o in ops], steps, warmup, use_graph)
+    ms = ws.bench.linear_chain([o[0] for o in ops], [o[1] for o in ops], [o[2] for o in ops], steps, warmup, use_graph)
     if ms < 0:
         raise RuntimeError(f"bench chain failed with code {ms}")
     return ms
@@ -396,7 +437,7 @@ def fp4_sweep(ws):
             sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             X, Y = ws.activation(1, K), ws.output(1, N)
             iters = max(20, min(400, (4 << 30) // per))
-            ms = ws.host.bench_fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr,
+            ms = ws.bench.fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr,
                                          N, 1, K, block, iters, 5)
             if ms < 0:
                 raise RuntimeError(f"fp4 chain failed: {ms}")
@@ -413,7 +454,7 @@ def cpu_baseline(pkg, threads, unit):
     on the linear layers of the decode workload at M=1, on a bounded sample: 12 of the 36 layers (the same seven
     weights walked 12 times: 2.3 GB of codes per walk, far beyond the host caches), timed three times."""
     import numpy as np
-    from oracle import oracle
+    from oracle import oracle, synth
     c = QWEN3_8B
     shapes = [(c["hidden"], c["q_out"]), (c["hidden"], c["kv_out"]), (c["hidden"], c["kv_out"]), (c["hidden"], c["q_out"]),
               (c["hidden"], c["inter"]), (c["hidden"], c["inter"]), (c["inter"], c["hidden"])]
@@ -422,7 +463,7 @@ def cpu_baseline(pkg, threads, unit):
     data = []
     for K, N in shapes:
         W = rng.integers(0, 0x7C, size=(N, K), dtype=np.uint8)
-        X = pkg.synth.activations(7, 1, K)
+        X = synth.activations(7, 1, K)
         data.append((W, X, K, N))
     layers_sampled = 12
     runs = []
@@ -510,8 +551,16 @@ def main():
         assert model.pos == DECODE_CTX
         model.reset(1, start + args.warmup)
         ms_other = model.run(args.steps, not use_graph)
+        # the same steps on the attention path that keeps every rounding point of the reference (BF16 probabilities)
+        model.set_exact_attention(True)
+        model.reset(1, start)
+        if args.warmup:
+            model.run(args.warmup, use_graph)
+        ms_exact = model.run(args.steps, use_graph)
+        model.set_exact_attention(False)
         ms_step = ms / args.steps
         value = 1000.0 / ms_step
+        extra["ms_per_step_exact_attention"] = round(ms_exact / args.steps, 4)
         metric, unit = "decode tok/s Qwen3-8B W8A16 bs=1", "tok/s"
         step_bytes = decode_step_bytes(DECODE_CTX - (args.steps - 1) / 2.0)
         extra["launch_mode"] = "hipGraph" if use_graph else "stream"
@@ -525,7 +574,7 @@ def main():
                     f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions")
         # dominant kernel: the fused RMSNorm + gate/up SwiGLU launch (two 4096 x 12288 weights), timed over the 36 layers' distinct weights
         K, N, M = 4096, 2 * 12288, 1
-        dom_us = model.bench_gate_up(10)
+        dom_us = ws.bench.gate_up_us(model, 10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
         del model
         torch.cuda.empty_cache()
@@ -587,7 +636,8 @@ def main():
     if args.workload == "decode_step":
         achieved = dom_bytes / dom_us * 1e-3
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    "traffic": GEMV_FUSED_GATE_UP_TRAFFIC_BYTES, "kernel": "gemv8_fused_kernel (RMSNorm + gate/up SwiGLU pair)",
+                    "traffic": GEMV_FUSED_GATE_UP_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE + "decode_step_qwen3_8b_ctx4096.md",
+                    "kernel": "gemv8_fused_kernel (RMSNorm + gate/up SwiGLU pair)",
                     "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3), "bytes_per_launch": dom_bytes}
     elif args.workload == "prefill":
         flops = 2.0 * M * K * N
@@ -601,6 +651,7 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "traffic": GEMV_GATE_UP_TRAFFIC_BYTES if (K, N, M) == (4096, 12288, 1) else None,
+                    "traffic_source": TRAFFIC_SOURCE + "gemv8_mfma_tiled_K4096_N12288_M1.md" if (K, N, M) == (4096, 12288, 1) else None,
                     "kernel": ws.lib.last_kernel(), "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
                     "bytes_per_launch": gemv_bytes(K, N, M)}
 

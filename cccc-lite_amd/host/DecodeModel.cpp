@@ -189,6 +189,35 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
     return rc;
 }
 
+int DecodeModel::saveNamedWeights(const std::string& filename)
+{
+    gpu_->setAsCurrent();
+    if (filename.empty() || hipDeviceSynchronize() != hipSuccess) { return -1; }
+    WeightFileWriter w;
+    // header: the first quantized tensor's type, else the first tensor's (cccc/Net.cpp:1243-1271)
+    const DataType head = Rocblas::isQuantized(lm_head_->getDataType()) || layers_.empty() ? lm_head_->getDataType() : layers_[0].wq->getDataType();
+    const char* names[] = { "auto", "float", "double", "half", "bfloat16", "fp8_e4m3", "fp8_e5m2", "fp4_e2m1" };
+    const DataType order[] = { CURRENT, FLOAT, DOUBLE, HALF, BFLOAT16, FP8_E4M3, FP8_E5M2, FP4_E2M1 };
+    std::string head_name = "auto";
+    for (int i = 0; i < 8; i++) { if (order[i] == head) { head_name = names[i]; } }
+    w.set_value("data_type", head_name);
+    w.set_value("named_weights", std::string("1"));
+    addNamedWeight(w, "W_emb", *emb_);
+    addNamedWeight(w, "W_rms_final", *rms_final_);
+    addNamedWeight(w, "W_lm_head", *lm_head_);
+    for (int i = 0; i < cfg_.layers; i++)
+    {
+        Layer& L = layers_[i];
+        const std::string n = std::to_string(i);
+        const std::pair<Matrix*, const char*> tensors[] = {
+            { L.rms_attn.get(), "W_rms_attn_" }, { L.wq.get(), "W_q_" }, { L.wk.get(), "W_k_" }, { L.wv.get(), "W_v_" },
+            { L.q_norm.get(), "W_qnorm_" }, { L.k_norm.get(), "W_knorm_" }, { L.wo.get(), "W_o_" }, { L.rms_ffn.get(), "W_rms_ffn_" },
+            { L.w_gate.get(), "W_gate_" }, { L.w_up.get(), "W_up_" }, { L.w_down.get(), "W_down_" } };
+        for (auto& [m, prefix] : tensors) { addNamedWeight(w, prefix + n, *m); }
+    }
+    return w.save(filename) > 0 ? 0 : -1;
+}
+
 size_t DecodeModel::weightBytes() const
 {
     const size_t q_out = (size_t)cfg_.n_q * cfg_.head_dim, kv_out = (size_t)cfg_.n_kv * cfg_.head_dim;
@@ -317,37 +346,6 @@ int DecodeModel::step()
     }
     if (rc == 0) { rc = hip_argmax_bf16(logits_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1, argmax_ws_->data()); }
     return rc;
-}
-
-double DecodeModel::benchGateUp(int reps)
-{
-    if (reps <= 0 || layers_.empty()) { return -2.0; }
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
-    const int sync_before = hip_quant_set_sync(0);
-    bool ok = true;
-    for (int rep = -1; rep < reps; rep++)    // pass -1 is the warm-up
-    {
-        if (rep == 0) { (void)hipEventRecord(e0, nullptr); }
-        for (auto& L : layers_)
-        {
-            hip_fused_linear gu = linear_desc(*L.w_gate, cfg_.inter, cfg_.hidden, r1_->data(), gated_->data());
-            gu.n_segments = 2;
-            gu.pair = 1;
-            gu.W[1] = L.w_up->data(); gu.n_out[1] = cfg_.inter; gu.w_scale[1] = L.w_up->getQuantScale();
-            gu.norm_weight = L.rms_ffn->data();
-            gu.norm_eps = cfg_.eps;
-            ok = (hip_quant_linear_fused(&gu) == 0) && ok;
-        }
-    }
-    (void)hipEventRecord(e1, nullptr);
-    ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
-    float ms = 0;
-    if (ok) { (void)hipEventElapsedTime(&ms, e0, e1); }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    hip_quant_set_sync(sync_before);
-    return ok ? (double)ms * 1000.0 / ((double)reps * layers_.size()) : -3.0;
 }
 
 double DecodeModel::run(int n_steps, int use_graph)

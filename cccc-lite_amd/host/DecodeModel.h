@@ -53,6 +53,13 @@ public:
     // -1 missing, -2 wrong size, -3 a type the fused decode kernels do not take (FP4, or too small to quantize).
     int loadNamedWeights(const WeightFile& file, DataType quantize_to = FP8_E5M2, std::string* failed = nullptr);
 
+    // Writes every tensor under the same names, as Net::saveNamedWeights does (cccc/Net.cpp:1235-1314): the header
+    // entry "data_type" (the linears' type), then per tensor "weight_<dtype>_<name>" with its bytes as they sit on the
+    // device, "scale_<name>" when the per-tensor scale is not 1 and "blockscale_<name>" for FP4.  This is the cache the
+    // reference writes after quantizing on load (save_fp8_file, cccc/MainProcess.cpp:362-378): loading it back gives
+    // the same bytes without quantizing again.  0 ok, -1 the file could not be written.
+    int saveNamedWeights(const std::string& filename);
+
     // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
     // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).
     void setExactAttention(bool exact) { exact_attention_ = exact; }
@@ -60,9 +67,6 @@ public:
     int step();                             // enqueues one decode step; the next token replaces the current one
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
     double run(int n_steps, int use_graph);
-    // Times `reps` passes over every layer's fused gate/up launch (norm + SwiGLU pair, distinct weights per
-    // layer) with events on the launch stream; returns the average microseconds per launch or < 0.
-    double benchGateUp(int reps);
     int currentToken();                     // blocking 4-byte read
     int currentPos();
     Matrix& logits() { return *logits_; }

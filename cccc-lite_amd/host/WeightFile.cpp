@@ -1,4 +1,5 @@
 #include "WeightFile.h"
+#include <cstdio>
 #include <cstring>
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -258,6 +259,92 @@ int WeightFile::loadNamed(Matrix& m, const std::string& name) const
     if ((int64_t)n_bytes != elems * (int64_t)typeBytes(wk.dt)) { return -1; }
     if (m.getDataType() != wk.dt) { m.retype(wk.dt); }
     return m.copyFromHost(bytes, n_bytes) == 0 ? 0 : -1;
+}
+
+// ------------------------------------------------------------------ writer
+
+void WeightFileWriter::set_value(const std::string& key, const void* bytes, size_t n)
+{
+    Entry e;
+    e.key = key;
+    e.host.assign((const uint8_t*)bytes, (const uint8_t*)bytes + n);
+    e.bytes = n;
+    entries_.push_back(std::move(e));
+}
+
+void WeightFileWriter::set_device_value(const std::string& key, const void* device_ptr, size_t n)
+{
+    Entry e;
+    e.key = key;
+    e.device = device_ptr;
+    e.bytes = n;
+    entries_.push_back(std::move(e));
+}
+
+long long WeightFileWriter::save(const std::string& filename) const
+{
+    std::string index;
+    uint64_t offset = 0;
+    for (const Entry& e : entries_)
+    {
+        index += e.key + " = " + std::to_string(offset) + "," + std::to_string(e.bytes) + "\n";
+        offset += e.bytes;
+    }
+    FILE* f = std::fopen(filename.c_str(), "wb");
+    if (!f) { return -1; }
+    uint8_t head[40] = {};
+    std::memcpy(head, kMagic, sizeof(kMagic) - 1);
+    const uint64_t index_len = index.size();
+    for (int i = 0; i < 8; i++) { head[32 + i] = (uint8_t)(index_len >> (8 * i)); }
+    bool ok = std::fwrite(head, 1, sizeof(head), f) == sizeof(head) && std::fwrite(index.data(), 1, index.size(), f) == index.size();
+    std::vector<uint8_t> slab;
+    for (const Entry& e : entries_)
+    {
+        if (!ok) { break; }
+        if (!e.device)
+        {
+            ok = e.bytes == 0 || std::fwrite(e.host.data(), 1, e.bytes, f) == e.bytes;
+            continue;
+        }
+        const size_t kSlab = (size_t)64 << 20;
+        slab.resize(e.bytes < kSlab ? e.bytes : kSlab);
+        for (size_t done = 0; ok && done < e.bytes; done += kSlab)
+        {
+            const size_t n = e.bytes - done < kSlab ? e.bytes - done : kSlab;
+            ok = GpuControl::copyDeviceToHost(slab.data(), (const uint8_t*)e.device + done, n) == 0 && std::fwrite(slab.data(), 1, n, f) == n;
+        }
+    }
+    ok = (std::fclose(f) == 0) && ok;
+    return ok ? (long long)(sizeof(head) + index.size() + offset) : -1;
+}
+
+const char* weightTypeSuffix(DataType dt)
+{
+    switch (dt)
+    {
+    case BFLOAT16: return "bf16";
+    case FLOAT: return "float";
+    case HALF: return "half";
+    case DOUBLE: return "double";
+    case FP8_E4M3: return "fp8_e4m3";
+    case FP8_E5M2: return "fp8_e5m2";
+    case FP4_E2M1: return "fp4_e2m1";
+    default: return "";
+    }
+}
+
+void addNamedWeight(WeightFileWriter& w, const std::string& name, const Matrix& m)
+{
+    const DataType dt = m.getDataType();
+    const size_t n_bytes = dt == FP4_E2M1 ? (size_t)((m.getDataSize() + 1) / 2) : (size_t)m.getDataSize() * typeBytes(dt);
+    const std::string suffix = weightTypeSuffix(dt);
+    w.set_device_value(suffix.empty() ? "weight_" + name : "weight_" + suffix + "_" + name, m.data(), n_bytes);
+    const float scale = m.getQuantScale();
+    if (scale != 1.0f) { w.set_value("scale_" + name, &scale, sizeof(float)); }
+    if (m.getBlockScaleData() && m.getBlockScaleCount() > 0)
+    {
+        w.set_device_value("blockscale_" + name, m.getBlockScaleData(), (size_t)m.getBlockScaleCount());
+    }
 }
 
 }    // namespace cccc

@@ -76,4 +76,39 @@ private:
     std::vector<std::string> order_;
 };
 
+// Writer of the same container: what the reference's INIReaderBin::set_value / save do for
+// Net::saveNamedWeights (cccc/Net.cpp:1235-1314), in the byte layout of scripts/convert_weights.py:54-83.
+// Entries are written in the order they were added.  A tensor entry is not buffered on the host: its bytes
+// are copied from the device in slabs while the file is written.
+class WeightFileWriter
+{
+public:
+    void set_value(const std::string& key, const void* bytes, size_t n);
+    void set_value(const std::string& key, const std::string& text) { set_value(key, text.data(), text.size()); }
+    // n bytes of device memory, read when save() runs (the memory must stay valid until then)
+    void set_device_value(const std::string& key, const void* device_ptr, size_t n);
+    // Bytes written, or -1 (cannot create / short write / device copy failed).
+    long long save(const std::string& filename) const;
+
+private:
+    struct Entry
+    {
+        std::string key;
+        std::vector<uint8_t> host;
+        const void* device = nullptr;
+        size_t bytes = 0;
+    };
+    std::vector<Entry> entries_;
+};
+
+// "weight_<dtype>_<name>" suffix of a data type (cccc/Net.cpp:222-235); empty for types without one.
+const char* weightTypeSuffix(DataType dt);
+
+// One named weight as Net::saveNamedWeights stores it (cccc/Net.cpp:1274-1303): the raw bytes under
+// "weight_<dtype>_<name>", "scale_<name>" (one float32) when the per-tensor scale is not 1, and
+// "blockscale_<name>" (one E4M3 byte per 16 elements) for FP4.  An FP4 blob is sized as the converter sizes it,
+// (elements + 1) / 2 bytes (scripts/convert_weights.py:363-365); the reference's own writer reserves one byte
+// per element there (cccc/Net.cpp:1284), of which only the first half is data.
+void addNamedWeight(WeightFileWriter& w, const std::string& name, const Matrix& m);
+
 }    // namespace cccc

@@ -212,6 +212,7 @@ Matrix Matrix::view(int w, int h, int c, int n) const
 int Matrix::copyFromHost(const void* src, size_t bytes)
 {
     if (!shared_data_ || bytes > shared_data_->sizeInByte()) { return 1; }
+    shared_data_->releaseTiled();    // a tiled copy of the old bytes must not outlive them; prepareTiled() builds a new one
     return GpuControl::copyHostToDevice(data_, src, bytes);
 }
 
@@ -235,6 +236,7 @@ void Matrix::loadQuantizedDirect(const uint8_t* host_data, int64_t n, float scal
     if (!gpu()) { return; }
     gpu()->setAsCurrent();
     // a storage of another type, or one too small for the upload, is replaced
+    shared_data_->releaseTiled();    // whatever tiled copy exists belongs to the bytes about to be replaced
     if (getDataType() != fp8_dt || (size_t)n > shared_data_->sizeInByte()) { shared_data_->resize(n, fp8_dt, true); }
     GpuControl::copyHostToDevice(shared_data_->data_, host_data, (size_t)n);
     shared_data_->quant_scale_ = scale;

@@ -1,6 +1,5 @@
 // Plain-C window onto the host mirror so that tests and the benchmark (Python, ctypes) drive the
-// same Matrix::mulBatched path a cccc graph would, plus a timing loop that runs a chain of linears
-// from native code (Python call overhead would otherwise dominate microsecond kernels).
+// same Matrix::mulBatched path a cccc graph would.
 #include "DecodeModel.h"
 #include <cstring>
 #include "Matrix.h"
@@ -88,128 +87,6 @@ unsigned long long cccc_gpu_allocated_bytes(void)
 {
     GpuControl* g = GpuControl::getCurrentGpu();
     return g ? (unsigned long long)g->allocatedBytes() : 0ull;
-}
-
-namespace
-{
-
-// Two timing events and the library's sync switch (off while timing), both put back on every way out.
-struct TimingScope
-{
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    int previous_sync;
-    bool ok;
-    TimingScope() : previous_sync(hip_quant_set_sync(0))
-    {
-        ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
-    }
-    ~TimingScope()
-    {
-        if (e0) { (void)hipEventDestroy(e0); }
-        if (e1) { (void)hipEventDestroy(e1); }
-        hip_quant_set_sync(previous_sync);
-    }
-    TimingScope(const TimingScope&) = delete;
-    TimingScope& operator=(const TimingScope&) = delete;
-};
-
-}    // namespace
-
-// Runs `steps` timed passes over a chain of n_ops linears  R[i] = W[i]^T X[i]  (Matrix::mulBatched
-// with TRANS / NO_TRANS, as the LLM graph calls it) after `warmup` untimed passes.  use_graph != 0
-// replays one captured hipGraph per pass instead of issuing the launches one by one.  Events are
-// recorded on the stream the kernels run on.  Returns elapsed milliseconds for all timed passes, or
-// a negative value on error.
-double cccc_bench_linear_chain(int n_ops, void** W, void** X, void** R, int steps, int warmup, int use_graph)
-{
-    auto one_pass = [&]() -> int {
-        int status = 0;
-        for (int i = 0; i < n_ops; i++)
-        {
-            const int rc = Matrix::mulBatched(*(Matrix*)W[i], *(Matrix*)X[i], *(Matrix*)R[i], MATRIX_TRANS, MATRIX_NO_TRANS, 1.0f, 0.0f);
-            if (rc != 0) { status = rc; }
-        }
-        return status;
-    };
-    hipStream_t stream = nullptr;
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
-    TimingScope timing;
-    if (!timing.ok) { return -1.0; }
-    const hipEvent_t e0 = timing.e0, e1 = timing.e1;
-    double result = -1.0;
-    for (int i = 0; i < warmup; i++) { if (one_pass() != 0) { return -2.0; } }
-    if (hipDeviceSynchronize() != hipSuccess) { return -3.0; }
-    if (use_graph)
-    {
-        if (hipStreamCreate(&stream) != hipSuccess) { return -4.0; }
-        hip_quant_set_stream(stream);
-        bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) == hipSuccess;
-        if (ok) { ok = one_pass() == 0; }
-        ok = (hipStreamEndCapture(stream, &graph) == hipSuccess) && ok;
-        hip_quant_set_stream(nullptr);
-        if (ok) { ok = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess; }
-        if (ok) { ok = hipGraphLaunch(exec, stream) == hipSuccess && hipStreamSynchronize(stream) == hipSuccess; }
-        if (ok)
-        {
-            (void)hipEventRecord(e0, stream);
-            for (int s = 0; s < steps; s++) { (void)hipGraphLaunch(exec, stream); }
-            (void)hipEventRecord(e1, stream);
-            ok = hipEventSynchronize(e1) == hipSuccess;
-        }
-        if (ok)
-        {
-            float ms = 0;
-            (void)hipEventElapsedTime(&ms, e0, e1);
-            result = ms;
-        }
-        if (exec) { (void)hipGraphExecDestroy(exec); }
-        if (graph) { (void)hipGraphDestroy(graph); }
-        (void)hipStreamDestroy(stream);
-    }
-    else
-    {
-        (void)hipEventRecord(e0, nullptr);
-        bool ok = true;
-        for (int s = 0; s < steps; s++) { ok = (one_pass() == 0) && ok; }
-        (void)hipEventRecord(e1, nullptr);
-        ok = (hipEventSynchronize(e1) == hipSuccess) && ok;
-        if (ok)
-        {
-            float ms = 0;
-            (void)hipEventElapsedTime(&ms, e0, e1);
-            result = ms;
-        }
-    }
-    return result;
-}
-
-// Times `iters` back-to-back FP4 block-scale linears  Y = W[i % n_w]^T X  issued straight through
-// hip_quant_gemm (the host mirror always passes the reference's block size 16; this loop lets the
-// benchmark also measure block 32).  Returns elapsed milliseconds or a negative value on error.
-double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n_out, int tokens, int K,
-                            unsigned int block, int iters, int warmup)
-{
-    TimingScope timing;
-    if (!timing.ok) { return -1.0; }
-    const hipEvent_t e0 = timing.e0, e1 = timing.e1;
-    int status = 0;
-    for (int i = 0; i < warmup + iters; i++)
-    {
-        if (i == warmup) { (void)hipEventRecord(e0, nullptr); }
-        const int rc = hip_quant_gemm(1, 0, n_out, tokens, K, 1.0f, W[i % n_w], (int)FP4_E2M1, K, 1.0f, X, (int)BFLOAT16, K, 1.0f,
-                                      0.0f, Y, (int)BFLOAT16, n_out, 0.0f, S[i % n_w], nullptr, block);
-        if (rc != 0) { status = rc; }
-    }
-    (void)hipEventRecord(e1, nullptr);
-    double result = -2.0;
-    if (hipEventSynchronize(e1) == hipSuccess && status == 0)
-    {
-        float ms = 0;
-        (void)hipEventElapsedTime(&ms, e0, e1);
-        result = ms;
-    }
-    return result;
 }
 
 // ---- weight container
@@ -309,6 +186,17 @@ int cccc_decode_load_named(void* m, void* f, int quantize_to, char* failed_out, 
     return rc;
 }
 
+int cccc_decode_save_named(void* m, const char* path) { return ((DecodeModel*)m)->saveNamedWeights(path); }
+
+// Writes one matrix as a named weight (with its scale / block scales) into a container of its own.
+int cccc_matrix_save_named(void* m, const char* name, const char* path)
+{
+    WeightFileWriter w;
+    w.set_value("named_weights", std::string("1"));
+    addNamedWeight(w, name, *(Matrix*)m);
+    return w.save(path) > 0 ? 0 : -1;
+}
+
 void cccc_decode_set_exact_attention(void* m, int exact) { ((DecodeModel*)m)->setExactAttention(exact != 0); }
 
 int cccc_decode_reset(void* m, int token, int pos) { return ((DecodeModel*)m)->reset(token, pos); }
@@ -345,8 +233,6 @@ void* cccc_decode_kv_data(void* m, int layer, int is_v)
     if (layer < 0 || layer >= d->config().layers) { return nullptr; }
     return (is_v ? d->vCache(layer) : d->kCache(layer)).data();
 }
-
-double cccc_decode_bench_gate_up(void* m, int reps) { return ((DecodeModel*)m)->benchGateUp(reps); }
 
 int cccc_decode_cos_table(void* m, void* host, unsigned long long bytes) { return ((DecodeModel*)m)->cosTable().copyToHost(host, (size_t)bytes); }
 

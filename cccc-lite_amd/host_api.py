@@ -37,10 +37,6 @@ class HostLibrary:
         L.cccc_matrix_mul.restype = i32; L.cccc_matrix_mul.argtypes = [vp, vp, vp, f32, f32, i32, i32]
         L.cccc_matrix_mul_batched.restype = i32; L.cccc_matrix_mul_batched.argtypes = [vp, vp, vp, i32, i32, f32, f32]
         L.cccc_gpu_allocated_bytes.restype = ctypes.c_ulonglong; L.cccc_gpu_allocated_bytes.argtypes = []
-        L.cccc_bench_linear_chain.restype = ctypes.c_double
-        L.cccc_bench_linear_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), i32, i32, i32]
-        L.cccc_bench_fp4_chain.restype = ctypes.c_double
-        L.cccc_bench_fp4_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_uint, i32, i32]
         u64 = ctypes.c_ulonglong
         L.cccc_decode_create.restype = vp; L.cccc_decode_create.argtypes = [i32] * 8 + [f32, f32]
         L.cccc_decode_destroy.restype = None; L.cccc_decode_destroy.argtypes = [vp]
@@ -66,10 +62,11 @@ class HostLibrary:
         L.cccc_host_float_to_e4m3.restype = ctypes.c_ubyte; L.cccc_host_float_to_e4m3.argtypes = [f32]
         L.cccc_host_half_to_bf16.restype = ctypes.c_ushort; L.cccc_host_half_to_bf16.argtypes = [ctypes.c_ushort]
         L.cccc_decode_load_named.restype = i32; L.cccc_decode_load_named.argtypes = [vp, vp, i32, ctypes.c_char_p, i32]
+        L.cccc_decode_save_named.restype = i32; L.cccc_decode_save_named.argtypes = [vp, ctypes.c_char_p]
+        L.cccc_matrix_save_named.restype = i32; L.cccc_matrix_save_named.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
         L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
-        L.cccc_decode_bench_gate_up.restype = ctypes.c_double; L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
         self.c = L
 
     def init(self, device: int = 0) -> None:
@@ -81,17 +78,6 @@ class HostLibrary:
 
     def matrix(self, w, h, c, n, dtype) -> "HostMatrix":
         return HostMatrix(self, self.c.cccc_matrix_create(w, h, c, n, dtype))
-
-    def bench_linear_chain(self, W, X, R, steps, warmup, use_graph) -> float:
-        n = len(W)
-        arr = lambda ms: (ctypes.c_void_p * n)(*[m.handle for m in ms])
-        return float(self.c.cccc_bench_linear_chain(n, arr(W), arr(X), arr(R), steps, warmup, 1 if use_graph else 0))
-
-
-    def bench_fp4_chain(self, W_ptrs, S_ptrs, X_ptr, Y_ptr, n_out, tokens, K, block, iters, warmup) -> float:
-        n = len(W_ptrs)
-        return float(self.c.cccc_bench_fp4_chain(n, (ctypes.c_void_p * n)(*W_ptrs), (ctypes.c_void_p * n)(*S_ptrs), X_ptr, Y_ptr,
-                                                 n_out, tokens, K, block, iters, warmup))
 
 
 class WeightFile:
@@ -185,6 +171,10 @@ class HostMatrix:
     def prepare_tiled(self) -> bool:
         return self.lib.c.cccc_matrix_prepare_tiled(self.handle) == 0
 
+    def save_named(self, name: str, path) -> None:
+        if self.lib.c.cccc_matrix_save_named(self.handle, name.encode(), str(path).encode()) != 0:
+            raise OSError(f"cannot write {path}")
+
     def quantize(self, dtype: int) -> None:
         self.lib.c.cccc_matrix_quantize(self.handle, dtype)
 
@@ -259,6 +249,11 @@ class DecodeModel:
         if rc != 0:
             raise ValueError(f"loading {failed.value.decode()!r} failed: {rc}")
 
+    def save_named(self, path) -> None:
+        """Every tensor under the converter's names, bytes as they sit on the device (DecodeModel::saveNamedWeights)."""
+        if self.lib.c.cccc_decode_save_named(self.handle, str(path).encode()) != 0:
+            raise OSError(f"cannot write {path}")
+
     def set_exact_attention(self, exact: bool) -> None:
         """True: separate norm / RoPE / append launch and BF16 probabilities (the reference's rounding
         points); False (default): the two-launch attention with FP32 probabilities."""
@@ -317,13 +312,6 @@ class DecodeModel:
 
     def kv_ptr(self, layer: int, is_v: bool) -> int:
         return self.lib.c.cccc_decode_kv_data(self.handle, layer, 1 if is_v else 0)
-
-    def bench_gate_up(self, reps: int) -> float:
-        """Average microseconds per fused gate/up launch over all layers' distinct weights."""
-        us = float(self.lib.c.cccc_decode_bench_gate_up(self.handle, reps))
-        if us < 0:
-            raise RuntimeError(f"gate/up timing failed: {us}")
-        return us
 
     @property
     def weight_bytes(self) -> int:

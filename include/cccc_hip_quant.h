@@ -129,8 +129,10 @@ C_EXPORT int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K,
  * (today: up to 16 tokens, except one or two tokens on weights under 8 MiB, and the GEMM of 48 tokens or
  * more when K is a multiple of 64): the matrix-core kernels want the 16 rows x 64 codes of one load
  * instruction to be one contiguous KiB.
- * Results agree with the row-major kernels up to the FP32 summation order.  hip_quant_weight_release forgets the key (before the
- * caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (FP4, K % 16 != 0, ...).
+ * Results agree with the row-major kernels up to the FP32 summation order.  The copy is keyed on the pointer, not
+ * on the bytes behind it: after any write to W the caller must call hip_quant_weight_prepare again (or
+ * hip_quant_weight_release), otherwise later calls compute from the stale copy.  hip_quant_weight_release forgets
+ * the key (before the caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (FP4, K % 16 != 0, ...).
  */
 C_EXPORT unsigned long long hip_quant_tiled_size(int type, int n_out, int K);
 C_EXPORT int hip_quant_weight_prepare(const void* W, int type, int n_out, int K, int ldw, void* dst_tiled);

@@ -2,6 +2,7 @@
 way cccc's graph does: Matrix::mulBatched(W, X, R, TRANS, NO_TRANS) on a weight loaded with
 loadQuantizedDirect / setBlockScaleFromHost, or quantized in place with quantizeWeights."""
 import numpy as np
+from oracle import synth
 import pytest
 
 from gpu_util import check_rows
@@ -26,8 +27,8 @@ def f64(oracle, bits):
 @pytest.mark.parametrize("tokens", [1, 4, 16, 64])
 def test_mul_batched_fp8_linear(host, pkg, oracle, tokens):
     n_out, K = 768, 1024
-    Wq = pkg.synth.weights_e5m2(11, n_out, K)
-    X = pkg.synth.activations(11, tokens, K)
+    Wq = synth.weights_e5m2(11, n_out, K)
+    X = synth.activations(11, tokens, K)
     W = host.matrix(K, n_out, 1, 1, BF16)                     # allocated as the activation type, re-typed on load
     W.load_quantized(Wq, 1.0, E5M2)
     assert W.dtype == E5M2 and W.quant_scale == 1.0
@@ -52,10 +53,10 @@ def test_mul_batched_fp4_two_batches_use_per_batch_offsets(host, pkg, oracle):
     n_out, K, tokens, batch = 128, 256, 3, 2
     nib, sc, Wd = [], [], []
     for b in range(batch):
-        n, s = pkg.synth.weights_fp4(20 + b, n_out, K)
+        n, s = synth.weights_fp4(20 + b, n_out, K)
         nib.append(n); sc.append(s)
         Wd.append(oracle.dequant_weight(n, oracle.FP4, n_out, K, blk_sc=s))
-    X = pkg.synth.activations(21, tokens * batch, K).reshape(batch, tokens, K)
+    X = synth.activations(21, tokens * batch, K).reshape(batch, tokens, K)
     W = host.matrix(K, n_out, 1, batch, BF16)
     W.load_quantized(np.concatenate([n.ravel() for n in nib]), 1.0, FP4)
     W.set_block_scale(np.concatenate([s.ravel() for s in sc]))
@@ -70,7 +71,7 @@ def test_mul_batched_fp4_two_batches_use_per_batch_offsets(host, pkg, oracle):
 
 def test_quantize_weights_in_place(host, pkg, oracle):
     n_out, K = 96, 128
-    w = pkg.synth.weights_f32(30, n_out, K)                   # exactly representable in BF16
+    w = synth.weights_f32(30, n_out, K)                   # exactly representable in BF16
     wb = oracle.f32_to_bf16(w)
     # FP8: per-tensor absmax scale, truncating encoder
     for target, top in ((E5M2, 57344.0), (E4M3, 448.0)):
@@ -97,8 +98,8 @@ def test_quantize_weights_in_place(host, pkg, oracle):
 
 def test_quantized_then_multiplied_matches_the_oracle(host, pkg, oracle):
     n_out, K, tokens = 256, 512, 2
-    w = pkg.synth.weights_f32(31, n_out, K)
-    X = pkg.synth.activations(31, tokens, K)
+    w = synth.weights_f32(31, n_out, K)
+    X = synth.activations(31, tokens, K)
     W = host.matrix(K, n_out, 1, 1, BF16); W.upload(oracle.f32_to_bf16(w))
     W.quantize(E5M2)
     codes = W.download(np.uint8, w.size).reshape(n_out, K)
@@ -119,3 +120,37 @@ def test_tracked_allocations_are_released(host, pkg):
     assert host.c.cccc_gpu_allocated_bytes() == base + 2 * 1024 * 1024
     del m
     assert host.c.cccc_gpu_allocated_bytes() == base
+
+
+def test_rewriting_a_prepared_weight_drops_its_tiled_copy(gpu, pkg, oracle):
+    """The tiled copy is keyed on the weight's pointer: every host path that writes the storage (a second
+    loadQuantizedDirect into the same allocation, a raw upload) must drop it, or the matrix-core GEMV would keep
+    computing from the old bytes."""
+    torch, dev, lib = gpu
+    host = pkg.host_api.host()
+    host.init(0)
+    host.set_repack(True)
+    n_out, K, tokens = 1024, 2048, 4
+    X = synth.activations(51, tokens, K)
+    xm = host.matrix(K, tokens, 1, 1, BF16)
+    xm.upload(X)
+    ym = host.matrix(n_out, tokens, 1, 1, BF16)
+    first, second, third = (synth.weights_e5m2(52 + i, n_out, K) for i in range(3))
+    wm = host.matrix(K, n_out, 1, 1, E5M2)
+
+    def run(codes, expect_kernel):
+        assert pkg.host_api.mul_batched(wm, xm, ym, ta=1, tb=0) == 0
+        assert lib.last_kernel() == expect_kernel
+        want = oracle.linear_exact(oracle.dequant_weight(codes, oracle.E5M2, n_out, K), X)
+        check_rows(oracle.bf16_to_f32(ym.download(np.uint16, tokens * n_out).reshape(tokens, n_out)).astype(np.float64), want, expect_kernel)
+
+    wm.load_quantized(first, 1.0, E5M2)
+    ptr = wm.data_ptr
+    run(first, "gemv_mfma_tiled")
+    wm.load_quantized(second, 1.0, E5M2)                 # same allocation, new bytes: a new tiled copy of the new bytes
+    assert wm.data_ptr == ptr
+    run(second, "gemv_mfma_tiled")
+    wm.upload(third)                                     # raw write: the copy is dropped, the row-major kernel reads the new bytes
+    run(third, "gemv_dot2")
+    assert wm.prepare_tiled()
+    run(third, "gemv_mfma_tiled")

@@ -3,6 +3,7 @@ DecodeModel::loadNamedWeights, against tensors set directly and against the CPU 
 import struct
 
 import numpy as np
+from oracle import synth, weight_file
 import pytest
 
 from gpu_util import check_rows
@@ -30,11 +31,11 @@ def test_fp8_and_fp4_weights_load_like_direct_uploads(tmp_path, gpu, pkg, host, 
     rng = np.random.default_rng(0)
     K, n_out = 512, 96
     x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
-    w = pkg.weight_file.BinWriter()
+    w = weight_file.BinWriter()
     codes8 = oracle.encode_e5m2_rne((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32))
     w.add("weight_fp8_e5m2_W_a", codes8); w.add_float("scale_W_a", 0.5); w.add_float("input_scale_W_a", 0.25)
     w.add("weight_W_legacy", codes8 & 0x7E)                                           # legacy key: FP8_E4M3, no scale entry -> 1.0
-    nib, sc = pkg.synth.pack_fp4_blockscale((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32), 16)
+    nib, sc = synth.pack_fp4_blockscale((rng.standard_normal((n_out, K)) * 0.02).astype(np.float32), 16)
     w.add("weight_fp4_e2m1_W_b", nib); w.add("blockscale_W_b", sc)
     w.add("weight_fp4_e2m1_W_c", nib); w.add("blockscale_W_c", np.concatenate([sc, np.full(sc.size, 0x7E, np.uint8)]))   # twice the scale bytes, as the reference's own writer leaves them
     sc_f32 = oracle.decode_table(E4M3)[sc].astype(np.float32)
@@ -71,7 +72,7 @@ def test_plain_weights_keep_or_convert_their_type(tmp_path, gpu, pkg, host, orac
     rng = np.random.default_rng(1)
     n = 4096
     vals = rng.standard_normal(n).astype(np.float32)
-    w = pkg.weight_file.BinWriter()
+    w = weight_file.BinWriter()
     w.add("weight_bf16_P", oracle.f32_to_bf16(vals))
     w.add("weight_half_Q", vals.astype(np.float16))
     w.add("weight_float_R", vals)
@@ -103,7 +104,7 @@ def test_decode_model_from_an_fp8_file_equals_direct_tensors(tmp_path, gpu, pkg,
     cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=64)
     weights = dec.make_model(cfg, 21)
     path = tmp_path / "model_fp8.bin"
-    pkg.weight_file.write_decode_model(path, weights, "fp8_e5m2")
+    weight_file.write_decode_model(path, weights, "fp8_e5m2")
     a, b = make_model(pkg, host, cfg), make_model(pkg, host, cfg)
     a.load(weights)
     b.load_named(pkg.host_api.WeightFile(host, path))
@@ -113,7 +114,7 @@ def test_decode_model_from_an_fp8_file_equals_direct_tensors(tmp_path, gpu, pkg,
         assert a.step() == b.step()
     assert np.array_equal(a.logits(), b.logits())
     # a file without some tensor is refused with its name
-    w = pkg.weight_file
+    w = weight_file
     path2 = tmp_path / "broken.bin"
     full = w.read_index(path)[0]
     bw = w.BinWriter()
@@ -140,7 +141,7 @@ def test_decode_model_quantizes_a_bf16_file_on_load(tmp_path, gpu, pkg, host, or
     file_model = {"emb": base["emb"], "rms_final": base["rms_final"], "lm_head": bf16_weight(base["lm_head"].shape),
                   "layers": [{k: (bf16_weight(v.shape) if k in linears else v) for k, v in base["layers"][0].items()}]}
     path = tmp_path / "model_bf16.bin"
-    pkg.weight_file.write_decode_model(path, file_model, "bf16")
+    weight_file.write_decode_model(path, file_model, "bf16")
     model = make_model(pkg, host, cfg)
     model.load_named(pkg.host_api.WeightFile(host, path), E5M2)
 
@@ -179,3 +180,119 @@ def test_decode_model_quantizes_a_bf16_file_on_load(tmp_path, gpu, pkg, host, or
         want_logits, token = orc.step(token, pos)
         got_logits = dec.f(model.logits())
         assert np.linalg.norm(got_logits - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+
+
+def test_quantize_on_load_then_save_then_reload_is_identical(tmp_path, gpu, pkg, host, oracle, dec):
+    """The weight_data_type + save_fp8_file route (cccc/MainProcess.cpp:362-378): a BF16 file is quantized on load,
+    DecodeModel::saveNamedWeights writes the cache, and a second model loaded from the cache holds the same bytes and
+    scales and decodes the same tokens without quantizing anything."""
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=500, t_kv=32)
+    rng = np.random.default_rng(9)
+    base = dec.make_model(cfg, 6)
+    linears = {"wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"}
+    bf16_weight = lambda shape: oracle.f32_to_bf16((rng.standard_normal(shape) * 0.02).astype(np.float32))
+    file_model = {"emb": base["emb"], "rms_final": base["rms_final"], "lm_head": bf16_weight(base["lm_head"].shape),
+                  "layers": [{k: (bf16_weight(v.shape) if k in linears else v) for k, v in L.items()} for L in base["layers"]]}
+    src = tmp_path / "model_bf16.bin"
+    weight_file.write_decode_model(src, file_model, "bf16")
+    a = make_model(pkg, host, cfg)
+    a.load_named(pkg.host_api.WeightFile(host, src), E5M2)
+    cache = tmp_path / "cache_fp8.bin"
+    a.save_named(cache)
+
+    # what the cache holds: header, typed keys, one float32 scale per quantized tensor, raw sizes
+    index, _ = weight_file.read_index(cache)
+    assert list(index)[:2] == ["data_type", "named_weights"] and weight_file.read_entry(cache, "data_type") == b"fp8_e5m2"
+    assert index["weight_bf16_W_emb"][1] == cfg.vocab * cfg.hidden * 2
+    assert index["weight_fp8_e5m2_W_lm_head"][1] == cfg.vocab * cfg.hidden and index["scale_W_lm_head"][1] == 4
+    for i in range(cfg.layers):
+        for name, n in (("W_q", cfg.q_out * cfg.hidden), ("W_k", cfg.kv_out * cfg.hidden), ("W_down", cfg.hidden * cfg.inter)):
+            assert index[f"weight_fp8_e5m2_{name}_{i}"][1] == n and index[f"scale_{name}_{i}"][1] == 4
+        assert index[f"weight_bf16_W_rms_attn_{i}"][1] == cfg.hidden * 2 and f"scale_W_rms_attn_{i}" not in index
+    # the saved scale is absmax / 57344 of the BF16 tensor, the saved codes its truncating quantization
+    w = oracle.bf16_to_f32(file_model["layers"][1]["w_down"])
+    amax = np.float32(np.abs(w).max())
+    assert struct.unpack("<f", weight_file.read_entry(cache, "scale_W_down_1"))[0] == np.float32(amax / np.float32(57344.0))
+    rc, codes = oracle.convert(w.reshape(-1), 0, 5, w.size, float(np.float32(57344.0) / amax))
+    assert rc == 0 and weight_file.read_entry(cache, "weight_fp8_e5m2_W_down_1") == codes.tobytes()
+
+    b = make_model(pkg, host, cfg)
+    b.load_named(pkg.host_api.WeightFile(host, cache), E5M2)
+    recache = tmp_path / "cache_again.bin"
+    b.save_named(recache)
+    assert cache.read_bytes() == recache.read_bytes()                     # same bytes, same scales, same order
+    for m in (a, b):
+        m.reset(11, 0)
+    for _ in range(6):
+        assert a.step() == b.step()
+    assert np.array_equal(a.logits(), b.logits())
+
+
+def test_fp4_matrix_saves_packed_codes_and_block_scales(tmp_path, gpu, pkg, host, oracle):
+    """quantizeWeights(FP4) on the device, then the named-weight writer: packed nibbles sized (elements + 1) / 2,
+    one E4M3 byte per 16 elements, both equal to the oracle's on-the-fly quantiser; reloading gives the same GEMV."""
+    K, n_out = 256, 80
+    w = synth.weights_f32(41, n_out, K)
+    m = host.matrix(K, n_out, 1, 1, BF16)
+    m.upload(oracle.f32_to_bf16(w))
+    m.quantize(FP4)
+    assert m.dtype == FP4
+    path = tmp_path / "fp4.bin"
+    m.save_named("W_x", path)
+    index, _ = weight_file.read_index(path)
+    assert index["weight_fp4_e2m1_W_x"][1] == n_out * K // 2 and index["blockscale_W_x"][1] == n_out * K // 16 and "scale_W_x" not in index
+    nib, sc = oracle.quantize_fp4_blockscale_kernel(w, 16)
+    assert weight_file.read_entry(path, "weight_fp4_e2m1_W_x") == nib.tobytes()
+    assert weight_file.read_entry(path, "blockscale_W_x") == sc.tobytes()
+    back = host.matrix(K, n_out, 1, 1, BF16)
+    assert pkg.host_api.WeightFile(host, path).load_named(back, "W_x") == 0 and back.dtype == FP4
+    x = synth.activations(41, 1, K)[0]
+    assert np.array_equal(linear_out(pkg, host, m, x, n_out, K), linear_out(pkg, host, back, x, n_out, K))
+
+
+def test_mixed_fp8_formats_in_one_file(tmp_path, gpu, pkg, host, oracle, dec):
+    """k stored as FP8_E4M3 with a scale next to E5M2 q and v: the step decodes each projection with its own format
+    (three launches instead of one).  Gate and up in two formats are refused by name."""
+    cfg = dec.DecodeConfig(layers=1, hidden=256, n_q=4, n_kv=2, inter=512, vocab=300, t_kv=16)
+    weights = dec.make_model(cfg, 31)
+    path = tmp_path / "mixed.bin"
+    weight_file.write_decode_model(path, weights, "fp8_e5m2")
+    wk_f32 = oracle.decode_table(oracle.E5M2)[weights["layers"][0]["wk"]]
+    scale = float(np.abs(wk_f32).max()) / 448.0
+    wk_e4m3 = oracle.encode_e4m3_rne((wk_f32 / np.float32(scale)).astype(np.float32))
+
+    def rewrite(replace_key, new_key, codes, scale_key):
+        bw = weight_file.BinWriter()
+        for k in weight_file.read_index(path)[0]:
+            if k == replace_key:
+                bw.add(new_key, codes)
+                bw.add_float(scale_key, scale)
+            else:
+                bw.add(k, weight_file.read_entry(path, k))
+        out = tmp_path / (new_key + ".bin")
+        bw.save(out)
+        return out
+
+    mixed = rewrite("weight_fp8_e5m2_W_k_0", "weight_fp8_e4m3_W_k_0", wk_e4m3, "scale_W_k_0")
+    model = make_model(pkg, host, cfg)
+    model.load_named(pkg.host_api.WeightFile(host, mixed))
+    model.set_exact_attention(True)
+
+    class MixedOracle(dec.DecodeOracle):
+        def deq(self, layer, name):
+            if name == "wk":
+                return oracle.dequant_fp8_to_bf16(wk_e4m3, oracle.E4M3, scale).reshape(wk_e4m3.shape)
+            return super().deq(layer, name)
+
+    orc = MixedOracle(cfg, weights)
+    token = 4
+    for pos in range(3):
+        model.reset(token, pos)
+        model.step()
+        want_logits, token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+    up_f32 = oracle.decode_table(oracle.E5M2)[weights["layers"][0]["w_up"]]
+    bad = rewrite("weight_fp8_e5m2_W_up_0", "weight_fp8_e4m3_W_up_0", oracle.encode_e4m3_rne((up_f32 / np.float32(scale)).astype(np.float32)), "scale_W_up_0")
+    with pytest.raises(ValueError, match="W_up_0"):
+        make_model(pkg, host, cfg).load_named(pkg.host_api.WeightFile(host, bad))
