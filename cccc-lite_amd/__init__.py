@@ -9,4 +9,4 @@ The directory name is not a Python identifier; load it as module `cccc_lite_amd`
 `__graft_entry__.load_package()`.
 """
 from .capi import DataType, QuantLibrary, library, library_path  # noqa: F401
-from . import host_api, synth, weight_file  # noqa: F401
+from . import host_api  # noqa: F401

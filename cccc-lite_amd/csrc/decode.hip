@@ -147,7 +147,11 @@ int hip_rms_norm_fwd(int type, void* X, void* Y, void* scale, void* invstd_out, 
         fprintf(stderr, "hip_rms_norm_fwd: null pointer\n");
         return 1;
     }
-    rms_norm_bf16_kernel<<<outer, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)scale, (float*)invstd_out, inner, epsilon);
+    const uint16_t *x = (const uint16_t*)X, *w = (const uint16_t*)scale;
+    uint16_t* y = (uint16_t*)Y;
+    if (inner > 64u * 8u * RMS_CHUNKS) { rms_norm_long_rows_kernel<<<outer, 256, 0, stream()>>>(x, y, w, (float*)invstd_out, inner, epsilon); }
+    else if (inner % 8 == 0 && aligned16(X) && aligned16(Y) && aligned16(scale)) { rms_norm_rows_kernel<true><<<(outer + 3) / 4, 256, 0, stream()>>>(x, y, w, (float*)invstd_out, outer, inner, epsilon); }
+    else { rms_norm_rows_kernel<false><<<(outer + 3) / 4, 256, 0, stream()>>>(x, y, w, (float*)invstd_out, outer, inner, epsilon); }
     return finish("rms_norm_fwd_bf16");
 }
 
@@ -170,7 +174,10 @@ int hip_rope_fwd(int type, const void* X, void* Y, const void* cos_tab, const vo
         fprintf(stderr, "hip_rope_fwd: null pointer\n");
         return 1;
     }
-    rope_bf16_kernel<<<(total + 255) / 256, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, D, T, B, pos_offset);
+    const bool vec = (D / 2) % 8 == 0 && aligned16(X) && aligned16(Y) && aligned16(cos_tab) && aligned16(sin_tab);
+    const unsigned items = vec ? total / 8 : total;
+    if (vec) { rope_rows_kernel<true><<<(items + 255) / 256, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, D, T, T * B, pos_offset); }
+    else { rope_rows_kernel<false><<<(items + 255) / 256, 256, 0, stream()>>>((const uint16_t*)X, (uint16_t*)Y, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, D, T, T * B, pos_offset); }
     return finish("rope_fwd_bf16");
 }
 

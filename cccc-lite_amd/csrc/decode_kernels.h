@@ -483,42 +483,124 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_mfma_kernel(const Fuse
 // ------------------------------------------------------------------------------------------
 // Standalone neighbours with the reference's signatures (BF16)
 
-static __global__ __launch_bounds__(256) void rms_norm_bf16_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ Y, const uint16_t* __restrict__ scale,
-                                                           float* __restrict__ invstd_out, unsigned inner, float eps)
+// RMSNorm of `outer` rows of `inner` BF16 values, one wave per row while a row fits the wave's registers
+// (inner <= 64 lanes x 8 values x RMS_CHUNKS), four rows per 256-thread workgroup: 128-bit loads, the row stays in
+// registers between the sum of squares and the scaling, the 64-lane sum is the DPP reduction.  Used for the per-head
+// norms (inner = 128) as well as whole hidden vectors up to 4096.  VEC = false: rows that are not whole 16-byte chunks
+// (or misaligned pointers) take the same structure with scalar accesses.
+constexpr int RMS_CHUNKS = 8;
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void rms_norm_rows_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ Y, const uint16_t* __restrict__ scale,
+                                                           float* __restrict__ invstd_out, unsigned outer, unsigned inner, float eps)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= outer) { return; }
+    const uint16_t* x = X + (size_t)row * inner;
+    uint16_t* y = Y + (size_t)row * inner;
+    float sumsq = 0.0f;
+    if constexpr (VEC)
+    {
+        const unsigned n_chunks = inner / 8u;               // 16-byte chunks of the row; chunk c belongs to lane c % 64
+        u32x4 v[RMS_CHUNKS];
+#pragma unroll
+        for (int j = 0; j < RMS_CHUNKS; j++)
+        {
+            const unsigned c = lane + 64u * j;
+            v[j] = u32x4{ 0u, 0u, 0u, 0u };
+            if (c < n_chunks) { v[j] = *(const u32x4*)(x + c * 8u); }
+            sumsq += sumsq8(v[j]);
+        }
+        const float invstd = rsqrtf(wave_sum(sumsq) / (float)inner + eps);
+        if (lane == 0 && invstd_out) { invstd_out[row] = invstd; }
+#pragma unroll
+        for (int j = 0; j < RMS_CHUNKS; j++)
+        {
+            const unsigned c = lane + 64u * j;
+            if (c < n_chunks) { *(u32x4*)(y + c * 8u) = normed8(v[j], *(const u32x4*)(scale + c * 8u), invstd); }
+        }
+    }
+    else
+    {
+        for (unsigned i = lane; i < inner; i += 64u)
+        {
+            const float f = bf16_bits_to_f32(x[i]);
+            sumsq = fmaf(f, f, sumsq);
+        }
+        const float invstd = rsqrtf(wave_sum(sumsq) / (float)inner + eps);
+        if (lane == 0 && invstd_out) { invstd_out[row] = invstd; }
+        for (unsigned i = lane; i < inner; i += 64u) { y[i] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(x[i]) * invstd * bf16_bits_to_f32(scale[i])); }
+    }
+}
+
+// Half-rotate RoPE of B x T heads of D values: lane = (head row, group of eight rotation pairs), so the left half, the
+// right half and the two table rows each arrive as one 128-bit load per lane and leave as one 128-bit store (D / 2 a
+// multiple of 8, the model case D = 128: eight lanes per head row); any other D takes one pair per lane.
+// Table row of head row r is (r % T) + pos_offset.
+template <bool VEC>
+__global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ Y, const uint16_t* __restrict__ cos_tab,
+                                                       const uint16_t* __restrict__ sin_tab, unsigned D, unsigned T, unsigned n_rows, unsigned pos_offset)
+{
+    const unsigned half = D / 2u;
+    const unsigned per_row = VEC ? half / 8u : half;         // work items per head row
+    const unsigned item = blockIdx.x * 256u + threadIdx.x;
+    const unsigned r = item / per_row;
+    if (r >= n_rows) { return; }
+    const unsigned p = (item - r * per_row) * (VEC ? 8u : 1u);      // first pair of this item
+    const uint16_t* x = X + (size_t)r * D + p;
+    uint16_t* y = Y + (size_t)r * D + p;
+    const size_t t = (size_t)(r % T + pos_offset) * half + p;
+    if constexpr (VEC)
+    {
+        const u32x4 l = *(const u32x4*)x, rt = *(const u32x4*)(x + half);
+        const u32x4 c = *(const u32x4*)(cos_tab + t), sn = *(const u32x4*)(sin_tab + t);
+        u32x4 ol, orr;
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+        {
+            uint32_t lo[2], hi[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+            {
+                const int sh = 16 * h;
+                const float a = bf16_bits_to_f32((l[d] >> sh) & 0xFFFFu), b = bf16_bits_to_f32((rt[d] >> sh) & 0xFFFFu);
+                const float cc = bf16_bits_to_f32((c[d] >> sh) & 0xFFFFu), ss = bf16_bits_to_f32((sn[d] >> sh) & 0xFFFFu);
+                lo[h] = f32_to_bf16_bits(a * cc - b * ss);
+                hi[h] = f32_to_bf16_bits(b * cc + a * ss);
+            }
+            ol[d] = lo[0] | (lo[1] << 16);
+            orr[d] = hi[0] | (hi[1] << 16);
+        }
+        *(u32x4*)y = ol;
+        *(u32x4*)(y + half) = orr;
+    }
+    else
+    {
+        const float a = bf16_bits_to_f32(x[0]), b = bf16_bits_to_f32(x[half]);
+        const float cc = bf16_bits_to_f32(cos_tab[t]), ss = bf16_bits_to_f32(sin_tab[t]);
+        y[0] = (uint16_t)f32_to_bf16_bits(a * cc - b * ss);
+        y[half] = (uint16_t)f32_to_bf16_bits(b * cc + a * ss);
+    }
+}
+
+// Rows longer than one wave's registers: a 256-thread workgroup per row, two passes over the row (the second one
+// comes out of the cache), block-wide sum through LDS.
+static __global__ __launch_bounds__(256) void rms_norm_long_rows_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ Y, const uint16_t* __restrict__ scale,
+                                                                float* __restrict__ invstd_out, unsigned inner, float eps)
 {
     __shared__ float red[4];
     const uint16_t* x = X + (size_t)blockIdx.x * inner;
     uint16_t* y = Y + (size_t)blockIdx.x * inner;
     float sumsq = 0.0f;
-    for (unsigned i = threadIdx.x; i < inner; i += 256)
+    for (unsigned i = threadIdx.x; i < inner; i += 256u)
     {
-        const float v = bf16_bits_to_f32(x[i]);
-        sumsq += v * v;
+        const float f = bf16_bits_to_f32(x[i]);
+        sumsq = fmaf(f, f, sumsq);
     }
     const float invstd = rsqrtf(block_sum<256>(sumsq, red) / (float)inner + eps);
     if (threadIdx.x == 0 && invstd_out) { invstd_out[blockIdx.x] = invstd; }
-    for (unsigned i = threadIdx.x; i < inner; i += 256)
-    {
-        const float sc = scale ? bf16_bits_to_f32(scale[i]) : 1.0f;
-        y[i] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(x[i]) * invstd * sc);
-    }
-}
-
-static __global__ __launch_bounds__(256) void rope_bf16_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ Y, const uint16_t* __restrict__ cos_tab,
-                                                       const uint16_t* __restrict__ sin_tab, unsigned D, unsigned T, unsigned B, unsigned pos_offset)
-{
-    const unsigned half_d = D / 2;
-    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= half_d * T * B) { return; }
-    const unsigned i = idx % half_d;
-    const unsigned bt = idx / half_d;
-    const unsigned t = bt % T;
-    const size_t base = (size_t)bt * D;
-    const size_t tab = (size_t)(t + pos_offset) * half_d + i;
-    const float c = bf16_bits_to_f32(cos_tab[tab]), s = bf16_bits_to_f32(sin_tab[tab]);
-    const float xl = bf16_bits_to_f32(X[base + i]), xr = bf16_bits_to_f32(X[base + half_d + i]);
-    Y[base + i] = (uint16_t)f32_to_bf16_bits(xl * c - xr * s);
-    Y[base + half_d + i] = (uint16_t)f32_to_bf16_bits(xr * c + xl * s);
+    for (unsigned i = threadIdx.x; i < inner; i += 256u) { y[i] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(x[i]) * invstd * bf16_bits_to_f32(scale[i])); }
 }
 
 // Embedding row copy: Y[t] = W[(int)ids[t]] (ids are floats in the reference); `d_token`, when given,

@@ -245,97 +245,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_kernel(const LinearArgs
 }
 
 // ------------------------------------------------------------------------------------------
-// FP8 GEMV, dot2 + DPP reduction, activations straight from global memory (no LDS, no barrier):
-// every lane loads the 32 bytes of x it needs per k-step itself; the 8..24 KiB activation vector is
-// shared by all waves and stays in the vector L1 / L2.  For MT == 1 only.
-
-template <int WT, int R, int U, int WAVES, bool SCALED, bool SKIP_MATH>
-__global__ __launch_bounds__(WAVES * 64) void gemv8_dot2_direct_kernel(const LinearArgs a)
-{
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int n_steps = (a.K + 1023) / 1024;
-    const int n_groups = (a.n_out + R - 1) / R;
-    const int last_row = a.n_out - 1;
-
-    for (int g = blockIdx.x * WAVES + wave; g < n_groups; g += gridDim.x * WAVES)
-    {
-        const uint8_t* wrow[R];
-#pragma unroll
-        for (int r = 0; r < R; r++)
-        {
-            const int row = min(g * R + r, last_row);
-            wrow[r] = a.W + (long long)row * a.ldw + lane * 16;
-        }
-        float acc[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) { acc[r] = 0.0f; }
-
-        for (int s0 = 0; s0 < n_steps; s0 += U)
-        {
-            u32x4 w[U][R];
-            u32x4 x[U][2];
-#pragma unroll
-            for (int u = 0; u < U; u++)
-            {
-                const int k = (s0 + u) * 1024 + lane * 16;
-                x[u][0] = x[u][1] = u32x4{ 0u, 0u, 0u, 0u };
-                if (k < a.K)
-                {
-                    x[u][0] = *(const u32x4*)(a.X + k);
-                    x[u][1] = *(const u32x4*)(a.X + k + 8);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++)
-            {
-                const int k = (s0 + u) * 1024 + lane * 16;
-#pragma unroll
-                for (int r = 0; r < R; r++)
-                {
-                    w[u][r] = u32x4{ 0u, 0u, 0u, 0u };
-                    if (k < a.K) { w[u][r] = __builtin_nontemporal_load((const u32x4*)(wrow[r] + (s0 + u) * 1024)); }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++)
-            {
-#pragma unroll
-                for (int r = 0; r < R; r++)
-                {
-                    if (SKIP_MATH)
-                    {
-                        acc[r] += __builtin_bit_cast(float, (w[u][r][0] ^ w[u][r][1] ^ w[u][r][2] ^ w[u][r][3] ^ x[u][0][0]) & 0x3F800000u);
-                    }
-                    else
-                    {
-#pragma unroll
-                        for (int d = 0; d < 4; d++)
-                        {
-                            bf16x2 p01, p23;
-                            fp8x4_to_bf16<WT, SCALED>(w[u][r][d], a.w_scale, p01, p23);
-                            acc[r] = dot2_bf16(p01, x[u][d >> 1][(d & 1) * 2 + 0], acc[r]);
-                            acc[r] = dot2_bf16(p23, x[u][d >> 1][(d & 1) * 2 + 1], acc[r]);
-                        }
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++)
-        {
-            const float total = wave_sum(acc[r]);
-            const int row = g * R + r;
-            if (lane == 0 && row < a.n_out)
-            {
-                uint16_t* y = a.Y + (long long)row * a.y_stride_out;
-                *y = finish_output(total, a.alpha, a.beta, y);
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
 // FP8 GEMV, dot2 + DPP reduction, software pipelined.  Same decomposition as gemv8_dot2_kernel, but
 // the (row group, k trip) pairs a wave walks are flattened into one sequence and the 128-bit loads
 // of the next pair are issued before the current pair is multiplied, so every wave always has

@@ -1,4 +1,5 @@
-"""Synthetic weights and activations of the benchmark configurations (seeded, reproducible).
+"""Synthetic weights and activations of the benchmark configurations (seeded, reproducible).  DATA MAKER for tests,
+the smoke test and the benchmark's CPU leg; not part of the shipped package.
 
 Weights: float32 N(0, 0.02) -> BF16 (RNE) -> FP8_E5M2 (RNE) with no extra scale, or the offline
 converter's FP4 block-scale packing (reference scripts/convert_weights.py:346-370, restated here

@@ -2,9 +2,9 @@
 
 Layout as scripts/convert_weights.py:54-83 writes it: 32 bytes "CFG_BIN INI" zero-padded, a
 little-endian uint64 with the length of the index text, the index text (ASCII lines
-"<key> = <offset>,<length>", offsets relative to the data area), then the data area.  The C++ reader
-the product uses is host/WeightFile.cpp; this module makes files for tests and tools and reads them
-back without the native library.
+"<key> = <offset>,<length>", offsets relative to the data area), then the data area.  The C++ reader and
+writer the product uses are cccc-lite_amd/host/WeightFile.cpp; this module is test infrastructure: it makes
+files for tests and reads them back without the native library.
 """
 from __future__ import annotations
 

@@ -6,6 +6,7 @@ sees the very bytes the kernels read, downloaded for the sampled rows."""
 import ctypes
 
 import numpy as np
+from oracle import synth
 import pytest
 
 from gpu_util import check_bf16_close, check_rows, from_dev, to_dev
@@ -61,7 +62,7 @@ def test_tiled_gemv_at_the_qwen3_8b_shapes(gpu, pkg, oracle, K, n_out):
         W_rows = wd[torch.from_numpy(rows).to(dev)].cpu().numpy()
         Wd_rows = oracle.dequant_fp8_to_bf16(W_rows, oracle.E5M2).reshape(W_rows.shape)
         for tokens in (1, 4, 16):
-            X = pkg.synth.activations(n_out + tokens, tokens, K)
+            X = synth.activations(n_out + tokens, tokens, K)
             xd = to_dev(torch, dev, X)
             yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
             assert lib.linear(wd.data_ptr(), E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
@@ -122,7 +123,7 @@ def test_fp4_gemv_at_the_llama_8b_shapes(gpu, pkg, oracle, K, n_out, block):
         w = (torch.randn(r, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16).to(torch.float32)
         nib[r0:r0 + r], sc[r0:r0 + r] = pack_fp4_on_device(torch, w, block)
         if r0 == 0:
-            want_nib, want_sc = pkg.synth.pack_fp4_blockscale(w[:64].cpu().numpy(), block)
+            want_nib, want_sc = synth.pack_fp4_blockscale(w[:64].cpu().numpy(), block)
             bad_nib = int((nib[:64].cpu().numpy().ravel() != want_nib).sum())
             bad_sc = int((sc[:64].cpu().numpy().ravel() != want_sc).sum())
             assert bad_nib == 0 and bad_sc == 0, f"device packer differs from the host packer: {bad_nib} code bytes, {bad_sc} scale bytes"
@@ -131,7 +132,7 @@ def test_fp4_gemv_at_the_llama_8b_shapes(gpu, pkg, oracle, K, n_out, block):
     nib_rows, sc_rows = nib[ridx].cpu().numpy(), sc[ridx].cpu().numpy()
     Wd_rows = oracle.dequant_weight(nib_rows, oracle.FP4, len(rows), K, blk_sc=sc_rows, block=block)
     for tokens in (1, 4):
-        X = pkg.synth.activations(n_out + tokens, tokens, K)
+        X = synth.activations(n_out + tokens, tokens, K)
         xd = to_dev(torch, dev, X)
         yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
         assert lib.linear(nib.data_ptr(), FP4, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, blk_sc=sc.data_ptr(), block_size=block) == 0

@@ -2,6 +2,7 @@
 oracle, through the C-ABI.  Expected values are the exact float64 contraction of the bit-exact
 dequantized BF16 weights (oracle.linear_exact); tolerances are the benchmark's (gpu_util)."""
 import numpy as np
+from oracle import synth
 import pytest
 
 from gpu_util import check_bf16_close, check_rows, from_dev, to_dev
@@ -44,9 +45,9 @@ def test_golden_linear_cases(gpu, pkg, oracle, golden_linear):
 @pytest.mark.parametrize("tokens", [1, 2, 3, 4, 5, 8, 16])
 @pytest.mark.parametrize("n_out,K", [(4096, 4096), (1024, 4096), (768, 12288), (1000, 2064), (7, 16)])
 def test_fp8_gemv_vs_oracle(gpu, pkg, oracle, tokens, n_out, K):
-    seed = pkg.synth.seed_for(2, n_out % 97 + tokens)
-    W = pkg.synth.weights_e5m2(seed, n_out, K)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(2, n_out % 97 + tokens)
+    W = synth.weights_e5m2(seed, n_out, K)
+    X = synth.activations(seed, tokens, K)
     y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K)
     want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X)
     check_rows(bf16_f64(oracle, y), want, f"{kernel} {n_out}x{K} M={tokens}")
@@ -94,14 +95,14 @@ def test_every_code_dequantizes_exactly_inside_the_gemv(gpu, pkg, oracle, tokens
 def test_per_tensor_scale_rounds_the_weight_to_bf16(gpu, pkg, oracle, tokens, w_type_name):
     """With invScale != 1 the weight entering the product is bf16(decode * invScale)."""
     n_out, K = 512, 1024
-    seed = pkg.synth.seed_for(2, 40 + tokens)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(2, 40 + tokens)
+    X = synth.activations(seed, tokens, K)
     if w_type_name == "e5m2":
-        wf = pkg.synth.weights_f32(seed, n_out, K)
+        wf = synth.weights_f32(seed, n_out, K)
         inv = float(np.abs(wf).max()) / 57344.0
         W, w_type = oracle.encode_e5m2_rne(wf / np.float32(inv)), oracle.E5M2
     else:
-        W, inv = pkg.synth.weights_e4m3(seed, n_out, K)
+        W, inv = synth.weights_e4m3(seed, n_out, K)
         w_type = oracle.E4M3
     y, kernel = run_linear(gpu, pkg, W, w_type, X, n_out, tokens, K, inv_scale=inv)
     want = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K, inv), X)
@@ -115,10 +116,10 @@ def test_per_tensor_scale_rounds_the_weight_to_bf16(gpu, pkg, oracle, tokens, w_
 def test_alpha_beta_epilogue(gpu, pkg, oracle):
     n_out, K = 640, 2048
     for tokens in (1, 4, 12, 48):
-        seed = pkg.synth.seed_for(2, 60 + tokens)
-        W = pkg.synth.weights_e5m2(seed, n_out, K)
-        X = pkg.synth.activations(seed, tokens, K)
-        Y0 = pkg.synth.activations(seed + 1, tokens, n_out)
+        seed = synth.seed_for(2, 60 + tokens)
+        W = synth.weights_e5m2(seed, n_out, K)
+        X = synth.activations(seed, tokens, K)
+        Y0 = synth.activations(seed + 1, tokens, n_out)
         y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K, alpha=0.5, beta=-2.0, Y0=Y0)
         want = 0.5 * oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X) - 2.0 * bf16_f64(oracle, Y0)
         check_rows(bf16_f64(oracle, y), want, kernel)
@@ -130,9 +131,9 @@ def test_alpha_beta_epilogue(gpu, pkg, oracle):
 @pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("n_out,K", [(4096, 4096), (1024, 4096), (512, 14336), (33, 64)])
 def test_fp4_gemv_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, block):
-    seed = pkg.synth.seed_for(3, n_out % 89 + tokens + block)
-    nib, sc = pkg.synth.weights_fp4(seed, n_out, K, block)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(3, n_out % 89 + tokens + block)
+    nib, sc = synth.weights_fp4(seed, n_out, K, block)
+    X = synth.activations(seed, tokens, K)
     y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, K, blk_sc=sc, block=block)
     want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block), X)
     check_rows(bf16_f64(oracle, y), want, f"{kernel} fp4 {n_out}x{K} M={tokens} b={block}")
@@ -161,11 +162,11 @@ def test_fp4_every_nibble_and_scale_inside_the_gemv(gpu, pkg, oracle):
 @pytest.mark.parametrize("tokens,n_out,K", [(128, 256, 512), (512, 768, 1024), (130, 200, 144), (17, 128, 64), (2048, 256, 256)])
 @pytest.mark.parametrize("fmt", ["e5m2", "fp4_16", "fp4_32"])
 def test_prefill_gemm_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, fmt):
-    seed = pkg.synth.seed_for(4, tokens % 83 + n_out % 7)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(4, tokens % 83 + n_out % 7)
+    X = synth.activations(seed, tokens, K)
     expect = "gemm_mfma"
     if fmt == "e5m2":
-        W = pkg.synth.weights_e5m2(seed, n_out, K)
+        W = synth.weights_e5m2(seed, n_out, K)
         y, kernel = run_linear(gpu, pkg, W, oracle.E5M2, X, n_out, tokens, K)
         Wd = oracle.dequant_weight(W, oracle.E5M2, n_out, K)
     else:
@@ -174,9 +175,9 @@ def test_prefill_gemm_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, fmt):
             # rows that are not whole 32-element loads (with blocks of 32 they even straddle rows: the scales run over
             # the flat element index) are served by the generic kernel
             expect = "generic"
-            nib, sc = pkg.synth.pack_fp4_blockscale(pkg.synth.weights_f32(seed, n_out, K), block)
+            nib, sc = synth.pack_fp4_blockscale(synth.weights_f32(seed, n_out, K), block)
         else:
-            nib, sc = pkg.synth.weights_fp4(seed, n_out, K, block)
+            nib, sc = synth.weights_fp4(seed, n_out, K, block)
         y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, K, blk_sc=sc, block=block)
         Wd = oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block)
     want = oracle.linear_exact(Wd, X)
@@ -195,15 +196,15 @@ def test_prefill_gemm_with_weights_kept_out_of_lds(gpu, pkg, oracle, tokens, n_o
     few output tiles that the k range is split over workgroups (2 and 8 ranges) and a second kernel adds
     the partial sums; n_out = 250 is not a multiple of 4 and never splits."""
     torch, dev, lib = gpu
-    seed = pkg.synth.seed_for(4, 300 + tokens % 89 + n_out % 13)
+    seed = synth.seed_for(4, 300 + tokens % 89 + n_out % 13)
     if w_type_name == "e5m2":
-        w_type, W = oracle.E5M2, pkg.synth.weights_e5m2(seed, n_out, K)
+        w_type, W = oracle.E5M2, synth.weights_e5m2(seed, n_out, K)
     else:
-        w_type, W = oracle.E4M3, pkg.synth.weights_e4m3(seed, n_out, K)[0]
-    X = pkg.synth.activations(seed, tokens, K)
+        w_type, W = oracle.E4M3, synth.weights_e4m3(seed, n_out, K)[0]
+    X = synth.activations(seed, tokens, K)
     want = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K), X)
     want_s = oracle.linear_exact(oracle.dequant_weight(W, w_type, n_out, K, 0.37), X)
-    c0 = pkg.synth.activations(seed + 1, tokens, n_out)
+    c0 = synth.activations(seed + 1, tokens, n_out)
     wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
     td = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
 
@@ -325,8 +326,8 @@ def test_random_shapes_with_padded_strides(gpu, pkg, oracle, case):
 def test_fp4_weight_as_B_with_block_scales(gpu, pkg, oracle):
     torch, dev, lib = gpu
     n_out, tokens, K = 64, 3, 128
-    nib, sc = pkg.synth.weights_fp4(5, n_out, K, 16)
-    Xb = pkg.synth.activations(5, tokens, K)
+    nib, sc = synth.weights_fp4(5, n_out, K, 16)
+    Xb = synth.activations(5, tokens, K)
     C0 = np.zeros((n_out, tokens), dtype=np.uint16)
     want = C0.copy()
     assert oracle.quant_gemm(1, 0, tokens, n_out, K, 1.0, Xb, oracle.BF16, K, 1.0, nib, oracle.FP4, K, 1.0, 0.0, want, tokens, None, sc, 16) == 0
@@ -389,7 +390,7 @@ def test_full_size_gemv_properties(gpu, pkg, oracle):
         rows = np.random.default_rng(n_out).choice(n_out, size=257, replace=False)
         Wd_rows = oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2)
         for tokens in (1, 4, 16):
-            X = pkg.synth.activations(n_out + tokens, tokens, K)
+            X = synth.activations(n_out + tokens, tokens, K)
             xd = to_dev(torch, dev, X)
             yd = torch.zeros(tokens, n_out, dtype=torch.int16, device=dev)
             assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K) == 0
@@ -413,7 +414,7 @@ def test_full_size_prefill_gemm_sampled(gpu, pkg, oracle):
     for tokens, n_out, K in ((512, 12288, 4096), (2048, 12288, 4096), (2048, 4096, 12288), (512, 4096, 12288)):
         g = torch.Generator(device="cpu").manual_seed(tokens + K)
         W = (torch.randn(n_out, K, generator=g) * 0.02).to(torch.bfloat16).to(torch.float8_e5m2).view(torch.uint8).numpy()
-        X = pkg.synth.activations(tokens, tokens, K)
+        X = synth.activations(tokens, tokens, K)
         wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
         rows = np.random.default_rng(tokens).choice(n_out, size=192, replace=False)
         want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W[rows], oracle.E5M2), X)
@@ -471,9 +472,9 @@ def test_prepared_weights_give_the_same_gemv(gpu, pkg, oracle, tokens, n_out, K)
     """Every launch configuration of the matrix-core kernel on the tiled copy (few / several / many row
     tiles per CU, short and long rows, ragged row counts and row lengths) against the exact contraction."""
     torch, dev, lib = gpu
-    seed = pkg.synth.seed_for(2, 200 + n_out % 91 + tokens)
-    W = pkg.synth.weights_e5m2(seed, n_out, K)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(2, 200 + n_out % 91 + tokens)
+    W = synth.weights_e5m2(seed, n_out, K)
+    X = synth.activations(seed, tokens, K)
     wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
     y0 = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
     assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y0.data_ptr(), n_out, tokens, K) == 0

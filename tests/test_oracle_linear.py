@@ -2,6 +2,7 @@
 the vectorised NumPy contraction and the float64 golden answers, one-hot and all-ones activations,
 and the converter-faithful FP4 packer against hand-computed blocks."""
 import numpy as np
+from oracle import synth
 import pytest
 import torch
 
@@ -84,7 +85,7 @@ def test_dispatcher_layouts_and_alpha_beta_vs_numpy(oracle):
 def test_converter_packer_by_hand(oracle, pkg):
     # one block, absmax 6 -> scale 1.0 (0x38), values on the grid map to themselves
     grid = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], dtype=np.float32)
-    for packer in (oracle.quantize_fp4_blockscale_converter, pkg.synth.pack_fp4_blockscale):
+    for packer in (oracle.quantize_fp4_blockscale_converter, synth.pack_fp4_blockscale):
         nib, sc = packer(grid, 16)
         assert sc.tolist() == [0x38]
         assert oracle.unpack_fp4(nib, 16).tolist() == [0, 1, 2, 3, 4, 5, 6, 7, 0, 9, 10, 11, 12, 13, 14, 15]   # sign of -0.0 is 0
@@ -145,9 +146,9 @@ def test_on_the_fly_fp4_quantiser_scale_byte_by_hand(oracle):
 
 
 def test_packers_agree_and_round_trip_is_bounded(oracle, pkg):
-    w = pkg.synth.weights_f32(3, 64, 256)
+    w = synth.weights_f32(3, 64, 256)
     a = oracle.quantize_fp4_blockscale_converter(w, 16)
-    b = pkg.synth.pack_fp4_blockscale(w, 16)
+    b = synth.pack_fp4_blockscale(w, 16)
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
     deq = oracle.bf16_to_f32(oracle.dequant_fp4_blockscale_to_bf16(a[0], a[1], w.size, 16)).reshape(w.shape)
     # scales land in E4M3's subnormal range (step 2^-9), so the error is bounded by the block scale error
@@ -157,8 +158,8 @@ def test_packers_agree_and_round_trip_is_bounded(oracle, pkg):
 
 
 def test_synthetic_e5m2_weights_are_rne(oracle, pkg):
-    w = pkg.synth.weights_f32(4, 32, 128)
-    q = pkg.synth.weights_e5m2(4, 32, 128)
+    w = synth.weights_f32(4, 32, 128)
+    q = synth.weights_e5m2(4, 32, 128)
     assert np.array_equal(q, oracle.encode_e5m2_rne(w))
     assert np.array_equal(q, torch.from_numpy(w).to(torch.float8_e5m2).view(torch.uint8).numpy())
     back = oracle.decode_table(oracle.E5M2)[q]
@@ -167,14 +168,14 @@ def test_synthetic_e5m2_weights_are_rne(oracle, pkg):
 
 def test_cpu_baseline_route_matches_the_oracle(oracle, pkg):
     n_out, tokens, K = 96, 2, 256
-    W = pkg.synth.weights_e5m2(5, n_out, K)
-    X = pkg.synth.activations(5, tokens, K)
+    W = synth.weights_e5m2(5, n_out, K)
+    X = synth.activations(5, tokens, K)
     want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X)
     fn, name = oracle.find_cblas_sgemm()
     for sgemm in (None, fn):
         Y, td, tg = oracle.cpu_linear(W, oracle.E5M2, 1.0, None, 16, X, n_out, tokens, K, sgemm=sgemm, threads=2)
         assert np.abs(f64(oracle, Y) - want).max() <= 2.0 ** -7 * np.abs(want).max(), name
-    nib, sc = pkg.synth.weights_fp4(6, n_out, K)
+    nib, sc = synth.weights_fp4(6, n_out, K)
     want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc), X)
     Y, _, _ = oracle.cpu_linear(nib, oracle.FP4, 1.0, sc, 16, X, n_out, tokens, K, sgemm=fn, threads=2)
     assert np.abs(f64(oracle, Y) - want).max() <= 2.0 ** -7 * np.abs(want).max()

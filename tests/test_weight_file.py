@@ -1,9 +1,10 @@
 """The CFG_BIN INI container reader of the host library (host/WeightFile.cpp) and its name-resolution
-rules, on files written by cccc-lite_amd/weight_file.py in the converter's layout
+rules, on files written by oracle/weight_file.py in the converter's layout
 (scripts/convert_weights.py:54-83).  Host code only: no GPU call is made."""
 import struct
 
 import numpy as np
+from oracle import weight_file
 import pytest
 
 
@@ -13,7 +14,7 @@ def host(pkg):
 
 
 def test_container_round_trip_and_key_order(tmp_path, pkg, host):
-    wf_mod = pkg.weight_file
+    wf_mod = weight_file
     w = wf_mod.BinWriter()
     rng = np.random.default_rng(0)
     blobs = {"data_type": b"fp8_e4m3", "named_weights": b"1", "weight_fp8_e5m2_W_q_0": rng.integers(0, 255, 4096, dtype=np.uint8),
@@ -38,7 +39,7 @@ def test_container_round_trip_and_key_order(tmp_path, pkg, host):
 
 def test_name_resolution_follows_the_reference_order(tmp_path, pkg, host):
     D = pkg.DataType
-    w = pkg.weight_file.BinWriter()
+    w = weight_file.BinWriter()
     one = np.zeros(16, dtype=np.uint8)
     w.add("weight_bf16_A", one); w.add("weight_fp8_e5m2_A", one)          # a quantized typed key is found through the suffix list in its order
     w.add("weight_half_B", one); w.add("weight_B", one)                   # legacy untyped key beats a plain typed key
@@ -62,7 +63,7 @@ def test_name_resolution_follows_the_reference_order(tmp_path, pkg, host):
 
 def test_malformed_files_are_refused(tmp_path, pkg, host):
     good = tmp_path / "g.bin"
-    w = pkg.weight_file.BinWriter()
+    w = weight_file.BinWriter()
     w.add("k", b"12345678")
     w.save(good)
     raw = bytearray(good.read_bytes())

@@ -3,6 +3,7 @@ C-ABI: same kernels, so the outputs must agree bit for bit; its k-split partial 
 device array that every call on the GPU shares, so the cases run back to back, a smaller one after a larger
 one, and a stale partial sum from the earlier call would show."""
 import numpy as np
+from oracle import synth
 import pytest
 
 from gpu_util import check_rows, from_dev, to_dev
@@ -14,19 +15,19 @@ E5M2, E4M3, FP4 = 5, 4, 6
 
 def both_ways(gpu, pkg, oracle, tokens, n_out, K, w_type=E5M2, expect=None, **kw):
     torch, dev, lib = gpu
-    seed = pkg.synth.seed_for(7, tokens % 61 + n_out % 17)
-    X = pkg.synth.activations(seed, tokens, K)
+    seed = synth.seed_for(7, tokens % 61 + n_out % 17)
+    X = synth.activations(seed, tokens, K)
     blk = {}
     if w_type == FP4:
-        W, sc = pkg.synth.weights_fp4(seed, n_out, K, 16)
+        W, sc = synth.weights_fp4(seed, n_out, K, 16)
         scd = to_dev(torch, dev, sc)
         blk = dict(blk_sc=scd.data_ptr(), block_size=16)
         Wd = oracle.dequant_weight(W, oracle.FP4, n_out, K, blk_sc=sc, block=16)
     else:
-        W = pkg.synth.weights_e5m2(seed, n_out, K)
+        W = synth.weights_e5m2(seed, n_out, K)
         Wd = oracle.dequant_weight(W, oracle.E5M2, n_out, K, kw.get("inv_scale", 1.0))
     wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
-    c0 = pkg.synth.activations(seed + 1, tokens, n_out)
+    c0 = synth.activations(seed + 1, tokens, n_out)
     outs = []
     for noalloc in (False, True):
         y = to_dev(torch, dev, np.concatenate([c0.ravel(), np.zeros(64, dtype=np.uint16)]))
