@@ -109,8 +109,9 @@ template <int WT, bool SCALED>
 bool gemv8_mfma(const LinearArgs& a)
 {
     const int cus = cu_count();
-    if (a.n_out >= cus * 32) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
-    else { gemv8_mfma_kernel<WT, 1, 2, 8, SCALED><<<(a.n_out + 15) / 16, 512, 0, stream()>>>(a); }
+    // row-major weight, 5..16 tokens: activations through LDS as on the tiled copy
+    if (a.n_out >= cus * 32) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED, false, true><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
+    else { gemv8_mfma_kernel<WT, 1, 2, 8, SCALED, false, true><<<(a.n_out + 15) / 16, 512, 0, stream()>>>(a); }
     return true;
 }
 
@@ -119,12 +120,15 @@ bool gemv8_mfma(const LinearArgs& a)
 // at every token count (lm_head, one token: 89.8 us against 92.7 for the dot2 kernel; 16 tokens:
 // 100 us against 125 for a variant that kept the activations in LDS).  Configurations tuned on
 // MI355X over the Qwen3-8B shapes with rotating weights.
-template <int WT, int RT, int U, int WAVES, bool SCALED>
+template <int WT, int RT, int U, int WAVES, bool SCALED, bool XLDS = false>
 void launch_ksplit_tiled(const LinearArgs& t)
 {
-    gemv8_mfma_kernel<WT, RT, U, WAVES, SCALED, true><<<(t.n_out + 16 * RT - 1) / (16 * RT), WAVES * 64, 0, stream()>>>(t);
+    gemv8_mfma_kernel<WT, RT, U, WAVES, SCALED, true, XLDS><<<(t.n_out + 16 * RT - 1) / (16 * RT), WAVES * 64, 0, stream()>>>(t);
 }
 
+// From five tokens on the activation operand goes through LDS (XLDS, see the kernel): fetched in operand order it
+// costs 16 cache lines per 256 bytes, and at 16 tokens that, not HBM, bounds the kernel (K = 12288, 4096 rows:
+// 15.2 -> 13.3 us; K = 4096, 1024 rows: 6.4 -> 5.3 us).
 template <int WT, bool SCALED>
 bool gemv8_mfma_ksplit_tiled(const LinearArgs& a, const uint8_t* tiled)
 {
@@ -133,25 +137,28 @@ bool gemv8_mfma_ksplit_tiled(const LinearArgs& a, const uint8_t* tiled)
     const int tiles_per_cu = ((a.n_out + 15) / 16) / cu_count();
     if (tiles_per_cu >= 16)
     {
-        if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED>(t); }
-        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED>(t); }
+        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED, true>(t); }
+        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED, true>(t); }
     }
     else if (tiles_per_cu >= 2)
     {
         if (a.tokens <= 2) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 1, 8, SCALED>(t); }
-        else { launch_ksplit_tiled<WT, 4, 1, 8, SCALED>(t); }
+        else if (a.tokens <= 4) { launch_ksplit_tiled<WT, 2, 1, 8, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED, true>(t); }
+        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED, true>(t); }
     }
     else if (a.K > 8192)
     {
-        if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
-        else { launch_ksplit_tiled<WT, 1, 2, 8, SCALED>(t); }
+        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED, true>(t); }
+        else { launch_ksplit_tiled<WT, 1, 4, 8, SCALED, true>(t); }
     }
     else
     {
         if (a.tokens <= 4) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
-        else { launch_ksplit_tiled<WT, 1, 2, 8, SCALED>(t); }
+        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED, true>(t); }
+        else { launch_ksplit_tiled<WT, 1, 4, 8, SCALED, true>(t); }
     }
     return true;
 }
