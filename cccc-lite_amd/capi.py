@@ -26,11 +26,16 @@ class FusedLinear(ctypes.Structure):
     _fields_ = [("w_type", ctypes.c_int), ("K", ctypes.c_int), ("n_segments", ctypes.c_int), ("pair", ctypes.c_int),
                 ("W", ctypes.c_void_p * 3), ("n_out", ctypes.c_int * 3), ("w_scale", ctypes.c_float * 3),
                 ("Y", ctypes.c_void_p * 3), ("X", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p),
-                ("norm_eps", ctypes.c_float), ("residual", ctypes.c_void_p)]
+                ("norm_eps", ctypes.c_float), ("residual", ctypes.c_void_p),
+                ("blk_sc", ctypes.c_void_p * 3), ("block_size", ctypes.c_uint)]
 
 
-def make_fused_linear(w_type, K, W, n_out, Y, X, scales=None, norm_weight=None, norm_eps=1e-6, residual=None, pair=False) -> FusedLinear:
+def make_fused_linear(w_type, K, W, n_out, Y, X, scales=None, norm_weight=None, norm_eps=1e-6, residual=None, pair=False,
+                      blk_sc=None, block_size=16) -> FusedLinear:
     d = FusedLinear()
+    d.block_size = block_size
+    for s, p in enumerate(blk_sc or []):
+        d.blk_sc[s] = p
     d.w_type, d.K, d.n_segments, d.pair = w_type, K, len(W), 1 if pair else 0
     for s in range(len(W)):
         d.W[s], d.n_out[s], d.Y[s] = W[s], n_out[s], Y[s]

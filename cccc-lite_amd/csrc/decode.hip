@@ -49,6 +49,25 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     return finish("quant_linear_fused");
 }
 
+// FP4 block-scale weights: two rows per wave, U = 2 batches for rows of up to 4096 elements (one k-step of 2048 per
+// lane and row is 1 KiB), 8-wave workgroups for very tall weights, as for FP8.
+template <int BLOCK>
+int launch_fused_fp4(const FusedLinearArgs& a, int n_groups)
+{
+    const size_t lds = (size_t)((a.K + 2047) / 2048) * 4096;
+    if (lds > 64 * 1024) { return -1; }
+    const int cus = cu_count();
+    const int want4 = (n_groups + 3) / 4;
+    if (n_groups >= cus * 64)
+    {
+        const int want = (n_groups + 7) / 8;
+        gemv4_fused_kernel<BLOCK, 2, 8><<<want < cus * 2 ? want : cus * 2, 512, lds, stream()>>>(a);
+    }
+    else if (a.K <= 8192) { gemv4_fused_kernel<BLOCK, 1, 4><<<want4 < cus * 4 ? want4 : cus * 4, 256, lds, stream()>>>(a); }
+    else { gemv4_fused_kernel<BLOCK, 2, 4><<<want4 < cus * 4 ? want4 : cus * 4, 256, lds, stream()>>>(a); }
+    return finish("quant_linear_fused");
+}
+
 // Matrix-core variant on the tiled copies.  Configurations from the tuning of gemv8_mfma_kernel at one token.
 template <int WT, int RT, int U, int WAVES, bool SCALED>
 void launch_fused_mfma_cfg(const FusedLinearArgs& a, int n_tiles, size_t lds)
@@ -74,8 +93,10 @@ int launch_fused_mfma(const FusedLinearArgs& a, int n_tiles)
 
 int hip_quant_linear_fused(const hip_fused_linear* d)
 {
-    if (!d || (d->w_type != DT_E4M3 && d->w_type != DT_E5M2)) { return -1; }
+    if (!d || (d->w_type != DT_E4M3 && d->w_type != DT_E5M2 && d->w_type != DT_FP4)) { return -1; }
     if (d->K <= 0 || d->K % 16 != 0 || d->n_segments < 1 || d->n_segments > 3 || !d->X || !aligned16(d->X)) { return -1; }
+    const bool fp4 = d->w_type == DT_FP4;
+    if (fp4 && (d->K % 32 != 0 || (d->block_size != 16 && d->block_size != 32))) { return -1; }
     if (d->pair && d->n_segments != 2) { return -1; }
     if (d->residual && !d->pair && d->n_segments != 1) { return -1; }
     if (d->norm_weight && !aligned16(d->norm_weight)) { return -1; }
@@ -86,7 +107,9 @@ int hip_quant_linear_fused(const hip_fused_linear* d)
     {
         if (!d->W[s] || !aligned16(d->W[s]) || d->n_out[s] <= 0) { return -1; }
         if (!d->pair && !d->Y[s]) { return -1; }
+        if (fp4 && (!d->blk_sc[s] || ((uintptr_t)d->blk_sc[s] & 1u))) { return -1; }
         a.W[s] = (const uint8_t*)d->W[s];
+        a.S[s] = fp4 ? (const uint8_t*)d->blk_sc[s] : nullptr;
         a.Y[s] = (uint16_t*)d->Y[s];
         a.n_out[s] = d->n_out[s];
         a.w_scale[s] = d->w_scale[s];
@@ -105,6 +128,12 @@ int hip_quant_linear_fused(const hip_fused_linear* d)
     a.norm_w = (const uint16_t*)d->norm_weight;
     a.norm_eps = d->norm_eps;
     a.residual = (const uint16_t*)d->residual;
+    a.block = d->block_size;
+    if (fp4)
+    {
+        note_kernel("gemv_fused_fp4");
+        return d->block_size == 16 ? launch_fused_fp4<16>(a, n_groups) : launch_fused_fp4<32>(a, n_groups);
+    }
     // every segment has a registered tiled copy (and this is not the SwiGLU pair): matrix-core variant
     if (!d->pair)
     {

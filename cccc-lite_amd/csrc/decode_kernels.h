@@ -51,6 +51,8 @@ struct FusedLinearArgs
     float norm_eps;
     const uint16_t* residual;  // bf16 [n_out[0]] or nullptr (single segment / pair only)
     const uint8_t* T[3];       // load-time tiled copies of W[s] (matrix-core variant only)
+    const uint8_t* S[3];       // FP4 only: E4M3 block scales of W[s], one byte per `block` elements of the flat index
+    unsigned block;            // FP4 only: 16 or 32
 };
 
 // Staging of the activation vector into LDS in the [step][half][lane] layout of the dot2 kernels,
@@ -65,10 +67,12 @@ struct StagedActivation
     u32x4 x[STAGE_PRE], w[STAGE_PRE];
 };
 
+// PARTS 16-byte pieces per lane and k-step: 2 for FP8 rows (a step is 1024 codes), 4 for FP4 rows (2048 codes)
+template <int PARTS = 2>
 __device__ __forceinline__ int stage_slot(int c)
 {
-    const int step = c >> 7, in_step = c & 127;
-    return (step * 2 + (in_step & 1)) * 64 + (in_step >> 1);
+    const int step = c / (64 * PARTS), in_step = c % (64 * PARTS);
+    return (step * PARTS + (in_step % PARTS)) * 64 + in_step / PARTS;
 }
 
 template <int THREADS>
@@ -113,11 +117,11 @@ __device__ __forceinline__ u32x4 normed8(const u32x4& v, const u32x4& w, float i
 }
 
 // `red` holds THREADS / 64 floats.  Ends with a barrier: xs is complete for every thread.
-template <int THREADS>
+template <int THREADS, int PARTS = 2>
 __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const StagedActivation& r, u32x4* xs, float* red)
 {
-    const int n_steps = (a.K + 1023) / 1024;
-    const int n_chunks = n_steps * 128;                      // 16-byte chunks incl. zero padding
+    const int n_steps = (a.K + 512 * PARTS - 1) / (512 * PARTS);
+    const int n_chunks = n_steps * 64 * PARTS;               // 16-byte chunks incl. zero padding
     float sumsq = 0.0f;
     if (a.norm_w)
     {
@@ -130,7 +134,7 @@ __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const Sta
         for (int j = 0; j < STAGE_PRE; j++)
         {
             const int c = threadIdx.x + j * THREADS;
-            if (c < n_chunks) { xs[stage_slot(c)] = r.x[j]; }
+            if (c < n_chunks) { xs[stage_slot<PARTS>(c)] = r.x[j]; }
         }
     }
     for (int c = threadIdx.x + STAGE_PRE * THREADS; c < n_chunks; c += THREADS)
@@ -138,7 +142,7 @@ __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const Sta
         u32x4 v = { 0u, 0u, 0u, 0u };
         if (c * 8 < a.K) { v = *(const u32x4*)(a.X + c * 8); }
         if (a.norm_w) { sumsq += sumsq8(v); }
-        xs[stage_slot(c)] = v;
+        xs[stage_slot<PARTS>(c)] = v;
     }
     if (a.norm_w)
     {
@@ -155,14 +159,40 @@ __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const Sta
         for (int j = 0; j < STAGE_PRE; j++)
         {
             const int c = threadIdx.x + j * THREADS;
-            if (c < n_chunks) { xs[stage_slot(c)] = normed8(r.x[j], r.w[j], invstd); }    // padding chunks are zero
+            if (c < n_chunks) { xs[stage_slot<PARTS>(c)] = normed8(r.x[j], r.w[j], invstd); }    // padding chunks are zero
         }
         for (int c = threadIdx.x + STAGE_PRE * THREADS; c < n_chunks; c += THREADS)
         {
-            if (c * 8 < a.K) { xs[stage_slot(c)] = normed8(xs[stage_slot(c)], *(const u32x4*)(a.norm_w + c * 8), invstd); }
+            if (c * 8 < a.K) { xs[stage_slot<PARTS>(c)] = normed8(xs[stage_slot<PARTS>(c)], *(const u32x4*)(a.norm_w + c * 8), invstd); }
         }
     }
     __syncthreads();
+}
+
+// What one lane does with the two finished sums of a row group: the SwiGLU pair bf16(silu(gate) * up) with the
+// reference's three roundings (group g = output g), or two plain outputs; the residual is added to a rounded value.
+__device__ __forceinline__ void fused_store(const FusedLinearArgs& a, int g, int seg, int row0, int row1, float t0, float t1)
+{
+    if (a.pair)
+    {
+        const float gate = bf16_round(t0), up = bf16_round(t1);
+        const float sig = bf16_round(1.0f / (1.0f + expf(-gate)));
+        const float silu = bf16_round(gate * sig);
+        float out = bf16_round(silu * up);
+        if (a.residual) { out = bf16_round(out + bf16_bits_to_f32(a.residual[g])); }
+        a.Y[0][g] = (uint16_t)f32_to_bf16_bits(out);
+    }
+    else
+    {
+        float o0 = bf16_round(t0), o1 = bf16_round(t1);
+        if (a.residual && seg == 0)
+        {
+            o0 = bf16_round(o0 + bf16_bits_to_f32(a.residual[row0]));
+            o1 = bf16_round(o1 + bf16_bits_to_f32(a.residual[row1]));
+        }
+        a.Y[seg][row0] = (uint16_t)f32_to_bf16_bits(o0);
+        if (row1 != row0) { a.Y[seg][row1] = (uint16_t)f32_to_bf16_bits(o1); }
+    }
 }
 
 // One wave owns a group of two rows at a time and walks its groups in batches of U KiB per row.  The
@@ -284,29 +314,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         {
             const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
             acc0 = acc1 = 0.0f;
-            if (lane == 0)
-            {
-                if (a.pair)
-                {
-                    const float gate = bf16_round(t0), up = bf16_round(t1);
-                    const float sig = bf16_round(1.0f / (1.0f + expf(-gate)));
-                    const float silu = bf16_round(gate * sig);
-                    float out = bf16_round(silu * up);
-                    if (a.residual) { out = bf16_round(out + bf16_bits_to_f32(a.residual[g])); }
-                    a.Y[0][g] = (uint16_t)f32_to_bf16_bits(out);
-                }
-                else
-                {
-                    float o0 = bf16_round(t0), o1 = bf16_round(t1);
-                    if (a.residual && cur.seg == 0)
-                    {
-                        o0 = bf16_round(o0 + bf16_bits_to_f32(a.residual[cur.row0]));
-                        o1 = bf16_round(o1 + bf16_bits_to_f32(a.residual[cur.row1]));
-                    }
-                    a.Y[cur.seg][cur.row0] = (uint16_t)f32_to_bf16_bits(o0);
-                    if (cur.row1 != cur.row0) { a.Y[cur.seg][cur.row1] = (uint16_t)f32_to_bf16_bits(o1); }
-                }
-            }
+            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1); }
         }
         g = ng;
         batch = nbatch;
@@ -321,6 +329,159 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
                 xa[u][0] = xn[u][0];
                 xa[u][1] = xn[u][1];
             }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// The fused one-token linear for FP4_E2M1 block-scale weights (cccc/cublas_real.h:952-955 dequantises them with
+// cuda_fp4_blockscale_to_bf16, cccc-cuda/cuda_functions.cu:2926-2939): same decomposition as gemv8_fused_kernel
+// -- a wave owns two rows, batches of U k-steps, the next batch requested before the current one is multiplied,
+// activation (normalised on the way when asked) staged once per workgroup -- with the arithmetic of
+// gemv4_dot2_kernel: a 128-bit load is 32 consecutive elements of a row, i.e. 32 / BLOCK scale blocks, and
+// fp4 * e4m3 is exact in BF16, so each block's dot product is taken on the bare FP4 values and multiplied by
+// its scale once.  Rows are K / 2 bytes, scales run over the flat element index; K % 32 == 0.
+// Dynamic LDS: ceil(K / 2048) * 4096 bytes.
+template <int BLOCK, int U, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv4_fused_kernel(const FusedLinearArgs a)
+{
+    static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    extern __shared__ u32x4 xs[];
+    __shared__ float red[WAVES];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_steps = (a.K + 2047) / 2048;
+    const int batches = (n_steps + U - 1) / U;
+    const int g0 = a.pair ? a.n_out[0] : (a.n_out[0] + 1) / 2;
+    const int g1 = (a.pair || a.n_segments < 2) ? g0 : g0 + (a.n_out[1] + 1) / 2;
+    const int n_groups = (a.pair || a.n_segments < 3) ? g1 : g1 + (a.n_out[2] + 1) / 2;
+    const int stride = gridDim.x * WAVES;
+
+    struct Rows
+    {
+        const uint8_t *w0, *w1, *s0, *s1;
+        int seg, row0, row1;
+    };
+    auto locate = [&](int g) {
+        Rows r;
+        r.seg = 0;
+        if (a.pair) { r.row0 = r.row1 = g; }
+        else
+        {
+            int local = g;
+            if (g >= g1) { r.seg = 2; local = g - g1; }
+            else if (g >= g0) { r.seg = 1; local = g - g0; }
+            r.row0 = local * 2;
+            r.row1 = min(local * 2 + 1, a.n_out[r.seg] - 1);
+        }
+        const int sa = a.pair ? 0 : r.seg, sb = a.pair ? 1 : r.seg;
+        r.w0 = a.W[sa] + (((long long)r.row0 * a.K) >> 1) + lane * 16;
+        r.w1 = a.W[sb] + (((long long)r.row1 * a.K) >> 1) + lane * 16;
+        r.s0 = a.S[sa] + ((long long)r.row0 * a.K) / BLOCK + lane * (32 / BLOCK);
+        r.s1 = a.S[sb] + ((long long)r.row1 * a.K) / BLOCK + lane * (32 / BLOCK);
+        return r;
+    };
+    auto request = [&](const Rows& r, int st0, u32x4* wa, u32x4* wb, uint32_t* sa, uint32_t* sb) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            wa[u] = wb[u] = u32x4{ 0u, 0u, 0u, 0u };
+            sa[u] = sb[u] = 0u;
+            if ((st0 + u) * 2048 + lane * 32 < a.K)
+            {
+                wa[u] = __builtin_nontemporal_load((const u32x4*)(r.w0 + (st0 + u) * 1024));
+                wb[u] = __builtin_nontemporal_load((const u32x4*)(r.w1 + (st0 + u) * 1024));
+                if (BLOCK == 16)
+                {
+                    sa[u] = *(const uint16_t*)(r.s0 + (st0 + u) * 128);
+                    sb[u] = *(const uint16_t*)(r.s1 + (st0 + u) * 128);
+                }
+                else
+                {
+                    sa[u] = r.s0[(st0 + u) * 64];
+                    sb[u] = r.s1[(st0 + u) * 64];
+                }
+            }
+        }
+    };
+    // sum over the 32 elements of one load of fp4 * x per scale block, times the block's scale
+    auto row_dot = [&](const u32x4& w, uint32_t sc, const u32x4 (&x)[4], float acc) {
+        float part[2] = { 0.0f, 0.0f };
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+        {
+            const bf16x2 q0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], 1.0f, 0);
+            const bf16x2 q1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], 1.0f, 1);
+            const bf16x2 q2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], 1.0f, 2);
+            const bf16x2 q3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], 1.0f, 3);
+            float p = part[d >> 1];
+            p = dot2_bf16(q0, x[d][0], p);
+            p = dot2_bf16(q1, x[d][1], p);
+            p = dot2_bf16(q2, x[d][2], p);
+            p = dot2_bf16(q3, x[d][3], p);
+            part[d >> 1] = p;
+        }
+        const float s_lo = e4m3_byte_to_f32(sc, 0);
+        const float s_hi = BLOCK == 16 ? e4m3_byte_to_f32(sc, 1) : s_lo;
+        return fmaf(s_hi, part[1], fmaf(s_lo, part[0], acc));
+    };
+
+    int g = blockIdx.x * WAVES + wave, batch = 0;
+    Rows cur{}, nxt{};
+    u32x4 wa[U], wb[U], na[U], nb[U];
+    uint32_t sa[U], sb[U], nsa[U], nsb[U];
+    StagedActivation staged;
+    stage_issue<WAVES * 64>(a, staged);
+    if (g < n_groups)
+    {
+        cur = locate(g);
+        request(cur, 0, wa, wb, sa, sb);
+    }
+    stage_finish<WAVES * 64, 4>(a, staged, xs, red);
+
+    float acc0 = 0.0f, acc1 = 0.0f;
+    while (g < n_groups)
+    {
+        int ng = g, nbatch = batch + 1;
+        if (nbatch == batches)
+        {
+            ng = g + stride;
+            nbatch = 0;
+        }
+        if (ng < n_groups)
+        {
+            nxt = nbatch == 0 ? locate(ng) : cur;
+            request(nxt, nbatch * U, na, nb, nsa, nsb);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int st = batch * U + u;
+            if (st < n_steps)
+            {
+                u32x4 x[4];
+#pragma unroll
+                for (int p = 0; p < 4; p++) { x[p] = xs[(st * 4 + p) * 64 + lane]; }
+                acc0 = row_dot(wa[u], sa[u], x, acc0);
+                acc1 = row_dot(wb[u], sb[u], x, acc1);
+            }
+        }
+        if (batch == batches - 1)
+        {
+            const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
+            acc0 = acc1 = 0.0f;
+            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1); }
+        }
+        g = ng;
+        batch = nbatch;
+        cur = nxt;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            wa[u] = na[u];
+            wb[u] = nb[u];
+            sa[u] = nsa[u];
+            sb[u] = nsb[u];
         }
     }
 }

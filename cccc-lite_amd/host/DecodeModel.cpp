@@ -99,6 +99,14 @@ Matrix* DecodeModel::tensor(int layer, int which)
     return (which >= 0 && which <= W_DOWN) ? table[which] : nullptr;
 }
 
+int DecodeModel::setBlockScales(int layer, int which, const void* host, size_t n_scales)
+{
+    Matrix* m = tensor(layer, which);
+    if (!m || m->getDataType() != FP4_E2M1 || (int64_t)n_scales != (m->getDataSize() + Matrix::fp4BlockSize() - 1) / Matrix::fp4BlockSize()) { return -1; }
+    m->setBlockScaleFromHost(host, (int64_t)n_scales);
+    return m->getBlockScaleData() ? 0 : 1;
+}
+
 Matrix* DecodeModel::activation(int which)
 {
     Matrix* table[] = { x_.get(), r1_.get(), q_.get(), k_.get(), v_.get(), att_.get(), gated_.get() };
@@ -111,7 +119,7 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     if (!m) { return -1; }
     if (Rocblas::isQuantized(dt))
     {
-        if ((int64_t)bytes != m->getDataSize()) { return -1; }
+        if ((int64_t)bytes != (dt == FP4_E2M1 ? (m->getDataSize() + 1) / 2 : m->getDataSize())) { return -1; }
         // only a tall weight (lm_head) is read through its tiled copy by the fused decode kernels
         m->setAllowRepack(which == LM_HEAD);
         m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
@@ -151,9 +159,10 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         if (!wk.valid()) { return fail(name, -1); }
         if (wk.is_quant)
         {
-            if (wk.dt == FP4_E2M1) { return fail(name, -3); }
             m.setAllowRepack(tiled);
-            return file.loadNamed(m, name) == 0 ? 0 : fail(name, -2);
+            if (file.loadNamed(m, name) != 0) { return fail(name, -2); }
+            if (wk.dt == FP4_E2M1 && !m.getBlockScaleData()) { return fail(name, -3); }    // FP4 without blockscale_<name>: no fused kernel
+            return 0;
         }
         Matrix tmp(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
         tmp.setAllowRepack(tiled);
@@ -167,7 +176,7 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
             tmp = bf;
         }
         tmp.quantizeWeights(quantize_to);
-        if (tmp.getDataType() != FP8_E4M3 && tmp.getDataType() != FP8_E5M2) { return fail(name, -3); }
+        if (!Rocblas::isQuantized(tmp.getDataType())) { return fail(name, -3); }
         m = tmp;
         return 0;
     };
@@ -254,6 +263,8 @@ static hip_fused_linear linear_desc(const Matrix& W, int n_out, int K, const voi
     d.W[0] = W.data();
     d.n_out[0] = n_out;
     d.w_scale[0] = W.getQuantScale();
+    d.blk_sc[0] = W.getBlockScaleData();
+    d.block_size = Matrix::fp4BlockSize();
     d.Y[0] = y;
     d.X = x;
     return d;
@@ -279,6 +290,8 @@ int DecodeModel::step()
             qkv.n_segments = 3;
             qkv.W[1] = L.wk->data(); qkv.n_out[1] = kv_out; qkv.w_scale[1] = L.wk->getQuantScale(); qkv.Y[1] = k_->data();
             qkv.W[2] = L.wv->data(); qkv.n_out[2] = kv_out; qkv.w_scale[2] = L.wv->getQuantScale(); qkv.Y[2] = v_->data();
+            qkv.blk_sc[1] = L.wk->getBlockScaleData();
+            qkv.blk_sc[2] = L.wv->getBlockScaleData();
             rc = hip_quant_linear_fused(&qkv);
         }
         else
@@ -325,6 +338,7 @@ int DecodeModel::step()
             gu.n_segments = 2;
             gu.pair = 1;
             gu.W[1] = L.w_up->data(); gu.n_out[1] = c.inter; gu.w_scale[1] = L.w_up->getQuantScale();
+            gu.blk_sc[1] = L.w_up->getBlockScaleData();
             gu.norm_weight = L.rms_ffn->data();
             gu.norm_eps = c.eps;
             rc = hip_quant_linear_fused(&gu);

@@ -42,15 +42,18 @@ public:
     Matrix* tensor(int layer, int which);
     Matrix* activation(int which);
 
-    // Uploads file bytes: FP8 codes for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
+    // Uploads file bytes: FP8 codes or packed FP4 nibbles for the linears (loadQuantizedDirect), BF16 bits for norms / embedding.
     int setTensor(int layer, int which, const void* host, size_t bytes, DataType dt, float scale);
+    // FP4 linears: the E4M3 block scales that go with the packed codes (one byte per 16 elements).
+    int setBlockScales(int layer, int which, const void* host, size_t n_scales);
 
     // Loads every tensor from a converted model file by the converter's names (scripts/convert_weights.py:142-166):
     // W_emb, W_rms_final, W_lm_head (W_emb when absent: tied), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
-    // W_qnorm_<i>, W_knorm_<i>, W_rms_ffn_<i>, W_gate_<i>, W_up_<i>, W_down_<i>.  FP8 linears are taken as stored;
+    // W_qnorm_<i>, W_knorm_<i>, W_rms_ffn_<i>, W_gate_<i>, W_up_<i>, W_down_<i>.  FP8 and FP4 linears are taken as stored;
     // linears stored as BF16 / HALF / FLOAT are quantized on load to `quantize_to` with a per-tensor absmax scale
     // (the reference's weight_data_type route, cccc/Matrix.cpp:301-355).  0 ok; otherwise `failed` names the tensor:
-    // -1 missing, -2 wrong size, -3 a type the fused decode kernels do not take (FP4, or too small to quantize).
+    // -1 missing, -2 wrong size, -3 something the fused decode kernels do not take (FP4 without block scales, gate and
+    // up in two formats, a tensor too small to quantize).  FP4_E2M1 linears load with their blockscale_<name> entries.
     int loadNamedWeights(const WeightFile& file, DataType quantize_to = FP8_E5M2, std::string* failed = nullptr);
 
     // Writes every tensor under the same names, as Net::saveNamedWeights does (cccc/Net.cpp:1235-1314): the header

@@ -160,6 +160,11 @@ int cccc_decode_set_tensor(void* m, int layer, int which, const void* host, unsi
     return ((DecodeModel*)m)->setTensor(layer, which, host, (size_t)bytes, (DataType)dtype, scale);
 }
 
+int cccc_decode_set_block_scales(void* m, int layer, int which, const void* host, unsigned long long n_scales)
+{
+    return ((DecodeModel*)m)->setBlockScales(layer, which, host, (size_t)n_scales);
+}
+
 void* cccc_decode_tensor_data(void* m, int layer, int which)
 {
     Matrix* t = ((DecodeModel*)m)->tensor(layer, which);

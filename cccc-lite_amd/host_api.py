@@ -41,6 +41,7 @@ class HostLibrary:
         L.cccc_decode_create.restype = vp; L.cccc_decode_create.argtypes = [i32] * 8 + [f32, f32]
         L.cccc_decode_destroy.restype = None; L.cccc_decode_destroy.argtypes = [vp]
         L.cccc_decode_set_tensor.restype = i32; L.cccc_decode_set_tensor.argtypes = [vp, i32, i32, vp, u64, i32, f32]
+        L.cccc_decode_set_block_scales.restype = i32; L.cccc_decode_set_block_scales.argtypes = [vp, i32, i32, vp, u64]
         L.cccc_decode_tensor_data.restype = vp; L.cccc_decode_tensor_data.argtypes = [vp, i32, i32]
         L.cccc_decode_reset.restype = i32; L.cccc_decode_reset.argtypes = [vp, i32, i32]
         L.cccc_decode_step.restype = i32; L.cccc_decode_step.argtypes = [vp]
@@ -226,6 +227,13 @@ class DecodeModel:
         if rc != 0:
             raise ValueError(f"set_tensor({layer}, {name}) failed: {rc}")
 
+    def set_block_scales(self, layer: int, name: str, scales: np.ndarray) -> None:
+        which = LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))
+        scales = np.ascontiguousarray(scales, dtype=np.uint8)
+        rc = self.lib.c.cccc_decode_set_block_scales(self.handle, layer, which, scales.ctypes.data, scales.size)
+        if rc != 0:
+            raise ValueError(f"set_block_scales({layer}, {name}) failed: {rc}")
+
     def tensor_ptr(self, layer: int, name: str) -> int:
         return self.lib.c.cccc_decode_tensor_data(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name)))
 
@@ -235,12 +243,19 @@ class DecodeModel:
         return self.lib.c.cccc_decode_tensor_prepare(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))) == 0
 
     def load(self, model: dict, fp8_dtype: int = 5) -> None:
-        """model: the dict layout of oracle.decode_oracle.make_model (uint8 codes / uint16 bf16 bits)."""
+        """model: the dict layout of oracle.decode_oracle.make_model (uint8 codes / uint16 bf16 bits); a quantized
+        tensor given as a (packed FP4 nibbles, E4M3 block scales) pair is loaded as FP4_E2M1."""
+        def put(li, name, value):
+            if isinstance(value, tuple):
+                self.set_tensor(li, name, value[0], 6)
+                self.set_block_scales(li, name, value[1])
+            else:
+                self.set_tensor(li, name, value, fp8_dtype if name in QUANTIZED else 3)
         for name in GLOBAL_TENSORS:
-            self.set_tensor(0, name, model[name], fp8_dtype if name in QUANTIZED else 3)
+            put(0, name, model[name])
         for li, L in enumerate(model["layers"]):
             for name in LAYER_TENSORS:
-                self.set_tensor(li, name, L[name], fp8_dtype if name in QUANTIZED else 3)
+                put(li, name, L[name])
 
     def load_named(self, wf: WeightFile, quantize_to: int = 5) -> None:
         """Every tensor from a converted model file by the converter's names; plain linears are quantized on load."""

@@ -159,12 +159,15 @@ C_EXPORT int hip_embed_fwd(int type, const void* ids, const void* W, void* Y, in
  * (`d_pos`, `d_token`: one int32 each) so that a step is a fixed launch sequence.
  */
 
-/* y_s = W_s * [rmsnorm](x) for 1..3 FP8 weights sharing x (q/k/v), or the SwiGLU pair
+/* y_s = W_s * [rmsnorm](x) for 1..3 quantized weights sharing x (q/k/v), or the SwiGLU pair
  * y = bf16(silu(W[0] x) * (W[1] x)) with silu(g) = bf16(g * bf16(sigmoid g)); optional residual
- * y = bf16(y + residual) on W[0]'s output.  Weights are [n_out][K], K contiguous, K % 16 == 0. */
+ * y = bf16(y + residual) on W[0]'s output.  Weights are [n_out][K], K contiguous, K % 16 == 0; FP4_E2M1
+ * weights (two elements per byte, K % 32 == 0) come with their E4M3 block scales, one byte per block_size
+ * (16 or 32) elements of the flat index, as cuda_fp4_blockscale_to_bf16 reads them
+ * (cccc-cuda/cuda_functions.cu:2926-2939); w_scale is ignored for them. */
 typedef struct hip_fused_linear
 {
-    int w_type;              /* 4 (FP8_E4M3) or 5 (FP8_E5M2) */
+    int w_type;              /* 4 (FP8_E4M3), 5 (FP8_E5M2) or 6 (FP4_E2M1 with block scales) */
     int K;
     int n_segments;          /* 1..3; 2 when pair != 0 */
     int pair;                /* 1: SwiGLU pair of W[0] (gate) and W[1] (up), both n_out[0] rows, into Y[0] */
@@ -176,6 +179,8 @@ typedef struct hip_fused_linear
     const void* norm_weight; /* bf16 [K] or NULL */
     float norm_eps;
     const void* residual;    /* bf16 [n_out[0]] or NULL */
+    const void* blk_sc[3];   /* FP4 only: block scales of W[s] */
+    unsigned int block_size; /* FP4 only: 16 or 32 */
 } hip_fused_linear;
 C_EXPORT int hip_quant_linear_fused(const hip_fused_linear* desc);
 

@@ -128,14 +128,27 @@ def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, pos: int,
     return out
 
 
-def make_model(cfg: DecodeConfig, seed: int = 0):
-    """Random-init model: FP8_E5M2 linears from N(0, 0.02) (round to nearest), BF16 norms near 1,
-    BF16 embedding N(0, 1)."""
+def dequant_linear(W) -> np.ndarray:
+    """BF16 bits [n_out, K] of a linear weight of the model dict: uint8 E5M2 codes [n_out, K], or a
+    (packed FP4 nibbles [n_out, K / 2], E4M3 block scales [n_out, K / 16]) pair."""
+    if isinstance(W, tuple):
+        nib, sc = W
+        n_out, K = nib.shape[0], nib.shape[1] * 2
+        return o.dequant_fp4_blockscale_to_bf16(nib, sc, n_out * K, K // sc.shape[1]).reshape(n_out, K)
+    return o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape)
+
+
+def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2"):
+    """Random-init model: linears from N(0, 0.02) as FP8_E5M2 codes (round to nearest) or, fmt = "fp4_e2m1", as the
+    converter's FP4 block-scale packing (blocks of 16); BF16 norms near 1, BF16 embedding N(0, 1)."""
     rng = np.random.default_rng(seed)
 
     def q8(n_out, K):
-        w = (rng.standard_normal((n_out, K), dtype=np.float32) * np.float32(0.02))
-        return o.encode_e5m2_rne(f(o.f32_to_bf16(w)))
+        w = f(o.f32_to_bf16(rng.standard_normal((n_out, K), dtype=np.float32) * np.float32(0.02)))
+        if fmt == "fp4_e2m1":
+            nib, sc = o.quantize_fp4_blockscale_converter(w, 16)
+            return nib.reshape(n_out, K // 2), sc.reshape(n_out, K // 16)
+        return o.encode_e5m2_rne(w)
 
     def norm_w(n):
         return o.f32_to_bf16((1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32))
@@ -165,7 +178,7 @@ class DecodeOracle:
         key = (layer, name)
         if key not in self._deq:
             W = self.model[name] if layer is None else self.model["layers"][layer][name]
-            self._deq[key] = o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape)
+            self._deq[key] = dequant_linear(W)
         return self._deq[key]
 
     def step(self, token: int, pos: int, trace: dict | None = None, logit_rows=None):

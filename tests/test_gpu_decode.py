@@ -384,3 +384,89 @@ def test_graph_replay_equals_eager_steps(small_model, dec):
     model.reset(3, 0)
     assert model.run(10, False) > 0
     assert model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
+
+
+# ------------------------------------------------------------------------------------------ FP4 block-scale weights
+
+@pytest.mark.parametrize("block", [16, 32])
+def test_fused_linear_fp4_variants(gpu, pkg, oracle, dec, block):
+    """hip_quant_linear_fused on FP4_E2M1 weights with E4M3 block scales: norm + three segments, single segment with
+    residual and no norm, the SwiGLU pair, rows longer than one k-step and row counts that are odd."""
+    from oracle import synth
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(block)
+    for K, (n0, n1, n2) in ((2048, (512, 128, 130)), (4608, (96, 33, 64)), (14336, (70, 16, 16))):
+        x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+        nw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+        packed = [synth.weights_fp4(int(rng.integers(1 << 20)), n, K, block) for n in (n0, n1, n2, n0)]
+        Wd = [oracle.dequant_weight(nib, oracle.FP4, nib.shape[0], K, blk_sc=sc, block=block) for nib, sc in packed]
+        nd = [to_dev(torch, dev, nib) for nib, _ in packed]
+        sd = [to_dev(torch, dev, sc) for _, sc in packed]
+        xd, nwd = to_dev(torch, dev, x), to_dev(torch, dev, nw)
+        xn = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6)
+        # (1) norm + three segments
+        ys = [torch.zeros(n + 8, dtype=torch.int16, device=dev) for n in (n0, n1, n2)]
+        d = pkg.capi.make_fused_linear(6, K, [w.data_ptr() for w in nd[:3]], [n0, n1, n2], [y.data_ptr() for y in ys], xd.data_ptr(),
+                                       norm_weight=nwd.data_ptr(), norm_eps=1e-6, blk_sc=[s_.data_ptr() for s_ in sd[:3]], block_size=block)
+        assert lib.quant_linear_fused(d) == 0 and lib.last_kernel() == "gemv_fused_fp4"
+        for s_, n in enumerate((n0, n1, n2)):
+            out = from_dev(ys[s_], np.uint16)
+            assert not out[n:].any()
+            assert ulp_close(out[:n], dec.linear(Wd[s_], xn), ulps=1.0, floor=2e-5).all(), (K, s_)
+        # (2) one segment, no norm, residual
+        res = oracle.f32_to_bf16(rng.standard_normal(n0).astype(np.float32))
+        rd = to_dev(torch, dev, res)
+        y = torch.zeros(n0, dtype=torch.int16, device=dev)
+        d = pkg.capi.make_fused_linear(6, K, [nd[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr(), residual=rd.data_ptr(),
+                                       blk_sc=[sd[0].data_ptr()], block_size=block)
+        assert lib.quant_linear_fused(d) == 0
+        lin = dec.linear(Wd[0], dec.f(x))
+        want = dec.r(lin + dec.f(res))
+        tol = np.maximum(np.maximum(np.abs(lin), np.abs(dec.f(res))), np.abs(want)) * 2.0 ** -7 + 1e-4
+        assert (np.abs(dec.f(from_dev(y, np.uint16)).astype(np.float64) - want) <= tol).all()
+        # (3) SwiGLU pair behind the norm
+        y = torch.zeros(n0, dtype=torch.int16, device=dev)
+        d = pkg.capi.make_fused_linear(6, K, [nd[0].data_ptr(), nd[3].data_ptr()], [n0, n0], [y.data_ptr(), None], xd.data_ptr(),
+                                       norm_weight=nwd.data_ptr(), norm_eps=1e-6, pair=True, blk_sc=[sd[0].data_ptr(), sd[3].data_ptr()], block_size=block)
+        assert lib.quant_linear_fused(d) == 0
+        want = dec.silu_mul(dec.linear(Wd[0], xn), dec.linear(Wd[3], xn))
+        out = from_dev(y, np.uint16)
+        assert ulp_close(out, want, ulps=3.0, floor=1e-4).all()
+        assert (out == oracle.f32_to_bf16(want)).mean() > 0.97
+    # refused: no block scales, a block length the kernels do not have, rows that are not whole 32-element loads
+    d = pkg.capi.make_fused_linear(6, K, [nd[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr(), block_size=block)
+    assert lib.quant_linear_fused(d) == -1
+    d = pkg.capi.make_fused_linear(6, K, [nd[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr(), blk_sc=[sd[0].data_ptr()], block_size=8)
+    assert lib.quant_linear_fused(d) == -1
+    d = pkg.capi.make_fused_linear(6, 48, [nd[0].data_ptr()], [n0], [y.data_ptr()], xd.data_ptr(), blk_sc=[sd[0].data_ptr()], block_size=block)
+    assert lib.quant_linear_fused(d) == -1
+
+
+def test_decode_steps_with_fp4_linears_follow_the_oracle(gpu, pkg, oracle, dec):
+    """The Llama-3.1-8B route of the reference (FP4_E2M1 block-scale linears, cccc/Net.cpp:1460-1481) through the
+    fused decode step: eight steps of a two-layer model against the oracle on the same nibbles and scale bytes."""
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=32)
+    weights = dec.make_model(cfg, 17, fmt="fp4_e2m1")
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    model.load(weights)
+    model.set_exact_attention(True)
+    orc = dec.DecodeOracle(cfg, weights)
+    token = 9
+    for pos in range(8):
+        model.reset(token, pos)
+        got_token = model.step()
+        want_logits, want_token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        top2 = np.sort(want_logits)[-2:]
+        if top2[1] - top2[0] > 2 * np.abs(got - want_logits).max():
+            assert got_token == want_token, pos
+        token = want_token
+    # graph replay == eager on this path too
+    model.reset(3, 0)
+    eager = [model.step() for _ in range(6)]
+    logits_eager = model.logits().copy()
+    model.reset(3, 0)
+    assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)

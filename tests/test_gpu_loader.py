@@ -296,3 +296,50 @@ def test_mixed_fp8_formats_in_one_file(tmp_path, gpu, pkg, host, oracle, dec):
     bad = rewrite("weight_fp8_e5m2_W_up_0", "weight_fp8_e4m3_W_up_0", oracle.encode_e4m3_rne((up_f32 / np.float32(scale)).astype(np.float32)), "scale_W_up_0")
     with pytest.raises(ValueError, match="W_up_0"):
         make_model(pkg, host, cfg).load_named(pkg.host_api.WeightFile(host, bad))
+
+
+def test_decode_model_from_an_fp4_file(tmp_path, gpu, pkg, host, oracle, dec):
+    """weight_fp4_e2m1_<name> + blockscale_<name> entries, as the converter writes a Llama FP4 model
+    (scripts/convert_weights.py:318-392): loading them gives the same steps as tensors set directly, and
+    saveNamedWeights writes the same entries back."""
+    cfg = dec.DecodeConfig(layers=1, hidden=256, n_q=4, n_kv=2, inter=512, vocab=400, t_kv=16)
+    weights = dec.make_model(cfg, 23, fmt="fp4_e2m1")
+    names = {"rms_attn": "W_rms_attn", "wq": "W_q", "wk": "W_k", "wv": "W_v", "q_norm": "W_qnorm", "k_norm": "W_knorm", "wo": "W_o",
+             "rms_ffn": "W_rms_ffn", "w_gate": "W_gate", "w_up": "W_up", "w_down": "W_down"}
+    w = weight_file.BinWriter()
+    w.add("data_type", b"fp4_e2m1")
+    w.add("named_weights", b"1")
+
+    def put(name, value):
+        if isinstance(value, tuple):
+            w.add(f"weight_fp4_e2m1_{name}", value[0])
+            w.add(f"blockscale_{name}", value[1])
+        else:
+            w.add(f"weight_bf16_{name}", value)
+
+    put("W_emb", weights["emb"]); put("W_rms_final", weights["rms_final"]); put("W_lm_head", weights["lm_head"])
+    for short, value in weights["layers"][0].items():
+        put(f"{names[short]}_0", value)
+    path = tmp_path / "model_fp4.bin"
+    w.save(path)
+    a, b = make_model(pkg, host, cfg), make_model(pkg, host, cfg)
+    a.load(weights)
+    b.load_named(pkg.host_api.WeightFile(host, path))
+    for m in (a, b):
+        m.reset(7, 0)
+    for _ in range(5):
+        assert a.step() == b.step()
+    assert np.array_equal(a.logits(), b.logits())
+    again = tmp_path / "model_fp4_again.bin"
+    b.save_named(again)
+    for key in weight_file.read_index(path)[0]:
+        assert weight_file.read_entry(again, key) == weight_file.read_entry(path, key), key
+    # an FP4 linear without its block scales cannot run on the fused kernels: refused by name
+    bw = weight_file.BinWriter()
+    for key in weight_file.read_index(path)[0]:
+        if key != "blockscale_W_o_0":
+            bw.add(key, weight_file.read_entry(path, key))
+    broken = tmp_path / "model_fp4_noscale.bin"
+    bw.save(broken)
+    with pytest.raises(ValueError, match="W_o_0"):
+        make_model(pkg, host, cfg).load_named(pkg.host_api.WeightFile(host, broken))
