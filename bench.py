@@ -424,29 +424,46 @@ def fp4_bytes(K, N, M, block):
     return K * N // 2 + K * N // block + 2 * M * K + 2 * M * N
 
 
-def fp4_sweep(ws):
-    """Llama-3.1-8B-shaped FP4 block-scale GEMVs at M=1, block 16 (the reference's format) and 32, weights
-    rotating over at least 512 MiB of distinct buffers."""
+def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
+    """BASELINE config 3: Llama-3.1-8B-shaped FP4 block-scale GEMVs, block 16 (the reference's format) and 32, weights
+    rotating over at least 512 MiB of distinct buffers, with their load-time tiled copies registered as the host mirror
+    registers them (unless --no-repack); M = 1 is the configuration's own row, 4 and 16 ride along.  Second list: the
+    FP4 prefill GEMM on the two MLP shapes (FLOPs 2 M K N against the BF16 matrix-core peak)."""
     t = ws.torch
-    out = []
+    out, prefill = [], []
     for (K, N) in LLAMA_SHAPES:
         for block in (16, 32):
             per = K * N // 2 + K * N // block
             n_w = max(2, min(48, (768 << 20) // per))
             nib = [t.randint(0, 256, (N, K // 2), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
-            X, Y = ws.activation(1, K), ws.output(1, N)
+            tiled = []
+            if ws.repack:
+                for w, s_ in zip(nib, sc):
+                    tiled.append(t.empty(ws.lib.tiled_size(FP4, N, K), dtype=t.uint8, device=ws.dev))
+                    assert ws.lib.weight_prepare_fp4(w.data_ptr(), s_.data_ptr(), block, N, K, tiled[-1].data_ptr()) == 0
             iters = max(20, min(400, (4 << 30) // per))
-            ms = ws.bench.fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr,
-                                         N, 1, K, block, iters, 5)
-            if ms < 0:
-                raise RuntimeError(f"fp4 chain failed: {ms}")
-            us = ms * 1000.0 / iters
-            gbs = fp4_bytes(K, N, 1, block) / us * 1e-3
-            out.append({"K": K, "N": N, "M": 1, "block": block, "us": round(us, 2), "GBps": round(gbs, 1),
-                        "frac": round(gbs / HBM_PEAK_GBS, 4), "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(per * n_w / 2 ** 20)})
-            del nib, sc
-    return out
+            mlp = (K, N) in ((4096, 14336), (14336, 4096))
+            for M in tuple(token_counts) + (tuple(prefill_tokens) if mlp and block == 16 else ()):
+                X, Y = ws.activation(M, K), ws.output(M, N)
+                n_it = iters if M <= 16 else 24
+                ms = ws.bench.fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr, N, M, K, block, n_it, 5)
+                if ms < 0:
+                    raise RuntimeError(f"fp4 chain failed: {ms}")
+                us = ms * 1000.0 / n_it
+                if M <= 16:
+                    gbs = fp4_bytes(K, N, M, block) / us * 1e-3
+                    out.append({"K": K, "N": N, "M": M, "block": block, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(per * n_w / 2 ** 20)})
+                else:
+                    tf = 2.0 * M * K * N / us * 1e-6
+                    prefill.append({"K": K, "N": N, "M": M, "block": block, "us": round(us, 2), "TFLOPs": round(tf, 1),
+                                    "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "kernel": ws.lib.last_kernel()})
+                del X, Y
+            for w in nib:
+                ws.lib.weight_release(w.data_ptr())
+            del nib, sc, tiled
+    return out, prefill
 
 
 def cpu_baseline(pkg, threads, unit):
@@ -591,7 +608,7 @@ def main():
                                    "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
             extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
             extra["prefill"] = prefill_cases(ws, by_shape)
-            extra["fp4_sweep"] = fp4_sweep(ws)
+            extra["fp4_sweep"], extra["fp4_prefill"] = fp4_sweep(ws)
     elif args.workload == "decode_linears":
         ops, by_shape = build_decode_model(ws, 1)
         step_bytes = sum(gemv_bytes(K, N, 1) for *_, K, N in ops)
@@ -613,7 +630,7 @@ def main():
         dom_us = dom_ms * 1000.0 / (10 * len(dom_ops))
         if not args.no_sweep:
             extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
-            extra["fp4_sweep"] = fp4_sweep(ws)
+            extra["fp4_sweep"], extra["fp4_prefill"] = fp4_sweep(ws)
     else:
         K, N = (int(v) for v in args.shape.split(","))
         M = args.tokens if args.workload == "gemv" else max(args.tokens, 512)

@@ -52,6 +52,7 @@ EXPORTS = (
     "hip_quant_gemm_noalloc",
     "hip_quant_tiled_size",
     "hip_quant_weight_prepare",
+    "hip_quant_weight_prepare_fp4",
     "hip_quant_weight_release",
     "hip_quant_linear_fused",
     "hip_rms_norm_fwd",
@@ -107,6 +108,8 @@ class QuantLibrary:
         L.hip_quant_tiled_size.argtypes = [i32, i32, i32]
         L.hip_quant_weight_prepare.restype = i32
         L.hip_quant_weight_prepare.argtypes = [vp, i32, i32, i32, i32, vp]
+        L.hip_quant_weight_prepare_fp4.restype = i32
+        L.hip_quant_weight_prepare_fp4.argtypes = [vp, vp, u32, i32, i32, vp]
         L.hip_quant_weight_release.restype = i32
         L.hip_quant_weight_release.argtypes = [vp]
         L.hip_quant_linear_fused.restype = i32
@@ -165,6 +168,9 @@ class QuantLibrary:
 
     def weight_prepare(self, W, w_type, n_out, K, ldw, dst_tiled) -> int:
         return self.c.hip_quant_weight_prepare(W, w_type, n_out, K, ldw, dst_tiled)
+
+    def weight_prepare_fp4(self, W, blk_sc, block_size, n_out, K, dst_tiled) -> int:
+        return self.c.hip_quant_weight_prepare_fp4(W, blk_sc, block_size, n_out, K, dst_tiled)
 
     def weight_release(self, W) -> int:
         return self.c.hip_quant_weight_release(W)

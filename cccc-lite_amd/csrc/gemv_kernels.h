@@ -684,6 +684,208 @@ static __global__ __launch_bounds__(256) void repack_tiled_kernel(const uint8_t*
 }
 
 // ------------------------------------------------------------------------------------------
+// FP4 block-scale GEMV on the matrix cores over a load-time tiled copy, tokens 1..16.
+//
+// fp4 * e4m3 is exact in BF16, but the hardware conversion only applies a power-of-two scale, so the block scale is
+// kept out of the operand: one v_mfma_f32_16x16x16_bf16 contracts exactly one 16-element scale block of 16 rows
+// against up to 16 tokens (FP32 sums of exact products), and the result is multiplied by the rows' block scales
+// and added to the accumulators.  For that the weight is the COLUMN operand: the output lane (n = lane % 16, g)
+// holds row n for tokens 4 g .. 4 g + 3 and needs one scale per instruction -- its own row's.
+//   A operand (rows)    = tokens:      lane (j, g) holds x[j][block + 4 g .. + 3]
+//   B operand (columns) = weight rows: lane (n, g) holds w[n][block + 4 g .. + 3]
+// Tiled copy (repack_tiled_fp4_kernel), per row tile t (16 rows) and chunk c (128 elements):
+//   codes   KiB (t * chunks + c): lane l = n + 16 g owns 16 bytes; byte pair m = 0..7 holds the four nibbles of
+//           row 16 t + n, elements 128 c + 16 m + 4 g .. + 3 (low nibble first, as in the file)
+//   scales  after all code KiBs, 16 * (128 / BLOCK) bytes per (t, c): row n's scales of the chunk, in order
+// so a wave reads one contiguous KiB of codes and one contiguous 128 (64) bytes of scales per chunk.
+// A workgroup owns RT row tiles and splits K over its waves in spans of 128 * U elements; every wave fetches the
+// activations of its span row-contiguously and turns them into operand order through a private LDS slab (8-byte
+// piece q of token t sits at piece q ^ 2 t of the token's 256-byte row: conflict free both ways).
+// MT = 4 or 16: tokens the slab and the fetch are sized for.  K % 32 == 0, X 16-byte aligned, ldx % 8 == 0.
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;        // operand type of the 16x16x16 BF16 matrix-core builtin
+
+template <int BLOCK, int RT, int U, int WAVES, int MT>
+__global__ __launch_bounds__(WAVES * 64) void gemv4_mfma_kernel(const LinearArgs a, const uint8_t* __restrict__ tiled_scales)
+{
+    static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    static_assert(MT == 4 || MT == 16, "token group");
+    constexpr int NS = 128 / BLOCK;                        // scale bytes per row and chunk
+    __shared__ float partial[WAVES][RT][64][4];
+    __shared__ u32x2 xstage[WAVES * U * MT * 32];          // per wave and chunk: MT token rows of 32 8-byte pieces
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int chunks = (a.K + 127) / 128;
+    const int n_tiles = (a.n_out + 15) / 16;
+    const int row_base = blockIdx.x * (16 * RT);
+
+    const uint8_t* wtile[RT];
+    const uint8_t* stile[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+    {
+        const long long tile = min((int)blockIdx.x * RT + rt, n_tiles - 1);      // a clamped tile is computed and dropped
+        wtile[rt] = a.W + tile * chunks * 1024 + lane * 16;
+        stile[rt] = tiled_scales + tile * chunks * (16 * NS) + n * NS;
+    }
+    u32x2* const slab = xstage + wave * (U * MT * 32);
+    const int xk = (lane & 15) * 8;                         // element offset of this lane's 16 bytes within a chunk row
+    const int xt = lane >> 4;                               // token of the first fetch; + 4 per further fetch
+
+    f32x4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) { acc[rt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+    const f32x4 zero = { 0.0f, 0.0f, 0.0f, 0.0f };
+
+    const int span = 128 * U;
+    for (int kb = wave * span; kb < a.K; kb += WAVES * span)
+    {
+        u32x4 xr[U][MT / 4];
+        u32x4 w[U][RT];
+        u32x2 sc[U][RT];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int k = kb + u * 128 + xk;
+#pragma unroll
+            for (int j = 0; j < MT / 4; j++)
+            {
+                xr[u][j] = u32x4{ 0u, 0u, 0u, 0u };
+                if (k < a.K && xt + 4 * j < a.tokens) { xr[u][j] = *(const u32x4*)(a.X + (long long)(xt + 4 * j) * a.ldx + k); }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const long long chunk = kb / 128 + u;
+            const bool in_k = kb + u * 128 < a.K;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+            {
+                w[u][rt] = u32x4{ 0u, 0u, 0u, 0u };
+                sc[u][rt] = u32x2{ 0u, 0u };
+                if (in_k)
+                {
+                    w[u][rt] = __builtin_nontemporal_load((const u32x4*)(wtile[rt] + chunk * 1024));
+                    if (NS == 8) { sc[u][rt] = *(const u32x2*)(stile[rt] + chunk * (16 * NS)); }
+                    else { sc[u][rt][0] = *(const uint32_t*)(stile[rt] + chunk * (16 * NS)); }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();                   // the reads of the previous trip are done (one wave, in-order LDS)
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int j = 0; j < MT / 4; j++)
+            {
+                const int t = xt + 4 * j;
+                *(u32x4*)&slab[(u * MT + t) * 32 + ((2 * (lane & 15)) ^ ((2 * t) & 31))] = xr[u][j];
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+#pragma unroll
+            for (int m = 0; m < 8; m++)
+            {
+                u32x2 xv = { 0u, 0u };
+                if (MT == 16 || n < MT) { xv = slab[(u * MT + (MT == 16 ? n : (n & (MT - 1)))) * 32 + ((4 * m + g) ^ ((2 * n) & 31))]; }
+                const s16x4 xa = __builtin_bit_cast(s16x4, xv);
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++)
+                {
+                    const uint32_t word = w[u][rt][m >> 1];
+                    const bf16x2 lo = (m & 1) ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 2) : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 0);
+                    const bf16x2 hi = (m & 1) ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 3) : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, 1);
+                    const bf16x4 wv = { lo[0], lo[1], hi[0], hi[1] };
+                    const f32x4 t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xa, __builtin_bit_cast(s16x4, wv), zero, 0, 0, 0);
+                    const int si = BLOCK == 16 ? m : (m >> 1);                  // scale byte of this block within the chunk
+                    const uint32_t sword = sc[u][rt][si >> 2];
+                    float s;
+                    switch (si & 3)
+                    {
+                    case 0: s = __builtin_amdgcn_cvt_f32_fp8(sword, 0); break;
+                    case 1: s = __builtin_amdgcn_cvt_f32_fp8(sword, 1); break;
+                    case 2: s = __builtin_amdgcn_cvt_f32_fp8(sword, 2); break;
+                    default: s = __builtin_amdgcn_cvt_f32_fp8(sword, 3); break;
+                    }
+#pragma unroll
+                    for (int c = 0; c < 4; c++) { acc[rt][c] = fmaf(s, t[c], acc[rt][c]); }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) { partial[wave][rt][lane][c] = acc[rt][c]; }
+    __syncthreads();
+
+    // D: lane (n, g) holds weight row n for tokens 4 g .. 4 g + 3
+    for (int v = threadIdx.x; v < RT * 256; v += WAVES * 64)
+    {
+        const int src_lane = v & 63;
+        const int c = (v >> 6) & 3;
+        const int rt = v >> 8;
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) { total += partial[w][rt][src_lane][c]; }
+        const int token = 4 * (src_lane >> 4) + c;
+        const int row = row_base + rt * 16 + (src_lane & 15);
+        if (token < a.tokens && row < a.n_out)
+        {
+            uint16_t* y = a.Y + (long long)token * a.y_stride_tok + (long long)row * a.y_stride_out;
+            *y = finish_output(total, a.alpha, a.beta, y);
+        }
+    }
+}
+
+// Builds the tiled copy of an FP4 weight (layout above) from the packed codes W [n_out][K / 2] and the block scales
+// S over the flat element index.  One thread per 16 destination bytes of codes; the scales of a (tile, chunk) are
+// written by its first 16 * NS threads... here: by the thread that owns lane n, g == 0.
+static __global__ __launch_bounds__(256) void repack_tiled_fp4_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ S, uint8_t* __restrict__ dst,
+                                                              int n_out, int K, int block)
+{
+    const int chunks = (K + 127) / 128;
+    const int ns = 128 / block;
+    const long long n_units = (long long)((n_out + 15) / 16) * chunks * 64;
+    uint8_t* const dst_scales = dst + (long long)((n_out + 15) / 16) * chunks * 1024;
+    for (long long q = (long long)blockIdx.x * 256 + threadIdx.x; q < n_units; q += (long long)gridDim.x * 256)
+    {
+        const int l = (int)(q & 63);
+        const long long tc = q >> 6;                        // tile * chunks + chunk
+        const int c = (int)(tc % chunks);
+        const int row = (int)(tc / chunks) * 16 + (l & 15);
+        const int g = l >> 4;
+        uint16_t out[8];
+#pragma unroll
+        for (int m = 0; m < 8; m++)
+        {
+            const int k = 128 * c + 16 * m + 4 * g;
+            out[m] = (row < n_out && k < K) ? *(const uint16_t*)(W + (((long long)row * K + k) >> 1)) : (uint16_t)0;
+        }
+        u32x4 v;
+#pragma unroll
+        for (int d = 0; d < 4; d++) { v[d] = (uint32_t)out[2 * d] | ((uint32_t)out[2 * d + 1] << 16); }
+        *(u32x4*)(dst + q * 16) = v;
+        if (g == 0)
+        {
+            for (int i = 0; i < ns; i++)
+            {
+                const int k = 128 * c + block * i;
+                dst_scales[tc * (16 * ns) + (l & 15) * ns + i] = (row < n_out && k < K) ? S[((long long)row * K + k) / block] : (uint8_t)0;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // Fallback for any layout / type / size the fast kernels do not take: one lane per output element,
 // software decode of the flat element index exactly as the reference's dequant kernels index it.
 //   element (o, k) of the weight is at flat index  o * w_stride_out + k * w_stride_k

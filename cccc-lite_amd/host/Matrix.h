@@ -33,7 +33,12 @@ public:
     void setQuantScale(float s) { shared_data_->quant_scale_ = s; }
     const void* getBlockScaleData() const { return shared_data_->block_scale_data_; }
     int64_t getBlockScaleCount() const { return shared_data_->block_scale_count_; }
-    void setBlockScaleFromHost(const void* src, int64_t n_scales) { shared_data_->setBlockScaleFromHost(src, n_scales); }
+    // Uploads the FP4 block scales; a [K x n_out] linear weight then gets its tiled copy (codes + scales)
+    void setBlockScaleFromHost(const void* src, int64_t n_scales)
+    {
+        shared_data_->setBlockScaleFromHost(src, n_scales);
+        if (number_ == 1 && channel_ == 1 && getDataType() == FP4_E2M1) { shared_data_->prepareTiled(height_, width_); }
+    }
     void getBlockScaleToHost(void* dst) const { shared_data_->getBlockScaleToHost(dst); }
     static unsigned int fp4BlockSize() { return MatrixData::fp4_block_size_; }
     void prepareTiled() { if (shared_data_ && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); } }

@@ -20,7 +20,7 @@ struct MatrixData
     int64_t block_scale_count_ = 0;
     static constexpr unsigned int fp4_block_size_ = 16;
     float input_scale_ = 0.0f;
-    // Load-time repacked (tiled) copy of an FP8 weight for the matrix-core GEMV; owned here, registered
+    // Load-time repacked (tiled) copy of an FP8 weight, or of an FP4 weight and its block scales, for the matrix-core GEMV; owned here, registered
     // with the kernel library under the key data_.  No counterpart in the reference.
     void* tiled_data_ = nullptr;
     static inline bool repack_weights = true;    // global switch
@@ -40,7 +40,7 @@ struct MatrixData
     void* resize(int64_t size, DataType data_type, bool force = false);
     void release();
 
-    // Builds / drops the tiled copy for a [n_out][K] FP8 weight stored in data_.
+    // Builds / drops the tiled copy for a [n_out][K] FP8 weight (or FP4 weight with block scales) stored in data_.
     void prepareTiled(int n_out, int K);
     void releaseTiled();
 

@@ -122,10 +122,15 @@ void* MatrixData::resize(int64_t size, DataType data_type, bool force)
 void MatrixData::prepareTiled(int n_out, int K)
 {
     releaseTiled();
-    if (!repack_weights || !allow_repack_ || !gpu_ || !data_ || (data_type_ != FP8_E4M3 && data_type_ != FP8_E5M2)) { return; }
+    if (!repack_weights || !allow_repack_ || !gpu_ || !data_ || !Rocblas::isQuantized(data_type_)) { return; }
+    const bool fp4 = data_type_ == FP4_E2M1;
+    // an FP4 weight is tiled together with its block scales: nothing to do until they have arrived
+    if (fp4 && (!block_scale_data_ || K % 32 != 0 || block_scale_count_ < ((int64_t)n_out * K + fp4_block_size_ - 1) / fp4_block_size_)) { return; }
     const unsigned long long bytes = hip_quant_tiled_size((int)data_type_, n_out, K);
     if (bytes == 0 || gpu_->malloc(&tiled_data_, (size_t)bytes) != 0) { tiled_data_ = nullptr; return; }
-    if (hip_quant_weight_prepare(data_, (int)data_type_, n_out, K, K, tiled_data_) != 0)
+    const int rc = fp4 ? hip_quant_weight_prepare_fp4(data_, block_scale_data_, fp4_block_size_, n_out, K, tiled_data_)
+                       : hip_quant_weight_prepare(data_, (int)data_type_, n_out, K, K, tiled_data_);
+    if (rc != 0)
     {
         gpu_->free(tiled_data_);
         tiled_data_ = nullptr;
@@ -168,6 +173,7 @@ void* MatrixData::allocBlockScaleGpu(int64_t n_scales)
 
 void MatrixData::setBlockScaleFromHost(const void* src, int64_t n_scales)
 {
+    releaseTiled();    // a tiled FP4 copy holds the old scales
     if (allocBlockScaleGpu(n_scales)) { GpuControl::copyHostToDevice(block_scale_data_, src, (size_t)n_scales); }
 }
 
@@ -284,7 +290,7 @@ void Matrix::quantizeWeights(DataType target_dt)
     }
     (void)hipDeviceSynchronize();    // float_buf is freed on return
     data_ = shared_data_->data_;
-    if (target_dt != FP4_E2M1 && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); }
+    if (number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); }
 }
 
 // The operand extents a column-major GEMM will touch, checked against what the tensors hold before

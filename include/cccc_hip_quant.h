@@ -132,11 +132,18 @@ C_EXPORT int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K,
  * Results agree with the row-major kernels up to the FP32 summation order.  The copy is keyed on the pointer, not
  * on the bytes behind it: after any write to W the caller must call hip_quant_weight_prepare again (or
  * hip_quant_weight_release), otherwise later calls compute from the stale copy.  hip_quant_weight_release forgets
- * the key (before the caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (FP4, K % 16 != 0, ...).
+ * the key (before the caller frees either buffer).  Returns 0 ok, 1 runtime error, -1 unsupported (K % 16 != 0, ...;
+ * FP4 weights have an entry point of their own below).
  */
 C_EXPORT unsigned long long hip_quant_tiled_size(int type, int n_out, int K);
 C_EXPORT int hip_quant_weight_prepare(const void* W, int type, int n_out, int K, int ldw, void* dst_tiled);
 C_EXPORT int hip_quant_weight_release(const void* W);
+/* The same for an FP4_E2M1 weight W ([n_out][K / 2] packed codes, K % 32 == 0) with its E4M3 block scales
+ * (one byte per block_size = 16 or 32 elements of the flat index): the tiled copy holds codes and scales
+ * (hip_quant_tiled_size(6, n_out, K) bytes) in the order the matrix-core GEMV for 1..16 tokens consumes
+ * them.  hip_quant_gemm uses it when the weight pointer, the block-scale pointer, the block size and the
+ * shape match.  Same rule: prepare again after any write to the codes or the scales. */
+C_EXPORT int hip_quant_weight_prepare_fp4(const void* W, const void* blk_sc, unsigned int block_size, int n_out, int K, void* dst_tiled);
 
 /* ------------------------------------------------------------------------------------------------
  * Decode-step neighbours of the linear (BF16 activations, one new token).

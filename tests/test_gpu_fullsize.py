@@ -131,19 +131,30 @@ def test_fp4_gemv_at_the_llama_8b_shapes(gpu, pkg, oracle, K, n_out, block):
     ridx = torch.from_numpy(rows).to(dev)
     nib_rows, sc_rows = nib[ridx].cpu().numpy(), sc[ridx].cpu().numpy()
     Wd_rows = oracle.dequant_weight(nib_rows, oracle.FP4, len(rows), K, blk_sc=sc_rows, block=block)
-    for tokens in (1, 4):
-        X = synth.activations(n_out + tokens, tokens, K)
-        xd = to_dev(torch, dev, X)
-        yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
-        assert lib.linear(nib.data_ptr(), FP4, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, blk_sc=sc.data_ptr(), block_size=block) == 0
-        kernel = lib.last_kernel()
-        assert kernel.startswith("gemv")
-        out = from_dev(yd, np.uint16)
-        assert not out[tokens * n_out:].any(), "wrote past the end"
-        y = out[:tokens * n_out].reshape(tokens, n_out)
-        want = oracle.linear_exact(Wd_rows, X)
-        check_rows(bf16_f64(oracle, y[:, rows]), want, f"{kernel} fp4 {n_out}x{K} M={tokens} block {block}")
-        check_bf16_close(y[:, rows], want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    # first on the bytes as the file holds them (dot2 kernel), then with the load-time tiled copy registered
+    # (matrix cores from three tokens on, and at one token for the long-row shape)
+    td = torch.zeros(lib.tiled_size(FP4, n_out, K), dtype=torch.uint8, device=dev)
+    for tiled in (False, True):
+        if tiled:
+            assert lib.weight_prepare_fp4(nib.data_ptr(), sc.data_ptr(), block, n_out, K, td.data_ptr()) == 0
+        try:
+            for tokens in (1, 4, 16):
+                X = synth.activations(n_out + tokens, tokens, K)
+                xd = to_dev(torch, dev, X)
+                yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+                assert lib.linear(nib.data_ptr(), FP4, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, blk_sc=sc.data_ptr(), block_size=block) == 0
+                kernel = lib.last_kernel()
+                on_cores = tiled and (tokens >= 3 or K > 8192)
+                assert kernel == ("gemv_mfma_tiled" if on_cores else "gemv_dot2")
+                out = from_dev(yd, np.uint16)
+                assert not out[tokens * n_out:].any(), "wrote past the end"
+                y = out[:tokens * n_out].reshape(tokens, n_out)
+                want = oracle.linear_exact(Wd_rows, X)
+                check_rows(bf16_f64(oracle, y[:, rows]), want, f"{kernel} fp4 {n_out}x{K} M={tokens} block {block}")
+                check_bf16_close(y[:, rows], want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+        finally:
+            if tiled:
+                assert lib.weight_release(nib.data_ptr()) == 0
     ones = np.full((1, K), 0x3F80, dtype=np.uint16)
     yd = torch.zeros(n_out, dtype=torch.int16, device=dev)
     assert lib.linear(nib.data_ptr(), FP4, to_dev(torch, dev, ones).data_ptr(), yd.data_ptr(), n_out, 1, K, blk_sc=sc.data_ptr(), block_size=block) == 0

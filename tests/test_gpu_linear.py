@@ -459,8 +459,7 @@ def test_weight_prepare_builds_the_tiled_layout(gpu, pkg, oracle, n_out, K):
     got = td.cpu().numpy()
     assert np.array_equal(got[:size], tiled_reference(W, n_out, K)) and np.all(got[size:] == 0xAA)
     assert lib.weight_release(wd.data_ptr()) == 0
-    # refused: FP4, K not a multiple of 16, null pointers
-    assert lib.tiled_size(oracle.FP4, n_out, K) == 0
+    # refused: FP4 through the FP8 entry point, K not a multiple of 16, null pointers
     assert lib.weight_prepare(wd.data_ptr(), oracle.FP4, n_out, K, K, td.data_ptr()) == -1
     assert lib.weight_prepare(wd.data_ptr(), oracle.E5M2, n_out, 24, 24, td.data_ptr()) == -1
     assert lib.weight_prepare(None, oracle.E5M2, n_out, K, K, td.data_ptr()) == -1
@@ -505,3 +504,82 @@ def test_prepared_weights_give_the_same_gemv(gpu, pkg, oracle, tokens, n_out, K)
     # after release the same call goes back to the plain kernels
     assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y0.data_ptr(), n_out, tokens, K) == 0
     assert lib.last_kernel() == plain_kernel
+
+
+# ------------------------------------------------------------------------------------------ FP4 tiled copy
+
+def tiled_reference_fp4(nib, sc, n_out, K, block):
+    """NumPy construction of the FP4 tiled copy: per row tile t (16 rows) and chunk c (128 elements) a KiB of codes
+    in which lane l = n + 16 g owns 16 bytes, byte pair m holding row 16 t + n, elements 128 c + 16 m + 4 g .. + 3;
+    after all code KiBs the scales, 16 * (128 / block) bytes per (t, c), row by row."""
+    n_tiles, chunks, ns = (n_out + 15) // 16, (K + 127) // 128, 128 // block
+    codes = np.zeros((n_tiles * 16, chunks * 64), dtype=np.uint8)
+    codes[:n_out, :K // 2] = nib.reshape(n_out, K // 2)
+    pieces = codes.view(np.uint16).reshape(n_tiles, 16, chunks, 8, 4)                    # [t][n][c][m][g]
+    codes_t = np.ascontiguousarray(pieces.transpose(0, 2, 4, 1, 3)).view(np.uint8)        # [t][c][g][n][m]
+    scales = np.zeros((n_tiles * 16, chunks * ns), dtype=np.uint8)
+    scales[:n_out, :K // block] = sc.reshape(n_out, K // block)
+    scales_t = np.ascontiguousarray(scales.reshape(n_tiles, 16, chunks, ns).transpose(0, 2, 1, 3))
+    return np.concatenate([codes_t.ravel(), scales_t.ravel()])
+
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("n_out,K", [(64, 128), (100, 2080), (4096, 4096)])
+def test_weight_prepare_fp4_builds_the_tiled_layout(gpu, oracle, n_out, K, block):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(6)
+    nib = rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8)
+    sc = rng.integers(0, 0x7F, size=(n_out, K // block), dtype=np.uint8)
+    nd, sd = to_dev(torch, dev, nib), to_dev(torch, dev, sc)
+    size = lib.tiled_size(oracle.FP4, n_out, K)
+    assert size == ((n_out + 15) // 16) * ((K + 127) // 128) * (1024 + 128)
+    td = torch.full((size + 64,), 0xAA, dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), block, n_out, K, td.data_ptr()) == 0
+    want = tiled_reference_fp4(nib, sc, n_out, K, block)
+    got = td.cpu().numpy()
+    assert np.array_equal(got[:want.size], want) and np.all(got[size:] == 0xAA)
+    assert lib.weight_release(nd.data_ptr()) == 0
+    assert lib.weight_prepare_fp4(nd.data_ptr(), None, block, n_out, K, td.data_ptr()) == -1
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), 8, n_out, K, td.data_ptr()) == -1
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), block, n_out, 48, td.data_ptr()) == -1
+
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 5, 9, 16])
+@pytest.mark.parametrize("n_out,K", [(300, 544), (4096, 4096), (1024, 4096), (512, 14336), (70000, 32), (8200, 1024), (65600, 160)])
+def test_prepared_fp4_weights_on_the_matrix_cores(gpu, pkg, oracle, tokens, n_out, K, block):
+    """Every launch shape of the FP4 matrix-core kernel on the tiled copy (few / several / many row tiles per CU, short
+    and long rows, ragged row counts, rows that end inside a 128-element chunk), 1..16 tokens, against the exact
+    contraction; alpha / beta; after release the call is back on the row-major kernel."""
+    torch, dev, lib = gpu
+    seed = synth.seed_for(3, 400 + n_out % 91 + tokens + block)
+    nib, sc = synth.weights_fp4(seed, n_out, K, block)
+    X = synth.activations(seed, tokens, K)
+    nd, sd, xd = to_dev(torch, dev, nib), to_dev(torch, dev, sc), to_dev(torch, dev, X)
+    td = torch.zeros(lib.tiled_size(oracle.FP4, n_out, K), dtype=torch.uint8, device=dev)
+    want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block), X)
+    c0 = synth.activations(seed + 1, tokens, n_out)
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), block, n_out, K, td.data_ptr()) == 0
+    try:
+        y = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
+        # one or two tokens stay on the dot2 kernel unless the rows are long and the row tiles few (256 CUs on the test GPU)
+        pays = tokens >= 3 or (K > 8192 and ((n_out + 15) // 16) // 256 < 2)
+        assert lib.last_kernel() == ("gemv_mfma_tiled" if pays else "gemv_dot2")
+        out = from_dev(y, np.uint16)
+        assert not out[tokens * n_out:].any(), "wrote past the end"
+        got = out[: tokens * n_out].reshape(tokens, n_out)
+        check_rows(bf16_f64(oracle, got), want, f"fp4 tiled {n_out}x{K} M={tokens} b={block}")
+        check_bf16_close(got, want, "fp4 tiled", slack_ulp=1.0, abs_floor=2e-5)
+        yb = to_dev(torch, dev, c0.reshape(-1))
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), yb.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block,
+                          alpha=0.5, beta=-2.0) == 0
+        check_rows(bf16_f64(oracle, from_dev(yb, np.uint16).reshape(tokens, n_out)), 0.5 * want - 2.0 * bf16_f64(oracle, c0), "fp4 tiled alpha beta")
+        # other block scales behind the same codes: the copy no longer applies
+        other = to_dev(torch, dev, sc)
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=other.data_ptr(), block_size=block) == 0
+        assert lib.last_kernel() == "gemv_dot2"
+    finally:
+        assert lib.weight_release(nd.data_ptr()) == 0
+    assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
+    assert lib.last_kernel() == "gemv_dot2"
