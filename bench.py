@@ -585,7 +585,7 @@ def main():
         extra["bytes_per_token"] = step_bytes
         extra["decode_step_GBps"] = round(step_bytes / ms_step * 1e-6, 1)
         extra["decode_step_frac_of_hbm_bound"] = round(step_bytes / ms_step * 1e-6 / HBM_PEAK_GBS, 4)
-        extra["launches_per_step"] = 6 * QWEN3_8B["layers"] + 4
+        extra["launches_per_step"] = 6 * QWEN3_8B["layers"] + 2
         extra["last_token"] = model.token
         workload = ("full random-init Qwen3-8B W8A16 decode step, batch 1, greedy: 36 layers, hidden 4096, 32 q / 8 kv heads x 128, qk RMSNorm, "
                     f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions")

@@ -27,13 +27,14 @@ class FusedLinear(ctypes.Structure):
                 ("W", ctypes.c_void_p * 3), ("n_out", ctypes.c_int * 3), ("w_scale", ctypes.c_float * 3),
                 ("Y", ctypes.c_void_p * 3), ("X", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p),
                 ("norm_eps", ctypes.c_float), ("residual", ctypes.c_void_p),
-                ("blk_sc", ctypes.c_void_p * 3), ("block_size", ctypes.c_uint)]
+                ("blk_sc", ctypes.c_void_p * 3), ("block_size", ctypes.c_uint), ("argmax_workspace", ctypes.c_void_p)]
 
 
 def make_fused_linear(w_type, K, W, n_out, Y, X, scales=None, norm_weight=None, norm_eps=1e-6, residual=None, pair=False,
-                      blk_sc=None, block_size=16) -> FusedLinear:
+                      blk_sc=None, block_size=16, argmax_workspace=None) -> FusedLinear:
     d = FusedLinear()
     d.block_size = block_size
+    d.argmax_workspace = argmax_workspace
     for s, p in enumerate(blk_sc or []):
         d.blk_sc[s] = p
     d.w_type, d.K, d.n_segments, d.pair = w_type, K, len(W), 1 if pair else 0
@@ -65,6 +66,7 @@ EXPORTS = (
     "hip_attention_decode_fused_bf16",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
+    "hip_argmax_pick_embed_bf16",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
     "hip_quant_last_kernel",
@@ -134,6 +136,8 @@ class QuantLibrary:
         L.hip_argmax_workspace_bytes.argtypes = [u32]
         L.hip_argmax_bf16.restype = i32
         L.hip_argmax_bf16.argtypes = [vp, u32, vp, vp, vp]
+        L.hip_argmax_pick_embed_bf16.restype = i32
+        L.hip_argmax_pick_embed_bf16.argtypes = [vp, u32, vp, vp, vp, vp, i32, i32]
         L.hip_quant_set_sync.restype = i32
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32

@@ -129,6 +129,8 @@ int hip_quant_linear_fused(const hip_fused_linear* d)
     a.norm_eps = d->norm_eps;
     a.residual = (const uint16_t*)d->residual;
     a.block = d->block_size;
+    if (d->argmax_workspace && (d->n_segments != 1 || d->pair || !aligned16(d->argmax_workspace))) { return -1; }
+    a.argmax_ws = d->argmax_workspace;
     if (fp4)
     {
         note_kernel("gemv_fused_fp4");
@@ -345,7 +347,22 @@ int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
     return finish("attention_decode_fused");
 }
 
-unsigned long long hip_argmax_workspace_bytes(unsigned int n) { return (unsigned long long)((n + ARGMAX_PER_BLOCK - 1) / ARGMAX_PER_BLOCK) * 8; }
+// room for either use: the per-block candidates of hip_argmax_bf16, or the candidate list a linear launch leaves
+unsigned long long hip_argmax_workspace_bytes(unsigned int n)
+{
+    const unsigned long long blocks = (n + ARGMAX_PER_BLOCK - 1) / ARGMAX_PER_BLOCK;
+    const unsigned long long list = 16ull + ((unsigned long long)n / 2 + 16) * 8;
+    return ((blocks * 8 > list ? blocks * 8 : list) + 255ull) & ~255ull;
+}
+
+int hip_argmax_pick_embed_bf16(const void* workspace, unsigned int n, void* d_index, void* d_pos, const void* embed_W, void* embed_y, int D, int n_rows)
+{
+    if (!workspace || !aligned16(workspace) || !d_index || n == 0) { return -1; }
+    if (embed_W && (!embed_y || D <= 0 || D % 8 != 0 || n_rows <= 0 || !aligned16(embed_W) || !aligned16(embed_y))) { return -1; }
+    const int blocks = embed_W ? (D / 8 + 255) / 256 : 1;
+    argmax_pick_embed_kernel<<<blocks < 1 ? 1 : blocks, 256, 0, stream()>>>(workspace, n, (int*)d_index, (int*)d_pos, (const uint16_t*)embed_W, (uint16_t*)embed_y, D, n_rows);
+    return finish("argmax_pick_embed");
+}
 
 int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos, void* workspace)
 {

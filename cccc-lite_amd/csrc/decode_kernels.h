@@ -19,6 +19,41 @@ namespace ccq
 
 __device__ __forceinline__ float bf16_round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// (value, index) order of the greedy pick: larger value first, lower index on ties; NaN never wins
+__device__ __forceinline__ bool better(float v, unsigned i, float bv, unsigned bi) { return v > bv || (v == bv && i < bi); }
+
+// best (value, index) over the 64 lanes of a wave, in every lane
+__device__ __forceinline__ void wave_argmax(float& bv, unsigned& bi)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+    {
+        const float ov = __shfl_xor(bv, off);
+        const unsigned oi = __shfl_xor(bi, off);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+}
+
+// Candidate list a linear kernel leaves for the greedy pick (optional, single-segment launches): one
+// (value, index) per wave or workgroup of the launch.  Layout: [0] count, [4..15] unused, then `capacity` floats,
+// then `capacity` indices, capacity = n_out / 2 + 16 (no launch shape has more waves than row pairs plus one workgroup).
+struct ArgmaxCandidates
+{
+    unsigned* count;
+    float* value;
+    unsigned* index;
+};
+
+__host__ __device__ __forceinline__ ArgmaxCandidates argmax_candidates(void* workspace, unsigned n)
+{
+    const unsigned capacity = n / 2u + 16u;
+    ArgmaxCandidates c;
+    c.count = (unsigned*)workspace;
+    c.value = (float*)((char*)workspace + 16);
+    c.index = (unsigned*)((char*)workspace + 16 + (size_t)capacity * 4);
+    return c;
+}
+
 // Sum over a workgroup of THREADS threads; every thread gets the result.  `scratch` holds THREADS / 64 floats.
 template <int THREADS>
 __device__ __forceinline__ float block_sum(float v, float* scratch)
@@ -53,6 +88,7 @@ struct FusedLinearArgs
     const uint8_t* T[3];       // load-time tiled copies of W[s] (matrix-core variant only)
     const uint8_t* S[3];       // FP4 only: E4M3 block scales of W[s], one byte per `block` elements of the flat index
     unsigned block;            // FP4 only: 16 or 32
+    void* argmax_ws;           // single segment only: candidate list of the outputs for the greedy pick, or nullptr
 };
 
 // Staging of the activation vector into LDS in the [step][half][lane] layout of the dot2 kernels,
@@ -171,7 +207,15 @@ __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const Sta
 
 // What one lane does with the two finished sums of a row group: the SwiGLU pair bf16(silu(gate) * up) with the
 // reference's three roundings (group g = output g), or two plain outputs; the residual is added to a rounded value.
-__device__ __forceinline__ void fused_store(const FusedLinearArgs& a, int g, int seg, int row0, int row1, float t0, float t1)
+__device__ __forceinline__ void store_candidate(const FusedLinearArgs& a, unsigned slot, unsigned n_slots, float v, unsigned i)
+{
+    const ArgmaxCandidates c = argmax_candidates(a.argmax_ws, (unsigned)a.n_out[0]);
+    c.value[slot] = v;
+    c.index[slot] = i;
+    if (slot == 0) { *c.count = n_slots; }
+}
+
+__device__ __forceinline__ void fused_store(const FusedLinearArgs& a, int g, int seg, int row0, int row1, float t0, float t1, float& best_v, unsigned& best_i)
 {
     if (a.pair)
     {
@@ -192,6 +236,9 @@ __device__ __forceinline__ void fused_store(const FusedLinearArgs& a, int g, int
         }
         a.Y[seg][row0] = (uint16_t)f32_to_bf16_bits(o0);
         if (row1 != row0) { a.Y[seg][row1] = (uint16_t)f32_to_bf16_bits(o1); }
+        // greedy candidates are taken on the values as stored (rounded to BF16)
+        if (better(o0, (unsigned)row0, best_v, best_i)) { best_v = o0; best_i = (unsigned)row0; }
+        if (better(o1, (unsigned)row1, best_v, best_i)) { best_v = o1; best_i = (unsigned)row1; }
     }
 }
 
@@ -275,6 +322,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
     if constexpr (!DIRECT_X) { stage_finish<WAVES * 64>(a, staged, xs, red); }
 
     float acc0 = 0.0f, acc1 = 0.0f;
+    float best_v = -INFINITY;                               // greedy candidate of this wave (lane 0 keeps it)
+    unsigned best_i = 0xFFFFFFFFu;
     while (g < n_groups)
     {
         int ng = g, nbatch = batch + 1;
@@ -314,7 +363,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         {
             const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
             acc0 = acc1 = 0.0f;
-            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1); }
+            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1, best_v, best_i); }
         }
         g = ng;
         batch = nbatch;
@@ -331,6 +380,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
             }
         }
     }
+    if (a.argmax_ws && lane == 0) { store_candidate(a, blockIdx.x * WAVES + wave, gridDim.x * WAVES, best_v, best_i); }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -440,6 +490,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv4_fused_kernel(const FusedLine
     stage_finish<WAVES * 64, 4>(a, staged, xs, red);
 
     float acc0 = 0.0f, acc1 = 0.0f;
+    float best_v = -INFINITY;
+    unsigned best_i = 0xFFFFFFFFu;
     while (g < n_groups)
     {
         int ng = g, nbatch = batch + 1;
@@ -470,7 +522,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv4_fused_kernel(const FusedLine
         {
             const float t0 = wave_sum(acc0), t1 = wave_sum(acc1);
             acc0 = acc1 = 0.0f;
-            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1); }
+            if (lane == 0) { fused_store(a, g, cur.seg, cur.row0, cur.row1, t0, t1, best_v, best_i); }
         }
         g = ng;
         batch = nbatch;
@@ -484,6 +536,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv4_fused_kernel(const FusedLine
             sb[u] = nsb[u];
         }
     }
+    if (a.argmax_ws && lane == 0) { store_candidate(a, blockIdx.x * WAVES + wave, gridDim.x * WAVES, best_v, best_i); }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -624,20 +677,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_mfma_kernel(const Fuse
             for (int c = 0; c < 4; c++) { partial[wave][rt][4 * g + c] = acc[rt][c]; }
     }
     __syncthreads();
-    for (int v = threadIdx.x; v < RT * 16; v += WAVES * 64)
+    static_assert(RT * 16 <= 64, "the outputs of a workgroup are finished by its first wave");
+    if (wave != 0) { return; }
+    float best_v = -INFINITY;
+    unsigned best_i = 0xFFFFFFFFu;
     {
+        const int v = lane;
         const int rt = v >> 4, r = v & 15;
         const int tile = (int)blockIdx.x * RT + rt;
-        if (tile >= n_tiles) { continue; }
         const int seg = tile >= t1 ? 2 : (tile >= t0 ? 1 : 0);
         const int row = (tile - (seg == 2 ? t1 : (seg == 1 ? t0 : 0))) * 16 + r;
-        if (row >= a.n_out[seg]) { continue; }
-        float total = 0.0f;
+        if (v < RT * 16 && tile < n_tiles && row < a.n_out[seg])
+        {
+            float total = 0.0f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; wv++) { total += partial[wv][rt][r]; }
-        float out = bf16_round(total);
-        if (a.residual && seg == 0) { out = bf16_round(out + bf16_bits_to_f32(a.residual[row])); }
-        a.Y[seg][row] = (uint16_t)f32_to_bf16_bits(out);
+            for (int wv = 0; wv < WAVES; wv++) { total += partial[wv][rt][r]; }
+            float out = bf16_round(total);
+            if (a.residual && seg == 0) { out = bf16_round(out + bf16_bits_to_f32(a.residual[row])); }
+            a.Y[seg][row] = (uint16_t)f32_to_bf16_bits(out);
+            best_v = out;
+            best_i = (unsigned)row;
+            if (!(out == out)) { best_v = -INFINITY; best_i = 0xFFFFFFFFu; }      // NaN never wins
+        }
+    }
+    if (a.argmax_ws)
+    {
+        wave_argmax(best_v, best_i);
+        if (lane == 0) { store_candidate(a, blockIdx.x, gridDim.x, best_v, best_i); }
     }
 }
 
@@ -1302,18 +1368,11 @@ static __global__ __launch_bounds__(256) void attn_rescale_combine_kernel(const 
 }
 
 // Arg-max of BF16 values, lowest index on ties, in two launches: per-block candidates, then the pick.
-__device__ __forceinline__ bool better(float v, unsigned i, float bv, unsigned bi) { return v > bv || (v == bv && i < bi); }
 
 template <int THREADS>
 __device__ __forceinline__ void block_argmax(float& bv, unsigned& bi, float* best_v, unsigned* best_i)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-    {
-        const float ov = __shfl_xor(bv, off);
-        const unsigned oi = __shfl_xor(bi, off);
-        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
-    }
+    wave_argmax(bv, bi);
     if ((threadIdx.x & 63) == 0) { best_v[threadIdx.x >> 6] = bv; best_i[threadIdx.x >> 6] = bi; }
     __syncthreads();
     if (threadIdx.x == 0)
@@ -1365,6 +1424,42 @@ static __global__ __launch_bounds__(256) void argmax_pick_kernel(const float* __
     {
         *d_index = (int)(bi == 0xFFFFFFFFu ? 0u : bi);
         if (d_pos) { *d_pos += 1; }
+    }
+}
+
+// The greedy pick from the candidate list a linear launch left behind, the step counter, and the embedding row of
+// the picked token for the next step -- one launch.  The first workgroup writes the token and advances *d_pos; every
+// workgroup works the pick out for itself (the list is a few KiB) and copies its share of the embedding row.
+static __global__ __launch_bounds__(256) void argmax_pick_embed_kernel(const void* __restrict__ workspace, unsigned n, int* __restrict__ d_index, int* __restrict__ d_pos,
+                                                               const uint16_t* __restrict__ W, uint16_t* __restrict__ y, int D, int n_rows)
+{
+    __shared__ float best_v[4];
+    __shared__ unsigned best_i[4];
+    __shared__ unsigned picked;
+    const ArgmaxCandidates c = argmax_candidates((void*)workspace, n);
+    const unsigned n_cand = min(*c.count, n / 2u + 16u);
+    float bv = -INFINITY;
+    unsigned bi = 0xFFFFFFFFu;
+    for (unsigned k = threadIdx.x; k < n_cand; k += 256)
+    {
+        if (better(c.value[k], c.index[k], bv, bi)) { bv = c.value[k]; bi = c.index[k]; }
+    }
+    block_argmax<256>(bv, bi, best_v, best_i);
+    if (threadIdx.x == 0)
+    {
+        picked = bi == 0xFFFFFFFFu ? 0u : bi;
+        if (blockIdx.x == 0)
+        {
+            *d_index = (int)picked;
+            if (d_pos) { *d_pos += 1; }
+        }
+    }
+    __syncthreads();
+    if (!W) { return; }
+    const int id = min((int)picked, n_rows - 1);
+    for (int ch = blockIdx.x * 256 + threadIdx.x; ch * 8 < D; ch += gridDim.x * 256)
+    {
+        *(u32x4*)(y + ch * 8) = *(const u32x4*)(W + (size_t)id * D + ch * 8);
     }
 }
 

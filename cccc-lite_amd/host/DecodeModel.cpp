@@ -237,7 +237,9 @@ size_t DecodeModel::weightBytes() const
 int DecodeModel::reset(int token, int pos)
 {
     const int state[2] = { token, pos };
-    return GpuControl::copyHostToDevice(d_state_, state, sizeof(state));
+    if (GpuControl::copyHostToDevice(d_state_, state, sizeof(state)) != 0) { return 1; }
+    // a step starts from the embedding of its token: the previous step's greedy pick leaves it behind, a reset fetches it
+    return hip_embed_token_bf16(d_state_, emb_->data(), x_->data(), cfg_.hidden, cfg_.vocab);
 }
 
 int DecodeModel::currentToken()
@@ -274,9 +276,8 @@ int DecodeModel::step()
 {
     const DecodeConfig& c = cfg_;
     const int q_out = c.n_q * c.head_dim, kv_out = c.n_kv * c.head_dim;
-    const int* d_token = d_state_;
     const int* d_pos = d_state_ + 1;
-    int rc = hip_embed_token_bf16(d_token, emb_->data(), x_->data(), c.hidden, c.vocab);
+    int rc = 0;
     for (int li = 0; li < c.layers && rc == 0; li++)
     {
         Layer& L = layers_[li];
@@ -356,9 +357,11 @@ int DecodeModel::step()
         hip_fused_linear head = linear_desc(*lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
         head.norm_weight = rms_final_->data();
         head.norm_eps = c.eps;
+        head.argmax_workspace = argmax_ws_->data();        // the launch leaves the greedy candidates of its logits
         rc = hip_quant_linear_fused(&head);
     }
-    if (rc == 0) { rc = hip_argmax_bf16(logits_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1, argmax_ws_->data()); }
+    // pick, advance the position, and fetch the next step's embedding row: one launch
+    if (rc == 0) { rc = hip_argmax_pick_embed_bf16(argmax_ws_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1, emb_->data(), x_->data(), c.hidden, c.vocab); }
     return rc;
 }
 

@@ -2,7 +2,7 @@
 // the host mirror: what the reference does per token through MainProcess::testExternalData ->
 // Net::inference -> MatrixOp::forward (cccc/MainProcess.cpp:1171-1239, cccc/Net.cpp:1748-1792,
 // cccc/MatrixOp.cpp:12-26) for the graph of scripts/convert_weights.py:488-692, collapsed into
-// six launches per layer.  Token id and position live in device memory, so a step is a fixed
+// six launches per layer and two per token (lm_head with the greedy candidates; pick + next embedding).  Token id and position live in device memory, so a step is a fixed
 // launch sequence that can be replayed as one hipGraph.
 #pragma once
 #include "Matrix.h"
@@ -66,7 +66,7 @@ public:
     // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
     // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).
     void setExactAttention(bool exact) { exact_attention_ = exact; }
-    int reset(int token, int pos);          // sets the device-side token / position (KV caches are kept)
+    int reset(int token, int pos);          // sets the device-side token / position and fetches the token's embedding (KV caches are kept)
     int step();                             // enqueues one decode step; the next token replaces the current one
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
     double run(int n_steps, int use_graph);

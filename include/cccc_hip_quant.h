@@ -188,6 +188,9 @@ typedef struct hip_fused_linear
     const void* residual;    /* bf16 [n_out[0]] or NULL */
     const void* blk_sc[3];   /* FP4 only: block scales of W[s] */
     unsigned int block_size; /* FP4 only: 16 or 32 */
+    void* argmax_workspace;  /* single segment, no pair: the launch also leaves the greedy-pick candidates of its
+                              * outputs here (hip_argmax_workspace_bytes(n_out[0]) bytes, 16-byte aligned) for
+                              * hip_argmax_pick_embed_bf16; NULL: none */
 } hip_fused_linear;
 C_EXPORT int hip_quant_linear_fused(const hip_fused_linear* desc);
 
@@ -232,6 +235,12 @@ C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, i
  * hip_argmax_workspace_bytes(n) bytes of device memory for the per-block candidates. */
 C_EXPORT unsigned long long hip_argmax_workspace_bytes(unsigned int n);
 C_EXPORT int hip_argmax_bf16(const void* x, unsigned int n, void* d_index, void* d_pos, void* workspace);
+/* The same pick in one launch from the candidate list a hip_quant_linear_fused launch left in `workspace`
+ * (its argmax_workspace; n = that launch's n_out[0]) -- the reference does this on the host after copying the
+ * logits back (cccc-llm/cccc-llm.cpp:546).  When embed_W is not NULL the launch also copies row *d_index of the
+ * BF16 table embed_W [n_rows][D] to embed_y: the embedding of the next step. */
+C_EXPORT int hip_argmax_pick_embed_bf16(const void* workspace, unsigned int n, void* d_index, void* d_pos,
+                                        const void* embed_W, void* embed_y, int D, int n_rows);
 
 /*
  * Library controls (no counterpart in the reference, which always uses the null stream and always

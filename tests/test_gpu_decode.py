@@ -470,3 +470,54 @@ def test_decode_steps_with_fp4_linears_follow_the_oracle(gpu, pkg, oracle, dec):
     logits_eager = model.logits().copy()
     model.reset(3, 0)
     assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
+
+
+@pytest.mark.parametrize("n_out,K,fmt", [(300, 1024, "e5m2"), (5000, 2048, "e5m2"), (70000, 1024, "e5m2 tiled"), (151936, 256, "e5m2 tiled"),
+                                         (4100, 2048, "fp4"), (66000, 512, "fp4")])
+def test_greedy_pick_from_the_linear_epilogue(gpu, pkg, oracle, n_out, K, fmt):
+    """hip_quant_linear_fused leaves the greedy candidates of its outputs, hip_argmax_pick_embed_bf16 picks among them,
+    advances the position and copies the embedding row: the token is the lowest index of the largest stored logit."""
+    from oracle import synth
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(n_out)
+    x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+    xd = to_dev(torch, dev, x)
+    kw = {}
+    if fmt == "fp4":
+        nib, sc = synth.weights_fp4(n_out, n_out, K, 16)
+        wd, sd = to_dev(torch, dev, nib), to_dev(torch, dev, sc)
+        w_type, kw = 6, dict(blk_sc=[sd.data_ptr()], block_size=16)
+    else:
+        W = synth.weights_e5m2(n_out, n_out, K)
+        W[n_out - 1] = W[3]                                        # two equal rows: equal logits, the lower index must win if they are the maximum
+        wd, w_type = to_dev(torch, dev, W), E5M2
+    copies = TiledCopies(torch, dev, lib, [wd], E5M2, K) if fmt.endswith("tiled") else None
+    ws = torch.full((lib.c.hip_argmax_workspace_bytes(n_out),), 0xEE, dtype=torch.uint8, device=dev)
+    y = torch.zeros(n_out, dtype=torch.int16, device=dev)
+    D = 64
+    emb = oracle.f32_to_bf16(rng.standard_normal((n_out, D)).astype(np.float32))
+    ed = to_dev(torch, dev, emb)
+    ey = torch.zeros(D, dtype=torch.int16, device=dev)
+    st = torch.tensor([-1, 41], dtype=torch.int32, device=dev)
+    d = pkg.capi.make_fused_linear(w_type, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(), argmax_workspace=ws.data_ptr(), **kw)
+    assert lib.quant_linear_fused(d) == 0
+    assert lib.last_kernel() == {"e5m2": "gemv_fused", "e5m2 tiled": "gemv_fused_mfma", "fp4": "gemv_fused_fp4"}[fmt]
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert lib.c.hip_argmax_pick_embed_bf16(ptr(ws), n_out, ptr(st), ctypes.c_void_p(st.data_ptr() + 4), ptr(ed), ptr(ey), D, n_out) == 0
+    if copies:
+        copies.release()
+    logits = oracle.bf16_to_f32(from_dev(y, np.uint16))
+    want = int(np.argmax(logits))                                    # first occurrence of the maximum
+    assert st.cpu().tolist() == [want, 42]
+    assert np.array_equal(from_dev(ey, np.uint16), emb[want])
+    # forced tie at the top: rows 3 and n_out - 1 of the logits made the largest by scaling x would need new weights; instead check
+    # the tie rule on the stored values directly: equal maxima -> lowest index
+    ties = np.flatnonzero(logits == logits.max())
+    assert want == ties[0]
+    # without an embedding table the launch only picks
+    assert lib.c.hip_argmax_pick_embed_bf16(ptr(ws), n_out, ptr(st), None, None, None, 0, 0) == 0
+    assert st.cpu().tolist() == [want, 42]
+    # refused: a candidate list on a multi-segment or pair launch
+    bad = pkg.capi.make_fused_linear(w_type, K, [wd.data_ptr(), wd.data_ptr()], [n_out, n_out], [y.data_ptr(), y.data_ptr()], xd.data_ptr(),
+                                     argmax_workspace=ws.data_ptr(), **({} if fmt != "fp4" else dict(blk_sc=[sd.data_ptr(), sd.data_ptr()], block_size=16)))
+    assert lib.quant_linear_fused(bad) == -1
