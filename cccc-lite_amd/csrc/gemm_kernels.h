@@ -271,10 +271,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // SPLIT: blockIdx.y selects one of gridDim.y equal ranges of k-tiles; the FP32 partial sums of range s go
 // to partial[s][token][feature] (no alpha / beta) and gemm_splitk_combine_kernel finishes them.  Used when
 // the output has too few tiles to fill the machine.
-template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16>
+// NB: 16-feature blocks per wave (a workgroup owns 64 NB features): 4 by default; 3 or 2 give the launch more, smaller
+// workgroups when the output has too few 256-feature tiles to fill the machine evenly.
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, float* __restrict__ partial)
 {
-    constexpr int NB = 4;                       // 16-feature blocks per wave
     constexpr int BTOK = MB * 16;               // tokens per workgroup
     constexpr int BK = 64, CPR = 8;
     constexpr int X_PER_THREAD = BTOK * CPR / 256;
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_tile = blockIdx.x % n_tiles;
     const int m_tile = blockIdx.x / n_tiles;
-    const int out_base = n_tile * 256 + wave * 64;
+    const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
     const int g = lane >> 4;
@@ -505,17 +506,17 @@ __global__ __launch_bounds__(256) void gemm_splitk_combine_kernel(const float* _
 }
 
 // splits > 1: `partial` holds splits * tokens * n_out floats
-template <int WT, int MB, bool TILED, int AT = DT_BF16>
+template <int WT, int MB, bool TILED, int AT = DT_BF16, int NB = 4>
 void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial = nullptr)
 {
-    const int n_tiles = (a.n_out + 255) / 256;
+    const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
     const dim3 grid(n_tiles * m_tiles, splits);
     const bool scaled = a.w_scale != 1.0f;
     if (splits > 1)
     {
-        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
-        else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
         const long long groups = (long long)a.tokens * (a.n_out / 4);
         const long long blocks = (groups + 255) / 256;
         const long long cap = (long long)cu_count() * 16;
@@ -523,8 +524,8 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
     }
     else
     {
-        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
-        else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+        else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
     }
 }
 
@@ -560,12 +561,34 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }
             const int cus = cu_count();
+            // Tile shape: 64 NB features x 16 MB tokens per workgroup.  What a shape costs, measured on MI355X: a CU wants
+            // two resident workgroups (one alone reaches ~85 % of the rate), the workgroups should spread evenly over the
+            // CUs (384 tiles on 256 CUs leave half of them with twice the work: 36 % of peak where 512 even tiles reach
+            // 42 %), and 48-feature waves with 64-token tiles cost ~5 % against the larger tiles.
+            struct Shape { int nb, mb; double quality; };
+            const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, 1.0 }, { 3, 8, 1.0 }, { 3, 4, 0.95 } };
+            int nb = 4, mb = 4;
+            double best = -1.0;
+            for (const Shape& sh : shapes)
+            {
+                if (sh.mb == 8 && a.tokens <= 64) { continue; }
+                const long long tiles = (long long)((a.n_out + 64 * sh.nb - 1) / (64 * sh.nb)) * ((a.tokens + 16 * sh.mb - 1) / (16 * sh.mb));
+                const double balance = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
+                const double occupancy = tiles >= 2LL * cus ? 1.0 : (tiles > cus ? 0.95 : 0.85);
+                const double score = sh.quality * balance * occupancy;
+                if (score > best + 1e-9)
+                {
+                    best = score;
+                    nb = sh.nb;
+                    mb = sh.mb;
+                }
+            }
+            int splits = 1;
+            float* partial = nullptr;
+            // too few tiles in every shape: split the k range over workgroups instead (256-feature tiles)
             const long long n_tiles = (a.n_out + 255) / 256;
             const long long tiles8 = n_tiles * ((a.tokens + 127) / 128), tiles4 = n_tiles * ((a.tokens + 63) / 64);
-            int mb = 4, splits = 1;
-            float* partial = nullptr;
-            if (a.tokens > 64 && tiles8 >= 2LL * cus) { mb = 8; }
-            else if (tiles4 * 4 < 5LL * cus && a.n_out % 4 == 0)
+            if (best < 0.6 && tiles4 * 4 < 5LL * cus && a.n_out % 4 == 0)
             {
                 const long long base = a.tokens > 64 ? tiles8 : tiles4;
                 long long s = (cus + base / 2) / base;
@@ -585,17 +608,20 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
                 if (partial)
                 {
                     splits = (int)s;
+                    nb = 4;
                     mb = a.tokens > 64 ? 8 : 4;
                 }
             }
             if (tiled)
             {
-                if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial); }
+                if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, true, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, true, AT, 3>(d); }
+                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial); }
                 else { launch_gemm_mfma_direct<WT, 4, true, AT>(d, splits, partial); }
             }
             else
             {
-                if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial); }
+                if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, false, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, false, AT, 3>(d); }
+                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial); }
                 else { launch_gemm_mfma_direct<WT, 4, false, AT>(d, splits, partial); }
             }
             return true;

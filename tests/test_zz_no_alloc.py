@@ -59,10 +59,10 @@ def test_noalloc_entry_point_matches_hip_quant_gemm(gpu, pkg, oracle):
 
 
 def test_noalloc_entry_point_refuses_what_does_not_fit(gpu, pkg, oracle, capfd):
-    """1100 tokens x 4096 features split K in two: 2 * 1100 * 4096 * 4 bytes = 36 MB of partial sums, more than
+    """512 tokens x 4352 features split K in four: 4 * 512 * 4352 * 4 bytes = 35.7 MB of partial sums, more than
     the static 32 MiB.  The call says so, launches nothing and leaves C alone; hip_quant_gemm takes the shape."""
     torch, dev, lib = gpu
-    tokens, n_out, K = 1100, 4096, 12288
+    tokens, n_out, K = 512, 4352, 12288
     w = torch.zeros(n_out * K, dtype=torch.uint8, device=dev)
     x = torch.zeros(tokens * K, dtype=torch.int16, device=dev)
     y = torch.full((tokens * n_out,), 0x1234, dtype=torch.int16, device=dev)
