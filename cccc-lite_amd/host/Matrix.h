@@ -18,6 +18,12 @@ public:
 
     // A view of the same storage with other dims (element count must not grow).
     Matrix view(int w, int h, int c, int n) const;
+    // Rows [row0, row0 + n_rows) of a (W x H) matrix as a (W x n_rows) matrix on the same storage -- for a linear
+    // weight stored [n_out][K] these are output features row0 .. row0 + n_rows - 1 with their block scales.  This is
+    // how several projections that share an input (q, k, v; gate, up) can live in ONE storage that a single GEMV
+    // reads while each keeps a tensor of its own (the reference's view mechanics: cccc/MatrixOp.cpp:1370-1396).
+    // An empty Matrix when the range does not fit or the matrix is not 2-D.
+    Matrix rowsView(int row0, int n_rows) const;
 
     int getWidth() const { return width_; }
     int getHeight() const { return height_; }
@@ -31,7 +37,10 @@ public:
 
     float getQuantScale() const { return shared_data_->quant_scale_; }
     void setQuantScale(float s) { shared_data_->quant_scale_ = s; }
-    const void* getBlockScaleData() const { return shared_data_->block_scale_data_; }
+    const void* getBlockScaleData() const
+    {
+        return shared_data_->block_scale_data_ ? (const uint8_t*)shared_data_->block_scale_data_ + scale_offset_ : nullptr;
+    }
     int64_t getBlockScaleCount() const { return shared_data_->block_scale_count_; }
     // Uploads the FP4 block scales; a [K x n_out] linear weight then gets its tiled copy (codes + scales)
     void setBlockScaleFromHost(const void* src, int64_t n_scales)
@@ -74,6 +83,7 @@ private:
 
     std::shared_ptr<MatrixData> shared_data_;
     void* data_ = nullptr;
+    int64_t scale_offset_ = 0;    // first block scale of this view within the storage's scale array
     int width_ = 0, height_ = 0, channel_ = 0, number_ = 0, row_ = 0;
 };
 

@@ -261,6 +261,49 @@ int WeightFile::loadNamed(Matrix& m, const std::string& name) const
     return m.copyFromHost(bytes, n_bytes) == 0 ? 0 : -1;
 }
 
+int WeightFile::loadNamedGroup(Matrix& m, const std::vector<std::string>& names) const
+{
+    const int K = m.getWidth();
+    const int64_t elems = m.getDataSize();
+    if (names.empty() || K <= 0 || m.getChannel() != 1 || m.getNumber() != 1) { return -1; }
+    DataType dt = CURRENT;
+    float scale = 1.0f;
+    std::vector<uint8_t> codes, scales;
+    for (const std::string& name : names)
+    {
+        const WeightKey wk = resolve(name);
+        if (!wk.valid()) { return 1; }
+        auto [bytes, n_bytes] = get_value(wk.key);
+        if (!wk.is_quant || !bytes || n_bytes == 0) { return -1; }
+        const float s = loadFloat("scale_" + wk.source, 1.0f);
+        if (dt == CURRENT) { dt = wk.dt; scale = s; }
+        else if (wk.dt != dt || s != scale) { return -1; }
+        const int64_t per_row = dt == FP4_E2M1 ? K / 2 : K;              // bytes per row
+        if (dt == FP4_E2M1 && K % (2 * (int)Matrix::fp4BlockSize()) != 0) { return -1; }
+        // whole rows only; an FP4 blob sized by elements (the reference's own writer) carries its data in the first half
+        int64_t data_bytes = (int64_t)n_bytes;
+        if (dt == FP4_E2M1 && data_bytes % (2 * per_row) == 0 && has_value("blockscale_" + wk.source) &&
+            (int64_t)get_value("blockscale_" + wk.source).second * (int64_t)Matrix::fp4BlockSize() == data_bytes)
+        {
+            data_bytes /= 2;
+        }
+        if (data_bytes % per_row != 0) { return -1; }
+        codes.insert(codes.end(), bytes, bytes + data_bytes);
+        if (dt == FP4_E2M1)
+        {
+            auto [bs, bs_bytes] = get_value("blockscale_" + wk.source);
+            const int64_t n_blocks = data_bytes * 2 / (int64_t)Matrix::fp4BlockSize();
+            if (!bs || (int64_t)bs_bytes < n_blocks) { return -1; }
+            scales.insert(scales.end(), bs, bs + n_blocks);
+        }
+    }
+    const int64_t want = dt == FP4_E2M1 ? elems / 2 : elems;
+    if ((int64_t)codes.size() != want) { return -1; }
+    m.loadQuantizedDirect(codes.data(), want, scale, dt);
+    if (dt == FP4_E2M1) { m.setBlockScaleFromHost(scales.data(), (int64_t)scales.size()); }
+    return 0;
+}
+
 // ------------------------------------------------------------------ writer
 
 void WeightFileWriter::set_value(const std::string& key, const void* bytes, size_t n)

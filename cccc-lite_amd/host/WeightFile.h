@@ -62,6 +62,13 @@ public:
     // 0 loaded; 1 not in the file; -1 byte count does not fit the tensor.
     int loadNamed(Matrix& m, const std::string& name) const;
 
+    // Loads several quantized linear weights that share their input width into ONE storage, row ranges in the
+    // order given (m is K x sum of their rows): the file bytes are uploaded unchanged, one after the other, FP4 block
+    // scales likewise, and the storage gets one tiled copy.  A GEMV on m then serves all of them in one launch and
+    // Matrix::rowsView hands each projection its own tensor.  All members must have the same data type and the same
+    // per-tensor scale (the one GEMM call has one).  0 ok; 1 a name is missing; -1 sizes, types or scales do not fit.
+    int loadNamedGroup(Matrix& m, const std::vector<std::string>& names) const;
+
 private:
     struct Entry
     {

@@ -215,6 +215,19 @@ Matrix Matrix::view(int w, int h, int c, int n) const
     return m;
 }
 
+Matrix Matrix::rowsView(int row0, int n_rows) const
+{
+    if (!shared_data_ || channel_ != 1 || number_ != 1 || row0 < 0 || n_rows <= 0 || row0 + n_rows > height_) { return Matrix(); }
+    const int64_t first = (int64_t)row0 * width_;                       // first element of the range
+    const DataType dt = getDataType();
+    if (dt == FP4_E2M1 && (first % 2 != 0 || first % fp4BlockSize() != 0)) { return Matrix(); }
+    Matrix m = *this;
+    m.setDim(width_, n_rows, 1, 1);
+    m.data_ = (char*)data_ + (dt == FP4_E2M1 ? first / 2 : first * (int64_t)Rocblas::elemBytes(dt));
+    m.scale_offset_ = scale_offset_ + (dt == FP4_E2M1 ? first / fp4BlockSize() : 0);
+    return m;
+}
+
 int Matrix::copyFromHost(const void* src, size_t bytes)
 {
     if (!shared_data_ || bytes > shared_data_->sizeInByte()) { return 1; }

@@ -137,6 +137,21 @@ int cccc_weightfile_resolve(void* f, const char* name, char* key_out, int capaci
     return (int)wk.dt | (wk.is_quant ? 0x10000 : 0);
 }
 
+// names: NUL-separated list ending with an empty string
+int cccc_weightfile_load_named_group(void* f, void* m, const char* names)
+{
+    std::vector<std::string> list;
+    for (const char* p = names; p && *p; p += std::strlen(p) + 1) { list.emplace_back(p); }
+    return ((WeightFile*)f)->loadNamedGroup(*(Matrix*)m, list);
+}
+
+// A new Matrix handle viewing rows [row0, row0 + n_rows) of m (NULL when the range does not fit); destroy it like any other.
+void* cccc_matrix_rows_view(void* m, int row0, int n_rows)
+{
+    Matrix v = ((Matrix*)m)->rowsView(row0, n_rows);
+    return v.data() ? new Matrix(v) : nullptr;
+}
+
 int cccc_weightfile_load_named(void* f, void* m, const char* name) { return ((WeightFile*)f)->loadNamed(*(Matrix*)m, name); }
 
 unsigned char cccc_host_float_to_e4m3(float v) { return floatToE4m3Truncated(v); }

@@ -59,6 +59,8 @@ class HostLibrary:
         L.cccc_weightfile_key.restype = ctypes.c_char_p; L.cccc_weightfile_key.argtypes = [vp, i32]
         L.cccc_weightfile_get.restype = ctypes.c_longlong; L.cccc_weightfile_get.argtypes = [vp, ctypes.c_char_p, vp, u64]
         L.cccc_weightfile_resolve.restype = i32; L.cccc_weightfile_resolve.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p, i32]
+        L.cccc_weightfile_load_named_group.restype = i32; L.cccc_weightfile_load_named_group.argtypes = [vp, vp, ctypes.c_char_p]
+        L.cccc_matrix_rows_view.restype = vp; L.cccc_matrix_rows_view.argtypes = [vp, i32, i32]
         L.cccc_weightfile_load_named.restype = i32; L.cccc_weightfile_load_named.argtypes = [vp, vp, ctypes.c_char_p]
         L.cccc_host_float_to_e4m3.restype = ctypes.c_ubyte; L.cccc_host_float_to_e4m3.argtypes = [f32]
         L.cccc_host_half_to_bf16.restype = ctypes.c_ushort; L.cccc_host_half_to_bf16.argtypes = [ctypes.c_ushort]
@@ -119,6 +121,11 @@ class WeightFile:
     def load_named(self, m: "HostMatrix", name: str) -> int:
         return self.lib.c.cccc_weightfile_load_named(self.handle, m.handle, name.encode())
 
+    def load_named_group(self, m: "HostMatrix", names) -> int:
+        """Several quantized linears sharing their input into one storage, row ranges in the order given."""
+        packed = b"".join(n.encode() + b"\0" for n in names) + b"\0"
+        return self.lib.c.cccc_weightfile_load_named_group(self.handle, m.handle, packed)
+
 
 class HostMatrix:
     def __init__(self, lib: HostLibrary, handle):
@@ -171,6 +178,13 @@ class HostMatrix:
 
     def prepare_tiled(self) -> bool:
         return self.lib.c.cccc_matrix_prepare_tiled(self.handle) == 0
+
+    def rows_view(self, row0: int, n_rows: int) -> "HostMatrix":
+        """Rows [row0, row0 + n_rows) as a matrix of their own on the same storage (Matrix::rowsView)."""
+        handle = self.lib.c.cccc_matrix_rows_view(self.handle, row0, n_rows)
+        if not handle:
+            raise ValueError("row range does not fit")
+        return HostMatrix(self.lib, handle)
 
     def save_named(self, name: str, path) -> None:
         if self.lib.c.cccc_matrix_save_named(self.handle, name.encode(), str(path).encode()) != 0:

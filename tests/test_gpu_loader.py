@@ -343,3 +343,68 @@ def test_decode_model_from_an_fp4_file(tmp_path, gpu, pkg, host, oracle, dec):
     bw.save(broken)
     with pytest.raises(ValueError, match="W_o_0"):
         make_model(pkg, host, cfg).load_named(pkg.host_api.WeightFile(host, broken))
+
+
+@pytest.mark.parametrize("fmt", ["fp8_e5m2", "fp4_e2m1"])
+def test_projections_sharing_an_input_load_into_one_storage(tmp_path, gpu, pkg, host, oracle, fmt):
+    """q, k, v of one layer in ONE storage (WeightFile::loadNamedGroup): a single GEMV on it gives the three
+    projections back to back, bit for bit what three separately loaded weights give, and Matrix::rowsView hands
+    each projection out as a tensor of its own (codes, and for FP4 the block scales, at the right offsets)."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(12)
+    K, rows = 1024, (512, 128, 128)
+    names = ("W_q_0", "W_k_0", "W_v_0")
+    w = weight_file.BinWriter()
+    packed = []
+    for name, n in zip(names, rows):
+        wf = (rng.standard_normal((n, K)) * 0.02).astype(np.float32)
+        if fmt == "fp4_e2m1":
+            nib, sc = synth.pack_fp4_blockscale(wf, 16)
+            w.add(f"weight_fp4_e2m1_{name}", nib); w.add(f"blockscale_{name}", sc)
+            packed.append((nib, sc))
+        else:
+            codes = oracle.encode_e5m2_rne(wf)
+            w.add(f"weight_fp8_e5m2_{name}", codes)
+            packed.append((codes, None))
+    w.add("weight_fp8_e4m3_W_other", np.zeros((128, K), np.uint8))
+    w.add("weight_fp8_e5m2_W_scaled", np.zeros((128, K), np.uint8)); w.add_float("scale_W_scaled", 0.5)
+    path = tmp_path / "group.bin"
+    w.save(path)
+    f = pkg.host_api.WeightFile(host, path)
+    dtype = FP4 if fmt == "fp4_e2m1" else E5M2
+
+    total = sum(rows)
+    group = host.matrix(K, total, 1, 1, BF16)
+    assert f.load_named_group(group, names) == 0 and group.dtype == dtype
+    for tokens in (1, 4):
+        X = synth.activations(70 + tokens, tokens, K)
+        xm = host.matrix(K, tokens, 1, 1, BF16); xm.upload(X)
+        y_all = host.matrix(total, tokens, 1, 1, BF16)
+        assert pkg.host_api.mul_batched(group, xm, y_all, ta=1, tb=0) == 0
+        got = y_all.download(np.uint16, tokens * total).reshape(tokens, total)
+        row0 = 0
+        for name, n, (codes, sc) in zip(names, rows, packed):
+            single = host.matrix(K, n, 1, 1, BF16)
+            assert f.load_named(single, name) == 0
+            y1 = host.matrix(n, tokens, 1, 1, BF16)
+            assert pkg.host_api.mul_batched(single, xm, y1, ta=1, tb=0) == 0
+            want_bits = y1.download(np.uint16, tokens * n).reshape(tokens, n)
+            Wd = oracle.dequant_weight(codes, oracle.FP4 if sc is not None else oracle.E5M2, n, K, blk_sc=sc)
+            check_rows(oracle.bf16_to_f32(got[:, row0:row0 + n]).astype(np.float64), oracle.linear_exact(Wd, X), name)
+            assert np.abs(oracle.bf16_to_f32(got[:, row0:row0 + n]).astype(np.float64) - oracle.bf16_to_f32(want_bits).astype(np.float64)).max() \
+                <= 2.0 ** -7 * np.abs(oracle.bf16_to_f32(want_bits)).max()
+            # the projection as a tensor of its own on the shared storage
+            view = group.rows_view(row0, n)
+            assert view.dtype == dtype and view.data_ptr == group.data_ptr + (row0 * K // 2 if sc is not None else row0 * K)
+            yv = host.matrix(n, tokens, 1, 1, BF16)
+            assert pkg.host_api.mul_batched(view, xm, yv, ta=1, tb=0) == 0
+            check_rows(oracle.bf16_to_f32(yv.download(np.uint16, tokens * n).reshape(tokens, n)).astype(np.float64), oracle.linear_exact(Wd, X), name + " view")
+            row0 += n
+    # members of different types or scales, a missing name, a storage of the wrong size
+    if fmt == "fp8_e5m2":
+        assert f.load_named_group(host.matrix(K, 512 + 128, 1, 1, BF16), ("W_q_0", "W_other")) == -1
+        assert f.load_named_group(host.matrix(K, 512 + 128, 1, 1, BF16), ("W_q_0", "W_scaled")) == -1
+    assert f.load_named_group(host.matrix(K, total, 1, 1, BF16), ("W_q_0", "W_k_0", "W_nope")) == 1
+    assert f.load_named_group(host.matrix(K, total + 16, 1, 1, BF16), names) == -1
+    with pytest.raises(ValueError):
+        group.rows_view(total - 8, 16)
