@@ -134,13 +134,17 @@ bool gemv8_mfma_ksplit_tiled(const LinearArgs& a, const uint8_t* tiled)
 {
     LinearArgs t = a;
     t.W = tiled;
-    const int tiles_per_cu = ((a.n_out + 15) / 16) / cu_count();
+    const int n_tiles = (a.n_out + 15) / 16;
+    const int tiles_per_cu = n_tiles / cu_count();
     if (tiles_per_cu >= 16)
     {
         if (a.tokens <= 4) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED>(t); }
         else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED, true>(t); }
         else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED, true>(t); }
     }
+    // projections stored together (gate + up: 24576 rows, q + k + v: 6144 rows), one or two tokens
+    else if (tiles_per_cu >= 4 && a.tokens <= 2) { launch_ksplit_tiled<WT, 2, 2, 16, SCALED>(t); }
+    else if (tiles_per_cu < 2 && a.K <= 8192 && a.tokens <= 2 && 2 * n_tiles >= 3 * cu_count()) { launch_ksplit_tiled<WT, 2, 4, 8, SCALED>(t); }
     else if (tiles_per_cu >= 2)
     {
         if (a.tokens <= 2) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED>(t); }
