@@ -443,8 +443,11 @@ int quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
             }
             else if (ok && !launched)
             {
-                launched = a.block_size == 16 ? gemm_mfma<DT_FP4, 16>(a) : gemm_mfma<DT_FP4, 32>(a);
-                if (launched) { note_kernel("gemm_mfma"); }
+                // the register-fed kernel reads the tiled copy; it wants whole 128-element chunks and at least 48 tokens
+                const uint8_t* tiled = (K % 128 == 0 && a.tokens >= 48) ? find_tiled_fp4(a) : nullptr;
+                launched = a.block_size == 16 ? gemm_mfma<DT_FP4, 16>(a, tiled, split_scratch) : gemm_mfma<DT_FP4, 32>(a, tiled, split_scratch);
+                if (!launched) { return -2; }                    // only a fixed scratch buffer that is too small ends here
+                note_kernel(tiled ? "gemm_mfma_tiled" : "gemm_mfma");
             }
         }
         else

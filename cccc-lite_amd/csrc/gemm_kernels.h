@@ -505,6 +505,302 @@ __global__ __launch_bounds__(256) void gemm_splitk_combine_kernel(const float* _
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// The same GEMM for FP4 block-scale weights, on their load-time tiled copy (repack_tiled_fp4_kernel): per 16-row tile and
+// 128-element chunk one contiguous KiB of codes -- lane (n = lane % 16, g = lane / 16) owns 16 bytes whose dword d holds
+// row n's elements 32 d + 4 g .. + 3 (low 16 bits) and 32 d + 16 + 4 g .. + 3 (high 16 bits) of the chunk -- and, behind
+// all code KiBs, 128 / BLOCK scale bytes per row and chunk.  One dword is therefore the lane's row operand of one
+// v_mfma_f32_16x16x32_bf16 (k = those eight elements), dwords 0, 1 belong to the first 64-element half of the chunk and
+// 2, 3 to the second.  fp4 * e4m3 has at most six significant bits, so bf16(fp4 * s) is exact: the codes are converted
+// to FP32 (v_cvt_scalef32_pk_f32_fp4; the hardware conversion itself only applies a power-of-two scale), multiplied by
+// the block scale and packed to BF16 in registers -- 16 VALU instructions per dword, shared by the MB token blocks.
+// The activation tile of a 64-element half is staged in LDS already in that operand order: 16-byte piece 4 s + g of a
+// token row holds elements 32 s + 4 g .. + 3 and 32 s + 16 + 4 g .. + 3, so a fragment is one 16-byte read.
+// K % 128 == 0.  Tile shapes, k split and epilogue as in gemm_mfma_direct_kernel, except that the 128-token x 256-feature
+// tile is compiled for one workgroup per CU (its accumulators, two operand buffers and two raw chunks do not fit the
+// 256 registers a wave has when two workgroups share a CU; with the whole register file the accumulators sit in AGPRs).
+template <int BLOCK>
+__device__ __forceinline__ u32x4 dequant8_fp4_blocks(uint32_t w, float s_lo, float s_hi)
+{
+    uint32_t out[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+    {
+        f32x2 v;
+        switch (b)
+        {
+        case 0: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); break;
+        case 1: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); break;
+        case 2: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); break;
+        default: v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); break;
+        }
+        const float sc = (BLOCK == 16 && b >= 2) ? s_hi : s_lo;
+        const bf16x2 p = { (__bf16)(v.x * sc), (__bf16)(v.y * sc) };
+        out[b] = __builtin_bit_cast(uint32_t, p);
+    }
+    return u32x4{ out[0], out[1], out[2], out[3] };
+}
+
+template <int BLOCK, int MB, bool SPLIT, int NB = 4>
+__global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a, const uint8_t* __restrict__ tiled_scales, const int n_tiles,
+                                                                                        const int m_tiles, float* __restrict__ partial)
+{
+    static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    constexpr int NS = 128 / BLOCK;             // scale bytes per row and chunk
+    constexpr int BTOK = MB * 16;
+    constexpr int BK = 64, CPR = 8;
+    constexpr int X_PER_THREAD = BTOK * CPR / 256;
+    __shared__ u32x4 xs[2][BTOK * CPR];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // The hardware hands consecutive workgroups to the eight XCDs in turn, each with an L2 of its own.  XCD x takes the
+    // feature tiles x, x + 8, ... and walks all token tiles of one before the next: the workgroups that share a weight
+    // tile then run on one XCD at about the same time and the tile reaches that L2 once.
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int n_tile = xcd + 8 * (local / m_tiles);
+    const int m_tile = local % m_tiles;
+    if (n_tile >= n_tiles) { return; }          // the grid is padded to whole rounds of eight feature tiles
+    const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
+    const int tok_base = m_tile * BTOK;
+    const int i16 = lane & 15;
+    const int g = lane >> 4;
+    const int chunks_total = a.K / 128;
+    const int c_begin = SPLIT ? (int)((long long)chunks_total * blockIdx.y / gridDim.y) : 0;
+    const int n_chunks = SPLIT ? (int)((long long)chunks_total * (blockIdx.y + 1) / gridDim.y) - c_begin : chunks_total;
+    const int n_kt = 2 * n_chunks;
+    const uint8_t* const x_begin = (const uint8_t*)a.X + (long long)c_begin * 128 * 2;
+
+    f32x4 acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { acc[mb][nb] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+
+    // Every address in the loop is a wave-uniform base (scalar registers) plus a 32-bit per-lane byte offset fixed for
+    // the whole kernel.
+    long long w_base[NB], s_base[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+    {
+        const long long tile = min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1);     // a clamped tile is computed and dropped
+        w_base[nb] = (tile * chunks_total + c_begin) * 1024;
+        s_base[nb] = (tile * chunks_total + c_begin) * (16 * NS);
+    }
+    const uint32_t w_off = lane * 16, s_off = i16 * NS;
+    uint32_t x_off[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; i++)
+    {
+        const int q = tid + i * 256;
+        x_off[i] = (uint32_t)(((long long)min(tok_base + q / CPR, a.tokens - 1) * a.ldx + (q % CPR) * 8) * 2);
+    }
+    // LDS slot (in 8-byte units) of this thread's first activation piece: elements 8 q8 .. + 3 go to piece 4 s + g0 at
+    // half hb, elements 8 q8 + 4 .. + 7 to piece 4 s + g0 + 1 (g0 is even, so that is the slot with bit 1 flipped); the
+    // thread's further pieces are 32 rows apart, which leaves the swizzle unchanged
+    int x_store;
+    {
+        const int row = tid / CPR, q8 = tid % CPR;
+        const int st = q8 >> 2, hb = (q8 >> 1) & 1, g0 = 2 * (q8 & 1);
+        x_store = (row * CPR + swizzled_chunk_n<CPR>(row, 4 * st + g0)) * 2 + hb;
+    }
+
+    u32x4 wraw_a[NB], wraw_b[NB], xreg[X_PER_THREAD];
+    u32x2 sraw_a[NB], sraw_b[NB];
+    auto fetch_x = [&](int kt) {
+        const int k0 = min(kt, n_kt - 1) * BK;
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++) { xreg[i] = *(const u32x4*)(x_begin + (size_t)k0 * 2 + (size_t)x_off[i]); }
+    };
+    auto fetch_w = [&](int c, u32x4* wraw, u32x2* sraw) {
+        const long long cc = min(c, n_chunks - 1);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+        {
+            wraw[nb] = *(const u32x4*)(a.W + w_base[nb] + cc * 1024 + (size_t)w_off);
+            const uint8_t* sp = tiled_scales + s_base[nb] + cc * (16 * NS) + (size_t)s_off;
+            if constexpr (NS == 8) { sraw[nb] = *(const u32x2*)sp; }
+            else { sraw[nb] = u32x2{ *(const uint32_t*)sp, 0u }; }
+        }
+    };
+    auto stage = [&](int buf) {
+        u32x2* dst = (u32x2*)xs[buf];
+#pragma unroll
+        for (int i = 0; i < X_PER_THREAD; i++)
+        {
+            dst[x_store + i * (32 * CPR * 2)] = u32x2{ xreg[i][0], xreg[i][1] };
+            dst[(x_store ^ 2) + i * (32 * CPR * 2)] = u32x2{ xreg[i][2], xreg[i][3] };
+        }
+    };
+    // Half `half` (four elements, one scale block when BLOCK is 16) of dword d of the chunk, block nb -> two registers
+    // of the lane's matrix-core operand: 2 conversions to FP32, 4 multiplies by the block scale, 2 packs to BF16
+    auto dequant_half = [&](const u32x4* wraw, const u32x2* sraw, int nb, int d, int half, u32x4* wf) {
+        const int si = BLOCK == 16 ? 2 * d + half : d;               // scale byte of the chunk
+        const uint32_t sw = sraw[nb][si >> 2];
+        const float sc = (si & 3) == 0 ? __builtin_amdgcn_cvt_f32_fp8(sw, 0) : (si & 3) == 1 ? __builtin_amdgcn_cvt_f32_fp8(sw, 1)
+                       : (si & 3) == 2 ? __builtin_amdgcn_cvt_f32_fp8(sw, 2) : __builtin_amdgcn_cvt_f32_fp8(sw, 3);
+        const uint32_t w = wraw[nb][d];
+        const f32x2 v0 = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0) : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2);
+        const f32x2 v1 = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1) : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+        const bf16x2 p0 = { (__bf16)(v0.x * sc), (__bf16)(v0.y * sc) };
+        const bf16x2 p1 = { (__bf16)(v1.x * sc), (__bf16)(v1.y * sc) };
+        wf[nb][2 * half] = __builtin_bit_cast(uint32_t, p0);
+        wf[nb][2 * half + 1] = __builtin_bit_cast(uint32_t, p1);
+    };
+
+    // One 64-element half (h) of a chunk = two matrix-core steps of MB token blocks each.  The conversion of a step's
+    // weights runs one step ahead of its products, a piece (half a dword: 9 VALU instructions) at a time between the
+    // matrix-core instructions of one token block, so that neither pipe waits for the other: wf_a holds the operands of
+    // the half's first step on entry and is refilled, during the second step, for the next half's first step; wf_b is
+    // filled during the first step for the second.  Order: barrier | (first half: request the next chunk's codes and
+    // scales) | first step | store the next activation tile to LDS, request the one after | second step; activation
+    // fragments are read AHEAD token blocks in front of their use.  Scheduling fences keep that order.
+    constexpr int AHEAD = 2;
+    u32x4 wf_a[NB], wf_b[NB];
+    auto k_tile = [&](int kt, int h, const u32x4* wcur, const u32x2* scur, u32x4* wnext, u32x2* snext) {
+        __syncthreads();                                     // tile kt is in xs[kt & 1]; the other buffer is free
+        if (h == 0) { fetch_w(kt / 2 + 1, wnext, snext); }
+        const u32x4* xt = xs[kt & 1];
+        constexpr int FRAGS = 2 * MB;
+        constexpr int PIECES = 2 * NB;                       // per step
+        auto read_frag = [&](int f) {
+            const int row = (f % MB) * 16 + i16;
+            return xt[row * CPR + swizzled_chunk_n<CPR>(row, 4 * (f / MB) + g)];
+        };
+        u32x4 ring[AHEAD + 1];
+#pragma unroll
+        for (int f = 0; f < AHEAD; f++) { ring[f] = read_frag(f); }
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++)
+        {
+            __builtin_amdgcn_sched_barrier(0);
+            if (f == FRAGS / 2)
+            {
+                stage((kt + 1) & 1);
+                fetch_x(kt + 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
+            const bf16x8 xf = __builtin_bit_cast(bf16x8, ring[f % (AHEAD + 1)]);
+            const int st = f / MB, mb = f % MB;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+            {
+                const bf16x8 w = __builtin_bit_cast(bf16x8, st == 0 ? wf_a[nb] : wf_b[nb]);
+                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, xf, acc[mb][nb], 0, 0, 0);
+            }
+            // this token block's share of the next step's conversions
+            const int p_begin = mb * PIECES / MB, p_end = (mb + 1) * PIECES / MB;
+#pragma unroll
+            for (int p = p_begin; p < p_end; p++)
+            {
+                if (st == 0) { dequant_half(wcur, scur, p / 2, 2 * h + 1, p % 2, wf_b); }
+                else if (h == 0) { dequant_half(wcur, scur, p / 2, 2, p % 2, wf_a); }
+                else { dequant_half(wnext, snext, p / 2, 0, p % 2, wf_a); }
+            }
+            // one fragment read, then each matrix-core instruction followed by its share of the VALU work
+            if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+            constexpr int VALU_PER_MFMA = (9 * ((PIECES + MB - 1) / MB) + NB - 1) / NB;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    fetch_x(0);
+    fetch_w(0, wraw_a, sraw_a);
+    stage(0);
+    fetch_x(1);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+    {
+        dequant_half(wraw_a, sraw_a, nb, 0, 0, wf_a);
+        dequant_half(wraw_a, sraw_a, nb, 0, 1, wf_a);
+    }
+    for (int c = 0; c < n_chunks; c += 2)
+    {
+        k_tile(2 * c, 0, wraw_a, sraw_a, wraw_b, sraw_b);
+        k_tile(2 * c + 1, 1, wraw_a, sraw_a, wraw_b, sraw_b);
+        if (c + 1 < n_chunks)
+        {
+            k_tile(2 * c + 2, 0, wraw_b, sraw_b, wraw_a, sraw_a);
+            k_tile(2 * c + 3, 1, wraw_b, sraw_b, wraw_a, sraw_a);
+        }
+    }
+
+    const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+    {
+        const int tok = tok_base + mb * 16 + i16;
+        if (tok >= a.tokens) { continue; }
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+        {
+            const int out = out_base + nb * 16 + 4 * g;
+            if (out >= a.n_out) { continue; }
+            const f32x4 r = acc[mb][nb];
+            if constexpr (SPLIT)
+            {
+                float* p = partial + ((long long)blockIdx.y * a.tokens + tok) * a.n_out + out;
+                if (wide_store && out + 3 < a.n_out) { *(f32x4*)p = r; }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { p[v] = r[v]; }
+                    }
+                }
+            }
+            else
+            {
+                uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                if (wide_store && out + 3 < a.n_out)
+                {
+                    uint16_t old[4] = { 0, 0, 0, 0 };
+                    if (a.beta != 0.0f) { *(uint2*)old = *(const uint2*)y; }
+                    uint16_t o[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) { o[v] = finish_output_act<DT_BF16>(r[v], a.alpha, a.beta, &old[v]); }
+                    *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) };
+                }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { y[v * a.y_stride_out] = finish_output_act<DT_BF16>(r[v], a.alpha, a.beta, y + v * a.y_stride_out); }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// a.W = the tiled codes; splits > 1: `partial` holds splits * tokens * n_out floats
+template <int BLOCK, int MB, int NB = 4>
+void launch_gemm4_mfma_direct(const LinearArgs& a, const uint8_t* tiled_scales, int splits = 1, float* partial = nullptr)
+{
+    const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
+    const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
+    const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, splits);
+    if (splits > 1)
+    {
+        gemm4_mfma_direct_kernel<BLOCK, MB, true, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, m_tiles, partial);
+        const long long groups = (long long)a.tokens * (a.n_out / 4);
+        const long long blocks = (groups + 255) / 256;
+        const long long cap = (long long)cu_count() * 16;
+        gemm_splitk_combine_kernel<DT_BF16><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
+    }
+    else { gemm4_mfma_direct_kernel<BLOCK, MB, false, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, m_tiles, nullptr); }
+}
+
 // splits > 1: `partial` holds splits * tokens * n_out floats
 template <int WT, int MB, bool TILED, int AT = DT_BF16, int NB = 4>
 void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial = nullptr)
@@ -539,6 +835,103 @@ void launch_gemm_mfma(const LinearArgs& a)
     else { gemm_mfma_kernel<WT, BLOCK, BM, BN, false, BK, XCD, AT><<<grid, 256, 0, stream()>>>(a, n_tiles, m_tiles); }
 }
 
+// Tile shape and k split of the register-fed kernels (tuned on MI355X with the FP8 kernel): a workgroup owns 64 NB features x
+// 16 MB tokens.  A CU wants two resident workgroups (one alone reaches ~85 % of the rate), the workgroups should spread
+// evenly over the CUs (384 tiles on 256 CUs leave half of them with twice the work: 36 % of peak where 512 even tiles
+// reach 42 %), and 48-feature waves with 64-token tiles cost ~5 % against the larger tiles.  Too few tiles in every
+// shape: the k range is split over workgroups (256-feature tiles, about one workgroup per CU, 1024 elements of k or more
+// each) and a second kernel adds the partial sums.
+struct DirectPlan
+{
+    int nb, mb, splits;
+    float* partial;
+    bool refused;            // a fixed scratch buffer is too small for the k split this shape takes (SplitScratch::refused says how much)
+};
+
+// Gives the plan `s` k ranges and the FP32 scratch they need; false when a fixed scratch buffer is too small for them.
+inline bool attach_split(DirectPlan& plan, const LinearArgs& a, long long s, SplitScratch* scratch)
+{
+    if (s <= 1) { return true; }
+    const size_t need = (size_t)s * a.tokens * a.n_out * sizeof(float);
+    if (scratch && scratch->strict)
+    {
+        if (!scratch->fixed || need > scratch->fixed_bytes)
+        {
+            scratch->refused = need;
+            plan.refused = true;
+            return false;
+        }
+        plan.partial = scratch->fixed;
+    }
+    else { plan.partial = (float*)workspace(need); }
+    if (plan.partial) { plan.splits = (int)s; }
+    return true;
+}
+
+// big_tile: whether the 128-token x 256-feature tile takes part in the scoring
+inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool big_tile = true)
+{
+    const int cus = cu_count();
+    struct Shape { int nb, mb; double quality; };
+    const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, 1.0 }, { 3, 8, 1.0 }, { 3, 4, 0.95 } };
+    DirectPlan plan = { 4, 4, 1, nullptr, false };
+    double best = -1.0;
+    for (const Shape& sh : shapes)
+    {
+        if (sh.mb == 8 && (a.tokens <= 64 || (sh.nb == 4 && !big_tile))) { continue; }
+        const long long tiles = (long long)((a.n_out + 64 * sh.nb - 1) / (64 * sh.nb)) * ((a.tokens + 16 * sh.mb - 1) / (16 * sh.mb));
+        const double balance = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
+        const double occupancy = tiles >= 2LL * cus ? 1.0 : (tiles > cus ? 0.95 : 0.85);
+        const double score = sh.quality * balance * occupancy;
+        if (score > best + 1e-9)
+        {
+            best = score;
+            plan.nb = sh.nb;
+            plan.mb = sh.mb;
+        }
+    }
+    const long long n_tiles = (a.n_out + 255) / 256;
+    const long long tiles8 = n_tiles * ((a.tokens + 127) / 128), tiles4 = n_tiles * ((a.tokens + 63) / 64);
+    if (best < 0.6 && tiles4 * 4 < 5LL * cus && a.n_out % 4 == 0)
+    {
+        const long long base = a.tokens > 64 ? tiles8 : tiles4;
+        long long s = (cus + base / 2) / base;
+        if (s > 8) { s = 8; }
+        if (s > a.K / 1024) { s = a.K / 1024; }
+        if (!attach_split(plan, a, s, scratch)) { return plan; }
+        if (plan.splits > 1)
+        {
+            plan.nb = 4;
+            plan.mb = a.tokens > 64 ? 8 : 4;
+        }
+    }
+    return plan;
+}
+
+// FP4: the 128 x 256 tile needs the register file of a whole SIMD per wave, so a CU runs one such workgroup at a time
+// and nothing hides its prologue and epilogue: it pays when every tile gets a CU of its own (1009 TFLOP/s on
+// 2048 x 4096, K 14336, against 940 for 64 x 256 tiles; 767 against 1009 for 128 x 192 tiles on 2048 x 14336, where a CU
+// runs three or four of them in sequence), with the k range split when the tiles are few.
+inline DirectPlan plan_direct_fp4(const LinearArgs& a, SplitScratch* scratch)
+{
+    const int cus = cu_count();
+    const long long tiles = (long long)((a.n_out + 255) / 256) * ((a.tokens + 127) / 128);
+    if (a.tokens > 64 && tiles <= cus)
+    {
+        long long s = a.n_out % 4 == 0 ? (cus + tiles / 2) / tiles : 1;
+        if (s > 8) { s = 8; }
+        if (s > a.K / 1024) { s = a.K / 1024; }
+        if (s < 1) { s = 1; }
+        if (tiles * s * 5 >= 3LL * cus)
+        {
+            DirectPlan plan = { 4, 8, 1, nullptr, false };
+            attach_split(plan, a, s, scratch);
+            return plan;
+        }
+    }
+    return plan_direct(a, scratch, false);
+}
+
 // Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
 // kernel that keeps the weights out of LDS -- on the tiled copy of the weight when one is registered
 // (1.10-1.15x the row-major rate: a wave's load is then eight full cache lines instead of sixteen half
@@ -553,6 +946,22 @@ void launch_gemm_mfma(const LinearArgs& a)
 template <int WT, int BLOCK, int AT = DT_BF16>
 bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch* scratch = nullptr)
 {
+    if constexpr (WT == DT_FP4 && AT == DT_BF16)
+    {
+        // FP4 with a tiled copy (codes, then the scales behind all code KiBs): the register-fed kernel
+        if (tiled && a.K % 128 == 0 && a.tokens >= 48 && (long long)a.tokens * a.ldx * 2 < (1LL << 32))
+        {
+            LinearArgs d = a;
+            d.W = tiled;
+            const uint8_t* scales = tiled + (long long)((a.n_out + 15) / 16) * (a.K / 128) * 1024;
+            const DirectPlan plan = plan_direct_fp4(a, scratch);
+            if (plan.refused) { return false; }
+            if (plan.nb == 3) { plan.mb == 8 ? launch_gemm4_mfma_direct<BLOCK, 8, 3>(d, scales) : launch_gemm4_mfma_direct<BLOCK, 4, 3>(d, scales); }
+            else if (plan.mb == 8) { launch_gemm4_mfma_direct<BLOCK, 8>(d, scales, plan.splits, plan.partial); }
+            else { launch_gemm4_mfma_direct<BLOCK, 4>(d, scales, plan.splits, plan.partial); }
+            return true;
+        }
+    }
     if constexpr (WT != DT_FP4)
     {
         const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
@@ -560,58 +969,10 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
         {
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }
-            const int cus = cu_count();
-            // Tile shape: 64 NB features x 16 MB tokens per workgroup.  What a shape costs, measured on MI355X: a CU wants
-            // two resident workgroups (one alone reaches ~85 % of the rate), the workgroups should spread evenly over the
-            // CUs (384 tiles on 256 CUs leave half of them with twice the work: 36 % of peak where 512 even tiles reach
-            // 42 %), and 48-feature waves with 64-token tiles cost ~5 % against the larger tiles.
-            struct Shape { int nb, mb; double quality; };
-            const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, 1.0 }, { 3, 8, 1.0 }, { 3, 4, 0.95 } };
-            int nb = 4, mb = 4;
-            double best = -1.0;
-            for (const Shape& sh : shapes)
-            {
-                if (sh.mb == 8 && a.tokens <= 64) { continue; }
-                const long long tiles = (long long)((a.n_out + 64 * sh.nb - 1) / (64 * sh.nb)) * ((a.tokens + 16 * sh.mb - 1) / (16 * sh.mb));
-                const double balance = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
-                const double occupancy = tiles >= 2LL * cus ? 1.0 : (tiles > cus ? 0.95 : 0.85);
-                const double score = sh.quality * balance * occupancy;
-                if (score > best + 1e-9)
-                {
-                    best = score;
-                    nb = sh.nb;
-                    mb = sh.mb;
-                }
-            }
-            int splits = 1;
-            float* partial = nullptr;
-            // too few tiles in every shape: split the k range over workgroups instead (256-feature tiles)
-            const long long n_tiles = (a.n_out + 255) / 256;
-            const long long tiles8 = n_tiles * ((a.tokens + 127) / 128), tiles4 = n_tiles * ((a.tokens + 63) / 64);
-            if (best < 0.6 && tiles4 * 4 < 5LL * cus && a.n_out % 4 == 0)
-            {
-                const long long base = a.tokens > 64 ? tiles8 : tiles4;
-                long long s = (cus + base / 2) / base;
-                if (s > 8) { s = 8; }
-                if (s > a.K / 64 / 16) { s = a.K / 64 / 16; }
-                const size_t need = (size_t)s * a.tokens * a.n_out * sizeof(float);
-                if (s > 1 && scratch && scratch->strict)
-                {
-                    if (!scratch->fixed || need > scratch->fixed_bytes)
-                    {
-                        scratch->refused = need;
-                        return false;
-                    }
-                    partial = scratch->fixed;
-                }
-                else if (s > 1) { partial = (float*)workspace(need); }
-                if (partial)
-                {
-                    splits = (int)s;
-                    nb = 4;
-                    mb = a.tokens > 64 ? 8 : 4;
-                }
-            }
+            const DirectPlan plan = plan_direct(a, scratch);
+            if (plan.refused) { return false; }
+            const int nb = plan.nb, mb = plan.mb, splits = plan.splits;
+            float* const partial = plan.partial;
             if (tiled)
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, true, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, true, AT, 3>(d); }

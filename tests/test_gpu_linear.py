@@ -583,3 +583,63 @@ def test_prepared_fp4_weights_on_the_matrix_cores(gpu, pkg, oracle, tokens, n_ou
         assert lib.weight_release(nd.data_ptr()) == 0
     assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
     assert lib.last_kernel() == "gemv_dot2"
+
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("tokens,n_out,K", [(48, 256, 128), (64, 300, 384), (130, 776, 1152), (512, 1024, 2048), (200, 520, 4096),
+                                            (256, 4096, 1024), (1000, 12288, 256)])
+def test_prepared_fp4_weights_in_the_prefill_gemm(gpu, pkg, oracle, tokens, n_out, K, block):
+    """FP4 prefill on the tiled copy (codes and block scales fed to the matrix cores from registers): every tile shape
+    (64 / 128 tokens x 192 / 256 features), the k split (few output tiles, long K) and its combine, ragged token and
+    feature counts, against the exact contraction; alpha / beta; without whole 128-element chunks, or after release, the
+    two-operand kernel takes the call."""
+    torch, dev, lib = gpu
+    seed = synth.seed_for(3, 900 + n_out % 89 + tokens + block)
+    nib, sc = synth.weights_fp4(seed, n_out, K, block)
+    X = synth.activations(seed, tokens, K)
+    nd, sd, xd = to_dev(torch, dev, nib), to_dev(torch, dev, sc), to_dev(torch, dev, X)
+    td = torch.zeros(lib.tiled_size(oracle.FP4, n_out, K), dtype=torch.uint8, device=dev)
+    want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block), X)
+    c0 = synth.activations(seed + 1, tokens, n_out)
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), block, n_out, K, td.data_ptr()) == 0
+    try:
+        y = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
+        assert lib.last_kernel() == "gemm_mfma_tiled"
+        out = from_dev(y, np.uint16)
+        assert not out[tokens * n_out:].any(), "wrote past the end"
+        got = out[: tokens * n_out].reshape(tokens, n_out)
+        check_rows(bf16_f64(oracle, got), want, f"fp4 prefill {n_out}x{K} M={tokens} b={block}")
+        check_bf16_close(got, want, "fp4 prefill", slack_ulp=1.0, abs_floor=2e-5)
+        yb = to_dev(torch, dev, c0.reshape(-1))
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), yb.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block,
+                          alpha=0.5, beta=-2.0) == 0
+        check_rows(bf16_f64(oracle, from_dev(yb, np.uint16).reshape(tokens, n_out)), 0.5 * want - 2.0 * bf16_f64(oracle, c0), "fp4 prefill alpha beta")
+        # the entry point that allocates nothing takes the same route (its k split uses the static scratch)
+        yn = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), yn.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block, noalloc=True) == 0
+        assert lib.last_kernel() == "gemm_mfma_tiled"
+        assert np.array_equal(from_dev(yn, np.uint16), out[: tokens * n_out])
+    finally:
+        assert lib.weight_release(nd.data_ptr()) == 0
+    assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
+    assert lib.last_kernel() == "gemm_mfma"
+    check_rows(bf16_f64(oracle, from_dev(y, np.uint16)[: tokens * n_out].reshape(tokens, n_out)), want, "fp4 prefill, row-major")
+
+
+def test_fp4_prefill_without_whole_chunks_stays_on_the_two_operand_kernel(gpu, pkg, oracle):
+    torch, dev, lib = gpu
+    tokens, n_out, K, block = 64, 256, 160, 16
+    nib, sc = synth.weights_fp4(77, n_out, K, block)
+    X = synth.activations(77, tokens, K)
+    nd, sd, xd = to_dev(torch, dev, nib), to_dev(torch, dev, sc), to_dev(torch, dev, X)
+    td = torch.zeros(lib.tiled_size(oracle.FP4, n_out, K), dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare_fp4(nd.data_ptr(), sd.data_ptr(), block, n_out, K, td.data_ptr()) == 0
+    try:
+        y = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+        assert lib.linear(nd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, blk_sc=sd.data_ptr(), block_size=block) == 0
+        assert lib.last_kernel() == "gemm_mfma"
+        want = oracle.linear_exact(oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=block), X)
+        check_rows(bf16_f64(oracle, from_dev(y, np.uint16).reshape(tokens, n_out)), want, "fp4 K=160")
+    finally:
+        assert lib.weight_release(nd.data_ptr()) == 0
