@@ -543,6 +543,8 @@ def main():
     ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
+    ap.add_argument("--weights", default="fp8", choices=["fp8", "fp4"], help="weight format of --workload gemv / prefill (fp4: E2M1 codes + E4M3 block scales)")
+    ap.add_argument("--block", type=int, default=16, choices=[16, 32], help="FP4 block length")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -666,21 +668,40 @@ def main():
     else:
         K, N = (int(v) for v in args.shape.split(","))
         M = args.tokens if args.workload == "gemv" else max(args.tokens, 512)
-        n_w = max(2, min(64, (1 << 30) // (K * N)))
-        weights = [ws.weight_e5m2(N, K) for _ in range(n_w)]
         X, Y = ws.activation(M, K), ws.output(M, N)
-        ops = [(W, X, Y, K, N) for W in weights]
-        torch.cuda.synchronize()
-        ms = time_chain(ws, ops, args.steps, args.warmup, False)
-        torch.cuda.synchronize()
-        ms_step = ms / args.steps
-        step_bytes = sum(gemv_bytes(K, N, M) for _ in ops)
+        if args.weights == "fp4":
+            t, block = torch, args.block
+            per = K * N // 2 + K * N // block
+            n_w = max(2, min(48, (768 << 20) // per))
+            nib = [t.randint(0, 256, (N, K // 2), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
+            sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
+            tiled = []
+            if ws.repack:
+                for w, s_ in zip(nib, sc):
+                    tiled.append(t.empty(ws.lib.tiled_size(FP4, N, K), dtype=t.uint8, device=ws.dev))
+                    assert ws.lib.weight_prepare_fp4(w.data_ptr(), s_.data_ptr(), block, N, K, tiled[-1].data_ptr()) == 0
+            torch.cuda.synchronize()
+            ms = ws.bench.fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr, N, M, K, block, args.steps * n_w, args.warmup * n_w)
+            if ms < 0:
+                raise RuntimeError(f"fp4 chain failed: {ms}")
+            ms_step = ms / args.steps
+            step_bytes = n_w * fp4_bytes(K, N, M, block)
+            ops = []
+        else:
+            n_w = max(2, min(64, (1 << 30) // (K * N)))
+            weights = [ws.weight_e5m2(N, K) for _ in range(n_w)]
+            ops = [(W, X, Y, K, N) for W in weights]
+            torch.cuda.synchronize()
+            ms = time_chain(ws, ops, args.steps, args.warmup, False)
+            torch.cuda.synchronize()
+            ms_step = ms / args.steps
+            step_bytes = sum(gemv_bytes(K, N, M) for _ in ops)
         value = step_bytes / ms_step * 1e-6
-        dom_us = ms_step * 1000.0 / len(ops)
+        dom_us = ms_step * 1000.0 / n_w
         extra["launch_mode"] = "stream"
-        workload = f"{args.workload} K={K} N={N} M={M} over {n_w} distinct FP8_E5M2 weights"
+        workload = f"{args.workload} K={K} N={N} M={M} over {n_w} distinct " + (f"FP4_E2M1 block-{args.block} weights" if args.weights == "fp4" else "FP8_E5M2 weights")
 
-    if args.workload != "decode_step":
+    if args.workload != "decode_step" and ops:
         assert ws.lib.linear(ops[0][0].data_ptr, E5M2, ops[0][1].data_ptr, ops[0][2].data_ptr, ops[0][4], M if args.workload != "decode_linears" else 1, ops[0][3]) == 0
     if args.workload == "decode_step":
         achieved = dom_bytes / dom_us * 1e-3
@@ -693,19 +714,20 @@ def main():
         achieved = flops / dom_us * 1e-6
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                    "kernel": "gemm_mfma_direct_kernel" if ws.lib.last_kernel() == "gemm_mfma_tiled" or (K % 64 == 0 and M >= 48) else "gemm_mfma_kernel",
+                    "kernel": ("gemm4_mfma_direct_kernel" if args.weights == "fp4" and ws.lib.last_kernel() == "gemm_mfma_tiled" else
+                               "gemm_mfma_direct_kernel" if args.weights == "fp8" and (ws.lib.last_kernel() == "gemm_mfma_tiled" or (K % 64 == 0 and M >= 48)) else "gemm_mfma_kernel"),
                     "weight_layout": "tiled copy" if ws.lib.last_kernel() == "gemm_mfma_tiled" else "row-major", "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3)}
     else:
-        achieved = gemv_bytes(K, N, M) / dom_us * 1e-3
+        achieved = (fp4_bytes(K, N, M, args.block) if args.weights == "fp4" else gemv_bytes(K, N, M)) / dom_us * 1e-3
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    "traffic": GEMV_GATE_UP_TRAFFIC_BYTES if (K, N, M) == (4096, 12288, 1) else None,
-                    "traffic_source": TRAFFIC_SOURCE + "gemv8_mfma_tiled_K4096_N12288_M1.md" if (K, N, M) == (4096, 12288, 1) else None,
+                    "traffic": GEMV_GATE_UP_TRAFFIC_BYTES if (K, N, M, args.weights) == (4096, 12288, 1, "fp8") else None,
+                    "traffic_source": TRAFFIC_SOURCE + "gemv8_mfma_tiled_K4096_N12288_M1.md" if (K, N, M, args.weights) == (4096, 12288, 1, "fp8") else None,
                     "kernel": ws.lib.last_kernel(), "shape": {"K": K, "N": N, "M": M}, "us_per_launch": round(dom_us, 3),
-                    "bytes_per_launch": gemv_bytes(K, N, M)}
+                    "bytes_per_launch": fp4_bytes(K, N, M, args.block) if args.weights == "fp4" else gemv_bytes(K, N, M)}
 
     line = {
-        "metric": metric if args.workload != "prefill" else "W8A16 prefill GEMM algorithmic GB/s",
+        "metric": metric if args.workload != "prefill" else ("W4A16" if args.weights == "fp4" else "W8A16") + " prefill GEMM algorithmic GB/s",
         "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},

@@ -285,8 +285,13 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n_tile = blockIdx.x % n_tiles;
-    const int m_tile = blockIdx.x / n_tiles;
+    // The hardware hands consecutive workgroups to the eight XCDs in turn, each with an L2 of its own.  With the feature
+    // tiles padded to a multiple of eight, feature tile n always lands on XCD n % 8, and the workgroups an XCD runs at
+    // one time are a block of (n_pad / 8) feature tiles x several token tiles: both operands are shared inside the L2.
+    const int n_pad = (n_tiles + 7) & ~7;
+    const int n_tile = blockIdx.x % n_pad;
+    const int m_tile = blockIdx.x / n_pad;
+    if (n_tile >= n_tiles) { return; }          // padding
     const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
@@ -543,7 +548,7 @@ __device__ __forceinline__ u32x4 dequant8_fp4_blocks(uint32_t w, float s_lo, flo
 
 template <int BLOCK, int MB, bool SPLIT, int NB = 4>
 __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a, const uint8_t* __restrict__ tiled_scales, const int n_tiles,
-                                                                                        const int m_tiles, float* __restrict__ partial)
+                                                                                        float* __restrict__ partial)
 {
     static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
     constexpr int NS = 128 / BLOCK;             // scale bytes per row and chunk
@@ -555,13 +560,13 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // The hardware hands consecutive workgroups to the eight XCDs in turn, each with an L2 of its own.  XCD x takes the
-    // feature tiles x, x + 8, ... and walks all token tiles of one before the next: the workgroups that share a weight
-    // tile then run on one XCD at about the same time and the tile reaches that L2 once.
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int n_tile = xcd + 8 * (local / m_tiles);
-    const int m_tile = local % m_tiles;
-    if (n_tile >= n_tiles) { return; }          // the grid is padded to whole rounds of eight feature tiles
+    // The hardware hands consecutive workgroups to the eight XCDs in turn, each with an L2 of its own.  With the feature
+    // tiles padded to a multiple of eight, feature tile n always lands on XCD n % 8, and the workgroups an XCD runs at
+    // one time are a block of (n_pad / 8) feature tiles x several token tiles: both operands are shared inside the L2.
+    const int n_pad = (n_tiles + 7) & ~7;
+    const int n_tile = blockIdx.x % n_pad;
+    const int m_tile = blockIdx.x / n_pad;
+    if (n_tile >= n_tiles) { return; }          // padding
     const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
@@ -789,16 +794,16 @@ void launch_gemm4_mfma_direct(const LinearArgs& a, const uint8_t* tiled_scales, 
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
-    const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, splits);
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, splits);
     if (splits > 1)
     {
-        gemm4_mfma_direct_kernel<BLOCK, MB, true, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, m_tiles, partial);
+        gemm4_mfma_direct_kernel<BLOCK, MB, true, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, partial);
         const long long groups = (long long)a.tokens * (a.n_out / 4);
         const long long blocks = (groups + 255) / 256;
         const long long cap = (long long)cu_count() * 16;
         gemm_splitk_combine_kernel<DT_BF16><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
     }
-    else { gemm4_mfma_direct_kernel<BLOCK, MB, false, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, m_tiles, nullptr); }
+    else { gemm4_mfma_direct_kernel<BLOCK, MB, false, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, nullptr); }
 }
 
 // splits > 1: `partial` holds splits * tokens * n_out floats
@@ -807,7 +812,7 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
-    const dim3 grid(n_tiles * m_tiles, splits);
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, splits);
     const bool scaled = a.w_scale != 1.0f;
     if (splits > 1)
     {
@@ -868,12 +873,14 @@ inline bool attach_split(DirectPlan& plan, const LinearArgs& a, long long s, Spl
     return true;
 }
 
-// big_tile: whether the 128-token x 256-feature tile takes part in the scoring
-inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool big_tile = true)
+// fp4: the FP4 kernel's costs -- the 128-token x 256-feature tile stays out of the scoring (see plan_direct_fp4), and
+// 64-token tiles pay for converting every weight for half as many products (913 against 1037 TFLOP/s at equal balance).
+inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool fp4 = false)
 {
     const int cus = cu_count();
+    const bool big_tile = !fp4;
     struct Shape { int nb, mb; double quality; };
-    const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, 1.0 }, { 3, 8, 1.0 }, { 3, 4, 0.95 } };
+    const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, fp4 ? 0.88 : 1.0 }, { 3, 8, 1.0 }, { 3, 4, fp4 ? 0.84 : 0.95 } };
     DirectPlan plan = { 4, 4, 1, nullptr, false };
     double best = -1.0;
     for (const Shape& sh : shapes)
@@ -929,7 +936,7 @@ inline DirectPlan plan_direct_fp4(const LinearArgs& a, SplitScratch* scratch)
             return plan;
         }
     }
-    return plan_direct(a, scratch, false);
+    return plan_direct(a, scratch, true);
 }
 
 // Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
