@@ -33,10 +33,10 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM bytes per launch of the gate/up-shaped GEMV (K=4096, N=12288, M=1) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99979 and 1.0)
-GEMV_GATE_UP_TRAFFIC_BYTES = 50451344
+# WRITE_SIZE, each scaled by the same counter on a 256 MiB device copy (factors 1.99977 and 1.0)
+GEMV_GATE_UP_TRAFFIC_BYTES = 50450876
 # the same two counters for one launch of the fused RMSNorm + gate/up SwiGLU GEMV (two 4096 x 12288 weights)
-GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = 101012454
+GEMV_FUSED_GATE_UP_TRAFFIC_BYTES = 101017770
 
 # `roofline.traffic` is a constant from a counter run, not measured by this script (rocprofv3 --pmc needs a run of its own)
 TRAFFIC_SOURCE = "constant copied from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/"
