@@ -491,8 +491,9 @@ def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
 
 def cpu_baseline(pkg, threads, unit):
     """The reference CPU route (scalar dequantisation of the whole weight to float32 + cblas_sgemm, cccc/Matrix.cpp:1258-1267)
-    on the linear layers of the decode workload at M=1, on a bounded sample: 12 of the 36 layers (the same seven
-    weights walked 12 times: 2.3 GB of codes per walk, far beyond the host caches), timed three times."""
+    on the linear layers of the decode workload at M=1, on a bounded sample: 24 of the 36 layers (the same seven
+    weights walked 24 times: 4.6 GB of codes per walk, far beyond the host caches), timed three times -- about
+    ten seconds of CPU work."""
     import numpy as np
     from oracle import oracle, synth
     c = QWEN3_8B
@@ -505,7 +506,7 @@ def cpu_baseline(pkg, threads, unit):
         W = rng.integers(0, 0x7C, size=(N, K), dtype=np.uint8)
         X = synth.activations(7, 1, K)
         data.append((W, X, K, N))
-    layers_sampled = 12
+    layers_sampled = 24
     runs = []
     t_end = time.time() + 30.0
     for rep in range(4):
