@@ -241,7 +241,8 @@ int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v, const 
                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
 {
     if (head_dim != 128 || n_q_heads <= 0 || n_kv_heads <= 0 || t_kv <= 0 || !d_pos) { return -1; }
-    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_tab || !sin_tab || !q_out || !k_cache || !v_cache) { return -1; }
+    if (!q || !k || !v || !cos_tab || !sin_tab || !q_out || !k_cache || !v_cache) { return -1; }
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) { return -1; }          // both (Qwen3-style heads) or neither (Llama-style)
     qk_norm_rope_kv_kernel<<<n_q_heads + 2 * n_kv_heads, 64, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v,
                                                                            (const uint16_t*)q_norm_w, (const uint16_t*)k_norm_w,
                                                                            (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,
@@ -320,7 +321,8 @@ int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
                                     int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
 {
     if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || !d_pos) { return -1; }
-    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_tab || !sin_tab || !k_cache || !v_cache || !y || !workspace) { return -1; }
+    if (!q || !k || !v || !cos_tab || !sin_tab || !k_cache || !v_cache || !y || !workspace) { return -1; }
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) { return -1; }          // both (Qwen3-style heads) or neither (Llama-style)
     if (!aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace)) { return -1; }
     const AttentionWorkspace w = attention_workspace(n_q_heads, t_kv);
     if (workspace_bytes < w.total || w.n_blocks > ATT_MAX_BLOCKS) { return -1; }

@@ -872,9 +872,13 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_kernel(const uint16
     const uint16_t* src = (is_q ? q : k) + h * 128;
     const uint16_t* nw = is_q ? q_norm_w : k_norm_w;
     const float xl = bf16_bits_to_f32(src[lane]), xr = bf16_bits_to_f32(src[lane + 64]);
-    const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
-    const float nl = bf16_round(xl * invstd * bf16_bits_to_f32(nw[lane]));
-    const float nr = bf16_round(xr * invstd * bf16_bits_to_f32(nw[lane + 64]));
+    float nl = xl, nr = xr;                  // no norm weights (Llama-style heads): the projection output is rotated as it is
+    if (nw)
+    {
+        const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
+        nl = bf16_round(xl * invstd * bf16_bits_to_f32(nw[lane]));
+        nr = bf16_round(xr * invstd * bf16_bits_to_f32(nw[lane + 64]));
+    }
     const float c = bf16_bits_to_f32(cos_tab[(size_t)pos * 64 + lane]), s = bf16_bits_to_f32(sin_tab[(size_t)pos * 64 + lane]);
     uint16_t* dst = is_q ? q_out + h * 128 : k_cache + ((size_t)h * t_kv + pos) * 128;
     dst[lane] = (uint16_t)f32_to_bf16_bits(nl * c - nr * s);
@@ -1101,16 +1105,22 @@ struct HeadLoads
 __device__ __forceinline__ HeadLoads load_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
                                                const uint16_t* __restrict__ sin_row, int lane)
 {
-    return HeadLoads{ src[lane], src[lane + 64], cos_row[lane], sin_row[lane], nw[lane], nw[lane + 64] };
+    return HeadLoads{ src[lane], src[lane + 64], cos_row[lane], sin_row[lane], nw ? nw[lane] : (uint16_t)0, nw ? nw[lane + 64] : (uint16_t)0 };
 }
 
-__device__ __forceinline__ void norm_rope_finish(const HeadLoads& h, float eps, float& out_l, float& out_r)
+// normed == false (no per-head norm weights, Llama-style): the head is rotated as the projection left it
+__device__ __forceinline__ void norm_rope_finish(const HeadLoads& h, bool normed, float eps, float& out_l, float& out_r)
 {
     const float xl = bf16_bits_to_f32(h.xl), xr = bf16_bits_to_f32(h.xr);
     const float c = bf16_bits_to_f32(h.c), sn = bf16_bits_to_f32(h.sn);
-    const float wl = bf16_bits_to_f32(h.wl), wr = bf16_bits_to_f32(h.wr);
-    const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
-    const float nl = bf16_round(xl * invstd * wl), nr = bf16_round(xr * invstd * wr);
+    float nl = xl, nr = xr;
+    if (normed)
+    {
+        const float wl = bf16_bits_to_f32(h.wl), wr = bf16_bits_to_f32(h.wr);
+        const float invstd = rsqrtf(wave_sum(xl * xl + xr * xr) / 128.0f + eps);
+        nl = bf16_round(xl * invstd * wl);
+        nr = bf16_round(xr * invstd * wr);
+    }
     out_l = bf16_round(nl * c - nr * sn);
     out_r = bf16_round(nr * c + nl * sn);
 }
@@ -1118,7 +1128,7 @@ __device__ __forceinline__ void norm_rope_finish(const HeadLoads& h, float eps, 
 __device__ __forceinline__ void norm_rope_head(const uint16_t* __restrict__ src, const uint16_t* __restrict__ nw, const uint16_t* __restrict__ cos_row,
                                                const uint16_t* __restrict__ sin_row, float eps, int lane, float& out_l, float& out_r)
 {
-    norm_rope_finish(load_head(src, nw, cos_row, sin_row, lane), eps, out_l, out_r);
+    norm_rope_finish(load_head(src, nw, cos_row, sin_row, lane), nw != nullptr, eps, out_l, out_r);
 }
 
 template <int G>
@@ -1170,7 +1180,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
     if (wave < G)
     {
         float l, r;
-        norm_rope_finish(hq, eps, l, r);
+        norm_rope_finish(hq, q_norm_w != nullptr, eps, l, r);
         q_lds[wave][lane] = (uint16_t)f32_to_bf16_bits(l);
         q_lds[wave][lane + 64] = (uint16_t)f32_to_bf16_bits(r);
     }

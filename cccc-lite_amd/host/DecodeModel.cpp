@@ -180,6 +180,8 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         m = tmp;
         return 0;
     };
+    // a file without per-head norm weights is a model without them (scripts/convert_weights.py:231-239 decides the same way)
+    qk_norm_ = cfg_.layers == 0 || file.resolve("W_qnorm_0").valid() || file.resolve("W_knorm_0").valid();
     int rc = load_plain(*emb_, "W_emb");
     if (rc == 0) { rc = load_plain(*rms_final_, "W_rms_final"); }
     if (rc == 0) { rc = load_linear(*lm_head_, file.resolve("W_lm_head").valid() ? "W_lm_head" : "W_emb", true); }
@@ -190,7 +192,11 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         const std::pair<Matrix*, const char*> plain[] = { { L.rms_attn.get(), "W_rms_attn_" }, { L.q_norm.get(), "W_qnorm_" }, { L.k_norm.get(), "W_knorm_" }, { L.rms_ffn.get(), "W_rms_ffn_" } };
         const std::pair<Matrix*, const char*> linear[] = { { L.wq.get(), "W_q_" }, { L.wk.get(), "W_k_" }, { L.wv.get(), "W_v_" }, { L.wo.get(), "W_o_" },
                                                           { L.w_gate.get(), "W_gate_" }, { L.w_up.get(), "W_up_" }, { L.w_down.get(), "W_down_" } };
-        for (auto& [m, prefix] : plain) { if (rc == 0) { rc = load_plain(*m, prefix + n); } }
+        for (auto& [m, prefix] : plain)
+        {
+            const bool head_norm = m == L.q_norm.get() || m == L.k_norm.get();
+            if (rc == 0 && (qk_norm_ || !head_norm)) { rc = load_plain(*m, prefix + n); }
+        }
         for (auto& [m, prefix] : linear) { if (rc == 0) { rc = load_linear(*m, prefix + n); } }
         // gate and up are decoded by one launch with one format
         if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType()) { rc = fail("W_up_" + n, -3); }
@@ -222,7 +228,11 @@ int DecodeModel::saveNamedWeights(const std::string& filename)
             { L.rms_attn.get(), "W_rms_attn_" }, { L.wq.get(), "W_q_" }, { L.wk.get(), "W_k_" }, { L.wv.get(), "W_v_" },
             { L.q_norm.get(), "W_qnorm_" }, { L.k_norm.get(), "W_knorm_" }, { L.wo.get(), "W_o_" }, { L.rms_ffn.get(), "W_rms_ffn_" },
             { L.w_gate.get(), "W_gate_" }, { L.w_up.get(), "W_up_" }, { L.w_down.get(), "W_down_" } };
-        for (auto& [m, prefix] : tensors) { addNamedWeight(w, prefix + n, *m); }
+        for (auto& [m, prefix] : tensors)
+        {
+            if (!qk_norm_ && (m == L.q_norm.get() || m == L.k_norm.get())) { continue; }
+            addNamedWeight(w, prefix + n, *m);
+        }
     }
     return w.save(filename) > 0 ? 0 : -1;
 }
@@ -307,16 +317,18 @@ int DecodeModel::step()
                 rc = hip_quant_linear_fused(&kv);
             }
         }
-        // 2-3. per-head q/k norm, RoPE, KV append and attention over the cache
+        // 2-3. per-head q/k norm (models that have one), RoPE, KV append and attention over the cache
+        const void* q_norm_w = qk_norm_ ? L.q_norm->data() : nullptr;
+        const void* k_norm_w = qk_norm_ ? L.k_norm->data() : nullptr;
         if (rc == 0 && !exact_attention_)
         {
-            rc = hip_attention_decode_fused_bf16(q_->data(), k_->data(), v_->data(), L.q_norm->data(), L.k_norm->data(), cos_->data(), sin_->data(),
+            rc = hip_attention_decode_fused_bf16(q_->data(), k_->data(), v_->data(), q_norm_w, k_norm_w, cos_->data(), sin_->data(),
                                                  k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(), attn_ws_bytes_,
                                                  c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
         }
         else if (rc == 0)
         {
-            rc = hip_qk_norm_rope_kv_bf16(q_->data(), k_->data(), v_->data(), L.q_norm->data(), L.k_norm->data(), cos_->data(), sin_->data(),
+            rc = hip_qk_norm_rope_kv_bf16(q_->data(), k_->data(), v_->data(), q_norm_w, k_norm_w, cos_->data(), sin_->data(),
                                           q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
             if (rc == 0)
             {

@@ -49,7 +49,8 @@ public:
 
     // Loads every tensor from a converted model file by the converter's names (scripts/convert_weights.py:142-166):
     // W_emb, W_rms_final, W_lm_head (W_emb when absent: tied), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
-    // W_qnorm_<i>, W_knorm_<i>, W_rms_ffn_<i>, W_gate_<i>, W_up_<i>, W_down_<i>.  FP8 and FP4 linears are taken as stored;
+    // W_qnorm_<i>, W_knorm_<i> (a file without them loads as a model without per-head norms), W_rms_ffn_<i>, W_gate_<i>,
+    // W_up_<i>, W_down_<i>.  FP8 and FP4 linears are taken as stored;
     // linears stored as BF16 / HALF / FLOAT are quantized on load to `quantize_to` with a per-tensor absmax scale
     // (the reference's weight_data_type route, cccc/Matrix.cpp:301-355).  0 ok; otherwise `failed` names the tensor:
     // -1 missing, -2 wrong size, -3 something the fused decode kernels do not take (FP4 without block scales, gate and
@@ -66,6 +67,11 @@ public:
     // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
     // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).
     void setExactAttention(bool exact) { exact_attention_ = exact; }
+    // Per-head RMSNorm of q and k in front of the rotation: on for Qwen3-style models (default), off for models without
+    // W_qnorm / W_knorm such as Llama-3.1 (has_qknorm in scripts/convert_weights.py:488-530).  loadNamedWeights sets it
+    // from what the file holds.
+    void setQkNorm(bool on) { qk_norm_ = on; }
+    bool qkNorm() const { return qk_norm_; }
     int reset(int token, int pos);          // sets the device-side token / position and fetches the token's embedding (KV caches are kept)
     int step();                             // enqueues one decode step; the next token replaces the current one
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
@@ -91,6 +97,7 @@ private:
     std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, attn_ws_, argmax_ws_;
     unsigned long long attn_ws_bytes_ = 0;
     bool exact_attention_ = false;
+    bool qk_norm_ = true;
     int* d_state_ = nullptr;    // [0] token, [1] position
 };
 

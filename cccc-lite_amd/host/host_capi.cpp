@@ -218,6 +218,8 @@ int cccc_matrix_save_named(void* m, const char* name, const char* path)
 }
 
 void cccc_decode_set_exact_attention(void* m, int exact) { ((DecodeModel*)m)->setExactAttention(exact != 0); }
+void cccc_decode_set_qk_norm(void* m, int on) { ((DecodeModel*)m)->setQkNorm(on != 0); }
+int cccc_decode_qk_norm(void* m) { return ((DecodeModel*)m)->qkNorm() ? 1 : 0; }
 
 int cccc_decode_reset(void* m, int token, int pos) { return ((DecodeModel*)m)->reset(token, pos); }
 

@@ -68,6 +68,8 @@ class HostLibrary:
         L.cccc_decode_save_named.restype = i32; L.cccc_decode_save_named.argtypes = [vp, ctypes.c_char_p]
         L.cccc_matrix_save_named.restype = i32; L.cccc_matrix_save_named.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
+        L.cccc_decode_set_qk_norm.restype = None; L.cccc_decode_set_qk_norm.argtypes = [vp, i32]
+        L.cccc_decode_qk_norm.restype = i32; L.cccc_decode_qk_norm.argtypes = [vp]
         L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         self.c = L
@@ -267,9 +269,11 @@ class DecodeModel:
                 self.set_tensor(li, name, value, fp8_dtype if name in QUANTIZED else 3)
         for name in GLOBAL_TENSORS:
             put(0, name, model[name])
+        self.set_qk_norm(all("q_norm" in L for L in model["layers"]))
         for li, L in enumerate(model["layers"]):
             for name in LAYER_TENSORS:
-                put(li, name, L[name])
+                if name in L:
+                    put(li, name, L[name])
 
     def load_named(self, wf: WeightFile, quantize_to: int = 5) -> None:
         """Every tensor from a converted model file by the converter's names; plain linears are quantized on load."""
@@ -287,6 +291,14 @@ class DecodeModel:
         """True: separate norm / RoPE / append launch and BF16 probabilities (the reference's rounding
         points); False (default): the two-launch attention with FP32 probabilities."""
         self.lib.c.cccc_decode_set_exact_attention(self.handle, 1 if exact else 0)
+
+    def set_qk_norm(self, on: bool) -> None:
+        """Per-head RMSNorm of q and k in front of the rotation (Qwen3: on, the default; Llama-3.1: off)."""
+        self.lib.c.cccc_decode_set_qk_norm(self.handle, 1 if on else 0)
+
+    @property
+    def qk_norm(self) -> bool:
+        return self.lib.c.cccc_decode_qk_norm(self.handle) != 0
 
     def reset(self, token: int, pos: int) -> None:
         assert self.lib.c.cccc_decode_reset(self.handle, token, pos) == 0

@@ -195,7 +195,9 @@ typedef struct hip_fused_linear
 C_EXPORT int hip_quant_linear_fused(const hip_fused_linear* desc);
 
 /* Per-head RMSNorm of q and k, RoPE at row *d_pos of the tables, append of k and v to the caches
- * (layout [kv_head][t_kv][128], the reference's (128, T_kv, 1, Hkv) cache).  head_dim is 128. */
+ * (layout [kv_head][t_kv][128], the reference's (128, T_kv, 1, Hkv) cache).  head_dim is 128.
+ * q_norm_w and k_norm_w both NULL: no per-head norm, the projections are rotated as they are (the
+ * graph scripts/convert_weights.py:488-530 emits with has_qknorm = False, e.g. Llama-3.1). */
 C_EXPORT int hip_qk_norm_rope_kv_bf16(const void* q, const void* k, const void* v,
                                       const void* q_norm_w, const void* k_norm_w,
                                       const void* cos_tab, const void* sin_tab,
@@ -218,7 +220,8 @@ C_EXPORT int hip_attention_decode_bf16(const void* q, const void* k_cache, const
  * raw projections ([n_q_heads][128], [n_kv_heads][128]); row *d_pos of both caches is written.  Same
  * workspace as above.  Scores are rounded to BF16 as in the reference; the softmax probabilities stay
  * FP32 (the reference rounds them to BF16 before the product with V), so outputs can differ from
- * hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 by about one BF16 ulp.  t_kv <= 65536. */
+ * hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 by about one BF16 ulp.  t_kv <= 65536.
+ * q_norm_w and k_norm_w both NULL: no per-head norm, as above. */
 C_EXPORT int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
                                              const void* q_norm_w, const void* k_norm_w,
                                              const void* cos_tab, const void* sin_tab,

@@ -138,9 +138,10 @@ def dequant_linear(W) -> np.ndarray:
     return o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape)
 
 
-def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2"):
+def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2", qk_norm: bool = True):
     """Random-init model: linears from N(0, 0.02) as FP8_E5M2 codes (round to nearest) or, fmt = "fp4_e2m1", as the
-    converter's FP4 block-scale packing (blocks of 16); BF16 norms near 1, BF16 embedding N(0, 1)."""
+    converter's FP4 block-scale packing (blocks of 16); BF16 norms near 1, BF16 embedding N(0, 1).
+    qk_norm = False: no per-head norm weights (has_qknorm = False in scripts/convert_weights.py:488-530, Llama-style)."""
     rng = np.random.default_rng(seed)
 
     def q8(n_out, K):
@@ -162,6 +163,9 @@ def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2"):
             "w_up": q8(cfg.inter, cfg.hidden), "w_down": q8(cfg.hidden, cfg.inter)})
     model["rms_final"] = norm_w(cfg.hidden)
     model["lm_head"] = q8(cfg.vocab, cfg.hidden)
+    if not qk_norm:
+        for L in model["layers"]:
+            del L["q_norm"], L["k_norm"]
     return model
 
 
@@ -193,8 +197,10 @@ class DecodeOracle:
             q = linear(self.deq(li, "wq"), xn).reshape(c.n_q, c.head_dim)
             k = linear(self.deq(li, "wk"), xn).reshape(c.n_kv, c.head_dim)
             v = linear(self.deq(li, "wv"), xn).reshape(c.n_kv, c.head_dim)
-            q = rope(rms_norm(q, f(L["q_norm"]), c.eps), self.cos[pos], self.sin[pos])
-            k = rope(rms_norm(k, f(L["k_norm"]), c.eps), self.cos[pos], self.sin[pos])
+            if "q_norm" in L:            # Q_hHT -> rmsNorm -> permute -> rope, or straight to the rotation (scripts/convert_weights.py:494-503)
+                q, k = rms_norm(q, f(L["q_norm"]), c.eps), rms_norm(k, f(L["k_norm"]), c.eps)
+            q = rope(q, self.cos[pos], self.sin[pos])
+            k = rope(k, self.cos[pos], self.sin[pos])
             self.k[li, :, pos], self.v[li, :, pos] = k, v
             att = attention(q, self.k[li], self.v[li], pos, c.n_q, c.n_kv).reshape(-1)
             r1 = r(x + linear(self.deq(li, "wo"), att))

@@ -472,6 +472,95 @@ def test_decode_steps_with_fp4_linears_follow_the_oracle(gpu, pkg, oracle, dec):
     assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
 
 
+@pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 300)])
+def test_attention_without_per_head_norms(gpu, oracle, dec, n_q, n_kv, t_kv):
+    """Llama-style heads (has_qknorm = False, scripts/convert_weights.py:488-530): NULL norm weights make both attention
+    routes rotate the raw projections.  The appended key row is then exactly rope(k) -- no rsqrt in its way -- and both
+    routes follow the oracle; one NULL norm weight alone is refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(31)
+    cfg = dec.DecodeConfig(n_q=n_q, n_kv=n_kv, t_kv=t_kv, theta=5e5)
+    cos, sin = dec.rope_tables(cfg)
+    kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    ws_bytes = lib.c.hip_attention_decode_workspace_bytes(n_q, n_kv, t_kv)
+    ws = torch.full((ws_bytes,), 0xA5, dtype=torch.uint8, device=dev)
+    cd, sd = to_dev(torch, dev, cos), to_dev(torch, dev, sin)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    null = ctypes.c_void_p(0)
+    for pos in (0, 63, 64, 130, t_kv - 1):
+        q = oracle.f32_to_bf16((2 * rng.standard_normal((n_q, 128))).astype(np.float32))
+        k = oracle.f32_to_bf16((2 * rng.standard_normal((n_kv, 128))).astype(np.float32))
+        v = oracle.f32_to_bf16(rng.standard_normal((n_kv, 128)).astype(np.float32))
+        qd, knd, vnd = (to_dev(torch, dev, a) for a in (q, k, v))
+        pd = torch.tensor([pos], dtype=torch.int32, device=dev)
+        qr = dec.rope(dec.f(q), dec.f(cos[pos]), dec.f(sin[pos]))
+        k_ref, v_ref = dec.f(kc).copy(), dec.f(vc).copy()
+        k_ref[:, pos] = dec.rope(dec.f(k), dec.f(cos[pos]), dec.f(sin[pos]))
+        v_ref[:, pos] = dec.f(v)
+        want = dec.attention(qr, k_ref, v_ref, pos, n_q, n_kv)
+        # two-launch route
+        kd, vd = to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+        y = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        assert lib.c.hip_attention_decode_fused_bf16(ptr(qd), ptr(knd), ptr(vnd), null, null, ptr(cd), ptr(sd), ptr(kd), ptr(vd), ptr(y), ptr(ws), ws_bytes,
+                                                     n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == 0
+        assert np.array_equal(dec.f(from_dev(kd, np.uint16).reshape(n_kv, t_kv, 128)), k_ref), pos
+        assert np.array_equal(dec.f(from_dev(vd, np.uint16).reshape(n_kv, t_kv, 128)), v_ref), pos
+        got = from_dev(y, np.uint16).reshape(n_q, 128)
+        assert ulp_close(got, want, ulps=3.0, floor=4e-3 * np.abs(want).max()).all(), pos
+        # the route with the reference's rounding points
+        kd2, vd2 = to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+        q_rot = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        y2 = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        assert lib.c.hip_qk_norm_rope_kv_bf16(ptr(qd), ptr(knd), ptr(vnd), null, null, ptr(cd), ptr(sd), ptr(q_rot), ptr(kd2), ptr(vd2),
+                                              n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == 0
+        assert np.array_equal(dec.f(from_dev(q_rot, np.uint16).reshape(n_q, 128)), qr), pos
+        assert np.array_equal(dec.f(from_dev(kd2, np.uint16).reshape(n_kv, t_kv, 128)), k_ref), pos
+        assert lib.c.hip_attention_decode_bf16(ptr(q_rot), ptr(kd2), ptr(vd2), ptr(y2), ptr(ws), ws_bytes, n_q, n_kv, 128, t_kv, ptr(pd)) == 0
+        assert ulp_close(from_dev(y2, np.uint16).reshape(n_q, 128), want, ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), pos
+    # one norm weight without the other describes no model
+    w1 = to_dev(torch, dev, oracle.f32_to_bf16(np.ones(128, dtype=np.float32)))
+    assert lib.c.hip_attention_decode_fused_bf16(ptr(qd), ptr(knd), ptr(vnd), ptr(w1), null, ptr(cd), ptr(sd), ptr(kd), ptr(vd), ptr(y), ptr(ws), ws_bytes,
+                                                 n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == -1
+    assert lib.c.hip_qk_norm_rope_kv_bf16(ptr(qd), ptr(knd), ptr(vnd), null, ptr(w1), ptr(cd), ptr(sd), ptr(q_rot), ptr(kd2), ptr(vd2),
+                                          n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == -1
+
+
+@pytest.mark.parametrize("fmt,exact", [("fp4_e2m1", True), ("fp4_e2m1", False), ("fp8_e5m2", False)])
+def test_decode_steps_of_a_model_without_qk_norm(gpu, pkg, oracle, dec, fmt, exact):
+    """A Llama-3.1-shaped graph (no W_qnorm / W_knorm, RoPE theta 5e5; FP4 block-scale linears are the reference's Llama
+    route, cccc/Net.cpp:1460-1481) through the fused decode step against the oracle, then graph replay == eager."""
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=32, theta=5e5)
+    weights = dec.make_model(cfg, 29, fmt=fmt, qk_norm=False)
+    assert "q_norm" not in weights["layers"][0]
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
+    model.load(weights)
+    assert not model.qk_norm
+    model.set_exact_attention(exact)
+    orc = dec.DecodeOracle(cfg, weights)
+    token = 9
+    for pos in range(8):
+        model.reset(token, pos)
+        got_token = model.step()
+        want_logits, want_token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        # layer 0 sees the oracle's inputs up to the GEMV's summation order: its rotated key row within BF16 rounding
+        assert ulp_close(model.kv(0, False)[:, pos], orc.k[0, :, pos], ulps=2.0, floor=2e-3).all()
+        top2 = np.sort(want_logits)[-2:]
+        if top2[1] - top2[0] > 2 * np.abs(got - want_logits).max():
+            assert got_token == want_token, pos
+        token = want_token
+    # graph replay == eager on this route too
+    model.reset(3, 0)
+    eager = [model.step() for _ in range(6)]
+    logits_eager = model.logits().copy()
+    model.reset(3, 0)
+    assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
+
+
 @pytest.mark.parametrize("n_out,K,fmt", [(300, 1024, "e5m2"), (5000, 2048, "e5m2"), (70000, 1024, "e5m2 tiled"), (151936, 256, "e5m2 tiled"),
                                          (4100, 2048, "fp4"), (66000, 512, "fp4")])
 def test_greedy_pick_from_the_linear_epilogue(gpu, pkg, oracle, n_out, K, fmt):

@@ -408,3 +408,49 @@ def test_projections_sharing_an_input_load_into_one_storage(tmp_path, gpu, pkg, 
     assert f.load_named_group(host.matrix(K, total + 16, 1, 1, BF16), names) == -1
     with pytest.raises(ValueError):
         group.rows_view(total - 8, 16)
+
+
+def test_a_file_without_qk_norm_weights_loads_as_a_model_without_them(tmp_path, gpu, pkg, host, oracle, dec):
+    """The converter writes no W_qnorm / W_knorm for Llama (scripts/convert_weights.py:195-216): such a file loads, runs the
+    steps of the same tensors set directly with the per-head norm switched off, and is saved back without those entries."""
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=400, t_kv=16, theta=5e5)
+    weights = dec.make_model(cfg, 37, fmt="fp4_e2m1", qk_norm=False)
+    names = {"rms_attn": "W_rms_attn", "wq": "W_q", "wk": "W_k", "wv": "W_v", "wo": "W_o",
+             "rms_ffn": "W_rms_ffn", "w_gate": "W_gate", "w_up": "W_up", "w_down": "W_down"}
+    w = weight_file.BinWriter()
+    w.add("data_type", b"fp4_e2m1")
+    w.add("named_weights", b"1")
+
+    def put(name, value):
+        if isinstance(value, tuple):
+            w.add(f"weight_fp4_e2m1_{name}", value[0])
+            w.add(f"blockscale_{name}", value[1])
+        else:
+            w.add(f"weight_bf16_{name}", value)
+
+    put("W_emb", weights["emb"]); put("W_rms_final", weights["rms_final"]); put("W_lm_head", weights["lm_head"])
+    for li, L in enumerate(weights["layers"]):
+        for short, value in L.items():
+            put(f"{names[short]}_{li}", value)
+    path = tmp_path / "llama_like.bin"
+    w.save(path)
+
+    def fresh():
+        return pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
+
+    a, b = fresh(), fresh()
+    a.load(weights)
+    assert b.qk_norm
+    b.load_named(pkg.host_api.WeightFile(host, path))
+    assert not a.qk_norm and not b.qk_norm
+    for m in (a, b):
+        m.reset(7, 0)
+    for _ in range(5):
+        assert a.step() == b.step()
+    assert np.array_equal(a.logits(), b.logits())
+    again = tmp_path / "llama_like_again.bin"
+    b.save_named(again)
+    keys = weight_file.read_index(again)[0]
+    assert not any("norm_" in k and ("qnorm" in k or "knorm" in k) for k in keys)
+    for key in weight_file.read_index(path)[0]:
+        assert weight_file.read_entry(again, key) == weight_file.read_entry(path, key), key

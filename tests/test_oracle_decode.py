@@ -2,6 +2,7 @@
 implementation of the whole step (no intermediate rounding), which the BF16-rounded oracle must
 follow within BF16 noise."""
 import numpy as np
+import pytest
 import torch
 
 
@@ -87,8 +88,10 @@ def torch_step(model, cfg, oracle, d, tokens):
         x = B(model["emb"][tok])
         for li, L in enumerate(model["layers"]):
             xn = norm(x, B(L["rms_attn"]))
-            q = rot(norm((W(L["wq"]) @ xn).view(cfg.n_q, 128), B(L["q_norm"])), pos)
-            k = rot(norm((W(L["wk"]) @ xn).view(cfg.n_kv, 128), B(L["k_norm"])), pos)
+            q, k = (W(L["wq"]) @ xn).view(cfg.n_q, 128), (W(L["wk"]) @ xn).view(cfg.n_kv, 128)
+            if "q_norm" in L:
+                q, k = norm(q, B(L["q_norm"])), norm(k, B(L["k_norm"]))
+            q, k = rot(q, pos), rot(k, pos)
             ks[li][:, pos], vs[li][:, pos] = k, (W(L["wv"]) @ xn).view(cfg.n_kv, 128)
             rep = cfg.n_q // cfg.n_kv
             kk, vv = ks[li][:, :pos + 1].repeat_interleave(rep, 0), vs[li][:, :pos + 1].repeat_interleave(rep, 0)
@@ -101,10 +104,14 @@ def torch_step(model, cfg, oracle, d, tokens):
     return outs
 
 
-def test_oracle_follows_an_unrounded_float64_model(oracle):
+@pytest.mark.parametrize("qk_norm", [True, False])
+def test_oracle_follows_an_unrounded_float64_model(oracle, qk_norm):
+    """qk_norm = False is the graph without per-head norms (Llama-style, scripts/convert_weights.py:494-503): the two
+    cases must also differ from each other, or the switch would not be in the oracle's path."""
     from oracle import decode_oracle as d
-    cfg = d.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=500, t_kv=16)
-    model = d.make_model(cfg, 3)
+    cfg = d.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=500, t_kv=16, theta=1e6 if qk_norm else 5e5)
+    model = d.make_model(cfg, 3, qk_norm=qk_norm)
+    assert ("q_norm" in model["layers"][0]) == qk_norm
     tokens = [7, 123, 42, 499, 0]
     want = torch_step(model, cfg, oracle, d, tokens)
     orc = d.DecodeOracle(cfg, model)
