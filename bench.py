@@ -218,6 +218,84 @@ def build_decode_step(ws: Workspace, ctx: int):
     return model
 
 
+LLAMA31_8B = dict(layers=32, hidden=4096, n_q=32, n_kv=8, q_out=4096, kv_out=1024, inter=14336, vocab=128256, theta=5e5)
+
+
+def build_llama_fp4_step(ws: Workspace, ctx: int, block: int = 16):
+    """Random-init Llama-3.1-8B-shaped model with FP4_E2M1 block-scale linears (the reference's Llama FP4 route: codes and
+    one E4M3 scale byte per 16 elements as scripts/convert_weights.py:346-370 packs them), no per-head q/k norms, RoPE
+    theta 5e5, BF16 embedding and a KV cache already holding `ctx` positions.  Codes and scale bytes are uniform random
+    (scales in [2^-5, 2) so that no NaN code occurs); every layer gets its own device buffers, filled from one host
+    pattern rotated per layer."""
+    import numpy as np
+    t, c = ws.torch, LLAMA31_8B
+    model = ws.pkg.host_api.DecodeModel(ws.host, c["layers"], c["hidden"], c["n_q"], c["n_kv"], 128, c["inter"], c["vocab"], ctx, theta=c["theta"])
+    model.set_qk_norm(False)
+    rng = np.random.default_rng(4321)
+    shapes = {"wq": (c["q_out"], c["hidden"]), "wk": (c["kv_out"], c["hidden"]), "wv": (c["kv_out"], c["hidden"]),
+              "wo": (c["hidden"], c["q_out"]), "w_gate": (c["inter"], c["hidden"]), "w_up": (c["inter"], c["hidden"]),
+              "w_down": (c["hidden"], c["inter"]), "lm_head": (c["vocab"], c["hidden"])}
+    biggest = max(n * k for n, k in shapes.values())
+    codes = rng.integers(0, 256, size=biggest // 2 + 4096, dtype=np.uint8)
+    scales = rng.integers(0x10, 0x40, size=biggest // block + 4096, dtype=np.uint8)
+
+    def put(li, name):
+        n_out, K = shapes[name]
+        off = (li * 131 + len(name) * 17) % 4096
+        model.set_tensor(li, name, codes[off:off + n_out * K // 2], FP4)
+        model.set_block_scales(li, name, scales[off:off + n_out * K // block])
+
+    def fill_bf16(ptr, n, mean, std):
+        step = 1 << 26
+        for i0 in range(0, n, step):
+            m = min(step, n - i0)
+            v = (t.randn(m, device=ws.dev, generator=ws.gen) * std + mean).to(t.bfloat16)
+            assert ws.lib.convert(v.data_ptr(), BF16, ptr + i0 * 2, BF16, m * 2, 1.0) == 0
+            t.cuda.synchronize()
+
+    for li in range(c["layers"]):
+        for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+            put(li, name)
+        for name in ("rms_attn", "rms_ffn"):
+            fill_bf16(model.tensor_ptr(li, name), c["hidden"], 1.0, 0.1)
+        for is_v in (False, True):
+            fill_bf16(model.kv_ptr(li, is_v), c["n_kv"] * ctx * 128, 0.0, 1.0)
+    put(0, "lm_head")
+    fill_bf16(model.tensor_ptr(0, "rms_final"), c["hidden"], 1.0, 0.1)
+    fill_bf16(model.tensor_ptr(0, "emb"), c["vocab"] * c["hidden"], 0.0, 1.0)
+    return model
+
+
+def llama_fp4_step_bytes(ctx_mean: float, block: int = 16) -> int:
+    """Bytes one FP4 decode step must move: codes and scale bytes of every linear once, the keys and values attended to,
+    the embedding row, the norm weights and the logits."""
+    c = LLAMA31_8B
+    elems = c["layers"] * (c["hidden"] * (c["q_out"] + 2 * c["kv_out"]) + c["q_out"] * c["hidden"] + 3 * c["hidden"] * c["inter"]) + c["hidden"] * c["vocab"]
+    kv = int(c["layers"] * 2 * c["kv_out"] * 2 * ctx_mean)
+    small = c["layers"] * 2 * 2 * c["hidden"] + 2 * c["hidden"] * 2 + c["vocab"] * 2
+    return elems // 2 + elems // block + kv + small
+
+
+def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool):
+    """The FP4 decode step as a benchmark entry: tokens / s of the Llama-3.1-8B-shaped model at context DECODE_CTX."""
+    model = build_llama_fp4_step(ws, DECODE_CTX)
+    start = DECODE_CTX - steps - warmup
+    ws.torch.cuda.synchronize()
+    model.reset(1, start)
+    if warmup:
+        model.run(warmup, use_graph)
+    ms = model.run(steps, use_graph) / steps
+    assert model.pos == DECODE_CTX
+    nbytes = llama_fp4_step_bytes(DECODE_CTX - (steps - 1) / 2.0)
+    c = LLAMA31_8B
+    entry = {"workload": ("full random-init Llama-3.1-8B-shaped FP4_E2M1 block-16 decode step, batch 1, greedy: 32 layers, hidden 4096, 32 q / 8 kv heads x 128, "
+                          f"no qk norm, RoPE theta 5e5, SwiGLU 14336, vocab 128256, bf16 KV cache holding {DECODE_CTX} positions"),
+             "tok_s": round(1000.0 / ms, 1), "ms_per_step": round(ms, 4), "launch_mode": "hipGraph" if use_graph else "stream",
+             "bytes_per_token": nbytes, "GBps": round(nbytes / ms * 1e-6, 1), "frac_of_hbm_bound": round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
+             "launches_per_step": 6 * c["layers"] + 2, "last_token": model.token}
+    return entry, model
+
+
 def decode_step_bytes(ctx_mean: float) -> int:
     """Bytes one decode step must move: every linear weight once, the keys and values of the positions
     attended to, the embedding row, the norm weights and the logits."""
@@ -549,6 +627,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-fp4-step", action="store_true", help="skip the Llama-3.1-8B-shaped FP4 decode step")
     ap.add_argument("--sweep-tokens", default="1,4,16", help="token counts of the per-shape GEMV sweep")
     ap.add_argument("--no-baselines", action="store_true", help="skip the same-GPU BF16 baselines of the decode step")
     ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
@@ -619,6 +698,8 @@ def main():
         K, N, M = 4096, 2 * 12288, 1
         dom_us = ws.bench.gate_up_us(model, 10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
+        if not args.no_fp4_step:
+            extra["fp4_decode_step"], fp4_model = llama_fp4_decode(ws, args.steps, args.warmup, use_graph)
         if not args.no_sweep:
             # Nothing is freed until the last sweep has run: on this driver, freeing a few GB of device memory slows the
             # kernels that stream through the buffers still allocated (the 253-linear chain: 1.79 -> 1.91 ms per step

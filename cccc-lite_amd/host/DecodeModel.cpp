@@ -120,8 +120,8 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     if (Rocblas::isQuantized(dt))
     {
         if ((int64_t)bytes != (dt == FP4_E2M1 ? (m->getDataSize() + 1) / 2 : m->getDataSize())) { return -1; }
-        // only a tall weight (lm_head) is read through its tiled copy by the fused decode kernels
-        m->setAllowRepack(which == LM_HEAD);
+        // only a tall FP8 weight (lm_head) is read through its tiled copy by the fused decode kernels
+        m->setAllowRepack(which == LM_HEAD && dt != FP4_E2M1);
         m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
         return 0;
     }
@@ -159,18 +159,19 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         if (!wk.valid()) { return fail(name, -1); }
         if (wk.is_quant)
         {
-            m.setAllowRepack(tiled);
+            m.setAllowRepack(tiled && wk.dt != FP4_E2M1);      // the fused FP4 kernels read the file layout only
             if (file.loadNamed(m, name) != 0) { return fail(name, -2); }
             if (wk.dt == FP4_E2M1 && !m.getBlockScaleData()) { return fail(name, -3); }    // FP4 without blockscale_<name>: no fused kernel
             return 0;
         }
+        const bool tiled_q = tiled && quantize_to != FP4_E2M1;
         Matrix tmp(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
-        tmp.setAllowRepack(tiled);
+        tmp.setAllowRepack(tiled_q);
         if (file.loadNamed(tmp, name) != 0) { return fail(name, -2); }
         if (tmp.getDataType() == FLOAT)
         {
             Matrix bf(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
-            bf.setAllowRepack(tiled);
+            bf.setAllowRepack(tiled_q);
             if (hip_convert(tmp.data(), (int)FLOAT, bf.data(), (int)BFLOAT16, (unsigned)tmp.getDataSize(), 1.0f) != 0) { return fail(name, -3); }
             (void)hipDeviceSynchronize();
             tmp = bf;
