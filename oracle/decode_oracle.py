@@ -214,8 +214,7 @@ class DecodeOracle:
                     trace.update(xn=xn, q=q.copy(), att=att.copy(), r1=r1, gated=gated)
         xf = rms_norm(x, f(self.model["rms_final"]), c.eps)
         if logit_rows is not None:
-            W = self.model["lm_head"][np.asarray(logit_rows)]
-            logits = linear(o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape), xf)
+            logits = linear(dequant_linear(self.model["lm_head"][np.asarray(logit_rows)]), xf)
             return logits, int(np.asarray(logit_rows)[int(np.argmax(logits))])
         logits = linear(self.deq(None, "lm_head"), xf)
         return logits, int(np.argmax(logits))

@@ -239,33 +239,65 @@ def test_fused_linears_at_their_qwen3_8b_instantiations(gpu, pkg, oracle, dec, c
 # ------------------------------------------------------------------------------------------ decode step
 
 @pytest.mark.parametrize("exact_attention", [False, True])
-def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
+@pytest.mark.parametrize("arch", ["qwen3_8b_fp8", "llama31_8b_fp4"])
+def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention, arch):
     """Two layers of the Qwen3-8B shape (hidden 4096, 32 / 8 heads, intermediate 12288, vocabulary 151936,
     4096 cache rows) with caches already holding 4090 positions, two steps from position 4090: every launch
     configuration the benchmark's 36-layer model uses is reached.  The last layer's intermediate vectors, the
-    appended cache rows of both layers and 4096 sampled logits against the CPU oracle on the same bytes."""
+    appended cache rows of both layers and 4096 sampled logits against the CPU oracle on the same bytes.
+    llama31_8b_fp4: the same at the Llama-3.1-8B shape (intermediate 14336, vocabulary 128256, RoPE theta 5e5, no
+    per-head norms) with FP4_E2M1 block-16 linears packed as the converter packs them -- the launches of the
+    benchmark's fp4_decode_step."""
     torch, dev, lib = gpu
     host = pkg.host_api.host()
     host.init(0)
-    cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=12288, vocab=151936, t_kv=4096)
-    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    fp4 = arch == "llama31_8b_fp4"
+    if fp4:
+        cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=14336, vocab=128256, t_kv=4096, theta=5e5)
+    else:
+        cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=12288, vocab=151936, t_kv=4096)
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
     model.set_exact_attention(exact_attention)
+    model.set_qk_norm(not fp4)
     gen = torch.Generator(device=dev).manual_seed(8)
     copy = lambda src, dst, nbytes: lib.convert(src.data_ptr(), BF16, dst, BF16, nbytes, 1.0)      # same type: a byte copy on the device
+
+    def draw_fp4(n_out, K):
+        """(packed codes, E4M3 block scales) on the device, from N(0, 0.02) rounded to BF16, in slabs of rows"""
+        nibs, scs = [], []
+        rows = max(1, (1 << 25) // K)
+        for r0 in range(0, n_out, rows):
+            w = (torch.randn(min(rows, n_out - r0), K, device=dev, generator=gen) * 0.02).to(torch.bfloat16).float()
+            nib, sc = pack_fp4_on_device(torch, w, 16)
+            nibs.append(nib)
+            scs.append(sc)
+        return torch.cat(nibs), torch.cat(scs)
+
+    def put_linear(li, name, n_out, K):
+        """Draws one linear, hands it to the model, returns what the oracle's model dict holds for it"""
+        if fp4:
+            nib, sc = draw_fp4(n_out, K)
+            nib_h, sc_h = nib.cpu().numpy(), sc.cpu().numpy()
+            model.set_tensor(li, name, nib_h, 6)
+            model.set_block_scales(li, name, sc_h)
+            return (nib_h, sc_h), (nib, sc)
+        w = draw_e5m2(torch, dev, gen, n_out, K)
+        assert copy(w, model.tensor_ptr(li, name), n_out * K) == 0
+        return w.cpu().numpy(), w
 
     weights = {"layers": []}
     lin_shapes = {"wq": (cfg.q_out, cfg.hidden), "wk": (cfg.kv_out, cfg.hidden), "wv": (cfg.kv_out, cfg.hidden), "wo": (cfg.hidden, cfg.q_out),
                   "w_gate": (cfg.inter, cfg.hidden), "w_up": (cfg.inter, cfg.hidden), "w_down": (cfg.hidden, cfg.inter)}
-    norm_sizes = {"rms_attn": cfg.hidden, "rms_ffn": cfg.hidden, "q_norm": 128, "k_norm": 128}
+    norm_sizes = {"rms_attn": cfg.hidden, "rms_ffn": cfg.hidden}
+    if not fp4:
+        norm_sizes.update(q_norm=128, k_norm=128)
     start = 4090
     k_host = np.zeros((cfg.layers, cfg.n_kv, cfg.t_kv, 128), dtype=np.float32)
     v_host = np.zeros_like(k_host)
     for li in range(cfg.layers):
         L = {}
         for name, (n_out, K) in lin_shapes.items():
-            w = draw_e5m2(torch, dev, gen, n_out, K)
-            assert copy(w, model.tensor_ptr(li, name), n_out * K) == 0
-            L[name] = w.cpu().numpy()
+            L[name], _ = put_linear(li, name, n_out, K)
         for name, n in norm_sizes.items():
             v = draw_bf16(torch, dev, gen, (n,), mean=1.0, std=0.1)
             assert copy(v, model.tensor_ptr(li, name), n * 2) == 0
@@ -276,9 +308,9 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
             c[:, start:] = 0x7FC1                                    # rows not written yet hold NaN patterns
             assert copy(c, model.kv_ptr(li, is_v), c.numel() * 2) == 0
             dst[li] = dec.f(host_bits(c))
-    lm = draw_e5m2(torch, dev, gen, cfg.vocab, cfg.hidden)
-    assert copy(lm, model.tensor_ptr(0, "lm_head"), cfg.vocab * cfg.hidden) == 0
-    assert model.prepare_tiled(0, "lm_head")
+    lm_host, lm = put_linear(0, "lm_head", cfg.vocab, cfg.hidden)
+    if not fp4:
+        assert model.prepare_tiled(0, "lm_head")
     fin = draw_bf16(torch, dev, gen, (cfg.hidden,), mean=1.0, std=0.1)
     assert copy(fin, model.tensor_ptr(0, "rms_final"), cfg.hidden * 2) == 0
     emb_rows = {}
@@ -287,7 +319,10 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
     torch.cuda.synchronize()
 
     logit_rows = np.sort(np.random.default_rng(3).choice(cfg.vocab, size=4096, replace=False))
-    lm_rows = lm[torch.from_numpy(logit_rows).to(dev)].cpu().numpy()
+    if fp4:
+        lm_rows = (lm_host[0][logit_rows], lm_host[1][logit_rows])
+    else:
+        lm_rows = lm[torch.from_numpy(logit_rows).to(dev)].cpu().numpy()
 
     class Rows:
         """Stands in for a [vocab, hidden] array of which only a few rows were downloaded."""
@@ -300,7 +335,8 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
 
     weights["emb"] = Rows(lambda t: host_bits(emb[int(t)]))
     weights["rms_final"] = host_bits(fin)
-    weights["lm_head"] = Rows(lambda idx: lm_rows[np.searchsorted(logit_rows, np.asarray(idx))])
+    pick = lambda idx: np.searchsorted(logit_rows, np.asarray(idx))
+    weights["lm_head"] = Rows((lambda idx: (lm_rows[0][pick(idx)], lm_rows[1][pick(idx)])) if fp4 else (lambda idx: lm_rows[pick(idx)]))
     del emb_rows
     orc = dec.DecodeOracle(cfg, weights)
     orc.k[:], orc.v[:] = k_host, v_host
@@ -319,7 +355,10 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention):
             got = dec.f(model.activation(name))
             assert np.isfinite(got).all(), name
             err = np.linalg.norm(got - want.reshape(-1)) / np.linalg.norm(want)
-            assert err < 1e-2, (pos, name, err)
+            # The second layer's inputs already differ from the oracle's by the first layer's BF16 roundings (r1 of a
+            # single layer: 1e-3), which the softmax amplifies; on the route that keeps FP32 probabilities every element
+            # may sit one more ulp away (a single layer measures 3e-3 .. 4e-3 there, two layers up to 1.1e-2).
+            assert err < (2e-2 if name == "att" and not exact_attention else 1e-2), (pos, name, err)
         for li in range(cfg.layers):
             gk, gv = dec.f(model.kv(li, False)[:, pos]), dec.f(model.kv(li, True)[:, pos])
             tol = 2e-3 if li == 0 else 1e-2                          # layer 0 sees identical inputs
