@@ -64,6 +64,7 @@ EXPORTS = (
     "hip_attention_decode_bf16",
     "hip_attention_decode_workspace_bytes",
     "hip_attention_decode_fused_bf16",
+    "hip_attention_decode_exact_bf16",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_argmax_pick_embed_bf16",
@@ -130,6 +131,8 @@ class QuantLibrary:
         L.hip_attention_decode_bf16.argtypes = [vp] * 5 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp]
         L.hip_attention_decode_fused_bf16.restype = i32
         L.hip_attention_decode_fused_bf16.argtypes = [vp] * 11 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp, f32]
+        L.hip_attention_decode_exact_bf16.restype = i32
+        L.hip_attention_decode_exact_bf16.argtypes = [vp] * 11 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp, f32]
         L.hip_attention_decode_workspace_bytes.restype = ctypes.c_ulonglong
         L.hip_attention_decode_workspace_bytes.argtypes = [i32, i32, i32]
         L.hip_argmax_workspace_bytes.restype = ctypes.c_ulonglong

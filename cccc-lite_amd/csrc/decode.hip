@@ -349,6 +349,42 @@ int hip_attention_decode_fused_bf16(const void* q, const void* k, const void* v,
     return finish("attention_decode_fused");
 }
 
+int hip_attention_decode_exact_bf16(const void* q, const void* k, const void* v, const void* q_norm_w, const void* k_norm_w,
+                                    const void* cos_tab, const void* sin_tab, void* k_cache, void* v_cache, void* y,
+                                    void* workspace, unsigned long long workspace_bytes,
+                                    int n_q_heads, int n_kv_heads, int head_dim, int t_kv, const void* d_pos, float epsilon)
+{
+    if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || !d_pos) { return -1; }
+    if (!q || !k || !v || !cos_tab || !sin_tab || !k_cache || !v_cache || !y || !workspace) { return -1; }
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) { return -1; }
+    if (!aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace)) { return -1; }
+    const AttentionWorkspace w = attention_workspace(n_q_heads, t_kv);
+    if (workspace_bytes < w.total) { return -1; }
+    const dim3 grid(w.n_blocks, n_kv_heads);
+    uint16_t* scores = (uint16_t*)((char*)workspace + w.scores);
+    float2* stats = (float2*)((char*)workspace + w.stats);
+    float* partial = (float*)((char*)workspace + w.partial);
+    const float scale = 1.0f / sqrtf(128.0f);
+    const int* pos = (const int*)d_pos;
+#define CCQ_ATTN_EXACT(G)                                                                                                                            \
+    attn_fused_kernel<G, true><<<grid, 256, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_norm_w,   \
+                                                           (const uint16_t*)k_norm_w, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,          \
+                                                           (uint16_t*)k_cache, (uint16_t*)v_cache, stats, partial, t_kv, w.n_blocks, pos,          \
+                                                           n_q_heads, epsilon, scale, scores);                                                      \
+    attn_pv_kernel<G><<<grid, 256, 0, stream()>>>(scores, stats, (const uint16_t*)v_cache, partial, t_kv, w.n_blocks, pos, n_q_heads)
+    switch (n_q_heads / n_kv_heads)
+    {
+    case 1: CCQ_ATTN_EXACT(1); break;
+    case 2: CCQ_ATTN_EXACT(2); break;
+    case 4: CCQ_ATTN_EXACT(4); break;
+    default: return -1;
+    }
+#undef CCQ_ATTN_EXACT
+    const int n_out = n_q_heads * 128;
+    attn_combine_kernel<<<(n_out + 63) / 64, 256, 0, stream()>>>(partial, (uint16_t*)y, n_out, t_kv, pos);
+    return finish("attention_decode_exact");
+}
+
 // room for either use: the per-block candidates of hip_argmax_bf16, or the candidate list a linear launch leaves
 unsigned long long hip_argmax_workspace_bytes(unsigned int n)
 {

@@ -1131,13 +1131,17 @@ __device__ __forceinline__ void norm_rope_head(const uint16_t* __restrict__ src,
     norm_rope_finish(load_head(src, nw, cos_row, sin_row, lane), nw != nullptr, eps, out_l, out_r);
 }
 
-template <int G>
+// SCORES_ONLY: the front half alone -- norm, rotation, append, the block's BF16 scores written to scores[qh][t] and their
+// (max, sum expf(s - max)) to stats -- for the route that rounds the probabilities of the whole row to BF16 before they
+// meet V (attn_pv_kernel and attn_combine_kernel follow); no value row is read here.
+template <int G, bool SCORES_ONLY = false>
 __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
                                                         const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
                                                         const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab,
                                                         uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
                                                         float2* __restrict__ stats, float* __restrict__ partial,
-                                                        int t_kv, int n_blocks, const int* __restrict__ d_pos, int n_q, float eps, float scale)
+                                                        int t_kv, int n_blocks, const int* __restrict__ d_pos, int n_q, float eps, float scale,
+                                                        uint16_t* __restrict__ scores = nullptr)
 {
     __shared__ float acc_lds[16][G][128];   // [key slot in workgroup][head][dim]
     __shared__ float s_lds[G][ATT_KEYS];    // scores, then expf(s - block max)
@@ -1171,11 +1175,14 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
 #pragma unroll
         for (int c = 0; c < 4; c++) { kraw[c] = __builtin_nontemporal_load((const u32x4*)(k_cache + ((size_t)kvh * t_kv + t) * 128 + c * 32 + key_in_wave * 8)); }
     }
-#pragma unroll
-    for (int it = 0; it < ATT_ITS; it++)
+    if constexpr (!SCORES_ONLY)
     {
-        const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);
-        vraw[it] = __builtin_nontemporal_load((const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8));
+#pragma unroll
+        for (int it = 0; it < ATT_ITS; it++)
+        {
+            const int t = min(t0 + it * 16 + wave * 4 + key_in_wave, n_keys - 1);
+            vraw[it] = __builtin_nontemporal_load((const u32x4*)(v_cache + ((size_t)kvh * t_kv + t) * 128 + sub * 8));
+        }
     }
     if (wave < G)
     {
@@ -1223,7 +1230,12 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
             for (int v = 0; v < 4; v++)
             {
                 const int kl = wave * 16 + key_in_wave * 4 + v;
-                s_lds[sub][kl] = t0 + kl < n_keys ? bf16_round(scale * sc[v]) : -INFINITY;
+                const float sv = bf16_round(scale * sc[v]);
+                s_lds[sub][kl] = t0 + kl < n_keys ? sv : -INFINITY;
+                if constexpr (SCORES_ONLY)
+                {
+                    if (t0 + kl < n_keys) { scores[(size_t)(kvh * G + sub) * t_kv + t0 + kl] = (uint16_t)(__builtin_bit_cast(uint32_t, sv) >> 16); }
+                }
             }
         }
     }
@@ -1245,6 +1257,7 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(const uint16_t* __restr
         l = wave_sum(l);
         if (lane == 0) { stats[(size_t)(kvh * G + wave) * n_blocks + blk] = make_float2(m, l); }
     }
+    if constexpr (SCORES_ONLY) { return; }
     __syncthreads();
     float acc[G][8];
 #pragma unroll

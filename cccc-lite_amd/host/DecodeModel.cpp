@@ -46,7 +46,6 @@ DecodeModel::DecodeModel(const DecodeConfig& cfg, GpuControl* gpu) : cfg_(cfg), 
     q_ = make(q_out, 1, BFLOAT16, gpu);
     k_ = make(kv_out, 1, BFLOAT16, gpu);
     v_ = make(kv_out, 1, BFLOAT16, gpu);
-    q_rot_ = make(q_out, 1, BFLOAT16, gpu);
     att_ = make(q_out, 1, BFLOAT16, gpu);
     gated_ = make(cfg.inter, 1, BFLOAT16, gpu);
     attn_ws_bytes_ = hip_attention_decode_workspace_bytes(cfg.n_q, cfg.n_kv, cfg.t_kv);
@@ -329,13 +328,9 @@ int DecodeModel::step()
         }
         else if (rc == 0)
         {
-            rc = hip_qk_norm_rope_kv_bf16(q_->data(), k_->data(), v_->data(), q_norm_w, k_norm_w, cos_->data(), sin_->data(),
-                                          q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
-            if (rc == 0)
-            {
-                rc = hip_attention_decode_bf16(q_rot_->data(), k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(),
-                                               attn_ws_bytes_, c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos);
-            }
+            rc = hip_attention_decode_exact_bf16(q_->data(), k_->data(), v_->data(), q_norm_w, k_norm_w, cos_->data(), sin_->data(),
+                                                 k_cache_[li]->data(), v_cache_[li]->data(), att_->data(), attn_ws_->data(), attn_ws_bytes_,
+                                                 c.n_q, c.n_kv, c.head_dim, c.t_kv, d_pos, c.eps);
         }
         // 4. r1 = x + W_o att
         if (rc == 0)

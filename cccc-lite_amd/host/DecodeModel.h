@@ -65,7 +65,7 @@ public:
     int saveNamedWeights(const std::string& filename);
 
     // false (default): two-launch attention with the norm / RoPE / append folded in and FP32 probabilities;
-    // true: the reference's rounding points throughout (separate norm / RoPE / append launch, BF16 probabilities).
+    // true: the reference's rounding points throughout (BF16 probabilities over the whole row; three launches).
     void setExactAttention(bool exact) { exact_attention_ = exact; }
     // Per-head RMSNorm of q and k in front of the rotation: on for Qwen3-style models (default), off for models without
     // W_qnorm / W_knorm such as Llama-3.1 (has_qknorm in scripts/convert_weights.py:488-530).  loadNamedWeights sets it
@@ -94,7 +94,7 @@ private:
     std::vector<Layer> layers_;
     std::unique_ptr<Matrix> emb_, rms_final_, lm_head_, logits_, cos_, sin_;
     std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
-    std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, q_rot_, att_, gated_, attn_ws_, argmax_ws_;
+    std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, att_, gated_, attn_ws_, argmax_ws_;
     unsigned long long attn_ws_bytes_ = 0;
     bool exact_attention_ = false;
     bool qk_norm_ = true;

@@ -230,6 +230,18 @@ C_EXPORT int hip_attention_decode_fused_bf16(const void* q, const void* k, const
                                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
                                              const void* d_pos, float epsilon);
 
+/* hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16 in three launches instead of four: the norm, the rotation and the
+ * cache append ride in the launch that computes the scores; every rounding point of the reference is kept (BF16 q, k,
+ * scores and probabilities, cccc/MatrixEx.cpp:3018-3104, cccc-hip/hip_functions.cpp:776-804).  Arguments as
+ * hip_attention_decode_fused_bf16. */
+C_EXPORT int hip_attention_decode_exact_bf16(const void* q, const void* k, const void* v,
+                                             const void* q_norm_w, const void* k_norm_w,
+                                             const void* cos_tab, const void* sin_tab,
+                                             void* k_cache, void* v_cache, void* y,
+                                             void* workspace, unsigned long long workspace_bytes,
+                                             int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                             const void* d_pos, float epsilon);
+
 /* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
 C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);
 

@@ -472,6 +472,65 @@ def test_decode_steps_with_fp4_linears_follow_the_oracle(gpu, pkg, oracle, dec):
     assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
 
 
+@pytest.mark.parametrize("n_q,n_kv,t_kv,normed", [(4, 2, 200, True), (8, 2, 300, True), (2, 2, 130, True), (8, 2, 300, False), (4, 2, 6000, True)])
+def test_three_launch_attention_keeps_the_reference_rounding_points(gpu, oracle, dec, n_q, n_kv, t_kv, normed):
+    """hip_attention_decode_exact_bf16: norm, rotation and append in the scores launch.  The appended rows are the
+    oracle's, the BF16 scores it leaves in the workspace are the reference's rounding point (within one ulp of the exact
+    product sum: the summation order is the matrix cores'), and the outputs agree with the four-launch route
+    (hip_qk_norm_rope_kv_bf16 + hip_attention_decode_bf16) on the same inputs as closely as with the oracle."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(41)
+    cfg = dec.DecodeConfig(n_q=n_q, n_kv=n_kv, t_kv=t_kv)
+    cos, sin = dec.rope_tables(cfg)
+    qw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(128)).astype(np.float32))
+    kw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(128)).astype(np.float32))
+    kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    ws_bytes = lib.c.hip_attention_decode_workspace_bytes(n_q, n_kv, t_kv)
+    ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device=dev)
+    ws2 = torch.full((ws_bytes,), 0x5A, dtype=torch.uint8, device=dev)
+    qwd, kwd, cd, sd = (to_dev(torch, dev, a) for a in (qw, kw, cos, sin))
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    nq_w, nk_w = (ptr(qwd), ptr(kwd)) if normed else (ctypes.c_void_p(0), ctypes.c_void_p(0))
+    for pos in ((0, 4095, 4096, 4160, t_kv - 1) if t_kv > 4096 else (0, 1, 63, 64, 127, 128, t_kv - 1)):
+        q = oracle.f32_to_bf16((2 * rng.standard_normal((n_q, 128))).astype(np.float32))
+        k = oracle.f32_to_bf16((2 * rng.standard_normal((n_kv, 128))).astype(np.float32))
+        v = oracle.f32_to_bf16(rng.standard_normal((n_kv, 128)).astype(np.float32))
+        qd, knd, vnd = (to_dev(torch, dev, a) for a in (q, k, v))
+        pd = torch.tensor([pos], dtype=torch.int32, device=dev)
+        kd, vd = to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+        y = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        assert lib.c.hip_attention_decode_exact_bf16(ptr(qd), ptr(knd), ptr(vnd), nq_w, nk_w, ptr(cd), ptr(sd), ptr(kd), ptr(vd), ptr(y), ptr(ws), ws_bytes,
+                                                     n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == 0
+        # the four-launch route on copies of the same caches
+        kd2, vd2 = to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+        q_rot = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        y2 = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        assert lib.c.hip_qk_norm_rope_kv_bf16(ptr(qd), ptr(knd), ptr(vnd), nq_w, nk_w, ptr(cd), ptr(sd), ptr(q_rot), ptr(kd2), ptr(vd2),
+                                              n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == 0
+        assert lib.c.hip_attention_decode_bf16(ptr(q_rot), ptr(kd2), ptr(vd2), ptr(y2), ptr(ws2), ws_bytes, n_q, n_kv, 128, t_kv, ptr(pd)) == 0
+        got_k = from_dev(kd, np.uint16).reshape(n_kv, t_kv, 128)
+        # the appended rows: both routes run the same arithmetic on the same bytes
+        assert np.array_equal(got_k, from_dev(kd2, np.uint16).reshape(n_kv, t_kv, 128)), pos
+        assert np.array_equal(from_dev(vd, np.uint16), from_dev(vd2, np.uint16)), pos
+        qr = dec.f(from_dev(q_rot, np.uint16).reshape(n_q, 128))
+        # scores: BF16 of the exact sum, up to the last bit of an FP32 sum taken in another order
+        s = ws[:n_q * t_kv * 2].cpu().numpy().view(np.uint16).reshape(n_q, t_kv)[:, :pos + 1]
+        for h in range(n_q):
+            exact = dec.f(got_k)[h // (n_q // n_kv), :pos + 1].astype(np.float64) @ qr[h].astype(np.float64)
+            ref = dec.r(np.float32(1 / np.sqrt(np.float32(128))) * exact.astype(np.float32))
+            # (ulp_close measures in units of |want| * 2^-8, i.e. half a BF16 ulp at the bottom of a binade: 2.0 = one rounding flip)
+            assert ulp_close(s[h], ref, ulps=2.0, floor=1e-5).all(), (pos, h)
+            assert (s[h] == oracle.f32_to_bf16(ref)).mean() > 0.99
+        want = dec.attention(qr, dec.f(got_k), dec.f(from_dev(vd, np.uint16).reshape(n_kv, t_kv, 128)), pos, n_q, n_kv)
+        got = from_dev(y, np.uint16).reshape(n_q, 128)
+        assert ulp_close(got, want, ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), pos
+        assert ulp_close(got, dec.f(from_dev(y2, np.uint16).reshape(n_q, 128)), ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), pos
+    args = [ptr(qd), ptr(knd), ptr(vnd), nq_w, nk_w, ptr(cd), ptr(sd), ptr(kd), ptr(vd), ptr(y), ptr(ws)]
+    assert lib.c.hip_attention_decode_exact_bf16(*args, ws_bytes - 256, n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == -1
+    assert lib.c.hip_attention_decode_exact_bf16(*args, ws_bytes, 3 * n_kv, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == -1
+
+
 @pytest.mark.parametrize("n_q,n_kv,t_kv", [(4, 2, 200), (8, 2, 300)])
 def test_attention_without_per_head_norms(gpu, oracle, dec, n_q, n_kv, t_kv):
     """Llama-style heads (has_qknorm = False, scripts/convert_weights.py:488-530): NULL norm weights make both attention
