@@ -499,8 +499,8 @@ def prefill_cases(ws, by_shape):
         for M in (512, 2048):
             X, Y = ws.activation(M, K), ws.output(M, N)
             ops = [(W, X, Y, K, N) for W in weights]
-            ms = time_chain(ws, ops, 3, 1, False)
-            us = ms * 1000.0 / (3 * len(ops))
+            ms = time_chain(ws, ops, 10, 3, False)
+            us = ms * 1000.0 / (10 * len(ops))
             tf = 2.0 * M * K * N / us * 1e-6
             x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
             for rep in range(2):
@@ -546,7 +546,7 @@ def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
             mlp = (K, N) in ((4096, 14336), (14336, 4096))
             for M in tuple(token_counts) + (tuple(prefill_tokens) if mlp and block == 16 else ()):
                 X, Y = ws.activation(M, K), ws.output(M, N)
-                n_it = iters if M <= 16 else 24
+                n_it = iters if M <= 16 else 96
                 ms = ws.bench.fp4_chain([w.data_ptr() for w in nib], [s_.data_ptr() for s_ in sc], X.data_ptr, Y.data_ptr, N, M, K, block, n_it, 5)
                 if ms < 0:
                     raise RuntimeError(f"fp4 chain failed: {ms}")
