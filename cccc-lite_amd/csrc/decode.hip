@@ -49,6 +49,25 @@ int launch_fused(const FusedLinearArgs& a, int n_groups)
     return finish("quant_linear_fused");
 }
 
+// BF16 weights (a tied lm_head): the dot2 kernel on 2-byte elements; launch shapes as for FP8 rows of twice the length.
+int launch_fused_bf16(const FusedLinearArgs& a, int n_groups)
+{
+    const size_t lds = (size_t)((a.K + 511) / 512) * 1024;
+    if (lds > 64 * 1024) { return -1; }
+    const int cus = cu_count();
+    if (n_groups >= cus * 64)
+    {
+        const int want = (n_groups + 7) / 8;
+        gemv8_fused_kernel<DT_BF16, 4, 8, false><<<want < cus * 2 ? want : cus * 2, 512, lds, stream()>>>(a);
+    }
+    else
+    {
+        const int want4 = (n_groups + 3) / 4;
+        gemv8_fused_kernel<DT_BF16, 4, 4, false><<<want4 < cus * 4 ? want4 : cus * 4, 256, lds, stream()>>>(a);
+    }
+    return finish("quant_linear_fused");
+}
+
 // FP4 block-scale weights: two rows per wave, U = 2 batches for rows of up to 4096 elements (one k-step of 2048 per
 // lane and row is 1 KiB), 8-wave workgroups for very tall weights, as for FP8.
 template <int BLOCK>
@@ -93,7 +112,7 @@ int launch_fused_mfma(const FusedLinearArgs& a, int n_tiles)
 
 int hip_quant_linear_fused(const hip_fused_linear* d)
 {
-    if (!d || (d->w_type != DT_E4M3 && d->w_type != DT_E5M2 && d->w_type != DT_FP4)) { return -1; }
+    if (!d || (d->w_type != DT_E4M3 && d->w_type != DT_E5M2 && d->w_type != DT_FP4 && d->w_type != DT_BF16)) { return -1; }
     if (d->K <= 0 || d->K % 16 != 0 || d->n_segments < 1 || d->n_segments > 3 || !d->X || !aligned16(d->X)) { return -1; }
     const bool fp4 = d->w_type == DT_FP4;
     if (fp4 && (d->K % 32 != 0 || (d->block_size != 16 && d->block_size != 32))) { return -1; }
@@ -131,6 +150,12 @@ int hip_quant_linear_fused(const hip_fused_linear* d)
     a.block = d->block_size;
     if (d->argmax_workspace && (d->n_segments != 1 || d->pair || !aligned16(d->argmax_workspace))) { return -1; }
     a.argmax_ws = d->argmax_workspace;
+    if (d->w_type == DT_BF16)
+    {
+        if (scaled) { return -1; }                          // a plain BF16 weight carries no dequantisation scale
+        note_kernel("gemv_fused_bf16");
+        return launch_fused_bf16(a, n_groups);
+    }
     if (fp4)
     {
         note_kernel("gemv_fused_fp4");

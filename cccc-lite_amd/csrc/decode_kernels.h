@@ -255,14 +255,22 @@ struct FusedRows
 // DIRECT_X (no RMSNorm in front, K a multiple of 1024): the activation is not staged at all -- every lane requests
 // the 32 bytes of x it needs for a step together with the weights of that step (x is a few KiB and stays in
 // the CU's L1), so the kernel has no prologue, no LDS and no barrier.
+// WT == DT_BF16: the weight is not quantized at all (a tied lm_head is the embedding table, which the reference keeps in
+// BF16: cccc/Net.cpp:1158-1190) -- the same kernel with 2-byte elements: a lane's 16-byte load is eight elements, a k-step
+// 512 of them, and the products need no conversion.  Staged activation only.
 template <int WT, int U, int WAVES, bool SCALED, bool DIRECT_X = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLinearArgs a)
 {
+    constexpr bool PLAIN = WT == DT_BF16;
+    static_assert(!(PLAIN && (DIRECT_X || SCALED)), "BF16 weights: staged activation, no scale");
+    constexpr int STEP = PLAIN ? 512 : 1024;                // elements of a row one wave-wide load covers
+    constexpr int ELEM = PLAIN ? 2 : 1;                     // bytes per weight element
+    constexpr int PARTS = PLAIN ? 1 : 2;                    // 16-byte activation pieces per lane and k-step
     extern __shared__ u32x4 xs[];
     __shared__ float red[WAVES];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_steps = (a.K + 1023) / 1024;
+    const int n_steps = (a.K + STEP - 1) / STEP;
     const int batches = (n_steps + U - 1) / U;
     // row groups of two: in pair mode (gate row i, up row i); otherwise two consecutive rows of one segment
     const int g0 = a.pair ? a.n_out[0] : (a.n_out[0] + 1) / 2;
@@ -283,8 +291,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
             r.row1 = min(local * 2 + 1, a.n_out[r.seg] - 1);
         }
         const int sa = a.pair ? 0 : r.seg, sb = a.pair ? 1 : r.seg;
-        r.w0 = a.W[sa] + (long long)r.row0 * a.K;
-        r.w1 = a.W[sb] + (long long)r.row1 * a.K;
+        r.w0 = a.W[sa] + (long long)r.row0 * a.K * ELEM;
+        r.w1 = a.W[sb] + (long long)r.row1 * a.K * ELEM;
         r.s0 = a.w_scale[sa];
         r.s1 = a.w_scale[sb];
         return r;
@@ -295,7 +303,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         for (int u = 0; u < U; u++)
         {
             wa[u] = wb[u] = u32x4{ 0u, 0u, 0u, 0u };
-            const int k = (st0 + u) * 1024 + lane * 16;
+            const int k = (st0 + u) * STEP + lane * (16 / ELEM);
             if (k < a.K)
             {
                 if constexpr (DIRECT_X)
@@ -303,8 +311,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
                     xq[u][0] = *(const u32x4*)(a.X + k);
                     xq[u][1] = *(const u32x4*)(a.X + k + 8);
                 }
-                wa[u] = __builtin_nontemporal_load((const u32x4*)(r.w0 + k));
-                wb[u] = __builtin_nontemporal_load((const u32x4*)(r.w1 + k));
+                wa[u] = __builtin_nontemporal_load((const u32x4*)(r.w0 + (long long)k * ELEM));
+                wb[u] = __builtin_nontemporal_load((const u32x4*)(r.w1 + (long long)k * ELEM));
             }
         }
     };
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         cur = locate(g);
         request(cur, 0, wa, wb, xa);
     }
-    if constexpr (!DIRECT_X) { stage_finish<WAVES * 64>(a, staged, xs, red); }
+    if constexpr (!DIRECT_X) { stage_finish<WAVES * 64, PARTS>(a, staged, xs, red); }
 
     float acc0 = 0.0f, acc1 = 0.0f;
     float best_v = -INFINITY;                               // greedy candidate of this wave (lane 0 keeps it)
@@ -341,7 +349,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_fused_kernel(const FusedLine
         for (int u = 0; u < U; u++)
         {
             const int st = batch * U + u;
-            if (st < n_steps)
+            if constexpr (PLAIN)
+            {
+                if (st < n_steps)
+                {
+                    const u32x4 x0 = xs[st * 64 + lane];
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                    {
+                        const uint32_t w0 = wa[u][d], w1 = wb[u][d];       // (a bit cast straight from the vector element reads element 0)
+                        acc0 = dot2_bf16(__builtin_bit_cast(bf16x2, w0), x0[d], acc0);
+                        acc1 = dot2_bf16(__builtin_bit_cast(bf16x2, w1), x0[d], acc1);
+                    }
+                }
+            }
+            else if (st < n_steps)
             {
                 const u32x4 x0 = DIRECT_X ? xa[u][0] : xs[(st * 2 + 0) * 64 + lane];
                 const u32x4 x1 = DIRECT_X ? xa[u][1] : xs[(st * 2 + 1) * 64 + lane];

@@ -184,7 +184,10 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
     qk_norm_ = cfg_.layers == 0 || file.resolve("W_qnorm_0").valid() || file.resolve("W_knorm_0").valid();
     int rc = load_plain(*emb_, "W_emb");
     if (rc == 0) { rc = load_plain(*rms_final_, "W_rms_final"); }
-    if (rc == 0) { rc = load_linear(*lm_head_, file.resolve("W_lm_head").valid() ? "W_lm_head" : "W_emb", true); }
+    // no W_lm_head entry: tied embeddings -- the head multiplies by the embedding table, which the reference never quantizes
+    // (cccc/Net.cpp:1158-1190 skips EMBED tables and every view that shares their storage)
+    setTiedLmHead(!file.resolve("W_lm_head").valid());
+    if (rc == 0 && !tied_lm_head_) { rc = load_linear(*lm_head_, "W_lm_head", true); }
     for (int i = 0; i < cfg_.layers && rc == 0; i++)
     {
         Layer& L = layers_[i];
@@ -210,7 +213,7 @@ int DecodeModel::saveNamedWeights(const std::string& filename)
     if (filename.empty() || hipDeviceSynchronize() != hipSuccess) { return -1; }
     WeightFileWriter w;
     // header: the first quantized tensor's type, else the first tensor's (cccc/Net.cpp:1243-1271)
-    const DataType head = Rocblas::isQuantized(lm_head_->getDataType()) || layers_.empty() ? lm_head_->getDataType() : layers_[0].wq->getDataType();
+    const DataType head = (!tied_lm_head_ && Rocblas::isQuantized(lm_head_->getDataType())) || layers_.empty() ? lm_head_->getDataType() : layers_[0].wq->getDataType();
     const char* names[] = { "auto", "float", "double", "half", "bfloat16", "fp8_e4m3", "fp8_e5m2", "fp4_e2m1" };
     const DataType order[] = { CURRENT, FLOAT, DOUBLE, HALF, BFLOAT16, FP8_E4M3, FP8_E5M2, FP4_E2M1 };
     std::string head_name = "auto";
@@ -219,7 +222,7 @@ int DecodeModel::saveNamedWeights(const std::string& filename)
     w.set_value("named_weights", std::string("1"));
     addNamedWeight(w, "W_emb", *emb_);
     addNamedWeight(w, "W_rms_final", *rms_final_);
-    addNamedWeight(w, "W_lm_head", *lm_head_);
+    if (!tied_lm_head_) { addNamedWeight(w, "W_lm_head", *lm_head_); }
     for (int i = 0; i < cfg_.layers; i++)
     {
         Layer& L = layers_[i];
@@ -235,6 +238,15 @@ int DecodeModel::saveNamedWeights(const std::string& filename)
         }
     }
     return w.save(filename) > 0 ? 0 : -1;
+}
+
+void DecodeModel::setTiedLmHead(bool tied)
+{
+    if (tied == tied_lm_head_) { return; }
+    tied_lm_head_ = tied;
+    // the separate head's storage is only held while it is used
+    if (tied) { lm_head_ = std::make_unique<Matrix>(cfg_.hidden, 1, 1, 1, FP8_E5M2, gpu_); }
+    else { lm_head_ = std::make_unique<Matrix>(cfg_.hidden, cfg_.vocab, 1, 1, FP8_E5M2, gpu_); }
 }
 
 size_t DecodeModel::weightBytes() const
@@ -362,7 +374,7 @@ int DecodeModel::step()
     }
     if (rc == 0)
     {
-        hip_fused_linear head = linear_desc(*lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
+        hip_fused_linear head = linear_desc(tied_lm_head_ ? *emb_ : *lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
         head.norm_weight = rms_final_->data();
         head.norm_eps = c.eps;
         head.argmax_workspace = argmax_ws_->data();        // the launch leaves the greedy candidates of its logits

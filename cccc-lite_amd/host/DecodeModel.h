@@ -48,7 +48,7 @@ public:
     int setBlockScales(int layer, int which, const void* host, size_t n_scales);
 
     // Loads every tensor from a converted model file by the converter's names (scripts/convert_weights.py:142-166):
-    // W_emb, W_rms_final, W_lm_head (W_emb when absent: tied), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
+    // W_emb, W_rms_final, W_lm_head (absent: tied embeddings, the head then reads W_emb in BF16), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
     // W_qnorm_<i>, W_knorm_<i> (a file without them loads as a model without per-head norms), W_rms_ffn_<i>, W_gate_<i>,
     // W_up_<i>, W_down_<i>.  FP8 and FP4 linears are taken as stored;
     // linears stored as BF16 / HALF / FLOAT are quantized on load to `quantize_to` with a per-tensor absmax scale
@@ -71,6 +71,11 @@ public:
     // W_qnorm / W_knorm such as Llama-3.1 (has_qknorm in scripts/convert_weights.py:488-530).  loadNamedWeights sets it
     // from what the file holds.
     void setQkNorm(bool on) { qk_norm_ = on; }
+    // Tied embeddings (tie_word_embeddings, scripts/convert_weights.py:230-260: no W_lm_head entry in the file): the head
+    // multiplies by the BF16 embedding table itself, as the reference does -- it never quantizes an EMBED table nor a view
+    // sharing its storage (cccc/Net.cpp:1158-1190) -- and no separate head is stored.  loadNamedWeights sets it from the file.
+    void setTiedLmHead(bool tied);
+    bool tiedLmHead() const { return tied_lm_head_; }
     bool qkNorm() const { return qk_norm_; }
     int reset(int token, int pos);          // sets the device-side token / position and fetches the token's embedding (KV caches are kept)
     int step();                             // enqueues one decode step; the next token replaces the current one
@@ -98,6 +103,7 @@ private:
     unsigned long long attn_ws_bytes_ = 0;
     bool exact_attention_ = false;
     bool qk_norm_ = true;
+    bool tied_lm_head_ = false;
     int* d_state_ = nullptr;    // [0] token, [1] position
 };
 

@@ -70,6 +70,8 @@ class HostLibrary:
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
         L.cccc_decode_set_qk_norm.restype = None; L.cccc_decode_set_qk_norm.argtypes = [vp, i32]
         L.cccc_decode_qk_norm.restype = i32; L.cccc_decode_qk_norm.argtypes = [vp]
+        L.cccc_decode_set_tied_lm_head.restype = None; L.cccc_decode_set_tied_lm_head.argtypes = [vp, i32]
+        L.cccc_decode_tied_lm_head.restype = i32; L.cccc_decode_tied_lm_head.argtypes = [vp]
         L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         self.c = L
@@ -267,8 +269,10 @@ class DecodeModel:
                 self.set_block_scales(li, name, value[1])
             else:
                 self.set_tensor(li, name, value, fp8_dtype if name in QUANTIZED else 3)
+        self.set_tied_lm_head("lm_head" not in model)
         for name in GLOBAL_TENSORS:
-            put(0, name, model[name])
+            if name in model:
+                put(0, name, model[name])
         self.set_qk_norm(all("q_norm" in L for L in model["layers"]))
         for li, L in enumerate(model["layers"]):
             for name in LAYER_TENSORS:
@@ -295,6 +299,14 @@ class DecodeModel:
     def set_qk_norm(self, on: bool) -> None:
         """Per-head RMSNorm of q and k in front of the rotation (Qwen3: on, the default; Llama-3.1: off)."""
         self.lib.c.cccc_decode_set_qk_norm(self.handle, 1 if on else 0)
+
+    def set_tied_lm_head(self, tied: bool) -> None:
+        """Tied embeddings: the head reads the BF16 embedding table, no separate lm_head is stored."""
+        self.lib.c.cccc_decode_set_tied_lm_head(self.handle, 1 if tied else 0)
+
+    @property
+    def tied_lm_head(self) -> bool:
+        return self.lib.c.cccc_decode_tied_lm_head(self.handle) != 0
 
     @property
     def qk_norm(self) -> bool:

@@ -174,7 +174,9 @@ C_EXPORT int hip_embed_fwd(int type, const void* ids, const void* W, void* Y, in
  * (cccc-cuda/cuda_functions.cu:2926-2939); w_scale is ignored for them. */
 typedef struct hip_fused_linear
 {
-    int w_type;              /* 4 (FP8_E4M3), 5 (FP8_E5M2) or 6 (FP4_E2M1 with block scales) */
+    int w_type;              /* 4 (FP8_E4M3), 5 (FP8_E5M2), 6 (FP4_E2M1 with block scales), or 3 (BF16: a weight the
+                              * reference leaves unquantized -- a tied lm_head is the embedding table, cccc/Net.cpp:1158-1190;
+                              * w_scale must be 1) */
     int K;
     int n_segments;          /* 1..3; 2 when pair != 0 */
     int pair;                /* 1: SwiGLU pair of W[0] (gate) and W[1] (up), both n_out[0] rows, into Y[0] */

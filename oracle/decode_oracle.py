@@ -129,8 +129,10 @@ def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, pos: int,
 
 
 def dequant_linear(W) -> np.ndarray:
-    """BF16 bits [n_out, K] of a linear weight of the model dict: uint8 E5M2 codes [n_out, K], or a
-    (packed FP4 nibbles [n_out, K / 2], E4M3 block scales [n_out, K / 16]) pair."""
+    """BF16 bits [n_out, K] of a linear weight of the model dict: uint8 E5M2 codes [n_out, K], a
+    (packed FP4 nibbles [n_out, K / 2], E4M3 block scales [n_out, K / 16]) pair, or uint16 BF16 bits as they are."""
+    if not isinstance(W, tuple) and W.dtype == np.uint16:
+        return W                                            # already BF16 bits: a weight the reference leaves unquantized
     if isinstance(W, tuple):
         nib, sc = W
         n_out, K = nib.shape[0], nib.shape[1] * 2
@@ -138,7 +140,7 @@ def dequant_linear(W) -> np.ndarray:
     return o.dequant_fp8_to_bf16(W, o.E5M2).reshape(W.shape)
 
 
-def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2", qk_norm: bool = True):
+def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2", qk_norm: bool = True, tied: bool = False):
     """Random-init model: linears from N(0, 0.02) as FP8_E5M2 codes (round to nearest) or, fmt = "fp4_e2m1", as the
     converter's FP4 block-scale packing (blocks of 16); BF16 norms near 1, BF16 embedding N(0, 1).
     qk_norm = False: no per-head norm weights (has_qknorm = False in scripts/convert_weights.py:488-530, Llama-style)."""
@@ -166,6 +168,8 @@ def make_model(cfg: DecodeConfig, seed: int = 0, fmt: str = "fp8_e5m2", qk_norm:
     if not qk_norm:
         for L in model["layers"]:
             del L["q_norm"], L["k_norm"]
+    if tied:                                                # tie_word_embeddings: no separate head (scripts/convert_weights.py:230-260)
+        del model["lm_head"]
     return model
 
 
@@ -213,8 +217,10 @@ class DecodeOracle:
                 if li == 0:
                     trace.update(xn=xn, q=q.copy(), att=att.copy(), r1=r1, gated=gated)
         xf = rms_norm(x, f(self.model["rms_final"]), c.eps)
+        # tied embeddings (no "lm_head" in the model): the head multiplies by the BF16 embedding table (cccc/Net.cpp:1158-1190)
+        head = "lm_head" if "lm_head" in self.model else "emb"
         if logit_rows is not None:
-            logits = linear(dequant_linear(self.model["lm_head"][np.asarray(logit_rows)]), xf)
+            logits = linear(dequant_linear(self.model[head][np.asarray(logit_rows)]), xf)
             return logits, int(np.asarray(logit_rows)[int(np.argmax(logits))])
-        logits = linear(self.deq(None, "lm_head"), xf)
+        logits = linear(self.deq(None, head), xf)
         return logits, int(np.argmax(logits))

@@ -620,6 +620,102 @@ def test_decode_steps_of_a_model_without_qk_norm(gpu, pkg, oracle, dec, fmt, exa
     assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
 
 
+@pytest.mark.parametrize("K,n_out", [(2048, 512), (1520, 37), (272, 70000), (4096, 1000)])
+def test_fused_linear_on_an_unquantized_bf16_weight(gpu, pkg, oracle, dec, K, n_out):
+    """w_type 3: a weight the reference leaves in BF16 (a tied lm_head is the embedding table, cccc/Net.cpp:1158-1190).
+    Norm in front, plain, with a residual, the greedy candidates of a tall weight, and three segments; a one-hot
+    activation returns the weight's own column bit for bit.  A per-tensor scale is refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(K + n_out)
+    x = oracle.f32_to_bf16(rng.standard_normal(K).astype(np.float32))
+    nw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    W = oracle.f32_to_bf16((rng.standard_normal((n_out, K)) * 0.05).astype(np.float32))
+    xd, nwd, wd = to_dev(torch, dev, x), to_dev(torch, dev, nw), to_dev(torch, dev, W)
+    xn = dec.rms_norm(dec.f(x), dec.f(nw), 1e-6)
+    # norm in front + candidates
+    ws_bytes = lib.c.hip_argmax_workspace_bytes(n_out)
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    y = torch.zeros(n_out + 8, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(BF16, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(), norm_weight=nwd.data_ptr(), norm_eps=1e-6,
+                                   argmax_workspace=ws.data_ptr())
+    assert lib.quant_linear_fused(d) == 0 and lib.last_kernel() == "gemv_fused_bf16"
+    out = from_dev(y, np.uint16)
+    assert not out[n_out:].any()
+    want = dec.linear(W, xn)
+    assert ulp_close(out[:n_out], want, ulps=1.0, floor=2e-5).all()
+    idx = torch.zeros(2, dtype=torch.int32, device=dev)
+    assert lib.c.hip_argmax_pick_embed_bf16(ctypes.c_void_p(ws.data_ptr()), n_out, ctypes.c_void_p(idx.data_ptr()), None, None, None, 0, 0) == 0
+    got = dec.f(out[:n_out])
+    assert int(idx[0].item()) == int(np.flatnonzero(got == got.max())[0])
+    # plain + residual
+    res = oracle.f32_to_bf16(rng.standard_normal(n_out).astype(np.float32))
+    rd = to_dev(torch, dev, res)
+    y = torch.zeros(n_out, dtype=torch.int16, device=dev)
+    d = pkg.capi.make_fused_linear(BF16, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(), residual=rd.data_ptr())
+    assert lib.quant_linear_fused(d) == 0
+    assert ulp_close(from_dev(y, np.uint16), dec.r(dec.linear(W, dec.f(x)) + dec.f(res)), ulps=1.0, floor=2e-5).all()
+    # one-hot activations: y = W[:, k] exactly
+    for k in (0, 7, K // 2 + 3, K - 1):
+        e = np.zeros(K, dtype=np.uint16)
+        e[k] = 0x3F80
+        ed = to_dev(torch, dev, e)
+        y = torch.zeros(n_out, dtype=torch.int16, device=dev)
+        d = pkg.capi.make_fused_linear(BF16, K, [wd.data_ptr()], [n_out], [y.data_ptr()], ed.data_ptr())
+        assert lib.quant_linear_fused(d) == 0
+        assert np.array_equal(from_dev(y, np.uint16), W[:, k]), k
+    if n_out >= 96:
+        # three segments of one weight's rows
+        cuts = (0, n_out // 2, n_out // 2 + 33, n_out)
+        ys = [torch.zeros(cuts[i + 1] - cuts[i], dtype=torch.int16, device=dev) for i in range(3)]
+        d = pkg.capi.make_fused_linear(BF16, K, [wd.data_ptr() + cuts[i] * K * 2 for i in range(3)], [cuts[i + 1] - cuts[i] for i in range(3)],
+                                       [t.data_ptr() for t in ys], xd.data_ptr(), norm_weight=nwd.data_ptr(), norm_eps=1e-6)
+        # (segment starts are whole rows of K * 2 bytes: 16-byte aligned because K is a multiple of 16)
+        assert lib.quant_linear_fused(d) == 0
+        assert ulp_close(np.concatenate([from_dev(t, np.uint16) for t in ys]), want, ulps=1.0, floor=2e-5).all()
+    bad = pkg.capi.make_fused_linear(BF16, K, [wd.data_ptr()], [n_out], [y.data_ptr()], xd.data_ptr(), scales=[0.5])
+    assert lib.quant_linear_fused(bad) == -1
+
+
+def test_decode_steps_with_tied_embeddings(gpu, pkg, oracle, dec):
+    """tie_word_embeddings (Hy-MT2, small Qwen3 models): no separate head -- the logits are the BF16 embedding table times the
+    normalised state, as in the reference, which never quantizes an EMBED table (cccc/Net.cpp:1158-1190)."""
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=32)
+    weights = dec.make_model(cfg, 43, tied=True)
+    assert "lm_head" not in weights
+    model = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    model.load(weights)
+    assert model.tied_lm_head
+    orc = dec.DecodeOracle(cfg, weights)
+    token = 9
+    for pos in range(8):
+        model.reset(token, pos)
+        got_token = model.step()
+        want_logits, want_token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        top2 = np.sort(want_logits)[-2:]
+        if top2[1] - top2[0] > 2 * np.abs(got - want_logits).max():
+            assert got_token == want_token, pos
+        token = want_token
+    model.reset(3, 0)
+    eager = [model.step() for _ in range(6)]
+    logits_eager = model.logits().copy()
+    model.reset(3, 0)
+    assert model.run(6, True) > 0 and model.token == eager[-1] and np.array_equal(model.logits(), logits_eager)
+    # an untied head of the same values quantized to FP8 answers differently: the tied route really reads the BF16 table
+    untied = dict(weights)
+    untied["lm_head"] = oracle.encode_e5m2_rne(dec.f(weights["emb"]))
+    other = pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv)
+    other.load(untied)
+    assert not other.tied_lm_head
+    other.reset(3, 0)
+    model.reset(3, 0)
+    other.step(); model.step()
+    assert not np.array_equal(other.logits(), model.logits())
+
+
 @pytest.mark.parametrize("n_out,K,fmt", [(300, 1024, "e5m2"), (5000, 2048, "e5m2"), (70000, 1024, "e5m2 tiled"), (151936, 256, "e5m2 tiled"),
                                          (4100, 2048, "fp4"), (66000, 512, "fp4")])
 def test_greedy_pick_from_the_linear_epilogue(gpu, pkg, oracle, n_out, K, fmt):

@@ -454,3 +454,38 @@ def test_a_file_without_qk_norm_weights_loads_as_a_model_without_them(tmp_path, 
     assert not any("norm_" in k and ("qnorm" in k or "knorm" in k) for k in keys)
     for key in weight_file.read_index(path)[0]:
         assert weight_file.read_entry(again, key) == weight_file.read_entry(path, key), key
+
+
+def test_a_file_without_lm_head_loads_with_tied_embeddings(tmp_path, gpu, pkg, host, oracle, dec):
+    """tie_word_embeddings: the converter writes no W_lm_head (scripts/convert_weights.py:256-260).  The model then multiplies
+    by the BF16 embedding table (cccc/Net.cpp:1158-1190 keeps EMBED tables unquantized), steps as the same tensors set
+    directly, and is saved back without a head entry."""
+    cfg = dec.DecodeConfig(layers=1, hidden=256, n_q=4, n_kv=2, inter=512, vocab=400, t_kv=16)
+    weights = dec.make_model(cfg, 47, tied=True)
+    names = {"rms_attn": "W_rms_attn", "wq": "W_q", "wk": "W_k", "wv": "W_v", "q_norm": "W_qnorm", "k_norm": "W_knorm", "wo": "W_o",
+             "rms_ffn": "W_rms_ffn", "w_gate": "W_gate", "w_up": "W_up", "w_down": "W_down"}
+    w = weight_file.BinWriter()
+    w.add("data_type", b"fp8_e5m2")
+    w.add("named_weights", b"1")
+    w.add("weight_bf16_W_emb", weights["emb"])
+    w.add("weight_bf16_W_rms_final", weights["rms_final"])
+    for short, value in weights["layers"][0].items():
+        w.add(("weight_fp8_e5m2_" if value.dtype == np.uint8 else "weight_bf16_") + f"{names[short]}_0", value)
+    path = tmp_path / "tied.bin"
+    w.save(path)
+    a, b = make_model(pkg, host, cfg), make_model(pkg, host, cfg)
+    a.load(weights)
+    assert not b.tied_lm_head
+    b.load_named(pkg.host_api.WeightFile(host, path))
+    assert a.tied_lm_head and b.tied_lm_head
+    for m in (a, b):
+        m.reset(7, 0)
+    for _ in range(5):
+        assert a.step() == b.step()
+    assert np.array_equal(a.logits(), b.logits())
+    again = tmp_path / "tied_again.bin"
+    b.save_named(again)
+    keys = weight_file.read_index(again)[0]
+    assert not any("W_lm_head" in k for k in keys)
+    for key in weight_file.read_index(path)[0]:
+        assert weight_file.read_entry(again, key) == weight_file.read_entry(path, key), key
