@@ -65,6 +65,10 @@ EXPORTS = (
     "hip_attention_decode_workspace_bytes",
     "hip_attention_decode_fused_bf16",
     "hip_attention_decode_exact_bf16",
+    "hip_qk_norm_rope_kv_rows_bf16",
+    "hip_attention_prefill_bf16",
+    "hip_add_bf16",
+    "hip_swiglu_bf16",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_argmax_pick_embed_bf16",
@@ -133,6 +137,14 @@ class QuantLibrary:
         L.hip_attention_decode_fused_bf16.argtypes = [vp] * 11 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp, f32]
         L.hip_attention_decode_exact_bf16.restype = i32
         L.hip_attention_decode_exact_bf16.argtypes = [vp] * 11 + [ctypes.c_ulonglong, i32, i32, i32, i32, vp, f32]
+        L.hip_qk_norm_rope_kv_rows_bf16.restype = i32
+        L.hip_qk_norm_rope_kv_rows_bf16.argtypes = [vp] * 10 + [i32, i32, i32, i32, i32, i32, f32]
+        L.hip_attention_prefill_bf16.restype = i32
+        L.hip_attention_prefill_bf16.argtypes = [vp] * 4 + [i32, i32, i32, i32, i32, i32]
+        L.hip_add_bf16.restype = i32
+        L.hip_add_bf16.argtypes = [vp, vp, vp, ctypes.c_ulonglong]
+        L.hip_swiglu_bf16.restype = i32
+        L.hip_swiglu_bf16.argtypes = [vp, vp, vp, ctypes.c_ulonglong]
         L.hip_attention_decode_workspace_bytes.restype = ctypes.c_ulonglong
         L.hip_attention_decode_workspace_bytes.argtypes = [i32, i32, i32]
         L.hip_argmax_workspace_bytes.restype = ctypes.c_ulonglong

@@ -244,6 +244,35 @@ C_EXPORT int hip_attention_decode_exact_bf16(const void* q, const void* k, const
                                              int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
                                              const void* d_pos, float epsilon);
 
+/*
+ * The same neighbours for a whole prompt: T tokens at positions pos0 .. pos0 + T - 1 in one pass (what the reference's graph
+ * does when cccc-llm feeds it T tokens at once, cccc-llm/cccc-llm.cpp:589-618), between hip_quant_gemm calls with T columns.
+ * Activations are token-major BF16 ([T][features], i.e. the column-major [features x T] hip_quant_gemm writes).
+ */
+
+/* Per-head RMSNorm (NULL, NULL: none) and RoPE of q [T][n_q_heads][128] and k [T][n_kv_heads][128] at table rows
+ * pos0 + t; q_out as q; k and v [T][n_kv_heads][128] go to rows pos0 + t of the caches ([kv_head][t_kv][128]). */
+C_EXPORT int hip_qk_norm_rope_kv_rows_bf16(const void* q, const void* k, const void* v,
+                                           const void* q_norm_w, const void* k_norm_w,
+                                           const void* cos_tab, const void* sin_tab,
+                                           void* q_out, void* k_cache, void* v_cache,
+                                           int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                           int n_tokens, int pos0, float epsilon);
+
+/* Causal GQA attention of the T rotated queries q [T][n_q_heads][128] over cache rows 0 .. pos0 + t (rows pos0 .. pos0 + T - 1
+ * already appended): scores rounded to BF16, keys past the token's position masked, FP32 softmax over the row, BF16
+ * probabilities, y [T][n_q_heads][128] = bf16(V p) -- the rounding points of cccc/MatrixEx.cpp:3018-3104.  On the matrix
+ * cores; no workspace.  n_q_heads / n_kv_heads must be 1, 2 or 4. */
+C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, void* y,
+                                        int n_q_heads, int n_kv_heads, int head_dim, int t_kv,
+                                        int n_tokens, int pos0);
+
+/* y = bf16(a + b) and y = bf16(bf16(gate * bf16(sigmoid(gate))) * up) over n BF16 elements (n % 8 == 0, 16-byte aligned):
+ * the residual add and the SwiGLU product with the reference's roundings (cccc-hip/hip_functions.cpp:895-908, :722-732,
+ * :953-966; cccc/MatrixEx.cpp:756-762). */
+C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
+C_EXPORT int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n);
+
 /* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
 C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);
 

@@ -1,0 +1,113 @@
+"""Prompt-phase neighbours (T tokens at once) against the CPU oracle of the one-token step, through the C-ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import from_dev, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dec():
+    from oracle import decode_oracle
+    return decode_oracle
+
+
+def ulp_close(got_bits, want_vals, ulps=1.0, floor=1e-6):
+    got = (got_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    want = np.asarray(want_vals, dtype=np.float64)
+    tol = ulps * np.maximum(np.abs(want), 2.0 ** -120) * 2.0 ** -8 + floor
+    return np.abs(got - want) <= tol
+
+
+ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+
+
+@pytest.mark.parametrize("n_q,n_kv,normed", [(4, 2, True), (8, 2, True), (2, 2, False)])
+def test_rows_norm_rope_append_equals_the_one_token_kernel(gpu, oracle, dec, n_q, n_kv, normed):
+    """T tokens through hip_qk_norm_rope_kv_rows_bf16 leave the bytes T calls of hip_qk_norm_rope_kv_bf16 leave."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(3)
+    t_kv, T, pos0 = 96, 37, 11
+    cfg = dec.DecodeConfig(n_q=n_q, n_kv=n_kv, t_kv=t_kv)
+    cos, sin = dec.rope_tables(cfg)
+    q = oracle.f32_to_bf16((2 * rng.standard_normal((T, n_q, 128))).astype(np.float32))
+    k = oracle.f32_to_bf16((2 * rng.standard_normal((T, n_kv, 128))).astype(np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal((T, n_kv, 128)).astype(np.float32))
+    qw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(128)).astype(np.float32))
+    kw = oracle.f32_to_bf16((1 + 0.1 * rng.standard_normal(128)).astype(np.float32))
+    qd, kd, vd, qwd, kwd, cd, sd = (to_dev(torch, dev, a) for a in (q, k, v, qw, kw, cos, sin))
+    nq_w, nk_w = (ptr(qwd), ptr(kwd)) if normed else (ctypes.c_void_p(0), ctypes.c_void_p(0))
+    base = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    kc, vc = to_dev(torch, dev, base), to_dev(torch, dev, base[::-1].copy())
+    q_out = torch.zeros(T * n_q * 128, dtype=torch.int16, device=dev)
+    assert lib.c.hip_qk_norm_rope_kv_rows_bf16(ptr(qd), ptr(kd), ptr(vd), nq_w, nk_w, ptr(cd), ptr(sd), ptr(q_out), ptr(kc), ptr(vc),
+                                               n_q, n_kv, 128, t_kv, T, pos0, ctypes.c_float(1e-6)) == 0
+    kc2, vc2 = to_dev(torch, dev, base), to_dev(torch, dev, base[::-1].copy())
+    q_ref = np.zeros((T, n_q, 128), dtype=np.uint16)
+    for t in range(T):
+        q1 = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        pd = torch.tensor([pos0 + t], dtype=torch.int32, device=dev)
+        qt, kt, vt = (to_dev(torch, dev, a[t]) for a in (q, k, v))
+        assert lib.c.hip_qk_norm_rope_kv_bf16(ptr(qt), ptr(kt), ptr(vt), nq_w, nk_w, ptr(cd), ptr(sd), ptr(q1), ptr(kc2), ptr(vc2),
+                                              n_q, n_kv, 128, t_kv, ptr(pd), ctypes.c_float(1e-6)) == 0
+        q_ref[t] = from_dev(q1, np.uint16).reshape(n_q, 128)
+    assert np.array_equal(from_dev(q_out, np.uint16).reshape(T, n_q, 128), q_ref)
+    assert np.array_equal(from_dev(kc, np.uint16), from_dev(kc2, np.uint16))
+    assert np.array_equal(from_dev(vc, np.uint16), from_dev(vc2, np.uint16))
+    # a prompt that would run past the cache is refused
+    assert lib.c.hip_qk_norm_rope_kv_rows_bf16(ptr(qd), ptr(kd), ptr(vd), nq_w, nk_w, ptr(cd), ptr(sd), ptr(q_out), ptr(kc), ptr(vc),
+                                               n_q, n_kv, 128, t_kv, T, t_kv - T + 1, ctypes.c_float(1e-6)) == -1
+
+
+@pytest.mark.parametrize("n_q,n_kv,t_kv,T,pos0", [(4, 2, 200, 1, 0), (4, 2, 200, 5, 0), (4, 2, 200, 16, 3), (8, 2, 200, 17, 0), (8, 2, 300, 100, 70),
+                                                     (2, 2, 200, 64, 64), (8, 2, 1024, 130, 800), (2, 1, 128, 33, 95)])
+def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n_q, n_kv, t_kv, T, pos0):
+    """Every token of the prompt attends to the cache rows up to its own position: the oracle's one-token attention,
+    token by token, on the same caches.  Rows past the prompt hold NaN patterns and must not leak."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(T + pos0)
+    q = oracle.f32_to_bf16(rng.standard_normal((T, n_q, 128)).astype(np.float32))
+    kc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    vc = oracle.f32_to_bf16(rng.standard_normal((n_kv, t_kv, 128)).astype(np.float32))
+    kc[:, pos0 + T:] = 0x7FC1
+    vc[:, pos0 + T:] = 0xFFFF
+    qd, kd, vd = to_dev(torch, dev, q), to_dev(torch, dev, kc), to_dev(torch, dev, vc)
+    y = torch.zeros(T * n_q * 128 + 64, dtype=torch.int16, device=dev)
+    assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), n_q, n_kv, 128, t_kv, T, pos0) == 0
+    out = from_dev(y, np.uint16)
+    assert not out[T * n_q * 128:].any()
+    got = out[:T * n_q * 128].reshape(T, n_q, 128)
+    kf, vf = dec.f(kc), dec.f(vc)
+    kf[:, pos0 + T:], vf[:, pos0 + T:] = 0.0, 0.0               # masked in the oracle too; NaN * 0 would poison its matrix products
+    for t in range(T):
+        want = dec.attention(dec.f(q[t]), kf, vf, pos0 + t, n_q, n_kv)
+        assert np.isfinite(dec.f(got[t])).all(), t
+        assert ulp_close(got[t], want, ulps=2.0, floor=2e-3 * np.abs(want).max()).all(), t
+        assert np.linalg.norm(dec.f(got[t]) - want) <= 4e-3 * np.linalg.norm(want), t
+    assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), n_q, n_kv, 128, t_kv, T, t_kv - T + 1) == -1
+    assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), 3 * n_kv, n_kv, 128, t_kv, T, pos0) == -1
+
+
+def test_residual_add_and_swiglu_rows(gpu, oracle, dec):
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(9)
+    n = 8 * 4099
+    a = oracle.f32_to_bf16((3 * rng.standard_normal(n)).astype(np.float32))
+    b = oracle.f32_to_bf16((3 * rng.standard_normal(n)).astype(np.float32))
+    a[:4] = (0x7F80, 0xFF80, 0x0000, 0x8000)                    # +-inf and zeros ride along
+    ad, bd = to_dev(torch, dev, a), to_dev(torch, dev, b)
+    y = torch.zeros(n, dtype=torch.int16, device=dev)
+    assert lib.c.hip_add_bf16(ptr(ad), ptr(bd), ptr(y), n) == 0
+    with np.errstate(invalid="ignore"):
+        want = oracle.f32_to_bf16(dec.f(a) + dec.f(b))
+    assert np.array_equal(from_dev(y, np.uint16), want)
+    assert lib.c.hip_swiglu_bf16(ptr(ad), ptr(bd), ptr(y), n) == 0
+    got = from_dev(y, np.uint16)
+    want = dec.silu_mul(dec.f(a[4:]), dec.f(b[4:]))
+    # expf on the device and in numpy may differ in the last bit: one BF16 ulp at the two roundings behind it
+    assert ulp_close(got[4:], want, ulps=3.0, floor=1e-30).all()
+    assert (got[4:] == oracle.f32_to_bf16(want)).mean() > 0.99
+    assert lib.c.hip_add_bf16(ptr(ad), ptr(bd), ptr(y), n - 1) == -1
