@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 namespace cccc
 {
@@ -372,17 +373,98 @@ int DecodeModel::step()
             rc = hip_quant_linear_fused(&dn);
         }
     }
-    if (rc == 0)
-    {
-        hip_fused_linear head = linear_desc(tied_lm_head_ ? *emb_ : *lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
-        head.norm_weight = rms_final_->data();
-        head.norm_eps = c.eps;
-        head.argmax_workspace = argmax_ws_->data();        // the launch leaves the greedy candidates of its logits
-        rc = hip_quant_linear_fused(&head);
-    }
+    return rc == 0 ? head() : rc;
+}
+
+int DecodeModel::head()
+{
+    const DecodeConfig& c = cfg_;
+    hip_fused_linear head = linear_desc(tied_lm_head_ ? *emb_ : *lm_head_, c.vocab, c.hidden, x_->data(), logits_->data());
+    head.norm_weight = rms_final_->data();
+    head.norm_eps = c.eps;
+    head.argmax_workspace = argmax_ws_->data();            // the launch leaves the greedy candidates of its logits
+    int rc = hip_quant_linear_fused(&head);
     // pick, advance the position, and fetch the next step's embedding row: one launch
     if (rc == 0) { rc = hip_argmax_pick_embed_bf16(argmax_ws_->data(), (unsigned)c.vocab, d_state_, d_state_ + 1, emb_->data(), x_->data(), c.hidden, c.vocab); }
     return rc;
+}
+
+int DecodeModel::prefill(const int* tokens, int n_tokens, int pos0)
+{
+    constexpr int kPiece = 2048;
+    if (!tokens || n_tokens <= 0 || pos0 < 0 || (long long)pos0 + n_tokens > cfg_.t_kv) { return -1; }
+    for (int i = 0; i < n_tokens; i++)
+    {
+        if (tokens[i] < 0 || tokens[i] >= cfg_.vocab) { return -1; }
+    }
+    gpu_->setAsCurrent();
+    int rc = 0;
+    for (int t0 = 0; t0 < n_tokens && rc == 0; t0 += kPiece)
+    {
+        const int n = n_tokens - t0 < kPiece ? n_tokens - t0 : kPiece;
+        rc = prefillPiece(tokens + t0, n, pos0 + t0, t0 + n == n_tokens);
+    }
+    return rc;
+}
+
+int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
+{
+    const DecodeConfig& c = cfg_;
+    const int q_out = c.n_q * c.head_dim, kv_out = c.n_kv * c.head_dim;
+    if (pf_.tokens < n)
+    {
+        pf_.tokens = n;
+        pf_.ids = make(n, 1, FLOAT, gpu_);
+        for (auto* m : { &pf_.x, &pf_.xn, &pf_.o, &pf_.r1 }) { *m = make(c.hidden, n, BFLOAT16, gpu_); }
+        for (auto* m : { &pf_.q, &pf_.q_rot, &pf_.att }) { *m = make(q_out, n, BFLOAT16, gpu_); }
+        for (auto* m : { &pf_.k, &pf_.v }) { *m = make(kv_out, n, BFLOAT16, gpu_); }
+        for (auto* m : { &pf_.gate, &pf_.up, &pf_.gated }) { *m = make(c.inter, n, BFLOAT16, gpu_); }
+    }
+    std::vector<float> ids(tokens, tokens + n);
+    if (GpuControl::copyHostToDevice(pf_.ids->data(), ids.data(), (size_t)n * sizeof(float)) != 0) { return 1; }
+    int rc = hip_embed_fwd((int)BFLOAT16, pf_.ids->data(), emb_->data(), pf_.x->data(), c.hidden, n, 1);
+    // y [n][n_out] = x [n][K] W^T: the weight is the A operand, transposed, as cccc's batchedMul passes it (scripts/convert_weights.py:492)
+    auto linear = [&](const Matrix& W, int n_out, int K, const Matrix& x, Matrix& y) {
+        return gpu_->rocblas_->gemm(MATRIX_TRANS, MATRIX_NO_TRANS, n_out, n, K, 1.0f, W.data(), W.getDataType(), K, W.getQuantScale(),
+                                    x.data(), BFLOAT16, K, 1.0f, 0.0f, y.data(), BFLOAT16, n_out, 0.0f,
+                                    W.getDataType() == FP4_E2M1 ? (const uint8_t*)W.getBlockScaleData() : nullptr, nullptr);
+    };
+    auto norm = [&](Matrix& x, Matrix& y, Matrix& w) {
+        return hip_rms_norm_fwd((int)BFLOAT16, x.data(), y.data(), w.data(), nullptr, (unsigned)n, (unsigned)c.hidden, c.eps);
+    };
+    for (int li = 0; li < c.layers && rc == 0; li++)
+    {
+        Layer& L = layers_[li];
+        rc = norm(*pf_.x, *pf_.xn, *L.rms_attn);
+        if (rc == 0) { rc = linear(*L.wq, q_out, c.hidden, *pf_.xn, *pf_.q); }
+        if (rc == 0) { rc = linear(*L.wk, kv_out, c.hidden, *pf_.xn, *pf_.k); }
+        if (rc == 0) { rc = linear(*L.wv, kv_out, c.hidden, *pf_.xn, *pf_.v); }
+        if (rc == 0)
+        {
+            rc = hip_qk_norm_rope_kv_rows_bf16(pf_.q->data(), pf_.k->data(), pf_.v->data(), qk_norm_ ? L.q_norm->data() : nullptr,
+                                               qk_norm_ ? L.k_norm->data() : nullptr, cos_->data(), sin_->data(), pf_.q_rot->data(),
+                                               k_cache_[li]->data(), v_cache_[li]->data(), c.n_q, c.n_kv, c.head_dim, c.t_kv, n, pos0, c.eps);
+        }
+        if (rc == 0)
+        {
+            rc = hip_attention_prefill_bf16(pf_.q_rot->data(), k_cache_[li]->data(), v_cache_[li]->data(), pf_.att->data(),
+                                            c.n_q, c.n_kv, c.head_dim, c.t_kv, n, pos0);
+        }
+        if (rc == 0) { rc = linear(*L.wo, c.hidden, q_out, *pf_.att, *pf_.o); }
+        if (rc == 0) { rc = hip_add_bf16(pf_.x->data(), pf_.o->data(), pf_.r1->data(), (unsigned long long)n * c.hidden); }
+        if (rc == 0) { rc = norm(*pf_.r1, *pf_.xn, *L.rms_ffn); }
+        if (rc == 0) { rc = linear(*L.w_gate, c.inter, c.hidden, *pf_.xn, *pf_.gate); }
+        if (rc == 0) { rc = linear(*L.w_up, c.inter, c.hidden, *pf_.xn, *pf_.up); }
+        if (rc == 0) { rc = hip_swiglu_bf16(pf_.gate->data(), pf_.up->data(), pf_.gated->data(), (unsigned long long)n * c.inter); }
+        if (rc == 0) { rc = linear(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.o); }
+        if (rc == 0) { rc = hip_add_bf16(pf_.r1->data(), pf_.o->data(), pf_.x->data(), (unsigned long long)n * c.hidden); }
+    }
+    if (rc != 0 || !last) { return rc; }
+    // the head runs on the last token's state: its greedy pick becomes the current token at position pos0 + n
+    const int state[2] = { tokens[n - 1], pos0 + n - 1 };
+    if (hipMemcpyAsync(x_->data(), (const char*)pf_.x->data() + (size_t)(n - 1) * c.hidden * 2, (size_t)c.hidden * 2, hipMemcpyDeviceToDevice, nullptr) != hipSuccess) { return 1; }
+    if (GpuControl::copyHostToDevice(d_state_, state, sizeof(state)) != 0) { return 1; }
+    return head();
 }
 
 double DecodeModel::run(int n_steps, int use_graph)

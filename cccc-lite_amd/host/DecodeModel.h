@@ -79,6 +79,13 @@ public:
     bool qkNorm() const { return qk_norm_; }
     int reset(int token, int pos);          // sets the device-side token / position and fetches the token's embedding (KV caches are kept)
     int step();                             // enqueues one decode step; the next token replaces the current one
+    // The prompt phase: n tokens at positions pos0 .. pos0 + n - 1 in one pass per layer -- what the reference's graph does
+    // when cccc-llm feeds it the whole prompt (cccc-llm/cccc-llm.cpp:589-618): the linears through Rocblas::gemm with n
+    // columns (the matrix-core GEMM from 48 tokens on), the per-head norm / RoPE / cache append, the causal attention with
+    // the reference's rounding points, residual adds and the SwiGLU product as row kernels.  Afterwards the caches hold
+    // the prompt, the current token is the greedy pick after its last token and the position is pos0 + n: step() carries
+    // on from there.  Prompts longer than 2048 tokens go through in pieces of 2048.  0 ok, -1 bad arguments.
+    int prefill(const int* tokens, int n_tokens, int pos0);
     // Runs n steps; use_graph: capture one step and replay it.  Returns elapsed ms (events on the launch stream) or < 0.
     double run(int n_steps, int use_graph);
     int currentToken();                     // blocking 4-byte read
@@ -100,6 +107,14 @@ private:
     std::unique_ptr<Matrix> emb_, rms_final_, lm_head_, logits_, cos_, sin_;
     std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
     std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, att_, gated_, attn_ws_, argmax_ws_;
+    // activations of a prompt piece, grown on demand: [tokens][features] BF16, and the token ids as floats (hip_embed_fwd's input)
+    struct PromptBuffers
+    {
+        int tokens = 0;
+        std::unique_ptr<Matrix> ids, x, xn, q, k, v, q_rot, att, o, r1, gate, up, gated;
+    } pf_;
+    int prefillPiece(const int* tokens, int n, int pos0, bool last);
+    int head();                             // final norm + lm_head + greedy pick + next embedding on x_
     unsigned long long attn_ws_bytes_ = 0;
     bool exact_attention_ = false;
     bool qk_norm_ = true;

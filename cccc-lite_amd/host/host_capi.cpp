@@ -223,6 +223,8 @@ int cccc_decode_qk_norm(void* m) { return ((DecodeModel*)m)->qkNorm() ? 1 : 0; }
 void cccc_decode_set_tied_lm_head(void* m, int tied) { ((DecodeModel*)m)->setTiedLmHead(tied != 0); }
 int cccc_decode_tied_lm_head(void* m) { return ((DecodeModel*)m)->tiedLmHead() ? 1 : 0; }
 
+int cccc_decode_prefill(void* m, const int* tokens, int n_tokens, int pos0) { return ((DecodeModel*)m)->prefill(tokens, n_tokens, pos0); }
+
 int cccc_decode_reset(void* m, int token, int pos) { return ((DecodeModel*)m)->reset(token, pos); }
 
 int cccc_decode_step(void* m)

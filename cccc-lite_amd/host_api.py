@@ -68,6 +68,7 @@ class HostLibrary:
         L.cccc_decode_save_named.restype = i32; L.cccc_decode_save_named.argtypes = [vp, ctypes.c_char_p]
         L.cccc_matrix_save_named.restype = i32; L.cccc_matrix_save_named.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
         L.cccc_decode_set_exact_attention.restype = None; L.cccc_decode_set_exact_attention.argtypes = [vp, i32]
+        L.cccc_decode_prefill.restype = i32; L.cccc_decode_prefill.argtypes = [vp, ctypes.POINTER(ctypes.c_int), i32, i32]
         L.cccc_decode_set_qk_norm.restype = None; L.cccc_decode_set_qk_norm.argtypes = [vp, i32]
         L.cccc_decode_qk_norm.restype = i32; L.cccc_decode_qk_norm.argtypes = [vp]
         L.cccc_decode_set_tied_lm_head.restype = None; L.cccc_decode_set_tied_lm_head.argtypes = [vp, i32]
@@ -314,6 +315,15 @@ class DecodeModel:
 
     def reset(self, token: int, pos: int) -> None:
         assert self.lib.c.cccc_decode_reset(self.handle, token, pos) == 0
+
+    def prefill(self, tokens, pos0: int = 0) -> int:
+        """The prompt phase (DecodeModel::prefill): the caches take the prompt at positions pos0 .., the greedy pick after its
+        last token becomes the current token.  Returns that token."""
+        arr = (ctypes.c_int * len(tokens))(*[int(t) for t in tokens])
+        rc = self.lib.c.cccc_decode_prefill(self.handle, arr, len(tokens), pos0)
+        if rc != 0:
+            raise RuntimeError(f"prefill failed: {rc}")
+        return self.token
 
     def step(self) -> int:
         rc = self.lib.c.cccc_decode_step(self.handle)

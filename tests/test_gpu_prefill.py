@@ -111,3 +111,82 @@ def test_residual_add_and_swiglu_rows(gpu, oracle, dec):
     assert ulp_close(got[4:], want, ulps=3.0, floor=1e-30).all()
     assert (got[4:] == oracle.f32_to_bf16(want)).mean() > 0.99
     assert lib.c.hip_add_bf16(ptr(ad), ptr(bd), ptr(y), n - 1) == -1
+
+
+# ------------------------------------------------------------------------------------------ the whole prompt phase
+
+def _fresh(pkg, host, cfg):
+    return pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
+
+
+@pytest.mark.parametrize("variant", ["qwen3 fp8", "llama fp4", "tied fp8"])
+@pytest.mark.parametrize("T", [1, 5, 20, 60])
+def test_prompt_phase_of_the_decode_model_follows_the_oracle(gpu, pkg, oracle, dec, variant, T):
+    """DecodeModel::prefill (linears through the GEMM face with T columns, row kernels between them) against the oracle
+    fed the same prompt token by token: the cache rows of every layer and position, the logits after the last token and
+    the greedy pick; then three decode steps carry on from the prompt and still follow the oracle."""
+    host = pkg.host_api.host()
+    host.init(0)
+    fp4, tied = variant == "llama fp4", variant == "tied fp8"
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=96, theta=5e5 if fp4 else 1e6)
+    weights = dec.make_model(cfg, 53, fmt="fp4_e2m1" if fp4 else "fp8_e5m2", qk_norm=not fp4, tied=tied)
+    model = _fresh(pkg, host, cfg)
+    model.load(weights)
+    model.set_exact_attention(True)
+    rng = np.random.default_rng(T)
+    prompt = [int(t) for t in rng.integers(0, cfg.vocab, size=T)]
+    orc = dec.DecodeOracle(cfg, weights)
+    for pos, tok in enumerate(prompt):
+        want_logits, want_next = orc.step(tok, pos)
+    got_next = model.prefill(prompt)
+    assert model.pos == T
+    for li in range(cfg.layers):
+        for is_v, want_c in ((False, orc.k[li]), (True, orc.v[li])):
+            got_c = dec.f(model.kv(li, is_v)[:, :T])
+            assert np.isfinite(got_c).all()
+            err = np.linalg.norm(got_c - want_c[:, :T]) / np.linalg.norm(want_c[:, :T])
+            assert err <= (2e-3 if li == 0 else 1e-2), (li, is_v, err)
+    got = dec.f(model.logits())
+    assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits)
+    top2 = np.sort(want_logits)[-2:]
+    if top2[1] - top2[0] > 2 * np.abs(got - want_logits).max():
+        assert got_next == want_next
+    token = want_next
+    for pos in range(T, T + 3):
+        model.reset(token, pos)
+        got_token = model.step()
+        want_logits, want_token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        token = want_token
+
+
+def test_prompt_in_pieces_and_bad_arguments(gpu, pkg, oracle, dec):
+    """A prompt fed in two calls (the second at pos0 = length of the first) leaves what one call leaves, up to the
+    summation order of the linears (a piece of 7 tokens takes the GEMV kernels, one of 53 the GEMM); a prompt that does not fit
+    the cache, an empty one and a token outside the vocabulary are refused."""
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=64)
+    weights = dec.make_model(cfg, 59)
+    prompt = [int(t) for t in np.random.default_rng(5).integers(0, cfg.vocab, size=60)]
+    a, b = _fresh(pkg, host, cfg), _fresh(pkg, host, cfg)
+    a.load(weights); b.load(weights)
+    a.prefill(prompt)
+    b.prefill(prompt[:7])
+    b.prefill(prompt[7:], pos0=7)
+    assert a.pos == b.pos == 60
+    for li in range(cfg.layers):
+        for is_v in (False, True):
+            ca, cb = dec.f(a.kv(li, is_v)[:, :60]), dec.f(b.kv(li, is_v)[:, :60])
+            assert np.linalg.norm(ca - cb) <= 1e-2 * np.linalg.norm(ca)
+    la, lb = dec.f(a.logits()), dec.f(b.logits())
+    assert np.linalg.norm(la - lb) <= 1e-2 * np.linalg.norm(la)
+    with pytest.raises(RuntimeError):
+        a.prefill(prompt + [1, 2, 3, 4, 5])                    # 65 positions in a cache of 64
+    with pytest.raises(RuntimeError):
+        a.prefill([])
+    with pytest.raises(RuntimeError):
+        a.prefill([3, cfg.vocab, 4])
+    with pytest.raises(RuntimeError):
+        a.prefill([1, 2], pos0=63)
