@@ -296,6 +296,33 @@ def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool):
     return entry, model
 
 
+def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3):
+    """The prompt phase of the same model (DecodeModel::prefill, positions 0 .. T - 1): every linear is one quantized GEMM
+    with T columns -- BASELINE config 4's kernel on all seven shapes of a layer, on the row-major file bytes (a batch-1
+    DecodeModel keeps no tiled copies) -- with the row kernels and the causal attention between them.  Wall clock around the
+    call, device synchronised on both sides; best of `reps` after one warm-up call (which also allocates the activations)."""
+    import numpy as np
+    t, c = ws.torch, QWEN3_8B
+    lin_elems = c["layers"] * (c["hidden"] * (c["q_out"] + 2 * c["kv_out"]) + c["q_out"] * c["hidden"] + 3 * c["hidden"] * c["inter"])
+    out = []
+    for T in token_counts:
+        prompt = [int(v) for v in np.random.default_rng(T).integers(0, c["vocab"], size=T)]
+        model.prefill(prompt)
+        best = None
+        for _ in range(reps):
+            t.cuda.synchronize()
+            t0 = time.perf_counter()
+            model.prefill(prompt)
+            t.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        # linears 2 T K N each; attention 2 * 2 * 128 * n_q per (token, visible key) pair
+        flops = 2.0 * T * lin_elems + 4.0 * 128 * 32 * c["layers"] * (T * (T + 1) / 2) + 2.0 * c["hidden"] * c["vocab"]
+        out.append({"tokens": T, "ms": round(best * 1e3, 3), "tok_s": round(T / best, 1), "TFLOPs": round(flops / best * 1e-12, 1),
+                    "frac_of_bf16_mfma_peak": round(flops / best * 1e-12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    return out
+
+
 def decode_step_bytes(ctx_mean: float) -> int:
     """Bytes one decode step must move: every linear weight once, the keys and values of the positions
     attended to, the embedding row, the norm weights and the logits."""
@@ -628,6 +655,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-fp4-step", action="store_true", help="skip the Llama-3.1-8B-shaped FP4 decode step")
+    ap.add_argument("--no-prompt", action="store_true", help="skip the prompt-phase (prefill) measurement of the decode model")
     ap.add_argument("--sweep-tokens", default="1,4,16", help="token counts of the per-shape GEMV sweep")
     ap.add_argument("--no-baselines", action="store_true", help="skip the same-GPU BF16 baselines of the decode step")
     ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
@@ -698,6 +726,11 @@ def main():
         K, N, M = 4096, 2 * 12288, 1
         dom_us = ws.bench.gate_up_us(model, 10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
+        if not args.no_prompt:
+            extra["prompt_phase"] = {"workload": "prompt phase of the same Qwen3-8B W8A16 model from an empty cache (DecodeModel::prefill): per layer seven "
+                                                 "quantized GEMMs with T columns on the row-major weights, RMSNorm / RoPE / append rows, causal attention, "
+                                                 "residual adds, SwiGLU; then the head on the last token",
+                                     "cases": prompt_phase(ws, model)}
         if not args.no_fp4_step:
             extra["fp4_decode_step"], fp4_model = llama_fp4_decode(ws, args.steps, args.warmup, use_graph)
         if not args.no_sweep:

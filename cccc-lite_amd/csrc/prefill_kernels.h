@@ -48,145 +48,269 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 
 // ------------------------------------------------------------------------------------------
 // Causal GQA attention of T query tokens over cache rows 0 .. pos0 + t, head_dim 128, on the matrix cores, with the
-// reference's rounding points.  Grid (ceil(T / 16), kv heads); a workgroup of four waves owns 16 tokens, wave w the
-// query head kvh * G + w (waves >= G only help to stage V).  Two passes over the keys 0 .. pos0 + (last token of the
-// tile):
-//   pass 1  scores of 16 keys x 16 tokens per v_mfma_f32_16x16x32_bf16 x 4 (key rows straight from the cache as the row
-//           operand, the rotated queries as columns: D lane (token = lane % 16, g = lane / 16) holds keys 4 g .. 4 g + 3),
-//           rounded to BF16, masked, running (max, sum) per lane, merged over the four lane groups at the end;
-//   pass 2  the same scores again, p = bf16(expf(s - max) / sum) -- the probabilities of the whole row, as the reference
+// reference's rounding points.  Grid (ceil(T / 32), kv heads); a workgroup of four waves owns 32 tokens (two 16-token
+// tiles), wave w the query head kvh * G + w (waves >= G only help with the staging).  Keys and values go through LDS in
+// blocks of 64 rows, fetched once per workgroup and pass and shared by the G heads and both token tiles (fetched by every
+// wave for itself they cost four times the cache traffic, which bounded the kernel).  Two passes over the keys
+// 0 .. pos0 + (last token of the workgroup):
+//   pass 1  scores of 16 keys x 16 tokens per v_mfma_f32_16x16x32_bf16 x 4 (key rows as the row operand, the rotated
+//           queries as columns: D lane (token = lane % 16, g = lane / 16) holds keys 4 g .. 4 g + 3), rounded to BF16,
+//           masked, running (max, sum) per lane, merged over the four lane groups at the end;
+//   pass 2  the same scores again, p = bf16(exp(s - max) / sum) -- the probabilities of the whole row, as the reference
 //           rounds them -- and y += P V on the matrix cores: the eight probabilities a lane holds for its token (keys
 //           4 g .. + 3 and 16 + 4 g .. + 3 of a 32-key slab) are its row operand as they are, because a contraction does not
 //           care in which order k is visited when both operands agree; the value operand (column = dim, the same keys)
-//           comes from a transposed copy of the 64-key value block in LDS, shared by the G heads.
+//           comes from a transposed copy of the value block, two keys per dword.
 // Value rows past the last position written so far may hold anything: they are zeroed while staging (0 * NaN is NaN).
-constexpr int PF_KEYS = 64;                 // keys per staged value block
-constexpr int PF_PITCH = 66;                // elements per transposed row: 64 keys + 2 (33 dwords, spreads the rows over the banks)
+constexpr int PF_KEYS = 64;                 // keys per staged block
+constexpr int PF_PITCH = 66;                // elements per transposed value row: 64 keys + 2 (33 dwords: rows spread over the banks)
+constexpr int PF_KPITCH = 136;              // elements per staged key row: 128 dims + 8 (68 dwords: 16 rows x 16 bytes hit 64 distinct banks)
+constexpr int PF_TT = 1;                    // 16-token tiles per workgroup
+
+// expf through the hardware's 2^x (x * log2 e is rounded once more in front of it: a few FP32 ulps, against the BF16
+// rounding that follows every use here)
+__device__ __forceinline__ float pf_exp(float x) { return __expf(x); }
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load in flight (its
+// release fence drains the vector-memory counter on this target), which would cancel the two-blocks-ahead prefetch below:
+// the kernel then pays a trip to memory per block (1.3 us per 64 keys and pass, whatever the arithmetic costs).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int G>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
                                                           uint16_t* __restrict__ y, int n_q, int t_kv, int n_tokens, int pos0, float scale)
 {
+    __shared__ __attribute__((aligned(16))) uint16_t ks[PF_KEYS * PF_KPITCH];   // [key][dim] of the current block
     __shared__ __attribute__((aligned(16))) uint16_t vt[128 * PF_PITCH];        // [dim][key] of the current block
     const int kvh = blockIdx.y;
-    const int t0 = blockIdx.x * 16;
+    const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * (16 * PF_TT);       // the workgroups that see the most keys go first
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 15, g = lane >> 4;
-    const int last_token = min(t0 + 15, n_tokens - 1);
-    const int n_keys = pos0 + last_token + 1;                   // keys this tile can see
+    const int last_token = min(t0 + 16 * PF_TT - 1, n_tokens - 1);
+    const int n_keys = pos0 + last_token + 1;                   // keys this workgroup can see
     const int n_written = pos0 + n_tokens;                      // cache rows holding data
-    const int my_pos = pos0 + min(t0 + j, n_tokens - 1);        // position of this lane's token
+    const int n_blocks = (n_keys + PF_KEYS - 1) / PF_KEYS;
     const bool active = wave < G;
     const uint16_t* kbase = k_cache + (size_t)kvh * t_kv * 128;
     const uint16_t* vbase = v_cache + (size_t)kvh * t_kv * 128;
 
-    // the query operand: token j's head, dims 32 c + 8 g .. + 7
-    u32x4 qf[4];
-    if (active)
+    // the query operands: token tile tt, token j's head, dims 32 c + 8 g .. + 7
+    u32x4 qf[PF_TT][4];
+    int my_pos[PF_TT];
+#pragma unroll
+    for (int tt = 0; tt < PF_TT; tt++)
     {
-        const uint16_t* qrow = q + ((size_t)min(t0 + j, n_tokens - 1) * n_q + kvh * G + wave) * 128 + g * 8;
-#pragma unroll
-        for (int c = 0; c < 4; c++) { qf[c] = *(const u32x4*)(qrow + c * 32); }
-    }
-    // scores of key tile kt (16 keys) against the 16 tokens: lane gets keys kt * 16 + 4 g + v, v = 0..3, of token j
-    auto score_tile = [&](int kt, float (&s)[4]) {
-        const int row = min(kt * 16 + j, t_kv - 1);
-        const uint16_t* krow = kbase + (size_t)row * 128 + g * 8;
-        f32x4 acc = { 0.0f, 0.0f, 0.0f, 0.0f };
-#pragma unroll
-        for (int c = 0; c < 4; c++)
+        const int t = min(t0 + tt * 16 + j, n_tokens - 1);
+        my_pos[tt] = pos0 + t;
+        if (active)
         {
-            const u32x4 kf = *(const u32x4*)(krow + c * 32);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[c]), acc, 0, 0, 0);
+            const uint16_t* qrow = q + ((size_t)t * n_q + kvh * G + wave) * 128 + g * 8;
+#pragma unroll
+            for (int c = 0; c < 4; c++) { qf[tt][c] = *(const u32x4*)(qrow + c * 32); }
         }
+    }
+    // staging: thread -> rows and 16-byte pieces of a 64-row block (item = thread + 256 i: key pair 2 p, 2 p + 1 with
+    // p = item % 32, dims 8 c .. + 7 with c = item / 32); raw[2 i], raw[2 i + 1] are the two rows' pieces
+    auto load_rows = [&](const uint16_t* base, int b, int limit, u32x4 (&raw)[4]) {
 #pragma unroll
-        for (int v = 0; v < 4; v++)
+        for (int i = 0; i < 2; i++)
         {
-            const int key = kt * 16 + 4 * g + v;
-            s[v] = key <= my_pos ? bf16_round(scale * acc[v]) : -INFINITY;
+            const int item = threadIdx.x + i * 256;
+            const int row = b * PF_KEYS + 2 * (item & 31);
+            // no predicate on the loads (rows past the limit re-read its last row and are zeroed when stored), so that
+            // the number of requests in flight is known at every wait
+            raw[2 * i] = *(const u32x4*)(base + (size_t)min(row, limit - 1) * 128 + (item >> 5) * 8);
+            raw[2 * i + 1] = *(const u32x4*)(base + (size_t)min(row + 1, limit - 1) * 128 + (item >> 5) * 8);
         }
     };
-
-    // ---- pass 1: row maximum and sum of expf(s - max)
-    float m = -INFINITY, l = 0.0f;
-    if (active)
-    {
-        const int n_kt = (n_keys + 15) / 16;
-        for (int kt = 0; kt < n_kt; kt++)
-        {
-            float s[4];
-            score_tile(kt, s);
-            const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-            if (tm > m)
-            {
-                l *= expf(m - tm);                              // m = -inf: l is 0 and stays 0
-                m = tm;
-            }
-            if (m > -INFINITY)
-            {
+    const u32x4 zero4 = { 0u, 0u, 0u, 0u };
+    auto store_keys = [&](int b, int limit, const u32x4 (&raw)[4]) {
 #pragma unroll
-                for (int v = 0; v < 4; v++) { l += expf(s[v] - m); }
+        for (int i = 0; i < 2; i++)
+        {
+            const int item = threadIdx.x + i * 256;
+            const int row = b * PF_KEYS + 2 * (item & 31);
+            uint16_t* dst = ks + 2 * (item & 31) * PF_KPITCH + (item >> 5) * 8;
+            *(u32x4*)dst = row < limit ? raw[2 * i] : zero4;
+            *(u32x4*)(dst + PF_KPITCH) = row + 1 < limit ? raw[2 * i + 1] : zero4;
+        }
+    };
+    // transposed store, two keys per dword: dim 8 c + e gets (key 2 p, key 2 p + 1) at dword p of its row
+    auto store_values = [&](int b, int limit, const u32x4 (&raw)[4]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+        {
+            const int item = threadIdx.x + i * 256;
+            const int row = b * PF_KEYS + 2 * (item & 31);
+            uint32_t* dst = (uint32_t*)vt + (item >> 5) * 8 * (PF_PITCH / 2) + (item & 31);
+            const u32x4 lo = row < limit ? raw[2 * i] : zero4, hi = row + 1 < limit ? raw[2 * i + 1] : zero4;
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+            {
+                dst[(2 * d) * (PF_PITCH / 2)] = (lo[d] & 0xFFFFu) | (hi[d] << 16);
+                dst[(2 * d + 1) * (PF_PITCH / 2)] = (lo[d] >> 16) | (hi[d] & 0xFFFF0000u);
             }
         }
+    };
+    // scores of the block's four key tiles (16 keys each) against the token tiles: for tile kt the lane gets keys
+    // kt * 16 + 4 g + v, v = 0..3, of token j.  All sixteen key operands are read first and the products run over the
+    // tiles inside each 32-dim step, so that consecutive matrix-core instructions never wait for each other's sums.
+    auto score_block = [&](int b, bool masked, float (&s)[PF_KEYS / 16][PF_TT][4]) {
+        u32x4 kf[PF_KEYS / 16][4];
+#pragma unroll
+        for (int kt = 0; kt < PF_KEYS / 16; kt++)
+        {
+            const uint16_t* krow = ks + (kt * 16 + j) * PF_KPITCH + g * 8;
+#pragma unroll
+            for (int c = 0; c < 4; c++) { kf[kt][c] = *(const u32x4*)(krow + c * 32); }
+        }
+        f32x4 acc[PF_KEYS / 16][PF_TT];
+#pragma unroll
+        for (int kt = 0; kt < PF_KEYS / 16; kt++)
+#pragma unroll
+            for (int tt = 0; tt < PF_TT; tt++) { acc[kt][tt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int kt = 0; kt < PF_KEYS / 16; kt++)
+#pragma unroll
+                for (int tt = 0; tt < PF_TT; tt++)
+                {
+                    acc[kt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt][c]), __builtin_bit_cast(bf16x8, qf[tt][c]), acc[kt][tt], 0, 0, 0);
+                }
+#pragma unroll
+        for (int kt = 0; kt < PF_KEYS / 16; kt++)
+#pragma unroll
+            for (int tt = 0; tt < PF_TT; tt++)
+            {
+                // rounded to BF16 by the hardware conversion (round to nearest even, as the integer trick rounds finite values)
+                const f32x4 a = acc[kt][tt];
+                const bf16x2 r01 = { (__bf16)(scale * a[0]), (__bf16)(scale * a[1]) }, r23 = { (__bf16)(scale * a[2]), (__bf16)(scale * a[3]) };
+                const uint32_t w01 = __builtin_bit_cast(uint32_t, r01), w23 = __builtin_bit_cast(uint32_t, r23);
+                s[kt][tt][0] = __builtin_bit_cast(float, w01 << 16);
+                s[kt][tt][1] = __builtin_bit_cast(float, w01 & 0xFFFF0000u);
+                s[kt][tt][2] = __builtin_bit_cast(float, w23 << 16);
+                s[kt][tt][3] = __builtin_bit_cast(float, w23 & 0xFFFF0000u);
+                if (masked)                                     // only blocks that reach past the workgroup's first token need the test
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        const int key = b * PF_KEYS + kt * 16 + 4 * g + v;
+                        if (key > my_pos[tt]) { s[kt][tt][v] = -INFINITY; }
+                    }
+                }
+            }
+    };
+
+    // ---- pass 1: row maximum and sum of exp(s - max)
+    float m[PF_TT], l[PF_TT];
+#pragma unroll
+    for (int tt = 0; tt < PF_TT; tt++) { m[tt] = -INFINITY; l[tt] = 0.0f; }
+    // rows are requested two blocks ahead of their use (two register sets, alternating): one block of work does not cover
+    // the trip to memory
+    u32x4 kraw[2][4], vraw[2][4];
+    load_rows(kbase, 0, n_written, kraw[0]);
+    load_rows(kbase, min(1, n_blocks - 1), n_written, kraw[1]);
+    auto pass1_block = [&](int b, u32x4 (&kr)[4]) {
+        lds_barrier();                                        // the previous block's reads are done
+        store_keys(b, n_written, kr);
+        load_rows(kbase, min(b + 2, n_blocks - 1), n_written, kr);      // unconditional (clamped): the wait counts stay exact
+        lds_barrier();
+        if (!active) { return; }
+        const bool masked = b * PF_KEYS + PF_KEYS - 1 > pos0 + t0;      // some key of the block lies past the first token's position
+        // all four key tiles of the block at once: sixteen independent scores per lane and token tile keep the matrix cores
+        // and the VALU busy where one tile at a time is a single chain of dependent instructions
+        float s[PF_KEYS / 16][PF_TT][4];
+        score_block(b, masked, s);
+#pragma unroll
+        for (int tt = 0; tt < PF_TT; tt++)
+        {
+            float bm = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < PF_KEYS / 16; kt++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) { bm = fmaxf(bm, s[kt][tt][v]); }
+            if (bm > m[tt])
+            {
+                l[tt] *= pf_exp(m[tt] - bm);                    // m = -inf: l is 0 and stays 0
+                m[tt] = bm;
+            }
+            if (m[tt] > -INFINITY)
+            {
+                float sum = 0.0f;
+#pragma unroll
+                for (int kt = 0; kt < PF_KEYS / 16; kt++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) { sum += pf_exp(s[kt][tt][v] - m[tt]); }
+                l[tt] += sum;
+            }
+        }
+    };
+    for (int b = 0; b < n_blocks; b += 2)
+    {
+        pass1_block(b, kraw[0]);
+        if (b + 1 < n_blocks) { pass1_block(b + 1, kraw[1]); }
+    }
+    float inv[PF_TT];
+#pragma unroll
+    for (int tt = 0; tt < PF_TT; tt++)
+    {
         // merge the four lane groups of a token (lanes j, j + 16, j + 32, j + 48)
 #pragma unroll
         for (int off = 16; off < 64; off <<= 1)
         {
-            const float om = __shfl_xor(m, off), ol = __shfl_xor(l, off);
-            const float nm = fmaxf(m, om);
-            if (nm > -INFINITY) { l = l * expf(m - nm) + ol * expf(om - nm); }
-            m = nm;
+            const float om = __shfl_xor(m[tt], off), ol = __shfl_xor(l[tt], off);
+            const float nm = fmaxf(m[tt], om);
+            if (nm > -INFINITY) { l[tt] = l[tt] * pf_exp(m[tt] - nm) + ol * pf_exp(om - nm); }
+            m[tt] = nm;
         }
+        inv[tt] = l[tt] > 0.0f ? 1.0f / l[tt] : 0.0f;
     }
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
 
     // ---- pass 2: probabilities and P V
-    f32x4 out[8];
+    f32x4 out[PF_TT][8];
 #pragma unroll
-    for (int d = 0; d < 8; d++) { out[d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
-    const int n_blocks = (n_keys + PF_KEYS - 1) / PF_KEYS;
-    for (int b = 0; b < n_blocks; b++)
-    {
-        __syncthreads();                                        // the previous block's value reads are done
-        // stage V^T: thread -> (key = idx / 16, dims 8 (idx % 16) .. + 7), four keys per thread
+    for (int tt = 0; tt < PF_TT; tt++)
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-        {
-            const int idx = threadIdx.x + i * 256;
-            const int key = idx >> 4, dim0 = (idx & 15) * 8;
-            const int row = b * PF_KEYS + key;
-            u32x4 raw = { 0u, 0u, 0u, 0u };
-            if (row < n_written && row < t_kv) { raw = *(const u32x4*)(vbase + (size_t)row * 128 + dim0); }
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-            {
-                vt[(dim0 + 2 * d) * PF_PITCH + key] = (uint16_t)(raw[d] & 0xFFFFu);
-                vt[(dim0 + 2 * d + 1) * PF_PITCH + key] = (uint16_t)(raw[d] >> 16);
-            }
-        }
-        __syncthreads();
-        if (!active) { continue; }
+        for (int d = 0; d < 8; d++) { out[tt][d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+    load_rows(kbase, 0, n_written, kraw[0]);
+    load_rows(vbase, 0, n_written, vraw[0]);
+    load_rows(kbase, min(1, n_blocks - 1), n_written, kraw[1]);
+    load_rows(vbase, min(1, n_blocks - 1), n_written, vraw[1]);
+    auto pass2_block = [&](int b, u32x4 (&kr)[4], u32x4 (&vr)[4]) {
+        lds_barrier();
+        store_keys(b, n_written, kr);
+        store_values(b, n_written, vr);
+        load_rows(kbase, min(b + 2, n_blocks - 1), n_written, kr);
+        load_rows(vbase, min(b + 2, n_blocks - 1), n_written, vr);
+        lds_barrier();
+        if (!active) { return; }
+        const bool masked = b * PF_KEYS + PF_KEYS - 1 > pos0 + t0;
+        float s[PF_KEYS / 16][PF_TT][4];
+        score_block(b, masked, s);
+        // exp(-inf) is 0: a masked key gets probability 0 without a test; the pairs are rounded and packed by one conversion each
+        bf16x8 pa[PF_KEYS / 32][PF_TT];
 #pragma unroll
         for (int slab = 0; slab < PF_KEYS / 32; slab++)
-        {
-            const int key0 = b * PF_KEYS + slab * 32;
-            if (key0 >= n_keys) { break; }
-            float s0[4], s1[4];
-            score_tile(key0 / 16, s0);
-            score_tile(key0 / 16 + 1, s1);
-            uint32_t pw[4];
 #pragma unroll
-            for (int v = 0; v < 2; v++)
+            for (int tt = 0; tt < PF_TT; tt++)
             {
-                const float a0 = s0[2 * v] > -INFINITY ? bf16_round(expf(s0[2 * v] - m) * inv) : 0.0f;
-                const float a1 = s0[2 * v + 1] > -INFINITY ? bf16_round(expf(s0[2 * v + 1] - m) * inv) : 0.0f;
-                const float b0 = s1[2 * v] > -INFINITY ? bf16_round(expf(s1[2 * v] - m) * inv) : 0.0f;
-                const float b1 = s1[2 * v + 1] > -INFINITY ? bf16_round(expf(s1[2 * v + 1] - m) * inv) : 0.0f;
-                pw[v] = (__builtin_bit_cast(uint32_t, a0) >> 16) | (__builtin_bit_cast(uint32_t, a1) & 0xFFFF0000u);
-                pw[2 + v] = (__builtin_bit_cast(uint32_t, b0) >> 16) | (__builtin_bit_cast(uint32_t, b1) & 0xFFFF0000u);
+                uint32_t pw[4];
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+#pragma unroll
+                    for (int v = 0; v < 2; v++)
+                    {
+                        const float* sv = s[2 * slab + h][tt];
+                        const bf16x2 pp = { (__bf16)(pf_exp(sv[2 * v] - m[tt]) * inv[tt]), (__bf16)(pf_exp(sv[2 * v + 1] - m[tt]) * inv[tt]) };
+                        pw[2 * h + v] = __builtin_bit_cast(uint32_t, pp);
+                    }
+                const u32x4 pvec = { pw[0], pw[1], pw[2], pw[3] };      // keys 4 g .. + 3, then 16 + 4 g .. + 3 of the slab
+                pa[slab][tt] = __builtin_bit_cast(bf16x8, pvec);
             }
-            const u32x4 pvec = { pw[0], pw[1], pw[2], pw[3] };  // keys 4 g .. + 3, then 16 + 4 g .. + 3 of the slab
-            const bf16x8 pa = __builtin_bit_cast(bf16x8, pvec);
+#pragma unroll
+        for (int slab = 0; slab < PF_KEYS / 32; slab++)
 #pragma unroll
             for (int d = 0; d < 8; d++)
             {
@@ -195,22 +319,32 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __res
                 const uint32_t v0 = *(const uint32_t*)vrow, v1 = *(const uint32_t*)(vrow + 2);
                 const uint32_t v2 = *(const uint32_t*)(vrow + 16), v3 = *(const uint32_t*)(vrow + 18);
                 const u32x4 vvec = { v0, v1, v2, v3 };
-                out[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8, vvec), out[d], 0, 0, 0);
+#pragma unroll
+                for (int tt = 0; tt < PF_TT; tt++)
+                {
+                    out[tt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[slab][tt], __builtin_bit_cast(bf16x8, vvec), out[tt][d], 0, 0, 0);
+                }
             }
-        }
+    };
+    for (int b = 0; b < n_blocks; b += 2)
+    {
+        pass2_block(b, kraw[0], vraw[0]);
+        if (b + 1 < n_blocks) { pass2_block(b + 1, kraw[1], vraw[1]); }
     }
     if (!active) { return; }
-    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3
+    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3 of its tile
 #pragma unroll
-    for (int d = 0; d < 8; d++)
-    {
+    for (int tt = 0; tt < PF_TT; tt++)
 #pragma unroll
-        for (int v = 0; v < 4; v++)
+        for (int d = 0; d < 8; d++)
         {
-            const int t = t0 + 4 * g + v;
-            if (t < n_tokens) { y[((size_t)t * n_q + kvh * G + wave) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(out[d][v]); }
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+            {
+                const int t = t0 + tt * 16 + 4 * g + v;
+                if (t < n_tokens) { y[((size_t)t * n_q + kvh * G + wave) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(out[tt][d][v]); }
+            }
         }
-    }
 }
 
 // ------------------------------------------------------------------------------------------

@@ -372,3 +372,92 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention, 
         all_logits = dec.f(logits)
         assert got_token == int(np.argmax(all_logits))
         token = got_token
+
+
+# ------------------------------------------------------------------------------------------ prompt phase
+
+@pytest.mark.parametrize("arch", ["qwen3_8b_fp8", "llama31_8b_fp4"])
+def test_prompt_phase_at_full_widths_equals_token_by_token_decoding(gpu, pkg, oracle, dec, arch):
+    """DecodeModel::prefill at the benchmark's widths (two layers): 130 prompt tokens from position 0 in one call against the
+    same tokens fed one at a time through the decode step on the attention route with the reference's rounding points
+    (which the tests above hold against the CPU oracle at these widths).  Both read the same weight bytes; the linears run
+    as GEMMs with 130 columns here and as GEMVs there, so agreement is to summation order: cache rows, last logits,
+    and the greedy pick when its margin allows."""
+    torch, dev, lib = gpu
+    host = pkg.host_api.host()
+    host.init(0)
+    fp4 = arch == "llama31_8b_fp4"
+    if fp4:
+        cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=14336, vocab=128256, t_kv=256, theta=5e5)
+    else:
+        cfg = dec.DecodeConfig(layers=2, hidden=4096, n_q=32, n_kv=8, inter=12288, vocab=151936, t_kv=256)
+    gen = torch.Generator(device=dev).manual_seed(21)
+    copy = lambda src, dst, nbytes: lib.convert(src.data_ptr(), BF16, dst, BF16, nbytes, 1.0)
+    models = [pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
+              for _ in range(2)]
+    for m in models:
+        m.set_qk_norm(not fp4)
+        m.set_exact_attention(True)
+    lin_shapes = {"wq": (cfg.q_out, cfg.hidden), "wk": (cfg.kv_out, cfg.hidden), "wv": (cfg.kv_out, cfg.hidden), "wo": (cfg.hidden, cfg.q_out),
+                  "w_gate": (cfg.inter, cfg.hidden), "w_up": (cfg.inter, cfg.hidden), "w_down": (cfg.hidden, cfg.inter)}
+
+    def put_linear(li, name, n_out, K):
+        if fp4:
+            nibs, scs = [], []
+            rows = max(1, (1 << 25) // K)
+            for r0 in range(0, n_out, rows):
+                w = (torch.randn(min(rows, n_out - r0), K, device=dev, generator=gen) * 0.02).to(torch.bfloat16).float()
+                nib, sc = pack_fp4_on_device(torch, w, 16)
+                nibs.append(nib); scs.append(sc)
+            nib_h, sc_h = torch.cat(nibs).cpu().numpy(), torch.cat(scs).cpu().numpy()
+            for m in models:
+                m.set_tensor(li, name, nib_h, 6)
+                m.set_block_scales(li, name, sc_h)
+        else:
+            w = draw_e5m2(torch, dev, gen, n_out, K)
+            for m in models:
+                assert copy(w, m.tensor_ptr(li, name), n_out * K) == 0
+
+    def put_plain(li, name, shape, mean, std):
+        v = draw_bf16(torch, dev, gen, shape, mean=mean, std=std)
+        for m in models:
+            assert copy(v, m.tensor_ptr(li, name), v.numel() * 2) == 0
+
+    for li in range(cfg.layers):
+        for name, (n_out, K) in lin_shapes.items():
+            put_linear(li, name, n_out, K)
+        for name in ("rms_attn", "rms_ffn"):
+            put_plain(li, name, (cfg.hidden,), 1.0, 0.1)
+        if not fp4:
+            for name in ("q_norm", "k_norm"):
+                put_plain(li, name, (128,), 1.0, 0.1)
+    put_linear(0, "lm_head", cfg.vocab, cfg.hidden)
+    if not fp4:
+        for m in models:
+            assert m.prepare_tiled(0, "lm_head")
+    put_plain(0, "rms_final", (cfg.hidden,), 1.0, 0.1)
+    put_plain(0, "emb", (cfg.vocab, cfg.hidden), 0.0, 1.0)
+    torch.cuda.synchronize()
+
+    T = 130
+    prompt = [int(t) for t in np.random.default_rng(11).integers(0, cfg.vocab, size=T)]
+    a, b = models
+    next_a = a.prefill(prompt)
+    for pos, tok in enumerate(prompt):
+        b.reset(tok, pos)
+        next_b = b.step()
+    assert a.pos == b.pos == T
+    for li in range(cfg.layers):
+        for is_v in (False, True):
+            ca, cb = dec.f(a.kv(li, is_v)[:, :T]), dec.f(b.kv(li, is_v)[:, :T])
+            assert np.isfinite(ca).all()
+            err = np.linalg.norm(ca - cb) / np.linalg.norm(cb)
+            assert err <= (2e-3 if li == 0 else 1e-2), (li, is_v, err)
+            # per position too: no row may be off by more than BF16 noise
+            rows = np.linalg.norm((ca - cb).reshape(cfg.n_kv, T, -1), axis=2) / np.linalg.norm(cb.reshape(cfg.n_kv, T, -1), axis=2)
+            assert rows.max() <= 3e-2, (li, is_v, rows.max())
+    la, lb = dec.f(a.logits()), dec.f(b.logits())
+    assert np.linalg.norm(la - lb) <= 1e-2 * np.linalg.norm(lb)
+    top2 = np.sort(lb)[-2:]
+    if top2[1] - top2[0] > 2 * np.abs(la - lb).max():
+        assert next_a == next_b
