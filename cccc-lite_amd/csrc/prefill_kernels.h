@@ -63,7 +63,7 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 //           comes from a transposed copy of the value block, two keys per dword.
 // Value rows past the last position written so far may hold anything: they are zeroed while staging (0 * NaN is NaN).
 constexpr int PF_KEYS = 64;                 // keys per staged block
-constexpr int PF_PITCH = 66;                // elements per transposed value row: 64 keys + 2 (33 dwords: rows spread over the banks)
+constexpr int PF_PITCH = 68;                // elements per transposed value row: 64 keys + 4 (34 dwords: 8-byte reads of 16 rows hit 32 distinct banks)
 constexpr int PF_KPITCH = 136;              // elements per staged key row: 128 dims + 8 (68 dwords: 16 rows x 16 bytes hit 64 distinct banks)
 constexpr int PF_TT = 1;                    // 16-token tiles per workgroup
 
@@ -316,9 +316,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __res
             {
                 // value operand: dim 16 d + j, the same eight keys
                 const uint16_t* vrow = vt + (16 * d + j) * PF_PITCH + slab * 32 + 4 * g;
-                const uint32_t v0 = *(const uint32_t*)vrow, v1 = *(const uint32_t*)(vrow + 2);
-                const uint32_t v2 = *(const uint32_t*)(vrow + 16), v3 = *(const uint32_t*)(vrow + 18);
-                const u32x4 vvec = { v0, v1, v2, v3 };
+                const uint2 va = *(const uint2*)vrow, vb = *(const uint2*)(vrow + 16);
+                const u32x4 vvec = { va.x, va.y, vb.x, vb.y };
 #pragma unroll
                 for (int tt = 0; tt < PF_TT; tt++)
                 {
