@@ -296,7 +296,7 @@ def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool):
     return entry, model
 
 
-def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3):
+def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, layout: str = "row-major"):
     """The prompt phase of the same model (DecodeModel::prefill, positions 0 .. T - 1): every linear is one quantized GEMM
     with T columns -- BASELINE config 4's kernel on all seven shapes of a layer, on the row-major file bytes (a batch-1
     DecodeModel keeps no tiled copies) -- with the row kernels and the causal attention between them.  Wall clock around the
@@ -318,7 +318,7 @@ def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3):
             best = dt if best is None else min(best, dt)
         # linears 2 T K N each; attention 2 * 2 * 128 * n_q per (token, visible key) pair
         flops = 2.0 * T * lin_elems + 4.0 * 128 * 32 * c["layers"] * (T * (T + 1) / 2) + 2.0 * c["hidden"] * c["vocab"]
-        out.append({"tokens": T, "ms": round(best * 1e3, 3), "tok_s": round(T / best, 1), "TFLOPs": round(flops / best * 1e-12, 1),
+        out.append({"tokens": T, "weights": layout, "ms": round(best * 1e3, 3), "tok_s": round(T / best, 1), "TFLOPs": round(flops / best * 1e-12, 1),
                     "frac_of_bf16_mfma_peak": round(flops / best * 1e-12 / MFMA_BF16_PEAK_TFLOPS, 4)})
     return out
 
@@ -752,6 +752,11 @@ def main():
                                                  "quantized GEMMs with T columns on the row-major weights, RMSNorm / RoPE / append rows, causal attention, "
                                                  "residual adds, SwiGLU; then the head on the last token",
                                      "cases": prompt_phase(ws, model)}
+            # the same with the load-time tiled copy of every linear (DecodeModel::setRepackLinears: twice the weight memory)
+            for li in range(QWEN3_8B["layers"]):
+                for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+                    assert model.prepare_tiled(li, name)
+            extra["prompt_phase"]["cases"] += prompt_phase(ws, model, layout="tiled copies")
         del model
         if not args.no_baselines:
             torch.cuda.empty_cache()

@@ -121,7 +121,7 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     {
         if ((int64_t)bytes != (dt == FP4_E2M1 ? (m->getDataSize() + 1) / 2 : m->getDataSize())) { return -1; }
         // only a tall FP8 weight (lm_head) is read through its tiled copy by the fused decode kernels
-        m->setAllowRepack(which == LM_HEAD && dt != FP4_E2M1);
+        m->setAllowRepack(repack_linears_ || (which == LM_HEAD && dt != FP4_E2M1));
         m->loadQuantizedDirect((const uint8_t*)host, (int64_t)bytes, scale, dt);
         return 0;
     }
@@ -154,17 +154,18 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
         m = tmp;
         return 0;
     };
-    auto load_linear = [&](Matrix& m, const std::string& name, bool tiled = false) -> int {
+    auto load_linear = [&](Matrix& m, const std::string& name, bool head = false) -> int {
+        const bool tiled = head || repack_linears_;
         const auto wk = file.resolve(name);
         if (!wk.valid()) { return fail(name, -1); }
         if (wk.is_quant)
         {
-            m.setAllowRepack(tiled && wk.dt != FP4_E2M1);      // the fused FP4 kernels read the file layout only
+            m.setAllowRepack(repack_linears_ || (tiled && wk.dt != FP4_E2M1));      // the fused FP4 kernels read the file layout only
             if (file.loadNamed(m, name) != 0) { return fail(name, -2); }
             if (wk.dt == FP4_E2M1 && !m.getBlockScaleData()) { return fail(name, -3); }    // FP4 without blockscale_<name>: no fused kernel
             return 0;
         }
-        const bool tiled_q = tiled && quantize_to != FP4_E2M1;
+        const bool tiled_q = repack_linears_ || (tiled && quantize_to != FP4_E2M1);
         Matrix tmp(m.getWidth(), m.getHeight(), 1, 1, BFLOAT16, gpu_);
         tmp.setAllowRepack(tiled_q);
         if (file.loadNamed(tmp, name) != 0) { return fail(name, -2); }

@@ -220,6 +220,7 @@ int cccc_matrix_save_named(void* m, const char* name, const char* path)
 void cccc_decode_set_exact_attention(void* m, int exact) { ((DecodeModel*)m)->setExactAttention(exact != 0); }
 void cccc_decode_set_qk_norm(void* m, int on) { ((DecodeModel*)m)->setQkNorm(on != 0); }
 int cccc_decode_qk_norm(void* m) { return ((DecodeModel*)m)->qkNorm() ? 1 : 0; }
+void cccc_decode_set_repack_linears(void* m, int on) { ((DecodeModel*)m)->setRepackLinears(on != 0); }
 void cccc_decode_set_tied_lm_head(void* m, int tied) { ((DecodeModel*)m)->setTiedLmHead(tied != 0); }
 int cccc_decode_tied_lm_head(void* m) { return ((DecodeModel*)m)->tiedLmHead() ? 1 : 0; }
 

@@ -71,6 +71,7 @@ class HostLibrary:
         L.cccc_decode_prefill.restype = i32; L.cccc_decode_prefill.argtypes = [vp, ctypes.POINTER(ctypes.c_int), i32, i32]
         L.cccc_decode_set_qk_norm.restype = None; L.cccc_decode_set_qk_norm.argtypes = [vp, i32]
         L.cccc_decode_qk_norm.restype = i32; L.cccc_decode_qk_norm.argtypes = [vp]
+        L.cccc_decode_set_repack_linears.restype = None; L.cccc_decode_set_repack_linears.argtypes = [vp, i32]
         L.cccc_decode_set_tied_lm_head.restype = None; L.cccc_decode_set_tied_lm_head.argtypes = [vp, i32]
         L.cccc_decode_tied_lm_head.restype = i32; L.cccc_decode_tied_lm_head.argtypes = [vp]
         L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
@@ -300,6 +301,10 @@ class DecodeModel:
     def set_qk_norm(self, on: bool) -> None:
         """Per-head RMSNorm of q and k in front of the rotation (Qwen3: on, the default; Llama-3.1: off)."""
         self.lib.c.cccc_decode_set_qk_norm(self.handle, 1 if on else 0)
+
+    def set_repack_linears(self, on: bool) -> None:
+        """Keep the tiled copy of every linear set or loaded from now on (faster prompt-phase GEMMs, twice the weight memory)."""
+        self.lib.c.cccc_decode_set_repack_linears(self.handle, 1 if on else 0)
 
     def set_tied_lm_head(self, tied: bool) -> None:
         """Tied embeddings: the head reads the BF16 embedding table, no separate lm_head is stored."""

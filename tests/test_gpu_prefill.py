@@ -171,7 +171,9 @@ def test_prompt_in_pieces_and_bad_arguments(gpu, pkg, oracle, dec):
     weights = dec.make_model(cfg, 59)
     prompt = [int(t) for t in np.random.default_rng(5).integers(0, cfg.vocab, size=60)]
     a, b = _fresh(pkg, host, cfg), _fresh(pkg, host, cfg)
+    b.set_repack_linears(True)                                 # the second model also reads its linears through their tiled copies
     a.load(weights); b.load(weights)
+    assert b.prepare_tiled(0, "w_down") and not a.prepare_tiled(0, "w_down")      # only b's linears may carry the copy
     a.prefill(prompt)
     b.prefill(prompt[:7])
     b.prefill(prompt[7:], pos0=7)
