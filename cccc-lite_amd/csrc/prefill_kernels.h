@@ -48,11 +48,10 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 
 // ------------------------------------------------------------------------------------------
 // Causal GQA attention of T query tokens over cache rows 0 .. pos0 + t, head_dim 128, on the matrix cores, with the
-// reference's rounding points.  Grid (ceil(T / 32), kv heads); a workgroup of four waves owns 32 tokens (two 16-token
-// tiles), wave w the query head kvh * G + w (waves >= G only help with the staging).  Keys and values go through LDS in
-// blocks of 64 rows, fetched once per workgroup and pass and shared by the G heads and both token tiles (fetched by every
-// wave for itself they cost four times the cache traffic, which bounded the kernel).  Two passes over the keys
-// 0 .. pos0 + (last token of the workgroup):
+// reference's rounding points.  Grid ceil(T / 16) x kv heads, one-dimensional; a workgroup of four waves owns 16 tokens, wave w the
+// query head kvh * G + w (waves >= G only help with the staging).  Keys and values go through LDS in blocks of 64 rows,
+// fetched once per workgroup and pass and shared by the G heads.  Two passes over the keys 0 .. pos0 + (last token of
+// the workgroup):
 //   pass 1  scores of 16 keys x 16 tokens per v_mfma_f32_16x16x32_bf16 x 4 (key rows as the row operand, the rotated
 //           queries as columns: D lane (token = lane % 16, g = lane / 16) holds keys 4 g .. 4 g + 3), rounded to BF16,
 //           masked, running (max, sum) per lane, merged over the four lane groups at the end;
@@ -61,32 +60,47 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 //           4 g .. + 3 and 16 + 4 g .. + 3 of a 32-key slab) are its row operand as they are, because a contraction does not
 //           care in which order k is visited when both operands agree; the value operand (column = dim, the same keys)
 //           comes from a transposed copy of the value block, two keys per dword.
+// Both passes are software-pipelined over two LDS buffers: while the VALU turns the raw scores of block b into statistics
+// or probabilities, the matrix cores already multiply block b + 1, whose keys were staged one iteration earlier; the
+// rows of block b + 2 travel from memory meanwhile and are stored behind the iteration's single barrier.
 // Value rows past the last position written so far may hold anything: they are zeroed while staging (0 * NaN is NaN).
 constexpr int PF_KEYS = 64;                 // keys per staged block
 constexpr int PF_PITCH = 68;                // elements per transposed value row: 64 keys + 4 (34 dwords: 8-byte reads of 16 rows hit 32 distinct banks)
 constexpr int PF_KPITCH = 136;              // elements per staged key row: 128 dims + 8 (68 dwords: 16 rows x 16 bytes hit 64 distinct banks)
-constexpr int PF_TT = 1;                    // 16-token tiles per workgroup
+constexpr float PF_LOG2E = 1.4426950408889634f;
 
-// expf through the hardware's 2^x (x * log2 e is rounded once more in front of it: a few FP32 ulps, against the BF16
-// rounding that follows every use here)
-__device__ __forceinline__ float pf_exp(float x) { return __expf(x); }
+// 2^x on the hardware unit.  exp(s - m) is taken as 2^(s log2 e - m log2 e) with one fused multiply-add in front: a few FP32
+// ulps from expf, against the BF16 rounding that follows every use here.
+__device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Two FP32 values rounded to BF16 (nearest even) into one dword, low half first.  Spelled as the instruction because the
+// compiler, seeing the halves used separately afterwards, converts each value with an instruction of its own.
+__device__ __forceinline__ uint32_t pf_pack_bf16(float lo, float hi)
+{
+    uint32_t r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load in flight (its
-// release fence drains the vector-memory counter on this target), which would cancel the two-blocks-ahead prefetch below:
-// the kernel then pays a trip to memory per block (1.3 us per 64 keys and pass, whatever the arithmetic costs).
+// release fence drains the vector-memory counter on this target), which would cancel the prefetch below: the kernel
+// then pays a trip to memory per block.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int G>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
-                                                          uint16_t* __restrict__ y, int n_q, int t_kv, int n_tokens, int pos0, float scale)
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+                                                             uint16_t* __restrict__ y, int n_q, int t_kv, int n_tokens, int pos0, float scale)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t ks[PF_KEYS * PF_KPITCH];   // [key][dim] of the current block
-    __shared__ __attribute__((aligned(16))) uint16_t vt[128 * PF_PITCH];        // [dim][key] of the current block
-    const int kvh = blockIdx.y;
-    const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * (16 * PF_TT);       // the workgroups that see the most keys go first
+    __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KEYS * PF_KPITCH];   // [key][dim] of two blocks
+    __shared__ __attribute__((aligned(16))) uint16_t vt[2][128 * PF_PITCH];        // [dim][key] of two blocks
+    // Consecutive workgroups go to the eight XCDs in turn, each with an L2 of its own: with the kv head as the fastest index
+    // an XCD serves few heads (one, with eight of them) and their keys and values stay in its L2 for all token tiles.
+    const int n_kv = n_q / G;
+    const int kvh = blockIdx.x % n_kv;
+    const int t0 = ((int)gridDim.x / n_kv - 1 - (int)blockIdx.x / n_kv) * 16;   // the workgroups that see the most keys go first
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 15, g = lane >> 4;
-    const int last_token = min(t0 + 16 * PF_TT - 1, n_tokens - 1);
+    const int last_token = min(t0 + 15, n_tokens - 1);
     const int n_keys = pos0 + last_token + 1;                   // keys this workgroup can see
     const int n_written = pos0 + n_tokens;                      // cache rows holding data
     const int n_blocks = (n_keys + PF_KEYS - 1) / PF_KEYS;
@@ -94,207 +108,204 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __res
     const uint16_t* kbase = k_cache + (size_t)kvh * t_kv * 128;
     const uint16_t* vbase = v_cache + (size_t)kvh * t_kv * 128;
 
-    // the query operands: token tile tt, token j's head, dims 32 c + 8 g .. + 7
-    u32x4 qf[PF_TT][4];
-    int my_pos[PF_TT];
-#pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++)
+    // the query operand: token j's head, dims 32 c + 8 g .. + 7
+    u32x4 qf[4];
+    const int my_pos = pos0 + min(t0 + j, n_tokens - 1);
+    if (active)
     {
-        const int t = min(t0 + tt * 16 + j, n_tokens - 1);
-        my_pos[tt] = pos0 + t;
-        if (active)
-        {
-            const uint16_t* qrow = q + ((size_t)t * n_q + kvh * G + wave) * 128 + g * 8;
+        const uint16_t* qrow = q + ((size_t)min(t0 + j, n_tokens - 1) * n_q + kvh * G + wave) * 128 + g * 8;
 #pragma unroll
-            for (int c = 0; c < 4; c++) { qf[tt][c] = *(const u32x4*)(qrow + c * 32); }
-        }
+        for (int c = 0; c < 4; c++) { qf[c] = *(const u32x4*)(qrow + c * 32); }
     }
-    // staging: thread -> rows and 16-byte pieces of a 64-row block (item = thread + 256 i: key pair 2 p, 2 p + 1 with
-    // p = item % 32, dims 8 c .. + 7 with c = item / 32); raw[2 i], raw[2 i + 1] are the two rows' pieces
-    auto load_rows = [&](const uint16_t* base, int b, int limit, u32x4 (&raw)[4]) {
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-        {
-            const int item = threadIdx.x + i * 256;
-            const int row = b * PF_KEYS + 2 * (item & 31);
-            // no predicate on the loads (rows past the limit re-read its last row and are zeroed when stored), so that
-            // the number of requests in flight is known at every wait
-            raw[2 * i] = *(const u32x4*)(base + (size_t)min(row, limit - 1) * 128 + (item >> 5) * 8);
-            raw[2 * i + 1] = *(const u32x4*)(base + (size_t)min(row + 1, limit - 1) * 128 + (item >> 5) * 8);
-        }
+    // staging: a thread moves two 16-byte pieces (dims 8 c .. + 7 and 64 + 8 c .. + 7, c = thread / 32) of two rows (keys
+    // 2 p, 2 p + 1 of the block, p = thread % 32): raw[2 i], raw[2 i + 1] are the two rows' pieces i.  A block index past the
+    // last block is clamped to it; rows past the last written one re-read it (no predicate on the loads) and are zeroed
+    // when stored.  Addresses are a uniform base plus a 32-bit offset per lane.
+    const int p2 = 2 * (threadIdx.x & 31), c8 = (threadIdx.x >> 5) * 8;
+    auto load_rows = [&](const uint16_t* base, int b, u32x4 (&raw)[4]) {
+        const int row = min(b, n_blocks - 1) * PF_KEYS + p2;
+        const uint32_t o0 = (uint32_t)min(row, n_written - 1) * 256u + c8 * 2, o1 = (uint32_t)min(row + 1, n_written - 1) * 256u + c8 * 2;
+        const char* base8 = (const char*)base;
+        raw[0] = *(const u32x4*)(base8 + o0);
+        raw[1] = *(const u32x4*)(base8 + o1);
+        raw[2] = *(const u32x4*)(base8 + o0 + 128);
+        raw[3] = *(const u32x4*)(base8 + o1 + 128);
     };
     const u32x4 zero4 = { 0u, 0u, 0u, 0u };
-    auto store_keys = [&](int b, int limit, const u32x4 (&raw)[4]) {
-#pragma unroll
-        for (int i = 0; i < 2; i++)
+    auto store_keys = [&](int buf, int b, const u32x4 (&raw)[4]) {
+        const int row = min(b, n_blocks - 1) * PF_KEYS + p2;
+        uint16_t* dst = ks[buf] + p2 * PF_KPITCH + c8;
+        if (row + PF_KEYS <= n_written)                         // (a sufficient test: no row of the block needs zeroing)
         {
-            const int item = threadIdx.x + i * 256;
-            const int row = b * PF_KEYS + 2 * (item & 31);
-            uint16_t* dst = ks + 2 * (item & 31) * PF_KPITCH + (item >> 5) * 8;
-            *(u32x4*)dst = row < limit ? raw[2 * i] : zero4;
-            *(u32x4*)(dst + PF_KPITCH) = row + 1 < limit ? raw[2 * i + 1] : zero4;
+            *(u32x4*)dst = raw[0];
+            *(u32x4*)(dst + PF_KPITCH) = raw[1];
+            *(u32x4*)(dst + 64) = raw[2];
+            *(u32x4*)(dst + PF_KPITCH + 64) = raw[3];
+        }
+        else
+        {
+            const bool in0 = row < n_written, in1 = row + 1 < n_written;
+            *(u32x4*)dst = in0 ? raw[0] : zero4;
+            *(u32x4*)(dst + PF_KPITCH) = in1 ? raw[1] : zero4;
+            *(u32x4*)(dst + 64) = in0 ? raw[2] : zero4;
+            *(u32x4*)(dst + PF_KPITCH + 64) = in1 ? raw[3] : zero4;
         }
     };
     // transposed store, two keys per dword: dim 8 c + e gets (key 2 p, key 2 p + 1) at dword p of its row
-    auto store_values = [&](int b, int limit, const u32x4 (&raw)[4]) {
+    auto store_values = [&](int buf, int b, const u32x4 (&raw)[4]) {
+        const int row = min(b, n_blocks - 1) * PF_KEYS + p2;
+        const bool whole = (min(b, n_blocks - 1) + 1) * PF_KEYS <= n_written;       // uniform: no row of the block needs zeroing
+        const bool in0 = whole || row < n_written, in1 = whole || row + 1 < n_written;
 #pragma unroll
         for (int i = 0; i < 2; i++)
         {
-            const int item = threadIdx.x + i * 256;
-            const int row = b * PF_KEYS + 2 * (item & 31);
-            uint32_t* dst = (uint32_t*)vt + (item >> 5) * 8 * (PF_PITCH / 2) + (item & 31);
-            const u32x4 lo = row < limit ? raw[2 * i] : zero4, hi = row + 1 < limit ? raw[2 * i + 1] : zero4;
+            uint32_t* dst = (uint32_t*)vt[buf] + (c8 + 64 * i) * (PF_PITCH / 2) + (p2 >> 1);
+            u32x4 lo = raw[2 * i], hi = raw[2 * i + 1];
+            if (!whole)
+            {
+                lo = in0 ? lo : zero4;
+                hi = in1 ? hi : zero4;
+            }
 #pragma unroll
             for (int d = 0; d < 4; d++)
             {
-                dst[(2 * d) * (PF_PITCH / 2)] = (lo[d] & 0xFFFFu) | (hi[d] << 16);
-                dst[(2 * d + 1) * (PF_PITCH / 2)] = (lo[d] >> 16) | (hi[d] & 0xFFFF0000u);
+                dst[(2 * d) * (PF_PITCH / 2)] = __builtin_amdgcn_perm(hi[d], lo[d], 0x05040100u);       // low halves of both keys
+                dst[(2 * d + 1) * (PF_PITCH / 2)] = __builtin_amdgcn_perm(hi[d], lo[d], 0x07060302u);   // high halves
             }
         }
     };
-    // scores of the block's four key tiles (16 keys each) against the token tiles: for tile kt the lane gets keys
+    // raw scores of a staged block's four key tiles (16 keys each) against the token tile: for tile kt the lane gets keys
     // kt * 16 + 4 g + v, v = 0..3, of token j.  All sixteen key operands are read first and the products run over the
     // tiles inside each 32-dim step, so that consecutive matrix-core instructions never wait for each other's sums.
-    auto score_block = [&](int b, bool masked, float (&s)[PF_KEYS / 16][PF_TT][4]) {
+    auto score_products = [&](int buf, f32x4 (&acc)[PF_KEYS / 16]) {
         u32x4 kf[PF_KEYS / 16][4];
 #pragma unroll
         for (int kt = 0; kt < PF_KEYS / 16; kt++)
         {
-            const uint16_t* krow = ks + (kt * 16 + j) * PF_KPITCH + g * 8;
+            const uint16_t* krow = ks[buf] + (kt * 16 + j) * PF_KPITCH + g * 8;
 #pragma unroll
             for (int c = 0; c < 4; c++) { kf[kt][c] = *(const u32x4*)(krow + c * 32); }
         }
-        f32x4 acc[PF_KEYS / 16][PF_TT];
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++)
-#pragma unroll
-            for (int tt = 0; tt < PF_TT; tt++) { acc[kt][tt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+        for (int kt = 0; kt < PF_KEYS / 16; kt++) { acc[kt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
 #pragma unroll
         for (int c = 0; c < 4; c++)
 #pragma unroll
             for (int kt = 0; kt < PF_KEYS / 16; kt++)
-#pragma unroll
-                for (int tt = 0; tt < PF_TT; tt++)
-                {
-                    acc[kt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt][c]), __builtin_bit_cast(bf16x8, qf[tt][c]), acc[kt][tt], 0, 0, 0);
-                }
+            {
+                acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt][c]), __builtin_bit_cast(bf16x8, qf[c]), acc[kt], 0, 0, 0);
+            }
+    };
+    // scaled, rounded to BF16 by the hardware conversion (round to nearest even, as the integer trick rounds finite
+    // values) and masked: only blocks that reach past the workgroup's first token need the test
+    auto score_round = [&](const f32x4 (&acc)[PF_KEYS / 16], int b, auto masked_c, float (&s)[PF_KEYS / 16][4]) {
+        constexpr bool masked = decltype(masked_c)::value;
 #pragma unroll
         for (int kt = 0; kt < PF_KEYS / 16; kt++)
-#pragma unroll
-            for (int tt = 0; tt < PF_TT; tt++)
+        {
+            const f32x4 a = acc[kt];
+            const uint32_t w01 = pf_pack_bf16(scale * a[0], scale * a[1]), w23 = pf_pack_bf16(scale * a[2], scale * a[3]);
+            s[kt][0] = __builtin_bit_cast(float, w01 << 16);
+            s[kt][1] = __builtin_bit_cast(float, w01 & 0xFFFF0000u);
+            s[kt][2] = __builtin_bit_cast(float, w23 << 16);
+            s[kt][3] = __builtin_bit_cast(float, w23 & 0xFFFF0000u);
+            if (masked)
             {
-                // rounded to BF16 by the hardware conversion (round to nearest even, as the integer trick rounds finite values)
-                const f32x4 a = acc[kt][tt];
-                const bf16x2 r01 = { (__bf16)(scale * a[0]), (__bf16)(scale * a[1]) }, r23 = { (__bf16)(scale * a[2]), (__bf16)(scale * a[3]) };
-                const uint32_t w01 = __builtin_bit_cast(uint32_t, r01), w23 = __builtin_bit_cast(uint32_t, r23);
-                s[kt][tt][0] = __builtin_bit_cast(float, w01 << 16);
-                s[kt][tt][1] = __builtin_bit_cast(float, w01 & 0xFFFF0000u);
-                s[kt][tt][2] = __builtin_bit_cast(float, w23 << 16);
-                s[kt][tt][3] = __builtin_bit_cast(float, w23 & 0xFFFF0000u);
-                if (masked)                                     // only blocks that reach past the workgroup's first token need the test
-                {
 #pragma unroll
-                    for (int v = 0; v < 4; v++)
-                    {
-                        const int key = b * PF_KEYS + kt * 16 + 4 * g + v;
-                        if (key > my_pos[tt]) { s[kt][tt][v] = -INFINITY; }
-                    }
+                for (int v = 0; v < 4; v++)
+                {
+                    if (b * PF_KEYS + kt * 16 + 4 * g + v > my_pos) { s[kt][v] = -INFINITY; }
                 }
             }
+        }
     };
 
     // ---- pass 1: row maximum and sum of exp(s - max)
-    float m[PF_TT], l[PF_TT];
-#pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++) { m[tt] = -INFINITY; l[tt] = 0.0f; }
-    // rows are requested two blocks ahead of their use (two register sets, alternating): one block of work does not cover
-    // the trip to memory
-    u32x4 kraw[2][4], vraw[2][4];
-    load_rows(kbase, 0, n_written, kraw[0]);
-    load_rows(kbase, min(1, n_blocks - 1), n_written, kraw[1]);
-    auto pass1_block = [&](int b, u32x4 (&kr)[4]) {
-        lds_barrier();                                        // the previous block's reads are done
-        store_keys(b, n_written, kr);
-        load_rows(kbase, min(b + 2, n_blocks - 1), n_written, kr);      // unconditional (clamped): the wait counts stay exact
-        lds_barrier();
-        if (!active) { return; }
-        const bool masked = b * PF_KEYS + PF_KEYS - 1 > pos0 + t0;      // some key of the block lies past the first token's position
-        // all four key tiles of the block at once: sixteen independent scores per lane and token tile keep the matrix cores
-        // and the VALU busy where one tile at a time is a single chain of dependent instructions
-        float s[PF_KEYS / 16][PF_TT][4];
-        score_block(b, masked, s);
-#pragma unroll
-        for (int tt = 0; tt < PF_TT; tt++)
+    float m = -INFINITY, l = 0.0f;
+    u32x4 kraw[4], vraw[4];
+    f32x4 cur[PF_KEYS / 16], next[PF_KEYS / 16];
+    // blocks 0 .. n_plain - 1 end at or before the first token's position and need no mask test (one or two blocks do)
+    const int n_plain = min((pos0 + t0 + 1) / PF_KEYS, n_blocks);
+    // prologue: block 0 staged and multiplied, block 1 staged, block 2 on its way
+    load_rows(kbase, 0, kraw);
+    store_keys(0, 0, kraw);
+    load_rows(kbase, 1, kraw);
+    lds_barrier();
+    if (active) { score_products(0, cur); }
+    store_keys(1, 1, kraw);
+    load_rows(kbase, 2, kraw);
+    lds_barrier();
+    // iteration b: ks[(b + 1) & 1] holds block b + 1, `cur` the raw scores of block b, kraw block b + 2 in flight
+    auto pass1_block = [&](int b, auto masked_c) {
+        if (active)
         {
+            score_products((b + 1) & 1, next);
+            float s[PF_KEYS / 16][4];
+            score_round(cur, b, masked_c, s);
             float bm = -INFINITY;
 #pragma unroll
             for (int kt = 0; kt < PF_KEYS / 16; kt++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) { bm = fmaxf(bm, s[kt][tt][v]); }
-            if (bm > m[tt])
-            {
-                l[tt] *= pf_exp(m[tt] - bm);                    // m = -inf: l is 0 and stays 0
-                m[tt] = bm;
-            }
-            if (m[tt] > -INFINITY)
-            {
-                float sum = 0.0f;
+                for (int v = 0; v < 4; v++) { bm = fmaxf(bm, s[kt][v]); }
+            const float nm = fmaxf(m, bm);
+            // nm = -inf: nothing visible to this lane yet, every term below is 2^(-inf) = 0 with the offset at 0
+            const float off = nm > -INFINITY ? -nm * PF_LOG2E : 0.0f;
+            l = nm == m ? l : l * pf_exp2(fmaf(m, PF_LOG2E, off));
+            m = nm;
+            float sum = 0.0f;
 #pragma unroll
-                for (int kt = 0; kt < PF_KEYS / 16; kt++)
+            for (int kt = 0; kt < PF_KEYS / 16; kt++)
 #pragma unroll
-                    for (int v = 0; v < 4; v++) { sum += pf_exp(s[kt][tt][v] - m[tt]); }
-                l[tt] += sum;
-            }
+                for (int v = 0; v < 4; v++) { sum += pf_exp2(fmaf(s[kt][v], PF_LOG2E, off)); }
+            l += sum;
         }
+        store_keys(b & 1, b + 2, kraw);                         // block b's buffer: its reads ended before the last barrier
+        load_rows(kbase, b + 3, kraw);
+        lds_barrier();
+#pragma unroll
+        for (int kt = 0; kt < PF_KEYS / 16; kt++) { cur[kt] = next[kt]; }
     };
-    for (int b = 0; b < n_blocks; b += 2)
-    {
-        pass1_block(b, kraw[0]);
-        if (b + 1 < n_blocks) { pass1_block(b + 1, kraw[1]); }
-    }
-    float inv[PF_TT];
+    // two copies of the iteration, with and without the mask test, each one straight run of instructions
+    for (int b = 0; b < n_plain; b++) { pass1_block(b, std::false_type{}); }
+    for (int b = n_plain; b < n_blocks; b++) { pass1_block(b, std::true_type{}); }
+    // merge the four lane groups of a token (lanes j, j + 16, j + 32, j + 48)
 #pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++)
+    for (int off = 16; off < 64; off <<= 1)
     {
-        // merge the four lane groups of a token (lanes j, j + 16, j + 32, j + 48)
-#pragma unroll
-        for (int off = 16; off < 64; off <<= 1)
-        {
-            const float om = __shfl_xor(m[tt], off), ol = __shfl_xor(l[tt], off);
-            const float nm = fmaxf(m[tt], om);
-            if (nm > -INFINITY) { l[tt] = l[tt] * pf_exp(m[tt] - nm) + ol * pf_exp(om - nm); }
-            m[tt] = nm;
-        }
-        inv[tt] = l[tt] > 0.0f ? 1.0f / l[tt] : 0.0f;
+        const float om = __shfl_xor(m, off), ol = __shfl_xor(l, off);
+        const float nm = fmaxf(m, om);
+        if (nm > -INFINITY) { l = l * pf_exp2((m - nm) * PF_LOG2E) + ol * pf_exp2((om - nm) * PF_LOG2E); }
+        m = nm;
     }
+    // p = 2^(s log2 e - (m log2 e + log2 l)): the division by the sum rides in the exponent
+    const float poff = l > 0.0f ? -(m * PF_LOG2E + __builtin_amdgcn_logf(l)) : -INFINITY;
 
     // ---- pass 2: probabilities and P V
-    f32x4 out[PF_TT][8];
+    f32x4 out[8];
 #pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++)
+    for (int d = 0; d < 8; d++) { out[d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+    load_rows(kbase, 0, kraw);
+    load_rows(vbase, 0, vraw);
+    store_keys(0, 0, kraw);
+    load_rows(kbase, 1, kraw);
+    lds_barrier();
+    if (active) { score_products(0, cur); }
+    store_keys(1, 1, kraw);
+    store_values(0, 0, vraw);
+    load_rows(kbase, 2, kraw);
+    load_rows(vbase, 1, vraw);
+    lds_barrier();
+    // iteration b: ks[(b + 1) & 1] holds key block b + 1, vt[b & 1] value block b; kraw = keys b + 2, vraw = values b + 1 in flight
+    auto pass2_block = [&](int b, auto masked_c) {
+        if (active)
+        {
+            score_products((b + 1) & 1, next);
+            float s[PF_KEYS / 16][4];
+            score_round(cur, b, masked_c, s);
+            // 2^(-inf) is 0: a masked key gets probability 0 without a test; the pairs are rounded and packed by one conversion each
+            bf16x8 pa[PF_KEYS / 32];
 #pragma unroll
-        for (int d = 0; d < 8; d++) { out[tt][d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
-    load_rows(kbase, 0, n_written, kraw[0]);
-    load_rows(vbase, 0, n_written, vraw[0]);
-    load_rows(kbase, min(1, n_blocks - 1), n_written, kraw[1]);
-    load_rows(vbase, min(1, n_blocks - 1), n_written, vraw[1]);
-    auto pass2_block = [&](int b, u32x4 (&kr)[4], u32x4 (&vr)[4]) {
-        lds_barrier();
-        store_keys(b, n_written, kr);
-        store_values(b, n_written, vr);
-        load_rows(kbase, min(b + 2, n_blocks - 1), n_written, kr);
-        load_rows(vbase, min(b + 2, n_blocks - 1), n_written, vr);
-        lds_barrier();
-        if (!active) { return; }
-        const bool masked = b * PF_KEYS + PF_KEYS - 1 > pos0 + t0;
-        float s[PF_KEYS / 16][PF_TT][4];
-        score_block(b, masked, s);
-        // exp(-inf) is 0: a masked key gets probability 0 without a test; the pairs are rounded and packed by one conversion each
-        bf16x8 pa[PF_KEYS / 32][PF_TT];
-#pragma unroll
-        for (int slab = 0; slab < PF_KEYS / 32; slab++)
-#pragma unroll
-            for (int tt = 0; tt < PF_TT; tt++)
+            for (int slab = 0; slab < PF_KEYS / 32; slab++)
             {
                 uint32_t pw[4];
 #pragma unroll
@@ -302,48 +313,54 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const uint16_t* __res
 #pragma unroll
                     for (int v = 0; v < 2; v++)
                     {
-                        const float* sv = s[2 * slab + h][tt];
-                        const bf16x2 pp = { (__bf16)(pf_exp(sv[2 * v] - m[tt]) * inv[tt]), (__bf16)(pf_exp(sv[2 * v + 1] - m[tt]) * inv[tt]) };
+                        const float* sv = s[2 * slab + h];
+                        const bf16x2 pp = { (__bf16)pf_exp2(fmaf(sv[2 * v], PF_LOG2E, poff)), (__bf16)pf_exp2(fmaf(sv[2 * v + 1], PF_LOG2E, poff)) };
                         pw[2 * h + v] = __builtin_bit_cast(uint32_t, pp);
                     }
                 const u32x4 pvec = { pw[0], pw[1], pw[2], pw[3] };      // keys 4 g .. + 3, then 16 + 4 g .. + 3 of the slab
-                pa[slab][tt] = __builtin_bit_cast(bf16x8, pvec);
+                pa[slab] = __builtin_bit_cast(bf16x8, pvec);
             }
+            // value operands (dim 16 d + j, the same eight keys) of both slabs are read before the first product
+            u32x4 vf[PF_KEYS / 32][8];
 #pragma unroll
-        for (int slab = 0; slab < PF_KEYS / 32; slab++)
+            for (int slab = 0; slab < PF_KEYS / 32; slab++)
 #pragma unroll
-            for (int d = 0; d < 8; d++)
-            {
-                // value operand: dim 16 d + j, the same eight keys
-                const uint16_t* vrow = vt + (16 * d + j) * PF_PITCH + slab * 32 + 4 * g;
-                const uint2 va = *(const uint2*)vrow, vb = *(const uint2*)(vrow + 16);
-                const u32x4 vvec = { va.x, va.y, vb.x, vb.y };
-#pragma unroll
-                for (int tt = 0; tt < PF_TT; tt++)
+                for (int d = 0; d < 8; d++)
                 {
-                    out[tt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[slab][tt], __builtin_bit_cast(bf16x8, vvec), out[tt][d], 0, 0, 0);
+                    const uint16_t* vrow = vt[b & 1] + (16 * d + j) * PF_PITCH + slab * 32 + 4 * g;
+                    const uint2 va = *(const uint2*)vrow, vb = *(const uint2*)(vrow + 16);
+                    vf[slab][d] = u32x4{ va.x, va.y, vb.x, vb.y };
                 }
-            }
-    };
-    for (int b = 0; b < n_blocks; b += 2)
-    {
-        pass2_block(b, kraw[0], vraw[0]);
-        if (b + 1 < n_blocks) { pass2_block(b + 1, kraw[1], vraw[1]); }
-    }
-    if (!active) { return; }
-    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3 of its tile
 #pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++)
+            for (int slab = 0; slab < PF_KEYS / 32; slab++)
 #pragma unroll
-        for (int d = 0; d < 8; d++)
-        {
-#pragma unroll
-            for (int v = 0; v < 4; v++)
-            {
-                const int t = t0 + tt * 16 + 4 * g + v;
-                if (t < n_tokens) { y[((size_t)t * n_q + kvh * G + wave) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(out[tt][d][v]); }
-            }
+                for (int d = 0; d < 8; d++)
+                {
+                    out[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[slab], __builtin_bit_cast(bf16x8, vf[slab][d]), out[d], 0, 0, 0);
+                }
         }
+        store_keys(b & 1, b + 2, kraw);
+        store_values((b + 1) & 1, b + 1, vraw);                 // held value block b - 1, read before the last barrier
+        load_rows(kbase, b + 3, kraw);
+        load_rows(vbase, b + 2, vraw);
+        lds_barrier();
+#pragma unroll
+        for (int kt = 0; kt < PF_KEYS / 16; kt++) { cur[kt] = next[kt]; }
+    };
+    for (int b = 0; b < n_plain; b++) { pass2_block(b, std::false_type{}); }
+    for (int b = n_plain; b < n_blocks; b++) { pass2_block(b, std::true_type{}); }
+    if (!active) { return; }
+    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3 of the tile
+#pragma unroll
+    for (int d = 0; d < 8; d++)
+    {
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+        {
+            const int t = t0 + 4 * g + v;
+            if (t < n_tokens) { y[((size_t)t * n_q + kvh * G + wave) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(out[d][v]); }
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------
