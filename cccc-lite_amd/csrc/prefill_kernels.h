@@ -48,8 +48,10 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 
 // ------------------------------------------------------------------------------------------
 // Causal GQA attention of T query tokens over cache rows 0 .. pos0 + t, head_dim 128, on the matrix cores, with the
-// reference's rounding points.  Grid ceil(T / 16) x kv heads, one-dimensional; a workgroup of four waves owns 16 tokens, wave w the
-// query head kvh * G + w (waves >= G only help with the staging).  Keys and values go through LDS in blocks of 64 rows,
+// reference's rounding points.  Grid ceil(T / 16) x kv heads, one-dimensional; a workgroup of four waves owns 16 tokens of the
+// G query heads of one kv head: a wave takes two heads (one when G = 1) and one half -- 32 keys -- of every staged block, so
+// that a key or value operand read from LDS serves two products and the halves of a head meet once at the end (waves left
+// over only help with the staging).  Keys and values go through LDS in blocks of 64 rows,
 // fetched once per workgroup and pass and shared by the G heads.  Two passes over the keys 0 .. pos0 + (last token of
 // the workgroup):
 //   pass 1  scores of 16 keys x 16 tokens per v_mfma_f32_16x16x32_bf16 x 4 (key rows as the row operand, the rotated
@@ -65,7 +67,7 @@ static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const u
 // rows of block b + 2 travel from memory meanwhile and are stored behind the iteration's single barrier.
 // Value rows past the last position written so far may hold anything: they are zeroed while staging (0 * NaN is NaN).
 constexpr int PF_KEYS = 64;                 // keys per staged block
-constexpr int PF_PITCH = 68;                // elements per transposed value row: 64 keys + 4 (34 dwords: 8-byte reads of 16 rows hit 32 distinct banks)
+constexpr int PF_PITCH = 68;                // elements per transposed value row: 64 keys + 4 (34 dwords: 8-byte reads of 16 rows hit 32 distinct banks; 72 measured the same)
 constexpr int PF_KPITCH = 136;              // elements per staged key row: 128 dims + 8 (68 dwords: 16 rows x 16 bytes hit 64 distinct banks)
 constexpr float PF_LOG2E = 1.4426950408889634f;
 
@@ -91,8 +93,12 @@ template <int G>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
                                                              uint16_t* __restrict__ y, int n_q, int t_kv, int n_tokens, int pos0, float scale)
 {
+    constexpr int H = G >= 2 ? 2 : 1;           // query heads per wave
+    constexpr int NW = 2 * (G / H);             // waves that compute: (head group, key half)
+    static_assert(G == 1 || G == 2 || G == 4, "query heads per kv head");
     __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KEYS * PF_KPITCH];   // [key][dim] of two blocks
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][128 * PF_PITCH];        // [dim][key] of two blocks
+    __shared__ float2 stat[4][H][16];                                              // (max, sum) per wave, head and token
     // Consecutive workgroups go to the eight XCDs in turn, each with an L2 of its own: with the kv head as the fastest index
     // an XCD serves few heads (one, with eight of them) and their keys and values stay in its L2 for all token tiles.
     const int n_kv = n_q / G;
@@ -104,18 +110,24 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __
     const int n_keys = pos0 + last_token + 1;                   // keys this workgroup can see
     const int n_written = pos0 + n_tokens;                      // cache rows holding data
     const int n_blocks = (n_keys + PF_KEYS - 1) / PF_KEYS;
-    const bool active = wave < G;
+    const bool active = wave < NW;
+    const int hg = wave >> 1, kh = wave & 1;                    // head group; which 32 keys of every block
+    const int head0 = kvh * G + hg * H;                         // first of the wave's heads
     const uint16_t* kbase = k_cache + (size_t)kvh * t_kv * 128;
     const uint16_t* vbase = v_cache + (size_t)kvh * t_kv * 128;
 
-    // the query operand: token j's head, dims 32 c + 8 g .. + 7
-    u32x4 qf[4];
+    // the query operands: token j, head head0 + h, dims 32 c + 8 g .. + 7
+    u32x4 qf[H][4];
     const int my_pos = pos0 + min(t0 + j, n_tokens - 1);
     if (active)
     {
-        const uint16_t* qrow = q + ((size_t)min(t0 + j, n_tokens - 1) * n_q + kvh * G + wave) * 128 + g * 8;
 #pragma unroll
-        for (int c = 0; c < 4; c++) { qf[c] = *(const u32x4*)(qrow + c * 32); }
+        for (int h = 0; h < H; h++)
+        {
+            const uint16_t* qrow = q + ((size_t)min(t0 + j, n_tokens - 1) * n_q + head0 + h) * 128 + g * 8;
+#pragma unroll
+            for (int c = 0; c < 4; c++) { qf[h][c] = *(const u32x4*)(qrow + c * 32); }
+        }
     }
     // staging: a thread moves two 16-byte pieces (dims 8 c .. + 7 and 64 + 8 c .. + 7, c = thread / 32) of two rows (keys
     // 2 p, 2 p + 1 of the block, p = thread % 32): raw[2 i], raw[2 i + 1] are the two rows' pieces i.  A block index past the
@@ -174,56 +186,65 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __
             }
         }
     };
-    // raw scores of a staged block's four key tiles (16 keys each) against the token tile: for tile kt the lane gets keys
-    // kt * 16 + 4 g + v, v = 0..3, of token j.  All sixteen key operands are read first and the products run over the
-    // tiles inside each 32-dim step, so that consecutive matrix-core instructions never wait for each other's sums.
-    auto score_products = [&](int buf, f32x4 (&acc)[PF_KEYS / 16]) {
-        u32x4 kf[PF_KEYS / 16][4];
+    // raw scores of the wave's two key tiles (keys 32 kh + 16 kt + ..) of a staged block against the token tile, for its H
+    // heads: for tile kt the lane gets keys 32 kh + 16 kt + 4 g + v, v = 0..3, of token j.  A key operand read from LDS
+    // serves H products; all eight are read first and the products run over tiles and heads inside each 32-dim step, so
+    // that consecutive matrix-core instructions never wait for each other's sums.
+    auto score_products = [&](int buf, f32x4 (&acc)[H][2]) {
+        u32x4 kf[2][4];
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++)
+        for (int kt = 0; kt < 2; kt++)
         {
-            const uint16_t* krow = ks[buf] + (kt * 16 + j) * PF_KPITCH + g * 8;
+            const uint16_t* krow = ks[buf] + (kh * 32 + kt * 16 + j) * PF_KPITCH + g * 8;
 #pragma unroll
             for (int c = 0; c < 4; c++) { kf[kt][c] = *(const u32x4*)(krow + c * 32); }
         }
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++) { acc[kt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) { acc[h][kt] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
 #pragma unroll
         for (int c = 0; c < 4; c++)
 #pragma unroll
-            for (int kt = 0; kt < PF_KEYS / 16; kt++)
-            {
-                acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt][c]), __builtin_bit_cast(bf16x8, qf[c]), acc[kt], 0, 0, 0);
-            }
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int h = 0; h < H; h++)
+                {
+                    acc[h][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt][c]), __builtin_bit_cast(bf16x8, qf[h][c]), acc[h][kt], 0, 0, 0);
+                }
     };
     // scaled, rounded to BF16 by the hardware conversion (round to nearest even, as the integer trick rounds finite
     // values) and masked: only blocks that reach past the workgroup's first token need the test
-    auto score_round = [&](const f32x4 (&acc)[PF_KEYS / 16], int b, auto masked_c, float (&s)[PF_KEYS / 16][4]) {
+    auto score_round = [&](const f32x4 (&acc)[H][2], int b, auto masked_c, float (&s)[H][2][4]) {
         constexpr bool masked = decltype(masked_c)::value;
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++)
-        {
-            const f32x4 a = acc[kt];
-            const uint32_t w01 = pf_pack_bf16(scale * a[0], scale * a[1]), w23 = pf_pack_bf16(scale * a[2], scale * a[3]);
-            s[kt][0] = __builtin_bit_cast(float, w01 << 16);
-            s[kt][1] = __builtin_bit_cast(float, w01 & 0xFFFF0000u);
-            s[kt][2] = __builtin_bit_cast(float, w23 << 16);
-            s[kt][3] = __builtin_bit_cast(float, w23 & 0xFFFF0000u);
-            if (masked)
-            {
+        for (int h = 0; h < H; h++)
 #pragma unroll
-                for (int v = 0; v < 4; v++)
+            for (int kt = 0; kt < 2; kt++)
+            {
+                const f32x4 a = acc[h][kt];
+                const uint32_t w01 = pf_pack_bf16(scale * a[0], scale * a[1]), w23 = pf_pack_bf16(scale * a[2], scale * a[3]);
+                s[h][kt][0] = __builtin_bit_cast(float, w01 << 16);
+                s[h][kt][1] = __builtin_bit_cast(float, w01 & 0xFFFF0000u);
+                s[h][kt][2] = __builtin_bit_cast(float, w23 << 16);
+                s[h][kt][3] = __builtin_bit_cast(float, w23 & 0xFFFF0000u);
+                if (masked)
                 {
-                    if (b * PF_KEYS + kt * 16 + 4 * g + v > my_pos) { s[kt][v] = -INFINITY; }
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (b * PF_KEYS + kh * 32 + kt * 16 + 4 * g + v > my_pos) { s[h][kt][v] = -INFINITY; }
+                    }
                 }
             }
-        }
     };
 
-    // ---- pass 1: row maximum and sum of exp(s - max)
-    float m = -INFINITY, l = 0.0f;
+    // ---- pass 1: row maximum and sum of exp(s - max), per lane over its keys
+    float m[H], l[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) { m[h] = -INFINITY; l[h] = 0.0f; }
     u32x4 kraw[4], vraw[4];
-    f32x4 cur[PF_KEYS / 16], next[PF_KEYS / 16];
+    f32x4 cur[H][2], next[H][2];
     // blocks 0 .. n_plain - 1 end at or before the first token's position and need no mask test (one or two blocks do)
     const int n_plain = min((pos0 + t0 + 1) / PF_KEYS, n_blocks);
     // prologue: block 0 staged and multiplied, block 1 staged, block 2 on its way
@@ -240,50 +261,73 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __
         if (active)
         {
             score_products((b + 1) & 1, next);
-            float s[PF_KEYS / 16][4];
+            float s[H][2][4];
             score_round(cur, b, masked_c, s);
-            float bm = -INFINITY;
 #pragma unroll
-            for (int kt = 0; kt < PF_KEYS / 16; kt++)
+            for (int h = 0; h < H; h++)
+            {
+                float bm = -INFINITY;
 #pragma unroll
-                for (int v = 0; v < 4; v++) { bm = fmaxf(bm, s[kt][v]); }
-            const float nm = fmaxf(m, bm);
-            // nm = -inf: nothing visible to this lane yet, every term below is 2^(-inf) = 0 with the offset at 0
-            const float off = nm > -INFINITY ? -nm * PF_LOG2E : 0.0f;
-            l = nm == m ? l : l * pf_exp2(fmaf(m, PF_LOG2E, off));
-            m = nm;
-            float sum = 0.0f;
+                for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-            for (int kt = 0; kt < PF_KEYS / 16; kt++)
+                    for (int v = 0; v < 4; v++) { bm = fmaxf(bm, s[h][kt][v]); }
+                const float nm = fmaxf(m[h], bm);
+                // nm = -inf: nothing visible to this lane yet, every term below is 2^(-inf) = 0 with the offset at 0
+                const float off = nm > -INFINITY ? -nm * PF_LOG2E : 0.0f;
+                l[h] = nm == m[h] ? l[h] : l[h] * pf_exp2(fmaf(m[h], PF_LOG2E, off));
+                m[h] = nm;
+                float sum = 0.0f;
 #pragma unroll
-                for (int v = 0; v < 4; v++) { sum += pf_exp2(fmaf(s[kt][v], PF_LOG2E, off)); }
-            l += sum;
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) { sum += pf_exp2(fmaf(s[h][kt][v], PF_LOG2E, off)); }
+                l[h] += sum;
+            }
         }
         store_keys(b & 1, b + 2, kraw);                         // block b's buffer: its reads ended before the last barrier
         load_rows(kbase, b + 3, kraw);
         lds_barrier();
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++) { cur[kt] = next[kt]; }
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) { cur[h][kt] = next[h][kt]; }
     };
     // two copies of the iteration, with and without the mask test, each one straight run of instructions
     for (int b = 0; b < n_plain; b++) { pass1_block(b, std::false_type{}); }
     for (int b = n_plain; b < n_blocks; b++) { pass1_block(b, std::true_type{}); }
-    // merge the four lane groups of a token (lanes j, j + 16, j + 32, j + 48)
+    // merge the four lane groups of a token (lanes j, j + 16, j + 32, j + 48), then the two waves of a head group
+    auto merge = [&](float& ma, float& la, float mb, float lb) {
+        const float nm = fmaxf(ma, mb);
+        if (nm > -INFINITY) { la = la * pf_exp2((ma - nm) * PF_LOG2E) + lb * pf_exp2((mb - nm) * PF_LOG2E); }
+        ma = nm;
+    };
 #pragma unroll
-    for (int off = 16; off < 64; off <<= 1)
+    for (int h = 0; h < H; h++)
     {
-        const float om = __shfl_xor(m, off), ol = __shfl_xor(l, off);
-        const float nm = fmaxf(m, om);
-        if (nm > -INFINITY) { l = l * pf_exp2((m - nm) * PF_LOG2E) + ol * pf_exp2((om - nm) * PF_LOG2E); }
-        m = nm;
-    }
-    // p = 2^(s log2 e - (m log2 e + log2 l)): the division by the sum rides in the exponent
-    const float poff = l > 0.0f ? -(m * PF_LOG2E + __builtin_amdgcn_logf(l)) : -INFINITY;
-
-    // ---- pass 2: probabilities and P V
-    f32x4 out[8];
 #pragma unroll
-    for (int d = 0; d < 8; d++) { out[d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+        for (int off = 16; off < 64; off <<= 1) { merge(m[h], l[h], __shfl_xor(m[h], off), __shfl_xor(l[h], off)); }
+        if (active && g == 0) { stat[wave][h][j] = make_float2(m[h], l[h]); }
+    }
+    lds_barrier();
+    float poff[H];
+#pragma unroll
+    for (int h = 0; h < H; h++)
+    {
+        if (active)
+        {
+            const float2 other = stat[wave ^ 1][h][j];
+            merge(m[h], l[h], other.x, other.y);
+        }
+        // p = 2^(s log2 e - (m log2 e + log2 l)): the division by the sum rides in the exponent
+        poff[h] = l[h] > 0.0f ? -(m[h] * PF_LOG2E + __builtin_amdgcn_logf(l[h])) : -INFINITY;
+    }
+
+    // ---- pass 2: probabilities and P V, per wave over its half of the keys
+    f32x4 out[H][8];
+#pragma unroll
+    for (int h = 0; h < H; h++)
+#pragma unroll
+        for (int d = 0; d < 8; d++) { out[h][d] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
     load_rows(kbase, 0, kraw);
     load_rows(vbase, 0, vraw);
     store_keys(0, 0, kraw);
@@ -300,44 +344,41 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __
         if (active)
         {
             score_products((b + 1) & 1, next);
-            float s[PF_KEYS / 16][4];
+            // value operands (dim 16 d + j, the lane's eight keys 32 kh + 4 g .. + 3 and + 16) are read ahead of their use
+            u32x4 vf[8];
+#pragma unroll
+            for (int d = 0; d < 8; d++)
+            {
+                const uint16_t* vrow = vt[b & 1] + (16 * d + j) * PF_PITCH + kh * 32 + 4 * g;
+                const uint2 va = *(const uint2*)vrow, vb = *(const uint2*)(vrow + 16);
+                vf[d] = u32x4{ va.x, va.y, vb.x, vb.y };
+            }
+            float s[H][2][4];
             score_round(cur, b, masked_c, s);
             // 2^(-inf) is 0: a masked key gets probability 0 without a test; the pairs are rounded and packed by one conversion each
-            bf16x8 pa[PF_KEYS / 32];
 #pragma unroll
-            for (int slab = 0; slab < PF_KEYS / 32; slab++)
+            for (int h = 0; h < H; h++)
             {
                 uint32_t pw[4];
 #pragma unroll
-                for (int h = 0; h < 2; h++)
+                for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                     for (int v = 0; v < 2; v++)
                     {
-                        const float* sv = s[2 * slab + h];
-                        const bf16x2 pp = { (__bf16)pf_exp2(fmaf(sv[2 * v], PF_LOG2E, poff)), (__bf16)pf_exp2(fmaf(sv[2 * v + 1], PF_LOG2E, poff)) };
-                        pw[2 * h + v] = __builtin_bit_cast(uint32_t, pp);
+                        const float* sv = s[h][kt];
+                        // (converted by the compiler's own instruction, not pf_pack_bf16: the result feeds a matrix-core instruction, and
+                        // only for instructions it knows does the compiler keep the wait states between the two)
+                        const bf16x2 pp = { (__bf16)pf_exp2(fmaf(sv[2 * v], PF_LOG2E, poff[h])), (__bf16)pf_exp2(fmaf(sv[2 * v + 1], PF_LOG2E, poff[h])) };
+                        pw[2 * kt + v] = __builtin_bit_cast(uint32_t, pp);
                     }
-                const u32x4 pvec = { pw[0], pw[1], pw[2], pw[3] };      // keys 4 g .. + 3, then 16 + 4 g .. + 3 of the slab
-                pa[slab] = __builtin_bit_cast(bf16x8, pvec);
+                const u32x4 pvec = { pw[0], pw[1], pw[2], pw[3] };      // keys 4 g .. + 3, then 16 + 4 g .. + 3 of the wave's 32
+                const bf16x8 pa = __builtin_bit_cast(bf16x8, pvec);
+#pragma unroll
+                for (int d = 0; d < 8; d++)
+                {
+                    out[h][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8, vf[d]), out[h][d], 0, 0, 0);
+                }
             }
-            // value operands (dim 16 d + j, the same eight keys) of both slabs are read before the first product
-            u32x4 vf[PF_KEYS / 32][8];
-#pragma unroll
-            for (int slab = 0; slab < PF_KEYS / 32; slab++)
-#pragma unroll
-                for (int d = 0; d < 8; d++)
-                {
-                    const uint16_t* vrow = vt[b & 1] + (16 * d + j) * PF_PITCH + slab * 32 + 4 * g;
-                    const uint2 va = *(const uint2*)vrow, vb = *(const uint2*)(vrow + 16);
-                    vf[slab][d] = u32x4{ va.x, va.y, vb.x, vb.y };
-                }
-#pragma unroll
-            for (int slab = 0; slab < PF_KEYS / 32; slab++)
-#pragma unroll
-                for (int d = 0; d < 8; d++)
-                {
-                    out[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[slab], __builtin_bit_cast(bf16x8, vf[slab][d]), out[d], 0, 0, 0);
-                }
         }
         store_keys(b & 1, b + 2, kraw);
         store_values((b + 1) & 1, b + 1, vraw);                 // held value block b - 1, read before the last barrier
@@ -345,22 +386,41 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const uint16_t* __
         load_rows(vbase, b + 2, vraw);
         lds_barrier();
 #pragma unroll
-        for (int kt = 0; kt < PF_KEYS / 16; kt++) { cur[kt] = next[kt]; }
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) { cur[h][kt] = next[h][kt]; }
     };
     for (int b = 0; b < n_plain; b++) { pass2_block(b, std::false_type{}); }
     for (int b = n_plain; b < n_blocks; b++) { pass2_block(b, std::true_type{}); }
-    if (!active) { return; }
-    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3 of the tile
-#pragma unroll
-    for (int d = 0; d < 8; d++)
+    // the two key halves of a head group meet in LDS (the staging buffers are free now): lane-major, so that consecutive
+    // lanes touch consecutive words
+    float* red = (float*)&ks[0][0];
+    static_assert(sizeof(ks) >= (size_t)(NW / 2) * H * 8 * 4 * 64 * sizeof(float), "reduction buffer");
+    if (active && kh == 1)
     {
 #pragma unroll
-        for (int v = 0; v < 4; v++)
-        {
-            const int t = t0 + 4 * g + v;
-            if (t < n_tokens) { y[((size_t)t * n_q + kvh * G + wave) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(out[d][v]); }
-        }
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int d = 0; d < 8; d++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) { red[(((hg * H + h) * 8 + d) * 4 + v) * 64 + lane] = out[h][d][v]; }
     }
+    lds_barrier();
+    if (!active || kh == 1) { return; }
+    // D of the last product: lane (dim = 16 d + j, g) holds tokens 4 g .. 4 g + 3 of the tile
+#pragma unroll
+    for (int h = 0; h < H; h++)
+#pragma unroll
+        for (int d = 0; d < 8; d++)
+        {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+            {
+                const int t = t0 + 4 * g + v;
+                const float sum = out[h][d][v] + red[(((hg * H + h) * 8 + d) * 4 + v) * 64 + lane];
+                if (t < n_tokens) { y[((size_t)t * n_q + head0 + h) * 128 + 16 * d + j] = (uint16_t)f32_to_bf16_bits(sum); }
+            }
+        }
 }
 
 // ------------------------------------------------------------------------------------------
