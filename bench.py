@@ -43,7 +43,7 @@ TRAFFIC_SOURCE = "constant copied from the rocprofv3 --pmc FETCH_SIZE / WRITE_SI
 
 FLOAT, HALF, BF16, E4M3, E5M2, FP4 = 0, 2, 3, 4, 5, 6
 
-QWEN3_8B = dict(layers=36, hidden=4096, q_out=4096, kv_out=1024, inter=12288, vocab=151936)
+QWEN3_8B = dict(layers=36, hidden=4096, n_q=32, n_kv=8, q_out=4096, kv_out=1024, inter=12288, vocab=151936)
 QWEN_SHAPES = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096), (4096, 151936)]     # (K, N)
 
 
@@ -221,7 +221,7 @@ def build_decode_step(ws: Workspace, ctx: int):
 LLAMA31_8B = dict(layers=32, hidden=4096, n_q=32, n_kv=8, q_out=4096, kv_out=1024, inter=14336, vocab=128256, theta=5e5)
 
 
-def build_llama_fp4_step(ws: Workspace, ctx: int, block: int = 16):
+def build_llama_fp4_step(ws: Workspace, ctx: int, block: int = 16, repack: bool = False):
     """Random-init Llama-3.1-8B-shaped model with FP4_E2M1 block-scale linears (the reference's Llama FP4 route: codes and
     one E4M3 scale byte per 16 elements as scripts/convert_weights.py:346-370 packs them), no per-head q/k norms, RoPE
     theta 5e5, BF16 embedding and a KV cache already holding `ctx` positions.  Codes and scale bytes are uniform random
@@ -231,6 +231,7 @@ def build_llama_fp4_step(ws: Workspace, ctx: int, block: int = 16):
     t, c = ws.torch, LLAMA31_8B
     model = ws.pkg.host_api.DecodeModel(ws.host, c["layers"], c["hidden"], c["n_q"], c["n_kv"], 128, c["inter"], c["vocab"], ctx, theta=c["theta"])
     model.set_qk_norm(False)
+    model.set_repack_linears(repack)            # tiled copies beside the file layout: what the prompt phase's FP4 GEMM reads
     rng = np.random.default_rng(4321)
     shapes = {"wq": (c["q_out"], c["hidden"]), "wk": (c["kv_out"], c["hidden"]), "wv": (c["kv_out"], c["hidden"]),
               "wo": (c["hidden"], c["q_out"]), "w_gate": (c["inter"], c["hidden"]), "w_up": (c["inter"], c["hidden"]),
@@ -276,9 +277,9 @@ def llama_fp4_step_bytes(ctx_mean: float, block: int = 16) -> int:
     return elems // 2 + elems // block + kv + small
 
 
-def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool):
+def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool, repack: bool = False):
     """The FP4 decode step as a benchmark entry: tokens / s of the Llama-3.1-8B-shaped model at context DECODE_CTX."""
-    model = build_llama_fp4_step(ws, DECODE_CTX)
+    model = build_llama_fp4_step(ws, DECODE_CTX, repack=repack)
     start = DECODE_CTX - steps - warmup
     ws.torch.cuda.synchronize()
     model.reset(1, start)
@@ -296,13 +297,13 @@ def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool):
     return entry, model
 
 
-def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, layout: str = "row-major"):
+def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, layout: str = "row-major", c=None):
     """The prompt phase of the same model (DecodeModel::prefill, positions 0 .. T - 1): every linear is one quantized GEMM
     with T columns -- BASELINE config 4's kernel on all seven shapes of a layer, on the row-major file bytes (a batch-1
     DecodeModel keeps no tiled copies) -- with the row kernels and the causal attention between them.  Wall clock around the
     call, device synchronised on both sides; best of `reps` after one warm-up call (which also allocates the activations)."""
     import numpy as np
-    t, c = ws.torch, QWEN3_8B
+    t, c = ws.torch, (c or QWEN3_8B)
     lin_elems = c["layers"] * (c["hidden"] * (c["q_out"] + 2 * c["kv_out"]) + c["q_out"] * c["hidden"] + 3 * c["hidden"] * c["inter"])
     out = []
     for T in token_counts:
@@ -317,7 +318,7 @@ def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, 
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
         # linears 2 T K N each; attention 2 * 2 * 128 * n_q per (token, visible key) pair
-        flops = 2.0 * T * lin_elems + 4.0 * 128 * 32 * c["layers"] * (T * (T + 1) / 2) + 2.0 * c["hidden"] * c["vocab"]
+        flops = 2.0 * T * lin_elems + 4.0 * 128 * c["n_q"] * c["layers"] * (T * (T + 1) / 2) + 2.0 * c["hidden"] * c["vocab"]
         out.append({"tokens": T, "weights": layout, "ms": round(best * 1e3, 3), "tok_s": round(T / best, 1), "TFLOPs": round(flops / best * 1e-12, 1),
                     "frac_of_bf16_mfma_peak": round(flops / best * 1e-12 / MFMA_BF16_PEAK_TFLOPS, 4)})
     return out
@@ -727,7 +728,7 @@ def main():
         dom_us = ws.bench.gate_up_us(model, 10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
         if not args.no_fp4_step:
-            extra["fp4_decode_step"], fp4_model = llama_fp4_decode(ws, args.steps, args.warmup, use_graph)
+            extra["fp4_decode_step"], fp4_model = llama_fp4_decode(ws, args.steps, args.warmup, use_graph, repack=not args.no_prompt)
         if not args.no_sweep:
             # Nothing is freed until the last sweep has run: on this driver, freeing a few GB of device memory slows the
             # kernels that stream through the buffers still allocated (the 253-linear chain: 1.79 -> 1.91 ms per step
@@ -757,6 +758,9 @@ def main():
                 for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
                     assert model.prepare_tiled(li, name)
             extra["prompt_phase"]["cases"] += prompt_phase(ws, model, layout="tiled copies")
+            if not args.no_fp4_step:
+                # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
+                extra["fp4_decode_step"]["prompt_phase"] = prompt_phase(ws, fp4_model, layout="tiled copies", c=LLAMA31_8B)
         del model
         if not args.no_baselines:
             torch.cuda.empty_cache()
