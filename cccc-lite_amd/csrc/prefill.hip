@@ -32,6 +32,7 @@ int hip_attention_prefill_bf16(const void* q, const void* k_cache, const void* v
     if (head_dim != 128 || n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0 || t_kv <= 0 || n_tokens <= 0) { return -1; }
     if (pos0 < 0 || (long long)pos0 + n_tokens > t_kv || n_kv_heads > 65535) { return -1; }
     if (!q || !k_cache || !v_cache || !y || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) { return -1; }
+    if ((long long)((n_tokens + 15) / 16) * n_kv_heads > 0x7FFFFFFFLL) { return -1; }
     const dim3 grid((unsigned)((n_tokens + 15) / 16) * n_kv_heads);
     const float scale = 1.0f / sqrtf(128.0f);
 #define CCQ_ATTN_PREFILL(G)                                                                                                                  \
