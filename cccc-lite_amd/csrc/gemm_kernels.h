@@ -875,16 +875,25 @@ inline bool attach_split(DirectPlan& plan, const LinearArgs& a, long long s, Spl
 
 // fp4: the FP4 kernel's costs -- the 128-token x 256-feature tile stays out of the scoring (see plan_direct_fp4), and
 // 64-token tiles pay for converting every weight for half as many products (913 against 1037 TFLOP/s at equal balance).
-inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool fp4 = false)
+// row_major (FP8 only): the weight is read from the file layout, where a wave's load is sixteen half cache lines; 64-token
+// tiles then pay that fetch for half as many products, and a 128-token tile is worth having even at one workgroup per CU
+// (4096 x 4096 at 2048 tokens: 70 us against 91; K 12288: 196 against 244; on the tiled copy the two are level).
+// 64 tokens x 128 features (FP8, K < 8192, at most 2048 features) puts 256 or more workgroups on outputs as narrow as 1024
+// features (2048 tokens: 29 / 35 us tiled / row-major against 33 / 40).  Wider outputs with few tiles keep the k split: with
+// a long K it is far ahead (K 12288 at 512 tokens: 60 against 110 us), and on 512 tokens x 4096 x 4096, where the two
+// measure the same on weights that rotate through the memory-side cache, the split is 8 us ahead inside a whole model.
+inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool fp4 = false, bool row_major = false)
 {
     const int cus = cu_count();
     const bool big_tile = !fp4;
     struct Shape { int nb, mb; double quality; };
-    const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, fp4 ? 0.88 : 1.0 }, { 3, 8, 1.0 }, { 3, 4, fp4 ? 0.84 : 0.95 } };
+    const double q64 = row_major ? 0.8 : 1.0;            // what a 64-token tile is worth against a 128-token one
+    const Shape shapes[] = { { 4, 8, 1.0 }, { 4, 4, fp4 ? 0.88 : q64 }, { 3, 8, 1.0 }, { 3, 4, fp4 ? 0.84 : 0.95 * q64 }, { 2, 4, 0.9 * q64 } };
     DirectPlan plan = { 4, 4, 1, nullptr, false };
     double best = -1.0;
     for (const Shape& sh : shapes)
     {
+        if (sh.nb == 2 && (fp4 || a.K >= 8192 || a.n_out > 2048)) { continue; }
         if (sh.mb == 8 && (a.tokens <= 64 || (sh.nb == 4 && !big_tile))) { continue; }
         const long long tiles = (long long)((a.n_out + 64 * sh.nb - 1) / (64 * sh.nb)) * ((a.tokens + 16 * sh.mb - 1) / (16 * sh.mb));
         const double balance = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
@@ -942,8 +951,8 @@ inline DirectPlan plan_direct_fp4(const LinearArgs& a, SplitScratch* scratch)
 // Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
 // kernel that keeps the weights out of LDS -- on the tiled copy of the weight when one is registered
 // (1.10-1.15x the row-major rate: a wave's load is then eight full cache lines instead of sixteen half
-// lines).  128-token tiles when they give every CU two workgroups; else 64-token tiles when those fill the
-// machine; else the k range is split over workgroups (about one per CU, 16 k-tiles or more each) and a
+// lines).  The tile shape comes from plan_direct (128- or 64-token tiles of 256, 192 or 128 features, whichever spreads
+// most evenly over the CUs); when none fills the machine the k range is split over workgroups (about one per CU, 16 k-tiles or more each) and a
 // second kernel adds the partial sums -- 2x on 512 tokens x 4096 features x K 12288.  Everything else (FP4,
 // ragged K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they
 // give every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
@@ -976,11 +985,12 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
         {
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }
-            const DirectPlan plan = plan_direct(a, scratch);
+            const DirectPlan plan = plan_direct(a, scratch, false, tiled == nullptr);
             if (plan.refused) { return false; }
             const int nb = plan.nb, mb = plan.mb, splits = plan.splits;
             float* const partial = plan.partial;
-            if (tiled)
+            if (nb == 2) { tiled ? launch_gemm_mfma_direct<WT, 4, true, AT, 2>(d) : launch_gemm_mfma_direct<WT, 4, false, AT, 2>(d); }
+            else if (tiled)
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, true, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, true, AT, 3>(d); }
                 else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial); }
