@@ -119,19 +119,22 @@ def _fresh(pkg, host, cfg):
     return pkg.host_api.DecodeModel(host, cfg.layers, cfg.hidden, cfg.n_q, cfg.n_kv, cfg.head_dim, cfg.inter, cfg.vocab, cfg.t_kv, theta=cfg.theta)
 
 
-@pytest.mark.parametrize("variant", ["qwen3 fp8", "llama fp4", "tied fp8"])
+@pytest.mark.parametrize("variant", ["qwen3 fp8", "llama fp4", "tied fp8", "qwen3 fp8 tiled", "llama fp4 tiled"])
 @pytest.mark.parametrize("T", [1, 5, 20, 60])
 def test_prompt_phase_of_the_decode_model_follows_the_oracle(gpu, pkg, oracle, dec, variant, T):
     """DecodeModel::prefill (linears through the GEMM face with T columns, row kernels between them) against the oracle
     fed the same prompt token by token: the cache rows of every layer and position, the logits after the last token and
-    the greedy pick; then three decode steps carry on from the prompt and still follow the oracle."""
+    the greedy pick; then three decode steps carry on from the prompt and still follow the oracle.  "tiled": every linear
+    keeps its load-time tiled copy, which the GEMMs and GEMVs of the prompt phase then read."""
     host = pkg.host_api.host()
     host.init(0)
-    fp4, tied = variant == "llama fp4", variant == "tied fp8"
+    fp4, tied, tiled = variant.startswith("llama fp4"), variant == "tied fp8", variant.endswith("tiled")
     cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=96, theta=5e5 if fp4 else 1e6)
     weights = dec.make_model(cfg, 53, fmt="fp4_e2m1" if fp4 else "fp8_e5m2", qk_norm=not fp4, tied=tied)
     model = _fresh(pkg, host, cfg)
+    model.set_repack_linears(tiled)
     model.load(weights)
+    assert model.prepare_tiled(1, "w_up") == tiled
     model.set_exact_attention(True)
     rng = np.random.default_rng(T)
     prompt = [int(t) for t in rng.integers(0, cfg.vocab, size=T)]
