@@ -69,6 +69,7 @@ EXPORTS = (
     "hip_attention_prefill_bf16",
     "hip_add_bf16",
     "hip_swiglu_bf16",
+    "hip_add_rms_norm_bf16",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_argmax_pick_embed_bf16",
@@ -145,6 +146,8 @@ class QuantLibrary:
         L.hip_add_bf16.argtypes = [vp, vp, vp, ctypes.c_ulonglong]
         L.hip_swiglu_bf16.restype = i32
         L.hip_swiglu_bf16.argtypes = [vp, vp, vp, ctypes.c_ulonglong]
+        L.hip_add_rms_norm_bf16.restype = i32
+        L.hip_add_rms_norm_bf16.argtypes = [vp, vp, vp, vp, vp, u32, u32, ctypes.c_float]
         L.hip_attention_decode_workspace_bytes.restype = ctypes.c_ulonglong
         L.hip_attention_decode_workspace_bytes.argtypes = [i32, i32, i32]
         L.hip_argmax_workspace_bytes.restype = ctypes.c_ulonglong

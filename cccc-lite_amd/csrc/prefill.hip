@@ -19,8 +19,8 @@ int hip_qk_norm_rope_kv_rows_bf16(const void* q, const void* k, const void* v, c
     if (pos0 < 0 || (long long)pos0 + n_tokens > t_kv) { return -1; }
     if (!q || !k || !v || !cos_tab || !sin_tab || !q_out || !k_cache || !v_cache) { return -1; }
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) { return -1; }
-    const dim3 grid(n_q_heads + 2 * n_kv_heads, n_tokens);
-    qk_norm_rope_kv_rows_kernel<<<grid, 64, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_norm_w,
+    const dim3 grid((n_q_heads + 2 * n_kv_heads + 3) / 4, n_tokens);
+    qk_norm_rope_kv_rows_kernel<<<grid, 256, 0, stream()>>>((const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_norm_w,
                                                            (const uint16_t*)k_norm_w, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab,
                                                            (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, n_q_heads, n_kv_heads, t_kv, pos0, epsilon);
     return finish("qk_norm_rope_kv_rows");
@@ -56,6 +56,15 @@ int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n)
     const long long blocks = (chunks + 255) / 256, cap = (long long)cu_count() * 16;
     add_rows_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>((const u32x4*)a, (const u32x4*)b, (u32x4*)y, chunks);
     return finish("add_bf16");
+}
+
+int hip_add_rms_norm_bf16(const void* a, const void* b, void* sum, const void* norm_w, void* y, unsigned int rows, unsigned int inner, float epsilon)
+{
+    if (!a || !b || !sum || !norm_w || !y || rows == 0 || inner == 0 || inner % 8 != 0 || inner > 64u * 8u * RMS_CHUNKS) { return -1; }
+    if (!aligned16(a) || !aligned16(b) || !aligned16(sum) || !aligned16(norm_w) || !aligned16(y)) { return -1; }
+    add_rms_norm_rows_kernel<<<(rows + 3) / 4, 256, 0, stream()>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)sum, (const uint16_t*)norm_w,
+                                                                   (uint16_t*)y, rows, inner, epsilon);
+    return finish("add_rms_norm_bf16");
 }
 
 int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n)

@@ -14,25 +14,27 @@ namespace ccq
 {
 
 // ------------------------------------------------------------------------------------------
-// Per-head q/k RMSNorm + RoPE + cache append for T tokens.  Grid (n_q + 2 n_kv, T), one wave per (head, token).
+// Per-head q/k RMSNorm + RoPE + cache append for T tokens.  Grid (ceil((n_q + 2 n_kv) / 4), T), one wave per (head, token)
+// and four of them per workgroup (one wave per workgroup -- 98 k tiny workgroups for 2048 tokens -- ran at a quarter of
+// the rate).  The arithmetic per head is the one-token kernel's, lane for lane.
 //   q [T][n_q][128] -> q_out [T][n_q][128];  k [T][n_kv][128] -> k_cache[h][pos0 + t];  v -> v_cache[h][pos0 + t]
 // q_norm_w == nullptr: no per-head norm (both or neither).
-static __global__ __launch_bounds__(64) void qk_norm_rope_kv_rows_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
-                                                                 const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
-                                                                 const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab,
-                                                                 uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
-                                                                 int n_q, int n_kv, int t_kv, int pos0, float eps)
+static __global__ __launch_bounds__(256) void qk_norm_rope_kv_rows_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                                                                  const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
+                                                                  const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab,
+                                                                  uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+                                                                  int n_q, int n_kv, int t_kv, int pos0, float eps)
 {
-    const int head = blockIdx.x, t = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int head = blockIdx.x * 4 + (threadIdx.x >> 6), t = blockIdx.y;
+    const int lane = threadIdx.x & 63;
     const int pos = pos0 + t;
+    if (head >= n_q + 2 * n_kv) { return; }
     if (head >= n_q + n_kv)
     {
         const int h = head - n_q - n_kv;
-        const uint16_t* src = v + ((size_t)t * n_kv + h) * 128;
-        uint16_t* dst = v_cache + ((size_t)h * t_kv + pos) * 128;
+        const uint32_t* src = (const uint32_t*)(v + ((size_t)t * n_kv + h) * 128);
+        uint32_t* dst = (uint32_t*)(v_cache + ((size_t)h * t_kv + pos) * 128);
         dst[lane] = src[lane];
-        dst[lane + 64] = src[lane + 64];
         return;
     }
     const bool is_q = head < n_q;
@@ -462,6 +464,47 @@ static __global__ __launch_bounds__(256) void swiglu_rows_kernel(const u32x4* __
             o[d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
         }
         y[c] = o;
+    }
+}
+
+// r = bf16(a + b) and y = rmsnorm(r) * w for rows of at most 4096 values (a multiple of 8): the residual add and the norm
+// that follows it in one pass, with add_rows_kernel's rounding and rms_norm_rows_kernel's arithmetic (a wave per row, the
+// row stays in registers, the same order of the sum of squares), so the pair gives the same bits as the two launches.
+static __global__ __launch_bounds__(256) void add_rms_norm_rows_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ R,
+                                                               const uint16_t* __restrict__ scale, uint16_t* __restrict__ Y, unsigned outer, unsigned inner, float eps)
+{
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= outer) { return; }
+    const size_t base = (size_t)row * inner;
+    const unsigned n_chunks = inner / 8u;                   // 16-byte chunks of the row; chunk c belongs to lane c % 64
+    u32x4 v[RMS_CHUNKS];
+    float sumsq = 0.0f;
+#pragma unroll
+    for (int j = 0; j < RMS_CHUNKS; j++)
+    {
+        const unsigned c = lane + 64u * j;
+        v[j] = u32x4{ 0u, 0u, 0u, 0u };
+        if (c < n_chunks)
+        {
+            const u32x4 va = *(const u32x4*)(A + base + c * 8u), vb = *(const u32x4*)(B + base + c * 8u);
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+            {
+                const float lo = bf16_bits_to_f32(va[d] & 0xFFFFu) + bf16_bits_to_f32(vb[d] & 0xFFFFu);
+                const float hi = bf16_bits_to_f32(va[d] >> 16) + bf16_bits_to_f32(vb[d] >> 16);
+                v[j][d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+            }
+            *(u32x4*)(R + base + c * 8u) = v[j];
+        }
+        sumsq += sumsq8(v[j]);
+    }
+    const float invstd = rsqrtf(wave_sum(sumsq) / (float)inner + eps);
+#pragma unroll
+    for (int j = 0; j < RMS_CHUNKS; j++)
+    {
+        const unsigned c = lane + 64u * j;
+        if (c < n_chunks) { *(u32x4*)(Y + base + c * 8u) = normed8(v[j], *(const u32x4*)(scale + c * 8u), invstd); }
     }
 }
 

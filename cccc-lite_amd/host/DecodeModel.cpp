@@ -433,10 +433,17 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
     auto norm = [&](Matrix& x, Matrix& y, Matrix& w) {
         return hip_rms_norm_fwd((int)BFLOAT16, x.data(), y.data(), w.data(), nullptr, (unsigned)n, (unsigned)c.hidden, c.eps);
     };
+    // a residual add and the norm behind it go out as one launch where the row fits the kernel (hidden <= 4096)
+    const bool fused_norm = c.hidden % 8 == 0 && c.hidden <= 4096;
+    auto add_norm = [&](Matrix& a, Matrix& b, Matrix& sum, Matrix& w, Matrix& y) {
+        if (fused_norm) { return hip_add_rms_norm_bf16(a.data(), b.data(), sum.data(), w.data(), y.data(), (unsigned)n, (unsigned)c.hidden, c.eps); }
+        const int r = hip_add_bf16(a.data(), b.data(), sum.data(), (unsigned long long)n * c.hidden);
+        return r != 0 ? r : norm(sum, y, w);
+    };
+    if (rc == 0 && c.layers > 0) { rc = norm(*pf_.x, *pf_.xn, *layers_[0].rms_attn); }
     for (int li = 0; li < c.layers && rc == 0; li++)
     {
         Layer& L = layers_[li];
-        rc = norm(*pf_.x, *pf_.xn, *L.rms_attn);
         if (rc == 0) { rc = linear(*L.wq, q_out, c.hidden, *pf_.xn, *pf_.q); }
         if (rc == 0) { rc = linear(*L.wk, kv_out, c.hidden, *pf_.xn, *pf_.k); }
         if (rc == 0) { rc = linear(*L.wv, kv_out, c.hidden, *pf_.xn, *pf_.v); }
@@ -452,13 +459,14 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
                                             c.n_q, c.n_kv, c.head_dim, c.t_kv, n, pos0);
         }
         if (rc == 0) { rc = linear(*L.wo, c.hidden, q_out, *pf_.att, *pf_.o); }
-        if (rc == 0) { rc = hip_add_bf16(pf_.x->data(), pf_.o->data(), pf_.r1->data(), (unsigned long long)n * c.hidden); }
-        if (rc == 0) { rc = norm(*pf_.r1, *pf_.xn, *L.rms_ffn); }
+        if (rc == 0) { rc = add_norm(*pf_.x, *pf_.o, *pf_.r1, *L.rms_ffn, *pf_.xn); }
         if (rc == 0) { rc = linear(*L.w_gate, c.inter, c.hidden, *pf_.xn, *pf_.gate); }
         if (rc == 0) { rc = linear(*L.w_up, c.inter, c.hidden, *pf_.xn, *pf_.up); }
         if (rc == 0) { rc = hip_swiglu_bf16(pf_.gate->data(), pf_.up->data(), pf_.gated->data(), (unsigned long long)n * c.inter); }
         if (rc == 0) { rc = linear(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.o); }
-        if (rc == 0) { rc = hip_add_bf16(pf_.r1->data(), pf_.o->data(), pf_.x->data(), (unsigned long long)n * c.hidden); }
+        // x = r1 + ffn, and the next layer's first norm with it (the head normalises the last token's row itself)
+        if (rc == 0 && li + 1 < c.layers) { rc = add_norm(*pf_.r1, *pf_.o, *pf_.x, *layers_[li + 1].rms_attn, *pf_.xn); }
+        else if (rc == 0) { rc = hip_add_bf16(pf_.r1->data(), pf_.o->data(), pf_.x->data(), (unsigned long long)n * c.hidden); }
     }
     if (rc != 0 || !last) { return rc; }
     // the head runs on the last token's state: its greedy pick becomes the current token at position pos0 + n

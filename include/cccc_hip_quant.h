@@ -272,6 +272,11 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
  * :953-966; cccc/MatrixEx.cpp:756-762). */
 C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
 C_EXPORT int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n);
+/* sum = bf16(a + b) and y = rmsnorm(sum) * norm_w, rows of `inner` BF16 values (a multiple of 8, at most 4096; 16-byte
+ * aligned pointers, else -1): hip_add_bf16 followed by hip_rms_norm_fwd in one pass, the same bits.  `sum` and `y` are
+ * buffers of their own.  The residual add and the norm behind it in the reference's graph (hip_functions.cpp:895-908, :1506-1535). */
+C_EXPORT int hip_add_rms_norm_bf16(const void* a, const void* b, void* sum, const void* norm_w, void* y,
+                                   unsigned int rows, unsigned int inner, float epsilon);
 
 /* Embedding row of token *d_token (int32 in device memory) -> y bf16 [D]. */
 C_EXPORT int hip_embed_token_bf16(const void* d_token, const void* W, void* y, int D, int n_rows);

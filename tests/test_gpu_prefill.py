@@ -91,6 +91,27 @@ def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n
     assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), 3 * n_kv, n_kv, 128, t_kv, T, pos0) == -1
 
 
+@pytest.mark.parametrize("rows,inner", [(1, 256), (7, 4096), (130, 1024), (5, 136)])
+def test_add_and_rms_norm_in_one_pass_equals_the_two_calls(gpu, oracle, dec, rows, inner):
+    """hip_add_rms_norm_bf16 against hip_add_bf16 followed by hip_rms_norm_fwd on the same inputs: both outputs byte for
+    byte; rows that do not fit the kernel (longer than 4096, not a multiple of 8) are refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(rows + inner)
+    a = oracle.f32_to_bf16(rng.standard_normal((rows, inner)).astype(np.float32))
+    b = oracle.f32_to_bf16((rng.standard_normal((rows, inner)) * 3).astype(np.float32))
+    w = oracle.f32_to_bf16((1.0 + 0.1 * rng.standard_normal(inner)).astype(np.float32))
+    ad, bd, wd = to_dev(torch, dev, a), to_dev(torch, dev, b), to_dev(torch, dev, w)
+    s1, y1, s2, y2 = (torch.zeros(rows * inner + 64, dtype=torch.int16, device=dev) for _ in range(4))
+    assert lib.c.hip_add_bf16(ptr(ad), ptr(bd), ptr(s1), rows * inner) == 0
+    assert lib.c.hip_rms_norm_fwd(oracle.BF16, ptr(s1), ptr(y1), ptr(wd), None, rows, inner, ctypes.c_float(1e-6)) == 0
+    assert lib.c.hip_add_rms_norm_bf16(ptr(ad), ptr(bd), ptr(s2), ptr(wd), ptr(y2), rows, inner, ctypes.c_float(1e-6)) == 0
+    assert np.array_equal(from_dev(s1, np.uint16), from_dev(s2, np.uint16))
+    assert np.array_equal(from_dev(y1, np.uint16), from_dev(y2, np.uint16))
+    assert from_dev(y2, np.uint16)[:rows * inner].any() and not from_dev(y2, np.uint16)[rows * inner:].any()
+    assert lib.c.hip_add_rms_norm_bf16(ptr(ad), ptr(bd), ptr(s2), ptr(wd), ptr(y2), 1, 4104, ctypes.c_float(1e-6)) == -1
+    assert lib.c.hip_add_rms_norm_bf16(ptr(ad), ptr(bd), ptr(s2), ptr(wd), ptr(y2), 1, 100, ctypes.c_float(1e-6)) == -1
+
+
 def test_residual_add_and_swiglu_rows(gpu, oracle, dec):
     torch, dev, lib = gpu
     rng = np.random.default_rng(9)
