@@ -78,7 +78,9 @@ constexpr float PF_LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Two FP32 values rounded to BF16 (nearest even) into one dword, low half first.  Spelled as the instruction because the
-// compiler, seeing the halves used separately afterwards, converts each value with an instruction of its own.
+// compiler, seeing the halves used separately afterwards, converts each value with an instruction of its own.  Only for
+// results that VALU code consumes: fed straight into a matrix-core instruction the value arrived stale in some lanes (NaN
+// rows) -- the compiler keeps the wait states between a VALU write and a matrix-core read only for instructions it knows.
 __device__ __forceinline__ uint32_t pf_pack_bf16(float lo, float hi)
 {
     uint32_t r;
