@@ -509,6 +509,49 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                       blk_scA, blk_scB, block_size, nullptr);
 }
 
+int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
+                          float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy)
+{
+    if (w_type != DT_E5M2 && w_type != DT_E4M3) { return -1; }
+    if (n_out <= 0 || tokens < 48 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
+    if (!W_gate || !W_up || !X || !Y || !aligned16(W_gate) || !aligned16(W_up) || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
+    if ((long long)n_out * ldw >= (1LL << 32) || (long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
+    LinearArgs a{};
+    a.W = (const uint8_t*)W_gate;
+    a.W_pair = (const uint8_t*)W_up;
+    a.X = (const uint16_t*)X;
+    a.Y = (uint16_t*)Y;
+    a.ldw = ldw;
+    a.ldx = ldx;
+    a.y_stride_tok = ldy;
+    a.y_stride_out = 1;
+    a.n_out = n_out;
+    a.tokens = tokens;
+    a.K = K;
+    a.w_scale = inv_scale_gate;
+    a.w_scale_pair = inv_scale_up;
+    a.alpha = 1.0f;
+    a.beta = 0.0f;
+    // both weights on their tiled copies, or both on the file layout
+    const uint8_t* tg = ccq::lookup_tiled(W_gate, w_type, n_out, K, ldw);
+    const uint8_t* tu = tg ? ccq::lookup_tiled(W_up, w_type, n_out, K, ldw) : nullptr;
+    if (tg && tu)
+    {
+        a.W = tg;
+        a.W_pair = tu;
+        note_kernel("gemm_swiglu_tiled");
+        if (w_type == DT_E5M2) { launch_gemm_mfma_direct_pair<DT_E5M2, true>(a); }
+        else { launch_gemm_mfma_direct_pair<DT_E4M3, true>(a); }
+    }
+    else
+    {
+        note_kernel("gemm_swiglu");
+        if (w_type == DT_E5M2) { launch_gemm_mfma_direct_pair<DT_E5M2, false>(a); }
+        else { launch_gemm_mfma_direct_pair<DT_E4M3, false>(a); }
+    }
+    return finish("quant_gemm_swiglu");
+}
+
 int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K, float alpha,
                            const void* A, int typeA, int lda, float invScaleA,
                            const void* B, int typeB, int ldb, float invScaleB,

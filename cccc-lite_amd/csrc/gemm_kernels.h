@@ -273,9 +273,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // the output has too few tiles to fill the machine.
 // NB: 16-feature blocks per wave (a workgroup owns 64 NB features): 4 by default; 3 or 2 give the launch more, smaller
 // workgroups when the output has too few 256-feature tiles to fill the machine evenly.
-template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4>
+// PAIR: two weights of one shape (a.W = gate, a.W_pair = up) against the same activations; a wave's first NB / 2 feature
+// blocks are gate rows, the other NB / 2 the same rows of up, and the epilogue writes the reference's SwiGLU product
+// bf16(bf16(g * bf16(sigmoid g)) * u) of the two rounded linears (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732,
+// :953-966) -- one launch instead of two GEMMs and an elementwise pass over three [tokens][n_out] matrices.  A workgroup
+// then owns 32 NB output features; alpha = 1, beta = 0, BF16.
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, float* __restrict__ partial)
 {
+    static_assert(!PAIR || (!SPLIT && NB % 2 == 0 && AT == DT_BF16), "pair: unsplit, an even number of feature blocks, BF16");
+    constexpr int NBO = PAIR ? NB / 2 : NB;     // feature blocks of a wave in the output
     constexpr int BTOK = MB * 16;               // tokens per workgroup
     constexpr int BK = 64, CPR = 8;
     constexpr int X_PER_THREAD = BTOK * CPR / 256;
@@ -292,7 +299,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     const int n_tile = blockIdx.x % n_pad;
     const int m_tile = blockIdx.x / n_pad;
     if (n_tile >= n_tiles) { return; }          // padding
-    const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
+    const int out_base = n_tile * (64 * NBO) + wave * (16 * NBO);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
     const int g = lane >> 4;
@@ -318,16 +325,18 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
     {
+        const int ob = nb % NBO;                            // feature block within the wave's output
         if (TILED)
         {
-            w_tile_base[nb] = (long long)min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1) * n_kt_total * 1024;
+            w_tile_base[nb] = (long long)min(out_base / 16 + ob, (a.n_out + 15) / 16 - 1) * n_kt_total * 1024;
             w_off[nb] = lane * 16;
         }
         else
         {
             w_tile_base[nb] = 0;
-            w_off[nb] = (uint32_t)((long long)min(out_base + nb * 16 + i16, a.n_out - 1) * a.ldw + g * 16);
+            w_off[nb] = (uint32_t)((long long)min(out_base + ob * 16 + i16, a.n_out - 1) * a.ldw + g * 16);
         }
+        if (PAIR && nb >= NBO) { w_tile_base[nb] += (long long)((intptr_t)a.W_pair - (intptr_t)a.W); }      // the up weight, addressed from the gate weight's base
     }
     uint32_t x_off[X_PER_THREAD];
 #pragma unroll
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     auto k_tile = [&](int kt, u32x4* wcur, u32x4* wnext) {
         u32x4 wf[2][NB];
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) { dequant16_fp8<WT, SCALED, AT>(wcur[nb], a.w_scale, wf[0][nb], wf[1][nb]); }
+        for (int nb = 0; nb < NB; nb++) { dequant16_fp8<WT, SCALED, AT>(wcur[nb], PAIR && nb >= NBO ? a.w_scale_pair : a.w_scale, wf[0][nb], wf[1][nb]); }
         __syncthreads();                                     // tile kt is in xs[kt & 1]; the other buffer is free
         fetch_w(kt + 1, wnext);
         const u32x4* xt = xs[kt & 1];
@@ -429,6 +438,40 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     }
 
     const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
+    if constexpr (PAIR)
+    {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+        {
+            const int tok = tok_base + mb * 16 + i16;
+            if (tok >= a.tokens) { continue; }
+#pragma unroll
+            for (int nb = 0; nb < NBO; nb++)
+            {
+                const int out = out_base + nb * 16 + 4 * g;
+                if (out >= a.n_out) { continue; }
+                uint16_t o[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                {
+                    const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc[mb][nb][v])), up = bf16_bits_to_f32(f32_to_bf16_bits(acc[mb][nb + NBO][v]));
+                    const float sig = bf16_bits_to_f32(f32_to_bf16_bits(1.0f / (1.0f + expf(-gate))));
+                    o[v] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(f32_to_bf16_bits(gate * sig)) * up);
+                }
+                uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                if (wide_store && out + 3 < a.n_out) { *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) }; }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { y[v * a.y_stride_out] = o[v]; }
+                    }
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
     {
@@ -828,6 +871,17 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
         if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
         else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
     }
+}
+
+// gate / up pair with the SwiGLU product in the epilogue: 128 tokens x 128 output features per workgroup
+template <int WT, bool TILED>
+void launch_gemm_mfma_direct_pair(const LinearArgs& a)
+{
+    const int n_tiles = (a.n_out + 127) / 128;
+    const int m_tiles = (a.tokens + 127) / 128;
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles);
+    if (a.w_scale != 1.0f || a.w_scale_pair != 1.0f) { gemm_mfma_direct_kernel<WT, true, 8, false, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+    else { gemm_mfma_direct_kernel<WT, false, 8, false, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
 }
 
 template <int WT, int BLOCK, int BM, int BN, int BK = 64, bool XCD = false, int AT = DT_BF16>

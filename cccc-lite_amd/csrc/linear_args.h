@@ -23,6 +23,10 @@ struct LinearArgs
     float w_scale;            // per-tensor dequant multiplier (invScale); ignored when blk_sc is set
     float alpha;
     float beta;
+    // gate / up pair (gemm_mfma_direct_kernel<..., PAIR>): W is the gate weight, W_pair the up weight of the same shape
+    // and layout; the output is the SwiGLU product of the two linears
+    const uint8_t* W_pair;
+    float w_scale_pair;
 };
 
 }    // namespace ccq

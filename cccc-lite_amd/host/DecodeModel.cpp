@@ -460,9 +460,20 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         }
         if (rc == 0) { rc = linear(*L.wo, c.hidden, q_out, *pf_.att, *pf_.o); }
         if (rc == 0) { rc = add_norm(*pf_.x, *pf_.o, *pf_.r1, *L.rms_ffn, *pf_.xn); }
-        if (rc == 0) { rc = linear(*L.w_gate, c.inter, c.hidden, *pf_.xn, *pf_.gate); }
-        if (rc == 0) { rc = linear(*L.w_up, c.inter, c.hidden, *pf_.xn, *pf_.up); }
-        if (rc == 0) { rc = hip_swiglu_bf16(pf_.gate->data(), pf_.up->data(), pf_.gated->data(), (unsigned long long)n * c.inter); }
+        // gate, up and their SwiGLU product: one launch for two FP8 weights of one type, else the three calls
+        int fused = -1;
+        if (rc == 0 && L.w_gate->getDataType() == L.w_up->getDataType())
+        {
+            fused = hip_quant_gemm_swiglu(c.inter, n, c.hidden, L.w_gate->data(), L.w_up->data(), (int)L.w_gate->getDataType(), c.hidden,
+                                          L.w_gate->getQuantScale(), L.w_up->getQuantScale(), pf_.xn->data(), c.hidden, pf_.gated->data(), c.inter);
+            if (fused > 0) { rc = fused; }
+        }
+        if (fused < 0)
+        {
+            if (rc == 0) { rc = linear(*L.w_gate, c.inter, c.hidden, *pf_.xn, *pf_.gate); }
+            if (rc == 0) { rc = linear(*L.w_up, c.inter, c.hidden, *pf_.xn, *pf_.up); }
+            if (rc == 0) { rc = hip_swiglu_bf16(pf_.gate->data(), pf_.up->data(), pf_.gated->data(), (unsigned long long)n * c.inter); }
+        }
         if (rc == 0) { rc = linear(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.o); }
         // x = r1 + ffn, and the next layer's first norm with it (the head normalises the last token's row itself)
         if (rc == 0 && li + 1 < c.layers) { rc = add_norm(*pf_.r1, *pf_.o, *pf_.x, *layers_[li + 1].rms_attn, *pf_.xn); }

@@ -270,6 +270,14 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
 /* y = bf16(a + b) and y = bf16(bf16(gate * bf16(sigmoid(gate))) * up) over n BF16 elements (n % 8 == 0, 16-byte aligned):
  * the residual add and the SwiGLU product with the reference's roundings (cccc-hip/hip_functions.cpp:895-908, :722-732,
  * :953-966; cccc/MatrixEx.cpp:756-762). */
+/* y[t][o] = swiglu(gate[t][o], up[t][o]) with gate = bf16(W_gate x_t), up = bf16(W_up x_t): the gate and up linears of an
+ * MLP block (two FP8 weights of one shape [n_out][K], row pitch ldw, dequantisation multipliers as in hip_quant_gemm; both
+ * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product
+ * bf16(bf16(g * bf16(sigmoid g)) * u) (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732, :953-966) in one launch, with
+ * the bits of the three calls it replaces.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).
+ * -1 (nothing launched, use the separate calls): other weight types, fewer than 48 tokens, K not a multiple of 64. */
+C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
+                                   float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);
 C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
 C_EXPORT int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n);
 /* sum = bf16(a + b) and y = rmsnorm(sum) * norm_w, rows of `inner` BF16 values (a multiple of 8, at most 4096; 16-byte

@@ -91,6 +91,56 @@ def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n
     assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), 3 * n_kv, n_kv, 128, t_kv, T, pos0) == -1
 
 
+@pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", False), ("e4m3", True)])
+@pytest.mark.parametrize("tokens,n_out,K", [(60, 512, 256), (130, 200, 1024), (300, 1536, 512)])
+def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, w_type, tiled, tokens, n_out, K):
+    """hip_quant_gemm_swiglu against two hip_quant_gemm calls and hip_swiglu_bf16 on the same inputs, byte for byte (K is
+    short enough that no call splits its k range, so every sum runs in the same order), on the file layout and on the
+    tiled copies, with the per-tensor scales of an E4M3 file differing between gate and up; and against the oracle's
+    exact contraction.  Unsupported arguments are refused with -1."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + n_out + K)
+    wt = oracle.E5M2 if w_type == "e5m2" else oracle.E4M3
+    sg, su = (1.0, 1.0) if w_type == "e5m2" else (0.011, 0.017)
+    Wg = rng.integers(0, 256, size=(n_out, K), dtype=np.uint8)
+    Wu = rng.integers(0, 256, size=(n_out, K), dtype=np.uint8)
+    for W in (Wg, Wu):                                          # no NaN / Inf codes
+        if w_type == "e5m2": W[(W & 0x7C) == 0x7C] = 0x3C
+        else: W[(W & 0x7F) == 0x7F] = 0x38
+    X = oracle.f32_to_bf16((rng.standard_normal((tokens, K)) * (0.05 if w_type == "e5m2" else 1.0)).astype(np.float32))
+    gd, ud, xd = to_dev(torch, dev, Wg), to_dev(torch, dev, Wu), to_dev(torch, dev, X)
+    keep = []
+    if tiled:
+        for wd in (gd, ud):
+            t = torch.zeros(lib.tiled_size(wt, n_out, K), dtype=torch.uint8, device=dev)
+            assert lib.weight_prepare(wd.data_ptr(), wt, n_out, K, K, t.data_ptr()) == 0
+            keep.append(t)
+    try:
+        g, u, y3, y1 = (torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev) for _ in range(4))
+        assert lib.linear(gd.data_ptr(), wt, xd.data_ptr(), g.data_ptr(), n_out, tokens, K, sg) == 0
+        assert lib.linear(ud.data_ptr(), wt, xd.data_ptr(), u.data_ptr(), n_out, tokens, K, su) == 0
+        assert lib.c.hip_swiglu_bf16(ptr(g), ptr(u), ptr(y3), tokens * n_out) == (0 if (tokens * n_out) % 8 == 0 else -1)
+        assert lib.c.hip_quant_gemm_swiglu(n_out, tokens, K, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su),
+                                           ptr(xd), K, ptr(y1), n_out) == 0
+        assert lib.last_kernel() == ("gemm_swiglu_tiled" if tiled else "gemm_swiglu")
+        got = from_dev(y1, np.uint16)
+        assert not got[tokens * n_out:].any()
+        if (tokens * n_out) % 8 == 0:
+            assert np.array_equal(got, from_dev(y3, np.uint16))
+        gate = oracle.f32_to_bf16(oracle.linear_exact(oracle.dequant_fp8_to_bf16(Wg, wt, sg), X).astype(np.float32))
+        up = oracle.f32_to_bf16(oracle.linear_exact(oracle.dequant_fp8_to_bf16(Wu, wt, su), X).astype(np.float32))
+        want = dec.silu_mul(dec.f(gate), dec.f(up))
+        have = dec.f(got[:tokens * n_out].reshape(tokens, n_out))
+        assert np.linalg.norm(have - want) <= 1e-2 * np.linalg.norm(want)
+        bad = lambda *a: lib.c.hip_quant_gemm_swiglu(*a)
+        assert bad(n_out, 47, K, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
+        assert bad(n_out, tokens, K, ptr(gd), ptr(ud), oracle.FP4, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
+        assert bad(n_out, tokens, K - 32, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
+    finally:
+        if tiled:
+            assert lib.weight_release(gd.data_ptr()) == 0 and lib.weight_release(ud.data_ptr()) == 0
+
+
 @pytest.mark.parametrize("rows,inner", [(1, 256), (7, 4096), (130, 1024), (5, 136)])
 def test_add_and_rms_norm_in_one_pass_equals_the_two_calls(gpu, oracle, dec, rows, inner):
     """hip_add_rms_norm_bf16 against hip_add_bf16 followed by hip_rms_norm_fwd on the same inputs: both outputs byte for
