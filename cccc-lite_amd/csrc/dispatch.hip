@@ -509,6 +509,53 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                       blk_scA, blk_scB, block_size, nullptr);
 }
 
+int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale, void* const* Y, const int* ldy,
+                            int w_type, int tokens, int K, int ldw, const void* X, int ldx)
+{
+    if (w_type != DT_E5M2 && w_type != DT_E4M3) { return -1; }
+    if (n_segments < 1 || n_segments > 3 || !n_out || !W || !inv_scale || !Y || !ldy) { return -1; }
+    if (tokens < 48 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
+    if ((long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
+    LinearArgs a{};
+    a.X = (const uint16_t*)X;
+    a.ldw = ldw;
+    a.ldx = ldx;
+    a.y_stride_out = 1;
+    a.tokens = tokens;
+    a.K = K;
+    a.alpha = 1.0f;
+    a.beta = 0.0f;
+    a.n_segments = n_segments;
+    bool all_tiled = true;
+    const uint8_t* tiled[3] = { nullptr, nullptr, nullptr };
+    for (int s = 0; s < n_segments; s++)
+    {
+        if (n_out[s] <= 0 || !W[s] || !Y[s] || !aligned16(W[s]) || ldy[s] < n_out[s] || (long long)n_out[s] * ldw >= (1LL << 32)) { return -1; }
+        a.seg_W[s] = (const uint8_t*)W[s];
+        a.seg_Y[s] = (uint16_t*)Y[s];
+        a.seg_n_out[s] = n_out[s];
+        a.seg_w_scale[s] = inv_scale[s];
+        a.seg_y_stride_tok[s] = ldy[s];
+        tiled[s] = ccq::lookup_tiled(W[s], w_type, n_out[s], K, ldw);
+        all_tiled = all_tiled && tiled[s] != nullptr;
+    }
+    // every weight on its tiled copy, or every weight on the file layout
+    if (all_tiled)
+    {
+        for (int s = 0; s < n_segments; s++) { a.seg_W[s] = tiled[s]; }
+        note_kernel("gemm_segments_tiled");
+        if (w_type == DT_E5M2) { launch_gemm_mfma_direct_segments<DT_E5M2, true>(a); }
+        else { launch_gemm_mfma_direct_segments<DT_E4M3, true>(a); }
+    }
+    else
+    {
+        note_kernel("gemm_segments");
+        if (w_type == DT_E5M2) { launch_gemm_mfma_direct_segments<DT_E5M2, false>(a); }
+        else { launch_gemm_mfma_direct_segments<DT_E4M3, false>(a); }
+    }
+    return finish("quant_gemm_segments");
+}
+
 int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                           float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy)
 {

@@ -278,10 +278,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // bf16(bf16(g * bf16(sigmoid g)) * u) of the two rounded linears (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732,
 // :953-966) -- one launch instead of two GEMMs and an elementwise pass over three [tokens][n_out] matrices.  A workgroup
 // then owns 32 NB output features; alpha = 1, beta = 0, BF16.
-template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a, const int n_tiles, float* __restrict__ partial)
+// SEG: the launch covers up to three linears on the same activations (the q, k and v projections: the narrow ones alone
+// leave most CUs idle); a workgroup finds its segment from its feature tile and takes that segment's weight, output,
+// width and scale -- from there on it is the single-linear kernel.
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a_in, const int n_tiles, float* __restrict__ partial)
 {
     static_assert(!PAIR || (!SPLIT && NB % 2 == 0 && AT == DT_BF16), "pair: unsplit, an even number of feature blocks, BF16");
+    static_assert(!SEG || (!SPLIT && !PAIR), "segments: unsplit single linears");
     constexpr int NBO = PAIR ? NB / 2 : NB;     // feature blocks of a wave in the output
     constexpr int BTOK = MB * 16;               // tokens per workgroup
     constexpr int BK = 64, CPR = 8;
@@ -296,9 +300,20 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     // tiles padded to a multiple of eight, feature tile n always lands on XCD n % 8, and the workgroups an XCD runs at
     // one time are a block of (n_pad / 8) feature tiles x several token tiles: both operands are shared inside the L2.
     const int n_pad = (n_tiles + 7) & ~7;
-    const int n_tile = blockIdx.x % n_pad;
+    int n_tile = blockIdx.x % n_pad;
     const int m_tile = blockIdx.x / n_pad;
     if (n_tile >= n_tiles) { return; }          // padding
+    LinearArgs a = a_in;
+    if constexpr (SEG)
+    {
+        const int s = n_tile >= a_in.seg_tile0[2] ? 2 : (n_tile >= a_in.seg_tile0[1] ? 1 : 0);
+        a.W = a_in.seg_W[s];
+        a.Y = a_in.seg_Y[s];
+        a.n_out = a_in.seg_n_out[s];
+        a.w_scale = a_in.seg_w_scale[s];
+        a.y_stride_tok = a_in.seg_y_stride_tok[s];
+        n_tile -= a_in.seg_tile0[s];
+    }
     const int out_base = n_tile * (64 * NBO) + wave * (16 * NBO);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
@@ -870,6 +885,38 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
     {
         if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
         else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+    }
+}
+
+// up to three linears on the same activations in one launch: 64- or 128-token x 256-feature tiles, whichever gives the CUs
+// two rounds of workgroups or more evenly
+template <int WT, bool TILED>
+void launch_gemm_mfma_direct_segments(LinearArgs a)
+{
+    const int cus = cu_count();
+    int n_tiles = 0;
+    for (int s = 0; s < 3; s++)
+    {
+        a.seg_tile0[s] = n_tiles;
+        if (s < a.n_segments) { n_tiles += (a.seg_n_out[s] + 255) / 256; }
+    }
+    a.seg_tile0[3] = n_tiles;
+    for (int s = a.n_segments; s < 3; s++) { a.seg_tile0[s] = n_tiles; }       // empty segments start past the last tile
+    bool scaled = false;
+    for (int s = 0; s < a.n_segments; s++) { scaled = scaled || a.seg_w_scale[s] != 1.0f; }
+    const long long tiles8 = (long long)n_tiles * ((a.tokens + 127) / 128);
+    const int n_pad = (n_tiles + 7) & ~7;
+    if (a.tokens > 64 && tiles8 >= 2LL * cus)
+    {
+        const dim3 grid(n_pad * ((a.tokens + 127) / 128));
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, false, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+        else { gemm_mfma_direct_kernel<WT, false, 8, false, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+    }
+    else
+    {
+        const dim3 grid(n_pad * ((a.tokens + 63) / 64));
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, false, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+        else { gemm_mfma_direct_kernel<WT, false, 4, false, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
     }
 }
 

@@ -27,6 +27,16 @@ struct LinearArgs
     // and layout; the output is the SwiGLU product of the two linears
     const uint8_t* W_pair;
     float w_scale_pair;
+    // up to three linears of one K, type and layout on the same activations as one launch (gemm_mfma_direct_kernel<..., SEG>):
+    // segment s owns the feature tiles seg_tile0[s] .. seg_tile0[s + 1] - 1 of the grid and brings its own weight, output,
+    // width and scale; n_segments = 0 everywhere else
+    int n_segments;
+    const uint8_t* seg_W[3];
+    uint16_t* seg_Y[3];
+    int seg_n_out[3];
+    int seg_tile0[4];
+    float seg_w_scale[3];
+    long long seg_y_stride_tok[3];
 };
 
 }    // namespace ccq

@@ -444,9 +444,23 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
     for (int li = 0; li < c.layers && rc == 0; li++)
     {
         Layer& L = layers_[li];
-        if (rc == 0) { rc = linear(*L.wq, q_out, c.hidden, *pf_.xn, *pf_.q); }
-        if (rc == 0) { rc = linear(*L.wk, kv_out, c.hidden, *pf_.xn, *pf_.k); }
-        if (rc == 0) { rc = linear(*L.wv, kv_out, c.hidden, *pf_.xn, *pf_.v); }
+        // q, k, v: one launch for three FP8 weights of one type, else three calls
+        int qkv = -1;
+        if (rc == 0 && L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
+        {
+            const int widths[3] = { q_out, kv_out, kv_out };
+            const void* const weights[3] = { L.wq->data(), L.wk->data(), L.wv->data() };
+            const float scales[3] = { L.wq->getQuantScale(), L.wk->getQuantScale(), L.wv->getQuantScale() };
+            void* const outputs[3] = { pf_.q->data(), pf_.k->data(), pf_.v->data() };
+            qkv = hip_quant_gemm_segments(3, widths, weights, scales, outputs, widths, (int)L.wq->getDataType(), n, c.hidden, c.hidden, pf_.xn->data(), c.hidden);
+            if (qkv > 0) { rc = qkv; }
+        }
+        if (qkv < 0)
+        {
+            if (rc == 0) { rc = linear(*L.wq, q_out, c.hidden, *pf_.xn, *pf_.q); }
+            if (rc == 0) { rc = linear(*L.wk, kv_out, c.hidden, *pf_.xn, *pf_.k); }
+            if (rc == 0) { rc = linear(*L.wv, kv_out, c.hidden, *pf_.xn, *pf_.v); }
+        }
         if (rc == 0)
         {
             rc = hip_qk_norm_rope_kv_rows_bf16(pf_.q->data(), pf_.k->data(), pf_.v->data(), qk_norm_ ? L.q_norm->data() : nullptr,

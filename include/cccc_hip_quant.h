@@ -270,6 +270,14 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
 /* y = bf16(a + b) and y = bf16(bf16(gate * bf16(sigmoid(gate))) * up) over n BF16 elements (n % 8 == 0, 16-byte aligned):
  * the residual add and the SwiGLU product with the reference's roundings (cccc-hip/hip_functions.cpp:895-908, :722-732,
  * :953-966; cccc/MatrixEx.cpp:756-762). */
+/* Up to three linears on the same activations in one launch: Y[s][t][o] = bf16(W[s] x_t), s < n_segments <= 3, FP8 weights
+ * [n_out[s]][K] of one type, K and row pitch ldw (all on their registered tiled copies, or all on the file layout), BF16
+ * activations [tokens][K] and outputs with row pitch ldy[s] -- the q, k and v projections of a prompt, whose narrow members
+ * alone leave most of the GPU idle.  The bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not
+ * split their k range.  -1 (nothing launched): other weight types, fewer than 48 tokens, K not a multiple of 64.  No
+ * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
+C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
+                                     void* const* Y, const int* ldy, int w_type, int tokens, int K, int ldw, const void* X, int ldx);
 /* y[t][o] = swiglu(gate[t][o], up[t][o]) with gate = bf16(W_gate x_t), up = bf16(W_up x_t): the gate and up linears of an
  * MLP block (two FP8 weights of one shape [n_out][K], row pitch ldw, dequantisation multipliers as in hip_quant_gemm; both
  * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product

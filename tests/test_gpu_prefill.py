@@ -91,6 +91,52 @@ def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n
     assert lib.c.hip_attention_prefill_bf16(ptr(qd), ptr(kd), ptr(vd), ptr(y), 3 * n_kv, n_kv, 128, t_kv, T, pos0) == -1
 
 
+@pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", True)])
+@pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512), (48, (64,), 64)])
+def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(gpu, oracle, w_type, tiled, tokens, widths, K):
+    """hip_quant_gemm_segments (the q, k, v projections of a prompt as one launch) against one hip_quant_gemm call per
+    weight, byte for byte (K short enough that no call splits its k range), on the file layout and on tiled copies, with
+    a different per-tensor scale per weight for E4M3; unsupported arguments are refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + K + len(widths))
+    wt = oracle.E5M2 if w_type == "e5m2" else oracle.E4M3
+    scales = [1.0] * len(widths) if w_type == "e5m2" else [0.011, 0.017, 0.023][:len(widths)]
+    X = oracle.f32_to_bf16((rng.standard_normal((tokens, K)) * (0.05 if w_type == "e5m2" else 1.0)).astype(np.float32))
+    xd = to_dev(torch, dev, X)
+    wds, keep, sep, one = [], [], [], []
+    for n_out in widths:
+        W = rng.integers(0, 256, size=(n_out, K), dtype=np.uint8)
+        if w_type == "e5m2": W[(W & 0x7C) == 0x7C] = 0x3C
+        else: W[(W & 0x7F) == 0x7F] = 0x38
+        wds.append(to_dev(torch, dev, W))
+        if tiled:
+            t = torch.zeros(lib.tiled_size(wt, n_out, K), dtype=torch.uint8, device=dev)
+            assert lib.weight_prepare(wds[-1].data_ptr(), wt, n_out, K, K, t.data_ptr()) == 0
+            keep.append(t)
+        sep.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
+        one.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
+    try:
+        for wd, y, n_out, sc in zip(wds, sep, widths, scales):
+            assert lib.linear(wd.data_ptr(), wt, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, sc) == 0
+        n = len(widths)
+        arr_i = (ctypes.c_int * n)(*widths)
+        arr_w = (ctypes.c_void_p * n)(*[w.data_ptr() for w in wds])
+        arr_s = (ctypes.c_float * n)(*scales)
+        arr_y = (ctypes.c_void_p * n)(*[y.data_ptr() for y in one])
+        call = lambda toks, k, typ: lib.c.hip_quant_gemm_segments(n, arr_i, arr_w, arr_s, arr_y, arr_i, typ, toks, k, K, ptr(xd), K)
+        assert call(tokens, K, wt) == 0
+        assert lib.last_kernel() == ("gemm_segments_tiled" if tiled else "gemm_segments")
+        for y1, y3, n_out in zip(one, sep, widths):
+            got = from_dev(y1, np.uint16)
+            assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
+            assert np.array_equal(got, from_dev(y3, np.uint16))
+        assert call(47, K, wt) == -1 and call(tokens, K - 32, wt) == -1 and call(tokens, K, oracle.FP4) == -1
+    finally:
+        if tiled:
+            for wd in wds:
+                assert lib.weight_release(wd.data_ptr()) == 0
+
+
 @pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", False), ("e4m3", True)])
 @pytest.mark.parametrize("tokens,n_out,K", [(60, 512, 256), (130, 200, 1024), (300, 1536, 512)])
 def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, w_type, tiled, tokens, n_out, K):
