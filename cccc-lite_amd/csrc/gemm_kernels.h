@@ -906,7 +906,8 @@ void launch_gemm_mfma_direct_segments(LinearArgs a)
     for (int s = 0; s < a.n_segments; s++) { scaled = scaled || a.seg_w_scale[s] != 1.0f; }
     const long long tiles8 = (long long)n_tiles * ((a.tokens + 127) / 128);
     const int n_pad = (n_tiles + 7) & ~7;
-    if (a.tokens > 64 && tiles8 >= 2LL * cus)
+    // (on the file layout the 128-token tile is worth having from one workgroup per CU on, see plan_direct)
+    if (a.tokens > 64 && (tiles8 >= 2LL * cus || (!TILED && tiles8 >= cus)))
     {
         const dim3 grid(n_pad * ((a.tokens + 127) / 128));
         if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, false, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
