@@ -181,6 +181,14 @@ std::unordered_map<const void*, TiledWeight> g_tiled;
 
 const uint8_t* find_tiled(const LinearArgs& a, int type) { return ccq::lookup_tiled(a.W, type, a.n_out, a.K, a.ldw); }
 
+// block length the FP4 tiled copy registered under W was built with (0: none)
+unsigned tiled_block_of(const void* W)
+{
+    std::shared_lock<std::shared_mutex> lock(g_tiled_mutex);
+    const auto it = g_tiled.find(W);
+    return it == g_tiled.end() ? 0u : it->second.block;
+}
+
 // The tiled copy of an FP4 weight, if one was built from these codes, these block scales and this block length.
 const uint8_t* find_tiled_fp4(const LinearArgs& a)
 {
@@ -512,7 +520,9 @@ int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
 int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale, void* const* Y, const int* ldy,
                             int w_type, int tokens, int K, int ldw, const void* X, int ldx)
 {
-    if (w_type != DT_E5M2 && w_type != DT_E4M3) { return -1; }
+    const bool fp4 = w_type == DT_FP4;
+    if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
+    if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
     if (n_segments < 1 || n_segments > 3 || !n_out || !W || !inv_scale || !Y || !ldy) { return -1; }
     if (tokens < 48 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
@@ -538,6 +548,22 @@ int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const*
         a.seg_y_stride_tok[s] = ldy[s];
         tiled[s] = ccq::lookup_tiled(W[s], w_type, n_out[s], K, ldw);
         all_tiled = all_tiled && tiled[s] != nullptr;
+    }
+    if (fp4)
+    {
+        // FP4 runs on the tiled copies only (codes, then the scale bytes): the block length comes from the registration
+        if (!all_tiled) { return -1; }
+        const unsigned block = tiled_block_of(W[0]);
+        for (int s = 0; s < n_segments; s++)
+        {
+            if (tiled_block_of(W[s]) != block) { return -1; }
+            a.seg_W[s] = tiled[s];
+        }
+        note_kernel("gemm_segments_tiled");
+        if (block == 16) { launch_gemm4_mfma_direct_segments<16>(a); }
+        else if (block == 32) { launch_gemm4_mfma_direct_segments<32>(a); }
+        else { return -1; }
+        return finish("quant_gemm_segments");
     }
     // every weight on its tiled copy, or every weight on the file layout
     if (all_tiled)

@@ -604,10 +604,13 @@ __device__ __forceinline__ u32x4 dequant8_fp4_blocks(uint32_t w, float s_lo, flo
     return u32x4{ out[0], out[1], out[2], out[3] };
 }
 
-template <int BLOCK, int MB, bool SPLIT, int NB = 4>
-__global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a, const uint8_t* __restrict__ tiled_scales, const int n_tiles,
+// SEG: as in gemm_mfma_direct_kernel -- up to three linears on the same activations, a workgroup takes weight, scales,
+// output and width of the segment its feature tile belongs to (a.seg_W[s] = tiled codes with the scales behind them).
+template <int BLOCK, int MB, bool SPLIT, int NB = 4, bool SEG = false>
+__global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a_in, const uint8_t* scales_in, const int n_tiles,
                                                                                         float* __restrict__ partial)
 {
+    static_assert(!SEG || !SPLIT, "segments: unsplit");
     static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
     constexpr int NS = 128 / BLOCK;             // scale bytes per row and chunk
     constexpr int BTOK = MB * 16;
@@ -622,9 +625,21 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
     // tiles padded to a multiple of eight, feature tile n always lands on XCD n % 8, and the workgroups an XCD runs at
     // one time are a block of (n_pad / 8) feature tiles x several token tiles: both operands are shared inside the L2.
     const int n_pad = (n_tiles + 7) & ~7;
-    const int n_tile = blockIdx.x % n_pad;
+    int n_tile = blockIdx.x % n_pad;
     const int m_tile = blockIdx.x / n_pad;
     if (n_tile >= n_tiles) { return; }          // padding
+    LinearArgs a = a_in;
+    const uint8_t* tiled_scales = scales_in;
+    if constexpr (SEG)
+    {
+        const int s = n_tile >= a_in.seg_tile0[2] ? 2 : (n_tile >= a_in.seg_tile0[1] ? 1 : 0);
+        a.W = a_in.seg_W[s];
+        a.Y = a_in.seg_Y[s];
+        a.n_out = a_in.seg_n_out[s];
+        a.y_stride_tok = a_in.seg_y_stride_tok[s];
+        tiled_scales = a.W + (long long)((a.n_out + 15) / 16) * (a.K / 128) * 1024;
+        n_tile -= a_in.seg_tile0[s];
+    }
     const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
@@ -886,6 +901,22 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
         if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
         else { gemm_mfma_direct_kernel<WT, false, MB, false, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
     }
+}
+
+// FP4 (tiled copies, K % 128 == 0): 64-token x 256-feature tiles, two workgroups per CU
+template <int BLOCK>
+void launch_gemm4_mfma_direct_segments(LinearArgs a)
+{
+    int n_tiles = 0;
+    for (int s = 0; s < 3; s++)
+    {
+        a.seg_tile0[s] = n_tiles;
+        if (s < a.n_segments) { n_tiles += (a.seg_n_out[s] + 255) / 256; }
+    }
+    a.seg_tile0[3] = n_tiles;
+    for (int s = a.n_segments; s < 3; s++) { a.seg_tile0[s] = n_tiles; }
+    const dim3 grid(((n_tiles + 7) & ~7) * ((a.tokens + 63) / 64));
+    gemm4_mfma_direct_kernel<BLOCK, 4, false, 4, true><<<grid, 256, 0, stream()>>>(a, nullptr, n_tiles, nullptr);
 }
 
 // up to three linears on the same activations in one launch: 64- or 128-token x 256-feature tiles, whichever gives the CUs

@@ -274,7 +274,9 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
  * [n_out[s]][K] of one type, K and row pitch ldw (all on their registered tiled copies, or all on the file layout), BF16
  * activations [tokens][K] and outputs with row pitch ldy[s] -- the q, k and v projections of a prompt, whose narrow members
  * alone leave most of the GPU idle.  The bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not
- * split their k range.  -1 (nothing launched): other weight types, fewer than 48 tokens, K not a multiple of 64.  No
+ * split their k range.  FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
+ * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 48 tokens, K not a
+ * multiple of 64.  No
  * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
 C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
                                      void* const* Y, const int* ldy, int w_type, int tokens, int K, int ldw, const void* X, int ldx);

@@ -137,6 +137,47 @@ def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(g
                 assert lib.weight_release(wd.data_ptr()) == 0
 
 
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512)])
+def test_fp4_linears_that_share_their_input_in_one_launch(gpu, oracle, block, tokens, widths, K):
+    """hip_quant_gemm_segments on FP4 block-scale weights (tiled copies registered, which is what the FP4 GEMM reads) against
+    one hip_quant_gemm call per weight, byte for byte; without the tiled copies the call is refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + K + block)
+    X = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
+    xd = to_dev(torch, dev, X)
+    wds, sds, keep, sep, one = [], [], [], [], []
+    for n_out in widths:
+        wds.append(to_dev(torch, dev, rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8)))
+        sds.append(to_dev(torch, dev, rng.integers(0x20, 0x40, size=(n_out, K // block), dtype=np.uint8)))
+        sep.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
+        one.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
+    n = len(widths)
+    arr_i = (ctypes.c_int * n)(*widths)
+    arr_w = (ctypes.c_void_p * n)(*[w.data_ptr() for w in wds])
+    arr_s = (ctypes.c_float * n)(*([1.0] * n))
+    arr_y = (ctypes.c_void_p * n)(*[y.data_ptr() for y in one])
+    call = lambda: lib.c.hip_quant_gemm_segments(n, arr_i, arr_w, arr_s, arr_y, arr_i, oracle.FP4, tokens, K, K, ptr(xd), K)
+    assert call() == -1                                         # no tiled copies yet
+    for wd, sd, n_out in zip(wds, sds, widths):
+        t = torch.zeros(lib.tiled_size(oracle.FP4, n_out, K), dtype=torch.uint8, device=dev)
+        assert lib.weight_prepare_fp4(wd.data_ptr(), sd.data_ptr(), block, n_out, K, t.data_ptr()) == 0
+        keep.append(t)
+    try:
+        for wd, sd, y, n_out in zip(wds, sds, sep, widths):
+            assert lib.linear(wd.data_ptr(), oracle.FP4, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, 1.0, sd.data_ptr(), block) == 0
+            assert lib.last_kernel() == "gemm_mfma_tiled"
+        assert call() == 0
+        assert lib.last_kernel() == "gemm_segments_tiled"
+        for y1, y3, n_out in zip(one, sep, widths):
+            got = from_dev(y1, np.uint16)
+            assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
+            assert np.array_equal(got, from_dev(y3, np.uint16))
+    finally:
+        for wd in wds:
+            assert lib.weight_release(wd.data_ptr()) == 0
+
+
 @pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", False), ("e4m3", True)])
 @pytest.mark.parametrize("tokens,n_out,K", [(60, 512, 256), (130, 200, 1024), (300, 1536, 512)])
 def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, w_type, tiled, tokens, n_out, K):
