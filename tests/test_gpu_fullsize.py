@@ -376,6 +376,52 @@ def test_decode_step_at_qwen3_8b_widths(gpu, pkg, oracle, dec, exact_attention, 
 
 # ------------------------------------------------------------------------------------------ prompt phase
 
+@pytest.mark.parametrize("tiled", [False, True])
+def test_fused_prompt_gemms_at_qwen3_8b_shapes_equal_the_separate_calls(gpu, pkg, oracle, tiled):
+    """2048 tokens at Qwen3-8B widths: q, k, v as one launch against three hip_quant_gemm calls, and gate / up / SwiGLU as
+    one launch against two calls and hip_swiglu_bf16 -- byte for byte (none of these shapes splits its k range), on the
+    file layout and on tiled copies; sampled features of the q output against the exact contraction."""
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(77)
+    T, K = 2048, 4096
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    x = draw_bf16(torch, dev, gen, (T, K))
+    widths = (4096, 1024, 1024, 12288, 12288)                  # q, k, v, gate, up
+    ws = [draw_e5m2(torch, dev, gen, n, K) for n in widths]
+    keep = []
+    if tiled:
+        for w, n in zip(ws, widths):
+            td = torch.zeros(lib.tiled_size(E5M2, n, K), dtype=torch.uint8, device=dev)
+            assert lib.weight_prepare(w.data_ptr(), E5M2, n, K, K, td.data_ptr()) == 0
+            keep.append(td)
+    try:
+        sep = [torch.zeros(T * n, dtype=torch.int16, device=dev) for n in widths]
+        for w, y, n in zip(ws, sep, widths):
+            assert lib.linear(w.data_ptr(), E5M2, x.data_ptr(), y.data_ptr(), n, T, K) == 0
+            assert lib.last_kernel() == ("gemm_mfma_tiled" if tiled else "gemm_mfma")
+        one = [torch.zeros(T * n, dtype=torch.int16, device=dev) for n in widths[:3]]
+        arr_i = (ctypes.c_int * 3)(*widths[:3])
+        arr_w = (ctypes.c_void_p * 3)(*[w.data_ptr() for w in ws[:3]])
+        arr_s = (ctypes.c_float * 3)(1.0, 1.0, 1.0)
+        arr_y = (ctypes.c_void_p * 3)(*[y.data_ptr() for y in one])
+        assert lib.c.hip_quant_gemm_segments(3, arr_i, arr_w, arr_s, arr_y, arr_i, E5M2, T, K, K, ptr(x), K) == 0
+        for a, b in zip(one, sep[:3]):
+            assert torch.equal(a, b)
+        rows = np.random.default_rng(3).choice(4096, size=96, replace=False)
+        want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(ws[0][torch.as_tensor(rows, device=dev)].cpu().numpy(), E5M2), host_bits(x).reshape(T, K))
+        check_rows(bf16_f64(oracle, host_bits(one[0]).reshape(T, 4096)[:, rows]), want, "q of the q,k,v launch")
+        prod, fused = torch.zeros(T * 12288, dtype=torch.int16, device=dev), torch.zeros(T * 12288, dtype=torch.int16, device=dev)
+        assert lib.c.hip_swiglu_bf16(ptr(sep[3]), ptr(sep[4]), ptr(prod), T * 12288) == 0
+        assert lib.c.hip_quant_gemm_swiglu(12288, T, K, ptr(ws[3]), ptr(ws[4]), E5M2, K, ctypes.c_float(1.0), ctypes.c_float(1.0),
+                                           ptr(x), K, ptr(fused), 12288) == 0
+        assert lib.last_kernel() == ("gemm_swiglu_tiled" if tiled else "gemm_swiglu")
+        assert torch.equal(fused, prod) and bool(fused.any())
+    finally:
+        if tiled:
+            for w in ws:
+                assert lib.weight_release(w.data_ptr()) == 0
+
+
 @pytest.mark.parametrize("arch", ["qwen3_8b_fp8", "llama31_8b_fp4"])
 def test_prompt_phase_at_full_widths_equals_token_by_token_decoding(gpu, pkg, oracle, dec, arch):
     """DecodeModel::prefill at the benchmark's widths (two layers): 130 prompt tokens from position 0 in one call against the
