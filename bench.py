@@ -324,6 +324,28 @@ def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, 
     return out
 
 
+def generate_run(ws: Workspace, model, use_graph: bool, prompt_tokens: int = 2048, new_tokens: int = 128):
+    """Prompt and generation together, as a chat turn runs them: DecodeModel::prefill on a prompt from an empty cache, then
+    greedy decode steps that carry on from it (one captured step replayed; the capture is inside the clock).  Wall clock,
+    device synchronised around each phase; the model keeps the tiled copies of its linears at this point of the run."""
+    import numpy as np
+    t = ws.torch
+    prompt = [int(v) for v in np.random.default_rng(prompt_tokens + 1).integers(0, QWEN3_8B["vocab"], size=prompt_tokens)]
+    model.prefill(prompt)                                       # warm-up
+    t.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.prefill(prompt)
+    t.cuda.synchronize()
+    t1 = time.perf_counter()
+    model.run(new_tokens, use_graph)
+    t.cuda.synchronize()
+    t2 = time.perf_counter()
+    assert model.pos == prompt_tokens + new_tokens
+    return {"workload": f"{prompt_tokens}-token prompt, then {new_tokens} greedy tokens, Qwen3-8B W8A16, batch 1",
+            "time_to_first_token_ms": round((t1 - t0) * 1e3, 3), "decode_ms": round((t2 - t1) * 1e3, 3),
+            "decode_tok_s": round(new_tokens / (t2 - t1), 1), "total_ms": round((t2 - t0) * 1e3, 3), "last_token": model.token}
+
+
 def decode_step_bytes(ctx_mean: float) -> int:
     """Bytes one decode step must move: every linear weight once, the keys and values of the positions
     attended to, the embedding row, the norm weights and the logits."""
@@ -792,6 +814,7 @@ def main():
                 for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
                     assert model.prepare_tiled(li, name)
             extra["prompt_phase"]["cases"] += prompt_phase(ws, model, layout="tiled copies")
+            extra["generate"] = generate_run(ws, model, use_graph)
             if not args.no_fp4_step:
                 # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
                 extra["fp4_decode_step"]["prompt_phase"] = prompt_phase(ws, fp4_model, layout="tiled copies", c=LLAMA31_8B)
