@@ -813,7 +813,7 @@ def main():
             for li in range(QWEN3_8B["layers"]):
                 for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
                     assert model.prepare_tiled(li, name)
-            extra["prompt_phase"]["cases"] += prompt_phase(ws, model, layout="tiled copies")
+            extra["prompt_phase"]["cases"] += prompt_phase(ws, model, token_counts=(512, 2048, DECODE_CTX), layout="tiled copies")
             extra["generate"] = generate_run(ws, model, use_graph)
             if not args.no_fp4_step:
                 # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
