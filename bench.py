@@ -10,7 +10,7 @@ cccc's graph issues them (`quant_gemv`), the per-shape sweep over M in {1, 4, 16
 FP4 block-scale sweep (`fp4_sweep`); GB/s figures are algorithmic bytes (K*N + 2*M*K + 2*M*N per
 GEMV) / elapsed.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_linears|gemv|prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_linears|gemv|prefill|prompt_attention]
                     [--shape K,N] [--tokens M] [--no-graph] [--no-cpu] [--no-sweep]
 
 Prints ONE JSON line.  `roofline` is measured live on the dominant kernel (the fused RMSNorm +
@@ -703,7 +703,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy"])
+    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy", "prompt_attention"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--weights", default="fp8", choices=["fp8", "fp4"], help="weight format of --workload gemv / prefill (fp4: E2M1 codes + E4M3 block scales)")
@@ -736,6 +736,28 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"workload": "copy", "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launches": args.steps}))
+        return
+    if args.workload == "prompt_attention":
+        # the prompt phase's causal attention kernel alone (for counter runs): --tokens query tokens from position 0,
+        # Qwen3-8B heads (32 q / 8 kv x 128), --steps launches after --warmup
+        import ctypes
+        lib, dev = pkg.library(), torch.device("cuda:0")
+        T = max(args.tokens, 16)
+        q = torch.randn(T, 32, 128, device=dev).to(torch.bfloat16)
+        kc, vc = torch.randn(8, T, 128, device=dev).to(torch.bfloat16), torch.randn(8, T, 128, device=dev).to(torch.bfloat16)
+        y = torch.zeros(T, 32, 128, device=dev, dtype=torch.bfloat16)
+        p = lambda x: ctypes.c_void_p(x.data_ptr())
+        launch = lambda: lib.c.hip_attention_prefill_bf16(p(q), p(kc), p(vc), p(y), 32, 8, 128, T, T, 0)
+        for _ in range(args.warmup):
+            assert launch() == 0
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "prompt_attention", "tokens": T, "launches": args.steps, "us_per_launch": round(e0.elapsed_time(e1) * 1e3 / args.steps, 2)}))
         return
     ws = Workspace(pkg, torch)
     ws.repack = not args.no_repack
