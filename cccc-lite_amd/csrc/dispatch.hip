@@ -6,7 +6,7 @@
 //     FP8, tokens <= 4                             gemv_dot2 (dot2 + DPP, software pipelined for small weights)
 //     FP8, tokens 5..16                            gemv_mfma (matrix cores, row-major weight)
 //     FP8, tokens >= 17                            gemm_mfma: weights straight into the matrix-core operands when
-//                                                  tokens >= 48 and K % 64 == 0 (row-major or tiled copy, k split
+//                                                  tokens >= 17 and K % 64 == 0 (row-major or tiled copy, k split
 //                                                  over workgroups when the output has few tiles), else dequant-to-LDS
 //     FP4 block scales, tokens <= 16               gemv_dot2 in token groups of four
 //     FP4 block scales, tokens >= 17               gemm_mfma (dequant-to-LDS)
@@ -451,8 +451,8 @@ int quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
             }
             else if (ok && !launched)
             {
-                // the register-fed kernel reads the tiled copy; it wants whole 128-element chunks and at least 48 tokens
-                const uint8_t* tiled = (K % 128 == 0 && a.tokens >= 48) ? find_tiled_fp4(a) : nullptr;
+                // the register-fed kernel reads the tiled copy; it wants whole 128-element chunks
+                const uint8_t* tiled = (K % 128 == 0 && a.tokens >= 17) ? find_tiled_fp4(a) : nullptr;
                 launched = a.block_size == 16 ? gemm_mfma<DT_FP4, 16>(a, tiled, split_scratch) : gemm_mfma<DT_FP4, 32>(a, tiled, split_scratch);
                 if (!launched) { return -2; }                    // only a fixed scratch buffer that is too small ends here
                 note_kernel(tiled ? "gemm_mfma_tiled" : "gemm_mfma");
@@ -524,7 +524,7 @@ int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const*
     if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
     if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
     if (n_segments < 1 || n_segments > 3 || !n_out || !W || !inv_scale || !Y || !ldy) { return -1; }
-    if (tokens < 48 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
+    if (tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
     LinearArgs a{};
     a.X = (const uint16_t*)X;
@@ -586,7 +586,7 @@ int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, cons
                           float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy)
 {
     if (w_type != DT_E5M2 && w_type != DT_E4M3) { return -1; }
-    if (n_out <= 0 || tokens < 48 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
+    if (n_out <= 0 || tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
     if (!W_gate || !W_up || !X || !Y || !aligned16(W_gate) || !aligned16(W_up) || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)n_out * ldw >= (1LL << 32) || (long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
     LinearArgs a{};

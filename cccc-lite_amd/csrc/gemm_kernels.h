@@ -1081,13 +1081,13 @@ inline DirectPlan plan_direct_fp4(const LinearArgs& a, SplitScratch* scratch)
     return plan_direct(a, scratch, true);
 }
 
-// Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 48 tokens take the
+// Kernel choice (tuned on MI355X).  FP8 weights with K a multiple of 64 and at least 17 tokens take the
 // kernel that keeps the weights out of LDS -- on the tiled copy of the weight when one is registered
 // (1.10-1.15x the row-major rate: a wave's load is then eight full cache lines instead of sixteen half
 // lines).  The tile shape comes from plan_direct (128- or 64-token tiles of 256, 192 or 128 features, whichever spreads
 // most evenly over the CUs); when none fills the machine the k range is split over workgroups (about one per CU, 16 k-tiles or more each) and a
 // second kernel adds the partial sums -- 2x on 512 tokens x 4096 features x K 12288.  Everything else (FP4,
-// ragged K, 17-47 tokens) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they
+// ragged K) takes the two-operand kernel: 128 x 128 tiles with the XCD-aware order when they
 // give every CU at least two workgroups (k step 128 for long K, where it halves the barriers per FLOP),
 // otherwise 128 x 64 tiles to put more workgroups on the machine.
 // `scratch`: see SplitScratch; nullptr = the stream's grow-on-demand workspace.  Returns false (nothing launched)
@@ -1098,7 +1098,7 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
     if constexpr (WT == DT_FP4 && AT == DT_BF16)
     {
         // FP4 with a tiled copy (codes, then the scales behind all code KiBs): the register-fed kernel
-        if (tiled && a.K % 128 == 0 && a.tokens >= 48 && (long long)a.tokens * a.ldx * 2 < (1LL << 32))
+        if (tiled && a.K % 128 == 0 && a.tokens >= 17 && (long long)a.tokens * a.ldx * 2 < (1LL << 32))
         {
             LinearArgs d = a;
             d.W = tiled;
@@ -1114,7 +1114,7 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
     if constexpr (WT != DT_FP4)
     {
         const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
-        if (a.K % 64 == 0 && a.tokens >= 48 && small_offsets)
+        if (a.K % 64 == 0 && a.tokens >= 17 && small_offsets)
         {
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }

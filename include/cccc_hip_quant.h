@@ -88,7 +88,7 @@ C_EXPORT int hip_absmax(const void* src, int src_type, unsigned int n, void* d_r
  * C of type HALF; the weight is dequantised to half, FP32 accumulation, one rounding to half).
  * `act_scale` is accepted and ignored (it only drives the W8A8 route, cccc/cublas_real.h:871-873).
  * Anything else (both operands quantized, FP4 with HALF, mixed 16-bit types, other C types) returns -1.
- * Device memory: the one case in which the library allocates is an FP8 GEMM of 48 tokens or more whose
+ * Device memory: the one case in which the library allocates is an FP8 GEMM of 17 tokens or more whose
  * output has too few tiles to fill the GPU; it then splits K over workgroups and keeps FP32 partial sums in a
  * scratch buffer per (device, stream) that grows on demand and lives until the process ends (at most
  * 8 * M * N * 4 bytes).  While the stream is being captured into a graph the buffer is never grown: the
@@ -107,7 +107,7 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
  * partial sums: in a static device array of HIP_QUANT_NOALLOC_SCRATCH_BYTES inside the library (one per
  * GPU the library runs on, held until the process ends) instead of a buffer grown on demand.  The call
  * never allocates or frees device memory.  A shape whose k-split needs more than that (splits * M * N * 4
- * bytes, splits <= 8; only FP8 GEMMs of 48 tokens or more with few output tiles split at all) returns -1
+ * bytes, splits <= 8; only FP8 GEMMs of 17 tokens or more with few output tiles split at all) returns -1
  * with a message on stderr and launches nothing; 32 MiB covers 512 tokens x 4096 features.
  * Every call on a GPU shares the one array: calls that overlap on one GPU (two streams, two host
  * threads) race on it and must be ordered by the caller.  Nothing in it needs clearing between calls:
@@ -126,7 +126,7 @@ C_EXPORT int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K,
  * of an FP8 weight W ([n_out][ldw], K contiguous, as loadQuantizedDirect uploads it) into `dst_tiled`
  * -- caller-owned device memory of hip_quant_tiled_size(...) bytes -- and remembers it under the key
  * `W`.  Later hip_quant_gemm calls whose weight pointer, type and shape match may use the tiled copy
- * (today: up to 16 tokens, except one or two tokens on weights under 8 MiB, and the GEMM of 48 tokens or
+ * (today: up to 16 tokens, except one or two tokens on weights under 8 MiB, and the GEMM of 17 tokens or
  * more when K is a multiple of 64): the matrix-core kernels want the 16 rows x 64 codes of one load
  * instruction to be one contiguous KiB.
  * Results agree with the row-major kernels up to the FP32 summation order.  The copy is keyed on the pointer, not
@@ -275,7 +275,7 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
  * activations [tokens][K] and outputs with row pitch ldy[s] -- the q, k and v projections of a prompt, whose narrow members
  * alone leave most of the GPU idle.  The bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not
  * split their k range.  FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
- * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 48 tokens, K not a
+ * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 17 tokens, K not a
  * multiple of 64.  No
  * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
 C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
@@ -285,7 +285,7 @@ C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const voi
  * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product
  * bf16(bf16(g * bf16(sigmoid g)) * u) (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732, :953-966) in one launch, with
  * the bits of the three calls it replaces.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).
- * -1 (nothing launched, use the separate calls): other weight types, fewer than 48 tokens, K not a multiple of 64. */
+ * -1 (nothing launched, use the separate calls): other weight types, fewer than 17 tokens, K not a multiple of 64. */
 C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                                    float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);
 C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);

@@ -92,7 +92,7 @@ def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n
 
 
 @pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", True)])
-@pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512), (48, (64,), 64)])
+@pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512), (48, (64,), 64), (20, (512, 256), 256)])
 def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(gpu, oracle, w_type, tiled, tokens, widths, K):
     """hip_quant_gemm_segments (the q, k, v projections of a prompt as one launch) against one hip_quant_gemm call per
     weight, byte for byte (K short enough that no call splits its k range), on the file layout and on tiled copies, with
@@ -130,7 +130,7 @@ def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(g
             got = from_dev(y1, np.uint16)
             assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
             assert np.array_equal(got, from_dev(y3, np.uint16))
-        assert call(47, K, wt) == -1 and call(tokens, K - 32, wt) == -1 and call(tokens, K, oracle.FP4) == -1
+        assert call(16, K, wt) == -1 and call(tokens, K - 32, wt) == -1 and call(tokens, K, oracle.FP4) == -1
     finally:
         if tiled:
             for wd in wds:
@@ -220,7 +220,7 @@ def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, 
         have = dec.f(got[:tokens * n_out].reshape(tokens, n_out))
         assert np.linalg.norm(have - want) <= 1e-2 * np.linalg.norm(want)
         bad = lambda *a: lib.c.hip_quant_gemm_swiglu(*a)
-        assert bad(n_out, 47, K, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
+        assert bad(n_out, 16, K, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
         assert bad(n_out, tokens, K, ptr(gd), ptr(ud), oracle.FP4, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
         assert bad(n_out, tokens, K - 32, ptr(gd), ptr(ud), wt, K, ctypes.c_float(sg), ctypes.c_float(su), ptr(xd), K, ptr(y1), n_out) == -1
     finally:
