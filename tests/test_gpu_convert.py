@@ -154,3 +154,33 @@ def test_float_to_fp4_blockscale_vs_oracle(gpu, oracle):
         wn, ws = oracle.quantize_fp4_blockscale_kernel(x, block)
         assert np.array_equal(nib.cpu().numpy(), wn) and np.array_equal(sc.cpu().numpy(), ws), (n, block)
     assert lib.float_to_fp4_blockscale(xd.data_ptr(), nib.data_ptr(), sc.data_ptr(), 16, 3) == -1
+
+
+@pytest.mark.parametrize("src_type", ["float", "half", "bf16"])
+@pytest.mark.parametrize("n,offset", [(1, 0), (7, 0), (4099, 0), (4099, 1), (1 << 20, 0), ((1 << 22) + 5, 3)])
+def test_absmax_of_a_tensor(gpu, oracle, src_type, n, offset):
+    """hip_absmax (the per-tensor scale of the on-the-fly FP8 quantiser, cccc-cuda/cuda_functions.cu:2694-2733) against
+    numpy on FLOAT / HALF / BF16 tensors, including a start that is not 16-byte aligned, a ragged tail, a NaN (skipped)
+    and the largest value in the last element; the result buffer is cleared by the call."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(n + offset)
+    x = (rng.standard_normal(n + offset) * 3).astype(np.float32)
+    if n > 4:
+        x[offset + 2] = np.nan
+    x[offset + n - 1] = -77.5 if n > 1 else 0.25
+    if src_type == "float":
+        host, code, vals = x, oracle.FLOAT, x
+    elif src_type == "half":
+        host = x.astype(np.float16)
+        code, vals = oracle.HALF, host.astype(np.float32)
+    else:
+        bits = oracle.f32_to_bf16(np.nan_to_num(x, nan=0.0))
+        if n > 4:
+            bits[offset + 2] = 0x7FC0
+        host, code, vals = bits, oracle.BF16, oracle.bf16_to_f32(bits)
+    d = to_dev(torch, dev, host)
+    res = torch.full((2,), 123.0, dtype=torch.float32, device=dev)
+    assert lib.absmax(d.data_ptr() + offset * host.dtype.itemsize, code, n, res.data_ptr()) == 0
+    got = res.cpu().numpy()
+    assert got[1] == 123.0
+    assert got[0] == np.nanmax(np.abs(vals[offset:offset + n]))
