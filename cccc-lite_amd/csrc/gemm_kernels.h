@@ -1045,8 +1045,12 @@ inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool f
     {
         const long long base = a.tokens > 64 ? tiles8 : tiles4;
         long long s = (cus + base / 2) / base;
-        if (s > 8) { s = 8; }
-        if (s > a.K / 1024) { s = a.K / 1024; }
+        // up to 64 tokens the weight bytes bound the launch and finer k ranges put more workgroups on them (32 tokens:
+        // 4096 x 4096 17.3 -> 14.6 us, 1024 x 4096 16.3 -> 13.5, 4096 x 12288 28.5 -> 24.0); above that the FP32 partial
+        // sums weigh more and a range keeps 1024 elements of k or more
+        const long long s_max = a.tokens <= 64 ? 16 : 8, k_min = a.tokens <= 64 ? 512 : 1024;
+        if (s > s_max) { s = s_max; }
+        if (s > a.K / k_min) { s = a.K / k_min; }
         if (!attach_split(plan, a, s, scratch)) { return plan; }
         if (plan.splits > 1)
         {

@@ -107,7 +107,7 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
  * partial sums: in a static device array of HIP_QUANT_NOALLOC_SCRATCH_BYTES inside the library (one per
  * GPU the library runs on, held until the process ends) instead of a buffer grown on demand.  The call
  * never allocates or frees device memory.  A shape whose k-split needs more than that (splits * M * N * 4
- * bytes, splits <= 8; only FP8 GEMMs of 17 tokens or more with few output tiles split at all) returns -1
+ * bytes, splits <= 16; only FP8 GEMMs of 17 tokens or more with few output tiles split at all) returns -1
  * with a message on stderr and launches nothing; 32 MiB covers 512 tokens x 4096 features.
  * Every call on a GPU shares the one array: calls that overlap on one GPU (two streams, two host
  * threads) race on it and must be ordered by the caller.  Nothing in it needs clearing between calls:
