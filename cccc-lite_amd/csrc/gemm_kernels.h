@@ -284,8 +284,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a_in, const int n_tiles, float* __restrict__ partial)
 {
-    static_assert(!PAIR || (!SPLIT && NB % 2 == 0 && AT == DT_BF16), "pair: unsplit, an even number of feature blocks, BF16");
-    static_assert(!SEG || (!SPLIT && !PAIR), "segments: unsplit single linears");
+    static_assert(!PAIR || (NB % 2 == 0 && AT == DT_BF16), "pair: an even number of feature blocks, BF16");
+    static_assert(!SEG || !PAIR, "segments: single linears");
     constexpr int NBO = PAIR ? NB / 2 : NB;     // feature blocks of a wave in the output
     constexpr int BTOK = MB * 16;               // tokens per workgroup
     constexpr int BK = 64, CPR = 8;
@@ -313,6 +313,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         a.w_scale = a_in.seg_w_scale[s];
         a.y_stride_tok = a_in.seg_y_stride_tok[s];
         n_tile -= a_in.seg_tile0[s];
+        // the partial sums of a segment follow those of the segments before it
+        if constexpr (SPLIT) { partial += (long long)gridDim.y * a_in.tokens * ((s > 0 ? a_in.seg_n_out[0] : 0) + (s > 1 ? a_in.seg_n_out[1] : 0)); }
     }
     const int out_base = n_tile * (64 * NBO) + wave * (16 * NBO);
     const int tok_base = m_tile * BTOK;
@@ -453,7 +455,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
     }
 
     const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
-    if constexpr (PAIR)
+    if constexpr (PAIR && !SPLIT)
     {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -495,12 +497,13 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
         {
-            const int out = out_base + nb * 16 + 4 * g;
+            const int out = out_base + (nb % NBO) * 16 + 4 * g;
             if (out >= a.n_out) { continue; }
             const f32x4 r = acc[mb][nb];
             if constexpr (SPLIT)
             {
-                float* p = partial + ((long long)blockIdx.y * a.tokens + tok) * a.n_out + out;
+                // pair: the up weight's sums are a second set behind all of the gate weight's
+                float* p = partial + (((long long)(nb / NBO) * gridDim.y + blockIdx.y) * a.tokens + tok) * a.n_out + out;
                 if (wide_store && out + 3 < a.n_out) { *(f32x4*)p = r; }
                 else
                 {
@@ -538,19 +541,58 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
 
 // Sums the FP32 partial tiles of a k-split GEMM and applies alpha / beta and the one rounding.  One thread
 // per four consecutive features of a token (n_out is a multiple of 4 on this path).
-template <int AT>
-__global__ __launch_bounds__(256) void gemm_splitk_combine_kernel(const float* __restrict__ partial, const int splits, const LinearArgs a)
+// SEG: the partial sums of up to three linears, each laid out as its own k-split GEMM, one after the other; a thread finds
+// its segment from its feature.  PAIR: gate sums, then up sums; the thread adds both and writes the SwiGLU product with the
+// roundings of the unsplit pair kernel's epilogue.
+template <int AT, bool SEG = false, bool PAIR = false>
+__global__ __launch_bounds__(256) void gemm_splitk_combine_kernel(const float* __restrict__ partial, const int splits, const LinearArgs a_in)
 {
-    const long long groups = (long long)a.tokens * (a.n_out / 4);
-    const long long slice = (long long)a.tokens * a.n_out;
-    const bool wide_store = a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0;
+    LinearArgs a = a_in;
+    const int n_all = SEG ? a_in.seg_n_out[0] + a_in.seg_n_out[1] + a_in.seg_n_out[2] : a_in.n_out;
+    const long long groups = (long long)a.tokens * (n_all / 4);
     for (long long q = (long long)blockIdx.x * 256 + threadIdx.x; q < groups; q += (long long)gridDim.x * 256)
     {
-        const int tok = (int)(q / (a.n_out / 4));
-        const int out = (int)(q % (a.n_out / 4)) * 4;
-        f32x4 r = *(const f32x4*)(partial + q * 4);
-        for (int s = 1; s < splits; s++) { r += *(const f32x4*)(partial + s * slice + q * 4); }
+        const int tok = (int)(q / (n_all / 4));
+        int out = (int)(q % (n_all / 4)) * 4;
+        const float* p = partial;
+        if constexpr (SEG)
+        {
+            const int n0 = a_in.seg_n_out[0], n01 = n0 + a_in.seg_n_out[1];
+            const int s = out >= n01 ? 2 : (out >= n0 ? 1 : 0);
+            const int start = s == 2 ? n01 : (s == 1 ? n0 : 0);
+            a.Y = a_in.seg_Y[s];
+            a.n_out = a_in.seg_n_out[s];
+            a.y_stride_tok = a_in.seg_y_stride_tok[s];
+            p += (long long)splits * a.tokens * start;
+            out -= start;
+        }
+        const long long slice = (long long)a.tokens * a.n_out;
+        p += (long long)tok * a.n_out + out;
+        f32x4 r = *(const f32x4*)p;
+        for (int s = 1; s < splits; s++) { r += *(const f32x4*)(p + s * slice); }
+        const bool wide_store = a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0;
         uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+        if constexpr (PAIR)
+        {
+            const float* pu = p + splits * slice;
+            f32x4 u = *(const f32x4*)pu;
+            for (int s = 1; s < splits; s++) { u += *(const f32x4*)(pu + s * slice); }
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+            {
+                const float gate = bf16_bits_to_f32(f32_to_bf16_bits(r[v])), up = bf16_bits_to_f32(f32_to_bf16_bits(u[v]));
+                const float sig = bf16_bits_to_f32(f32_to_bf16_bits(1.0f / (1.0f + expf(-gate))));
+                o[v] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(f32_to_bf16_bits(gate * sig)) * up);
+            }
+            if (wide_store) { *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) }; }
+            else
+            {
+#pragma unroll
+                for (int v = 0; v < 4; v++) { y[v * a.y_stride_out] = o[v]; }
+            }
+            continue;
+        }
         if (wide_store)
         {
             uint16_t old[4] = { 0, 0, 0, 0 };
@@ -937,6 +979,43 @@ void launch_gemm_mfma_direct_segments(LinearArgs a)
     for (int s = 0; s < a.n_segments; s++) { scaled = scaled || a.seg_w_scale[s] != 1.0f; }
     const long long tiles8 = (long long)n_tiles * ((a.tokens + 127) / 128);
     const int n_pad = (n_tiles + 7) & ~7;
+    // Few tiles (q, k, v of a 4096-wide model are 24 feature tiles; up to 512 tokens that is under one workgroup for every
+    // second CU): the k range is split over workgroups as in plan_direct, every segment's partial sums laid out as its own
+    // split GEMM one after the other, and one combine launch finishes all of them (36-layer model, 128 tokens: 8.0 -> 7.0 ms;
+    // 256 tokens 8.4 -> 7.6; 512 tokens 10.8 -> 10.5).
+    {
+        int n_all = 0;
+        bool by4 = true;
+        for (int sg = 0; sg < 3; sg++)
+        {
+            if (sg >= a.n_segments) { a.seg_n_out[sg] = 0; }
+            n_all += a.seg_n_out[sg];
+            by4 = by4 && a.seg_n_out[sg] % 4 == 0;
+        }
+        const int mb = a.tokens > 64 ? 8 : 4;
+        const long long base = (long long)n_tiles * ((a.tokens + mb * 16 - 1) / (mb * 16));
+        long long splits = cus / base;
+        if (splits > (mb == 8 ? 8 : 16)) { splits = mb == 8 ? 8 : 16; }
+        if (splits > a.K / 512) { splits = a.K / 512; }
+        float* partial = splits >= 2 && by4 ? (float*)workspace((size_t)splits * a.tokens * n_all * sizeof(float)) : nullptr;
+        if (partial)
+        {
+            const dim3 grid(n_pad * ((a.tokens + mb * 16 - 1) / (mb * 16)), (unsigned)splits);
+            if (mb == 8)
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 8, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            else
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            const long long blocks = ((long long)a.tokens * (n_all / 4) + 255) / 256, cap = (long long)cus * 16;
+            gemm_splitk_combine_kernel<DT_BF16, true, false><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
+            return;
+        }
+    }
     // (on the file layout the 128-token tile is worth having from one workgroup per CU on, see plan_direct)
     if (a.tokens > 64 && (tiles8 >= 2LL * cus || (!TILED && tiles8 >= cus)))
     {
@@ -958,8 +1037,37 @@ void launch_gemm_mfma_direct_pair(const LinearArgs& a)
 {
     const int n_tiles = (a.n_out + 127) / 128;
     const int m_tiles = (a.tokens + 127) / 128;
+    const bool scaled = a.w_scale != 1.0f || a.w_scale_pair != 1.0f;
+    // Up to 128 tokens of a 12288-wide pair are 96 workgroups: the k range is split in two or more and the combine launch
+    // adds the gate and the up sums and writes the SwiGLU product with the same roundings (36-layer model, 128 tokens:
+    // 8.0 -> 7.3 ms; from 129 tokens on, 192 workgroups or more, the split only costs).
+    {
+        const int mb = a.tokens > 64 ? 8 : 4;
+        const int m_split = (a.tokens + mb * 16 - 1) / (mb * 16);
+        long long splits = cu_count() / ((long long)n_tiles * m_split);
+        if (splits > 8) { splits = 8; }
+        if (splits > a.K / 512) { splits = a.K / 512; }
+        float* partial = splits >= 2 && a.n_out % 4 == 0 ? (float*)workspace((size_t)2 * splits * a.tokens * a.n_out * sizeof(float)) : nullptr;
+        if (partial)
+        {
+            const dim3 grid(((n_tiles + 7) & ~7) * m_split, (unsigned)splits);
+            if (mb == 8)
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 8, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            else
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            const long long blocks = ((long long)a.tokens * (a.n_out / 4) + 255) / 256, cap = (long long)cu_count() * 16;
+            gemm_splitk_combine_kernel<DT_BF16, false, true><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
+            return;
+        }
+    }
     const dim3 grid(((n_tiles + 7) & ~7) * m_tiles);
-    if (a.w_scale != 1.0f || a.w_scale_pair != 1.0f) { gemm_mfma_direct_kernel<WT, true, 8, false, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
+    if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, false, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
     else { gemm_mfma_direct_kernel<WT, false, 8, false, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, nullptr); }
 }
 

@@ -444,12 +444,9 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
     for (int li = 0; li < c.layers && rc == 0; li++)
     {
         Layer& L = layers_[li];
-        // q, k, v: one launch for three weights of one type, else three calls.  Up to 64 tokens the FP8 GEMMs are bound by
-        // their weight bytes and each call alone splits its k range over more workgroups than the joint launch has tiles
-        // (32 tokens of a 36-layer 4096-wide model: 6.1 ms against 6.8; from 100 tokens on the joint launches are ahead)
-        const bool joint = n > 64 || L.wq->getDataType() == FP4_E2M1;
+        // q, k, v: one launch for three weights of one type, else three calls
         int qkv = -1;
-        if (rc == 0 && joint && L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
+        if (rc == 0 && L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
         {
             const int widths[3] = { q_out, kv_out, kv_out };
             const void* const weights[3] = { L.wq->data(), L.wk->data(), L.wv->data() };
@@ -479,7 +476,7 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         if (rc == 0) { rc = add_norm(*pf_.x, *pf_.o, *pf_.r1, *L.rms_ffn, *pf_.xn); }
         // gate, up and their SwiGLU product: one launch for two FP8 weights of one type, else the three calls
         int fused = -1;
-        if (rc == 0 && n > 64 && L.w_gate->getDataType() == L.w_up->getDataType())
+        if (rc == 0 && L.w_gate->getDataType() == L.w_up->getDataType())
         {
             fused = hip_quant_gemm_swiglu(c.inter, n, c.hidden, L.w_gate->data(), L.w_up->data(), (int)L.w_gate->getDataType(), c.hidden,
                                           L.w_gate->getQuantScale(), L.w_up->getQuantScale(), pf_.xn->data(), c.hidden, pf_.gated->data(), c.inter);

@@ -273,8 +273,10 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
 /* Up to three linears on the same activations in one launch: Y[s][t][o] = bf16(W[s] x_t), s < n_segments <= 3, FP8 weights
  * [n_out[s]][K] of one type, K and row pitch ldw (all on their registered tiled copies, or all on the file layout), BF16
  * activations [tokens][K] and outputs with row pitch ldy[s] -- the q, k and v projections of a prompt, whose narrow members
- * alone leave most of the GPU idle.  The bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not
- * split their k range.  FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
+ * alone leave most of the GPU idle.  With too few output tiles for the GPU (FP8, K >= 1024) the k range is split over
+ * workgroups, the FP32 partial sums go to a workspace the library grows on demand and one more launch adds them for all
+ * segments; otherwise the bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not split either.
+ * FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
  * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 17 tokens, K not a
  * multiple of 64.  No
  * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
@@ -284,7 +286,9 @@ C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const voi
  * MLP block (two FP8 weights of one shape [n_out][K], row pitch ldw, dequantisation multipliers as in hip_quant_gemm; both
  * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product
  * bf16(bf16(g * bf16(sigmoid g)) * u) (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732, :953-966) in one launch, with
- * the bits of the three calls it replaces.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).
+ * the bits of the three calls it replaces -- or, with too few output tiles for the GPU (K >= 1024), the k range split over
+ * workgroups and a second launch that adds the FP32 partial sums (workspace grown on demand) and writes the product with
+ * the same roundings.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).
  * -1 (nothing launched, use the separate calls): other weight types, fewer than 17 tokens, K not a multiple of 64. */
 C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                                    float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);

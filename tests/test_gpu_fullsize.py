@@ -422,6 +422,59 @@ def test_fused_prompt_gemms_at_qwen3_8b_shapes_equal_the_separate_calls(gpu, pkg
                 assert lib.weight_release(w.data_ptr()) == 0
 
 
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("T", [32, 128])
+def test_fused_prompt_gemms_of_a_short_prompt_at_qwen3_8b_shapes(gpu, pkg, oracle, dec, tiled, T):
+    """32 and 128 tokens at Qwen3-8B widths, where the q,k,v launch (24 feature tiles) and the gate / up pair (96) split
+    their k range over workgroups and a combine launch finishes them -- for the pair with the SwiGLU product: sampled
+    features of q, k, v and of the product against the exact contraction, nothing written past the outputs."""
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(78 + T)
+    K = 4096
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    x = draw_bf16(torch, dev, gen, (T, K))
+    widths = (4096, 1024, 1024, 12288, 12288)                  # q, k, v, gate, up
+    ws = [draw_e5m2(torch, dev, gen, n, K) for n in widths]
+    keep = []
+    if tiled:
+        for w, n in zip(ws, widths):
+            td = torch.zeros(lib.tiled_size(E5M2, n, K), dtype=torch.uint8, device=dev)
+            assert lib.weight_prepare(w.data_ptr(), E5M2, n, K, K, td.data_ptr()) == 0
+            keep.append(td)
+    try:
+        X = host_bits(x).reshape(T, K)
+        exact = lambda w, rows: oracle.linear_exact(oracle.dequant_fp8_to_bf16(w[torch.as_tensor(rows, device=dev)].cpu().numpy(), E5M2), X)
+        one = [torch.zeros(T * n + 64, dtype=torch.int16, device=dev) for n in widths[:3]]
+        arr_i = (ctypes.c_int * 3)(*widths[:3])
+        arr_w = (ctypes.c_void_p * 3)(*[w.data_ptr() for w in ws[:3]])
+        arr_s = (ctypes.c_float * 3)(1.0, 1.0, 1.0)
+        arr_y = (ctypes.c_void_p * 3)(*[y.data_ptr() for y in one])
+        assert lib.c.hip_quant_gemm_segments(3, arr_i, arr_w, arr_s, arr_y, arr_i, E5M2, T, K, K, ptr(x), K) == 0
+        assert lib.last_kernel() == ("gemm_segments_tiled" if tiled else "gemm_segments")
+        for y, w, n, name in zip(one, ws, widths, "qkv"):
+            bits = host_bits(y)
+            assert not bits[T * n:].any(), name
+            rows = np.random.default_rng(n + T).choice(n, size=64, replace=False)
+            check_rows(bf16_f64(oracle, bits[:T * n].reshape(T, n)[:, rows]), exact(w, rows), f"{name} of the q,k,v launch, {T} tokens")
+        fused = torch.zeros(T * 12288 + 64, dtype=torch.int16, device=dev)
+        assert lib.c.hip_quant_gemm_swiglu(12288, T, K, ptr(ws[3]), ptr(ws[4]), E5M2, K, ctypes.c_float(1.0), ctypes.c_float(1.0),
+                                           ptr(x), K, ptr(fused), 12288) == 0
+        assert lib.last_kernel() == ("gemm_swiglu_tiled" if tiled else "gemm_swiglu")
+        bits = host_bits(fused)
+        assert not bits[T * 12288:].any()
+        rows = np.random.default_rng(5 + T).choice(12288, size=64, replace=False)
+        gate = oracle.f32_to_bf16(exact(ws[3], rows).astype(np.float32))
+        up = oracle.f32_to_bf16(exact(ws[4], rows).astype(np.float32))
+        want = dec.silu_mul(dec.f(gate), dec.f(up))
+        have = dec.f(bits[:T * 12288].reshape(T, 12288)[:, rows])
+        assert np.isfinite(have).all() and have.any()
+        assert np.linalg.norm(have - want) <= 1e-2 * np.linalg.norm(want)
+    finally:
+        if tiled:
+            for w in ws:
+                assert lib.weight_release(w.data_ptr()) == 0
+
+
 @pytest.mark.parametrize("arch", ["qwen3_8b_fp8", "llama31_8b_fp4"])
 def test_prompt_phase_at_full_widths_equals_token_by_token_decoding(gpu, pkg, oracle, dec, arch):
     """DecodeModel::prefill at the benchmark's widths (two layers): 130 prompt tokens from position 0 in one call against the

@@ -4,7 +4,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from gpu_util import from_dev, to_dev
+from gpu_util import check_rows, from_dev, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -95,19 +95,22 @@ def test_prefill_attention_follows_the_oracle_token_by_token(gpu, oracle, dec, n
 @pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512), (48, (64,), 64), (20, (512, 256), 256)])
 def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(gpu, oracle, w_type, tiled, tokens, widths, K):
     """hip_quant_gemm_segments (the q, k, v projections of a prompt as one launch) against one hip_quant_gemm call per
-    weight, byte for byte (K short enough that no call splits its k range), on the file layout and on tiled copies, with
-    a different per-tensor scale per weight for E4M3; unsupported arguments are refused."""
+    weight and against the exact contraction, on the file layout and on tiled copies, with a different per-tensor scale per
+    weight for E4M3.  Byte for byte where K is too short for a k split (under 1024); at K = 1024 the joint launch splits
+    its few tiles in two k ranges with one combine for all segments, the separate calls do not, and the two differ by
+    the order of the FP32 sums only.  Unsupported arguments are refused."""
     torch, dev, lib = gpu
     rng = np.random.default_rng(tokens + K + len(widths))
     wt = oracle.E5M2 if w_type == "e5m2" else oracle.E4M3
     scales = [1.0] * len(widths) if w_type == "e5m2" else [0.011, 0.017, 0.023][:len(widths)]
     X = oracle.f32_to_bf16((rng.standard_normal((tokens, K)) * (0.05 if w_type == "e5m2" else 1.0)).astype(np.float32))
     xd = to_dev(torch, dev, X)
-    wds, keep, sep, one = [], [], [], []
+    wds, keep, sep, one, host_w = [], [], [], [], []
     for n_out in widths:
         W = rng.integers(0, 256, size=(n_out, K), dtype=np.uint8)
         if w_type == "e5m2": W[(W & 0x7C) == 0x7C] = 0x3C
         else: W[(W & 0x7F) == 0x7F] = 0x38
+        host_w.append(W)
         wds.append(to_dev(torch, dev, W))
         if tiled:
             t = torch.zeros(lib.tiled_size(wt, n_out, K), dtype=torch.uint8, device=dev)
@@ -126,10 +129,16 @@ def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(g
         call = lambda toks, k, typ: lib.c.hip_quant_gemm_segments(n, arr_i, arr_w, arr_s, arr_y, arr_i, typ, toks, k, K, ptr(xd), K)
         assert call(tokens, K, wt) == 0
         assert lib.last_kernel() == ("gemm_segments_tiled" if tiled else "gemm_segments")
-        for y1, y3, n_out in zip(one, sep, widths):
+        for y1, y3, n_out, W, sc in zip(one, sep, widths, host_w, scales):
             got = from_dev(y1, np.uint16)
             assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
-            assert np.array_equal(got, from_dev(y3, np.uint16))
+            if K < 1024:
+                assert np.array_equal(got, from_dev(y3, np.uint16))
+            have = oracle.bf16_to_f32(got[:tokens * n_out].reshape(tokens, n_out)).astype(np.float64)
+            other = oracle.bf16_to_f32(from_dev(y3, np.uint16)[:tokens * n_out].reshape(tokens, n_out)).astype(np.float64)
+            want = oracle.linear_exact(oracle.dequant_fp8_to_bf16(W, wt, sc), X)
+            check_rows(have, want, f"segment of {n_out} features")
+            assert (np.linalg.norm(have - other, axis=1) <= 2e-3 * np.linalg.norm(want, axis=1)).all()
         assert call(16, K, wt) == -1 and call(tokens, K - 32, wt) == -1 and call(tokens, K, oracle.FP4) == -1
     finally:
         if tiled:
@@ -181,10 +190,12 @@ def test_fp4_linears_that_share_their_input_in_one_launch(gpu, oracle, block, to
 @pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e5m2", True), ("e4m3", False), ("e4m3", True)])
 @pytest.mark.parametrize("tokens,n_out,K", [(60, 512, 256), (130, 200, 1024), (300, 1536, 512)])
 def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, w_type, tiled, tokens, n_out, K):
-    """hip_quant_gemm_swiglu against two hip_quant_gemm calls and hip_swiglu_bf16 on the same inputs, byte for byte (K is
-    short enough that no call splits its k range, so every sum runs in the same order), on the file layout and on the
-    tiled copies, with the per-tensor scales of an E4M3 file differing between gate and up; and against the oracle's
-    exact contraction.  Unsupported arguments are refused with -1."""
+    """hip_quant_gemm_swiglu against two hip_quant_gemm calls and hip_swiglu_bf16 on the same inputs -- byte for byte where K
+    is too short for a k split (under 1024), so every sum runs in the same order; at K = 1024 the pair launch splits its
+    few tiles in two k ranges and its combine launch writes the product, which may then differ from the three calls where
+    a gate or up sum lands on the other side of a BF16 rounding boundary -- and against the oracle's exact contraction, on
+    the file layout and on the tiled copies, with the per-tensor scales of an E4M3 file differing between gate and up.
+    Unsupported arguments are refused with -1."""
     torch, dev, lib = gpu
     rng = np.random.default_rng(tokens + n_out + K)
     wt = oracle.E5M2 if w_type == "e5m2" else oracle.E4M3
@@ -212,8 +223,10 @@ def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, 
         assert lib.last_kernel() == ("gemm_swiglu_tiled" if tiled else "gemm_swiglu")
         got = from_dev(y1, np.uint16)
         assert not got[tokens * n_out:].any()
-        if (tokens * n_out) % 8 == 0:
+        if (tokens * n_out) % 8 == 0 and K < 1024:
             assert np.array_equal(got, from_dev(y3, np.uint16))
+        elif (tokens * n_out) % 8 == 0:
+            assert np.mean(got != from_dev(y3, np.uint16)) < 0.02
         gate = oracle.f32_to_bf16(oracle.linear_exact(oracle.dequant_fp8_to_bf16(Wg, wt, sg), X).astype(np.float32))
         up = oracle.f32_to_bf16(oracle.linear_exact(oracle.dequant_fp8_to_bf16(Wu, wt, su), X).astype(np.float32))
         want = dec.silu_mul(dec.f(gate), dec.f(up))
