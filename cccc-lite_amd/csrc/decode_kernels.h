@@ -752,13 +752,24 @@ __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const uint16_t* __re
     if constexpr (VEC)
     {
         const unsigned n_chunks = inner / 8u;               // 16-byte chunks of the row; chunk c belongs to lane c % 64
-        u32x4 v[RMS_CHUNKS];
+        // every load is issued before the first use (a load inside a per-lane branch waits for the one before it: eight
+        // memory latencies in a row on a 4096-wide row); lanes past the row's end re-read its last chunk and drop it
+        u32x4 v[RMS_CHUNKS], w[RMS_CHUNKS];
+        const int n_j = n_chunks <= 64u ? 1 : RMS_CHUNKS;   // short rows (the per-head norms) are one chunk per lane at most
 #pragma unroll
         for (int j = 0; j < RMS_CHUNKS; j++)
         {
-            const unsigned c = lane + 64u * j;
-            v[j] = u32x4{ 0u, 0u, 0u, 0u };
-            if (c < n_chunks) { v[j] = *(const u32x4*)(x + c * 8u); }
+            if (j < n_j)
+            {
+                const unsigned c = min(lane + 64u * j, n_chunks - 1u);
+                v[j] = *(const u32x4*)(x + c * 8u);
+                w[j] = *(const u32x4*)(scale + c * 8u);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RMS_CHUNKS; j++)
+        {
+            if (j >= n_j || lane + 64u * j >= n_chunks) { v[j] = u32x4{ 0u, 0u, 0u, 0u }; }
             sumsq += sumsq8(v[j]);
         }
         const float invstd = rsqrtf(wave_sum(sumsq) / (float)inner + eps);
@@ -767,7 +778,7 @@ __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const uint16_t* __re
         for (int j = 0; j < RMS_CHUNKS; j++)
         {
             const unsigned c = lane + 64u * j;
-            if (c < n_chunks) { *(u32x4*)(y + c * 8u) = normed8(v[j], *(const u32x4*)(scale + c * 8u), invstd); }
+            if (j < n_j && c < n_chunks) { *(u32x4*)(y + c * 8u) = normed8(v[j], w[j], invstd); }
         }
     }
     else

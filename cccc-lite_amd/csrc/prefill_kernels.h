@@ -480,21 +480,34 @@ static __global__ __launch_bounds__(256) void add_rms_norm_rows_kernel(const uin
     if (row >= outer) { return; }
     const size_t base = (size_t)row * inner;
     const unsigned n_chunks = inner / 8u;                   // 16-byte chunks of the row; chunk c belongs to lane c % 64
-    u32x4 v[RMS_CHUNKS];
+    // every load is issued before the first use (a load inside a per-lane branch waits for the one before it); lanes past
+    // the row's end re-read its last chunk and drop it
+    u32x4 v[RMS_CHUNKS], va[RMS_CHUNKS], vb[RMS_CHUNKS], w[RMS_CHUNKS];
+    const int n_j = n_chunks <= 64u ? 1 : RMS_CHUNKS;
+#pragma unroll
+    for (int j = 0; j < RMS_CHUNKS; j++)
+    {
+        if (j < n_j)
+        {
+            const unsigned c = min(lane + 64u * j, n_chunks - 1u);
+            va[j] = *(const u32x4*)(A + base + c * 8u);
+            vb[j] = *(const u32x4*)(B + base + c * 8u);
+            w[j] = *(const u32x4*)(scale + c * 8u);
+        }
+    }
     float sumsq = 0.0f;
 #pragma unroll
     for (int j = 0; j < RMS_CHUNKS; j++)
     {
         const unsigned c = lane + 64u * j;
         v[j] = u32x4{ 0u, 0u, 0u, 0u };
-        if (c < n_chunks)
+        if (j < n_j && c < n_chunks)
         {
-            const u32x4 va = *(const u32x4*)(A + base + c * 8u), vb = *(const u32x4*)(B + base + c * 8u);
 #pragma unroll
             for (int d = 0; d < 4; d++)
             {
-                const float lo = bf16_bits_to_f32(va[d] & 0xFFFFu) + bf16_bits_to_f32(vb[d] & 0xFFFFu);
-                const float hi = bf16_bits_to_f32(va[d] >> 16) + bf16_bits_to_f32(vb[d] >> 16);
+                const float lo = bf16_bits_to_f32(va[j][d] & 0xFFFFu) + bf16_bits_to_f32(vb[j][d] & 0xFFFFu);
+                const float hi = bf16_bits_to_f32(va[j][d] >> 16) + bf16_bits_to_f32(vb[j][d] >> 16);
                 v[j][d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
             }
             *(u32x4*)(R + base + c * 8u) = v[j];
@@ -506,7 +519,7 @@ static __global__ __launch_bounds__(256) void add_rms_norm_rows_kernel(const uin
     for (int j = 0; j < RMS_CHUNKS; j++)
     {
         const unsigned c = lane + 64u * j;
-        if (c < n_chunks) { *(u32x4*)(Y + base + c * 8u) = normed8(v[j], *(const u32x4*)(scale + c * 8u), invstd); }
+        if (j < n_j && c < n_chunks) { *(u32x4*)(Y + base + c * 8u) = normed8(v[j], w[j], invstd); }
     }
 }
 
