@@ -830,12 +830,12 @@ def main():
             extra["prompt_phase"] = {"workload": "prompt phase of the same Qwen3-8B W8A16 model from an empty cache (DecodeModel::prefill): per layer seven "
                                                  "quantized GEMMs with T columns on the row-major weights, RMSNorm / RoPE / append rows, causal attention, "
                                                  "residual adds, SwiGLU; then the head on the last token",
-                                     "cases": prompt_phase(ws, model, token_counts=(32, 512, 2048))}
+                                     "cases": prompt_phase(ws, model, token_counts=(32, 128, 512, 2048))}
             # the same with the load-time tiled copy of every linear (DecodeModel::setRepackLinears: twice the weight memory)
             for li in range(QWEN3_8B["layers"]):
                 for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
                     assert model.prepare_tiled(li, name)
-            extra["prompt_phase"]["cases"] += prompt_phase(ws, model, token_counts=(512, 2048, DECODE_CTX), layout="tiled copies")
+            extra["prompt_phase"]["cases"] += prompt_phase(ws, model, token_counts=(32, 128, 512, 2048, DECODE_CTX), layout="tiled copies")
             extra["generate"] = generate_run(ws, model, use_graph)
             if not args.no_fp4_step:
                 # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
