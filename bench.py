@@ -839,7 +839,7 @@ def main():
             extra["generate"] = generate_run(ws, model, use_graph)
             if not args.no_fp4_step:
                 # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
-                extra["fp4_decode_step"]["prompt_phase"] = prompt_phase(ws, fp4_model, layout="tiled copies", c=LLAMA31_8B)
+                extra["fp4_decode_step"]["prompt_phase"] = prompt_phase(ws, fp4_model, token_counts=(32, 128, 512, 2048), layout="tiled copies", c=LLAMA31_8B)
         del model
         if not args.no_baselines:
             torch.cuda.empty_cache()

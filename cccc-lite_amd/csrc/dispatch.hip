@@ -585,7 +585,9 @@ int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const*
 int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                           float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy)
 {
-    if (w_type != DT_E5M2 && w_type != DT_E4M3) { return -1; }
+    const bool fp4 = w_type == DT_FP4;
+    if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
+    if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
     if (n_out <= 0 || tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
     if (!W_gate || !W_up || !X || !Y || !aligned16(W_gate) || !aligned16(W_up) || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)n_out * ldw >= (1LL << 32) || (long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
@@ -608,6 +610,20 @@ int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, cons
     // both weights on their tiled copies, or both on the file layout
     const uint8_t* tg = ccq::lookup_tiled(W_gate, w_type, n_out, K, ldw);
     const uint8_t* tu = tg ? ccq::lookup_tiled(W_up, w_type, n_out, K, ldw) : nullptr;
+    if (fp4)
+    {
+        // FP4 runs on the tiled copies only (codes, then the scale bytes), both of one block length
+        if (!tg || !tu) { return -1; }
+        const unsigned block = tiled_block_of(W_gate);
+        if (tiled_block_of(W_up) != block) { return -1; }
+        a.W = tg;
+        a.W_pair = tu;
+        note_kernel("gemm_swiglu_tiled");
+        if (block == 16) { launch_gemm4_mfma_direct_pair<16>(a); }
+        else if (block == 32) { launch_gemm4_mfma_direct_pair<32>(a); }
+        else { return -1; }
+        return finish("quant_gemm_swiglu");
+    }
     if (tg && tu)
     {
         a.W = tg;

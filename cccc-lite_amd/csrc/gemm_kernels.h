@@ -648,12 +648,16 @@ __device__ __forceinline__ u32x4 dequant8_fp4_blocks(uint32_t w, float s_lo, flo
 
 // SEG: as in gemm_mfma_direct_kernel -- up to three linears on the same activations, a workgroup takes weight, scales,
 // output and width of the segment its feature tile belongs to (a.seg_W[s] = tiled codes with the scales behind them).
-template <int BLOCK, int MB, bool SPLIT, int NB = 4, bool SEG = false>
+// PAIR: as in the FP8 kernel -- a.W = gate, a.W_pair = up, two tiled copies of one shape (so the up weight's codes and scale
+// bytes sit at the same offsets behind a.W_pair as the gate's behind a.W); a wave's first NB / 2 feature blocks are gate
+// rows, the others the same rows of up; SwiGLU product in the epilogue, or in the combine launch when the k range is split.
+template <int BLOCK, int MB, bool SPLIT, int NB = 4, bool SEG = false, bool PAIR = false>
 __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a_in, const uint8_t* scales_in, const int n_tiles,
                                                                                         float* __restrict__ partial)
 {
-    static_assert(!SEG || !SPLIT, "segments: unsplit");
     static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    static_assert(!PAIR || (NB % 2 == 0 && !SEG), "pair: an even number of feature blocks, one pair of weights");
+    constexpr int NBO = PAIR ? NB / 2 : NB;     // feature blocks of a wave in the output
     constexpr int NS = 128 / BLOCK;             // scale bytes per row and chunk
     constexpr int BTOK = MB * 16;
     constexpr int BK = 64, CPR = 8;
@@ -681,8 +685,10 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
         a.y_stride_tok = a_in.seg_y_stride_tok[s];
         tiled_scales = a.W + (long long)((a.n_out + 15) / 16) * (a.K / 128) * 1024;
         n_tile -= a_in.seg_tile0[s];
+        // the partial sums of a segment follow those of the segments before it
+        if constexpr (SPLIT) { partial += (long long)gridDim.y * a_in.tokens * ((s > 0 ? a_in.seg_n_out[0] : 0) + (s > 1 ? a_in.seg_n_out[1] : 0)); }
     }
-    const int out_base = n_tile * (64 * NB) + wave * (16 * NB);
+    const int out_base = n_tile * (64 * NBO) + wave * (16 * NBO);
     const int tok_base = m_tile * BTOK;
     const int i16 = lane & 15;
     const int g = lane >> 4;
@@ -704,9 +710,15 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
     {
-        const long long tile = min(out_base / 16 + nb, (a.n_out + 15) / 16 - 1);     // a clamped tile is computed and dropped
+        const long long tile = min(out_base / 16 + nb % NBO, (a.n_out + 15) / 16 - 1);     // a clamped tile is computed and dropped
         w_base[nb] = (tile * chunks_total + c_begin) * 1024;
         s_base[nb] = (tile * chunks_total + c_begin) * (16 * NS);
+        if (PAIR && nb >= NBO)
+        {
+            const long long up = (long long)((intptr_t)a.W_pair - (intptr_t)a.W);     // the up copy, addressed from the gate copy
+            w_base[nb] += up;
+            s_base[nb] += up;
+        }
     }
     const uint32_t w_off = lane * 16, s_off = i16 * NS;
     uint32_t x_off[X_PER_THREAD];
@@ -854,6 +866,40 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
     }
 
     const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
+    if constexpr (PAIR && !SPLIT)
+    {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+        {
+            const int tok = tok_base + mb * 16 + i16;
+            if (tok >= a.tokens) { continue; }
+#pragma unroll
+            for (int nb = 0; nb < NBO; nb++)
+            {
+                const int out = out_base + nb * 16 + 4 * g;
+                if (out >= a.n_out) { continue; }
+                uint16_t o[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                {
+                    const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc[mb][nb][v])), up = bf16_bits_to_f32(f32_to_bf16_bits(acc[mb][nb + NBO][v]));
+                    const float sig = bf16_bits_to_f32(f32_to_bf16_bits(1.0f / (1.0f + expf(-gate))));
+                    o[v] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(f32_to_bf16_bits(gate * sig)) * up);
+                }
+                uint16_t* y = a.Y + (long long)tok * a.y_stride_tok + (long long)out * a.y_stride_out;
+                if (wide_store && out + 3 < a.n_out) { *(uint2*)y = uint2{ (uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16) }; }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                    {
+                        if (out + v < a.n_out) { y[v * a.y_stride_out] = o[v]; }
+                    }
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
     {
@@ -862,12 +908,13 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
         {
-            const int out = out_base + nb * 16 + 4 * g;
+            const int out = out_base + (nb % NBO) * 16 + 4 * g;
             if (out >= a.n_out) { continue; }
             const f32x4 r = acc[mb][nb];
             if constexpr (SPLIT)
             {
-                float* p = partial + ((long long)blockIdx.y * a.tokens + tok) * a.n_out + out;
+                // pair: the up weight's sums are a second set behind all of the gate weight's
+                float* p = partial + (((long long)(nb / NBO) * gridDim.y + blockIdx.y) * a.tokens + tok) * a.n_out + out;
                 if (wide_store && out + 3 < a.n_out) { *(f32x4*)p = r; }
                 else
                 {
@@ -957,8 +1004,59 @@ void launch_gemm4_mfma_direct_segments(LinearArgs a)
     }
     a.seg_tile0[3] = n_tiles;
     for (int s = a.n_segments; s < 3; s++) { a.seg_tile0[s] = n_tiles; }
+    // few tiles: the k range split over workgroups and one combine launch for all segments, as for FP8 below
+    {
+        const int cus = cu_count();
+        int n_all = 0;
+        bool by4 = true;
+        for (int sg = 0; sg < 3; sg++)
+        {
+            if (sg >= a.n_segments) { a.seg_n_out[sg] = 0; }
+            n_all += a.seg_n_out[sg];
+            by4 = by4 && a.seg_n_out[sg] % 4 == 0;
+        }
+        const int mb = a.tokens > 64 ? 8 : 4;
+        const int m_tiles = (a.tokens + mb * 16 - 1) / (mb * 16);
+        long long splits = cus / ((long long)n_tiles * m_tiles);
+        if (splits > (mb == 8 ? 8 : 16)) { splits = mb == 8 ? 8 : 16; }
+        if (splits > a.K / 512) { splits = a.K / 512; }
+        float* partial = splits >= 2 && by4 ? (float*)workspace((size_t)splits * a.tokens * n_all * sizeof(float)) : nullptr;
+        if (partial)
+        {
+            const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, (unsigned)splits);
+            if (mb == 8) { gemm4_mfma_direct_kernel<BLOCK, 8, true, 4, true><<<grid, 256, 0, stream()>>>(a, nullptr, n_tiles, partial); }
+            else { gemm4_mfma_direct_kernel<BLOCK, 4, true, 4, true><<<grid, 256, 0, stream()>>>(a, nullptr, n_tiles, partial); }
+            const long long blocks = ((long long)a.tokens * (n_all / 4) + 255) / 256, cap = (long long)cus * 16;
+            gemm_splitk_combine_kernel<DT_BF16, true, false><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
+            return;
+        }
+    }
     const dim3 grid(((n_tiles + 7) & ~7) * ((a.tokens + 63) / 64));
     gemm4_mfma_direct_kernel<BLOCK, 4, false, 4, true><<<grid, 256, 0, stream()>>>(a, nullptr, n_tiles, nullptr);
+}
+
+// FP4 gate / up pair with the SwiGLU product (tiled copies; a.W / a.W_pair = the copies, codes then scale bytes): 64 tokens
+// x 128 output features per workgroup, the k range split when those are too few for the GPU
+template <int BLOCK>
+void launch_gemm4_mfma_direct_pair(const LinearArgs& a)
+{
+    const uint8_t* tiled_scales = a.W + (long long)((a.n_out + 15) / 16) * (a.K / 128) * 1024;
+    const int n_tiles = (a.n_out + 127) / 128;
+    const int m_tiles = (a.tokens + 63) / 64;
+    long long splits = cu_count() / ((long long)n_tiles * m_tiles);
+    if (splits > 8) { splits = 8; }
+    if (splits > a.K / 512) { splits = a.K / 512; }
+    float* partial = splits >= 2 && a.n_out % 4 == 0 ? (float*)workspace((size_t)2 * splits * a.tokens * a.n_out * sizeof(float)) : nullptr;
+    if (partial)
+    {
+        const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, (unsigned)splits);
+        gemm4_mfma_direct_kernel<BLOCK, 4, true, 4, false, true><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, partial);
+        const long long blocks = ((long long)a.tokens * (a.n_out / 4) + 255) / 256, cap = (long long)cu_count() * 16;
+        gemm_splitk_combine_kernel<DT_BF16, false, true><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
+        return;
+    }
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles);
+    gemm4_mfma_direct_kernel<BLOCK, 4, false, 4, false, true><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, nullptr);
 }
 
 // up to three linears on the same activations in one launch: 64- or 128-token x 256-feature tiles, whichever gives the CUs

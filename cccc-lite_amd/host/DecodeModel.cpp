@@ -474,7 +474,7 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         }
         if (rc == 0) { rc = linear(*L.wo, c.hidden, q_out, *pf_.att, *pf_.o); }
         if (rc == 0) { rc = add_norm(*pf_.x, *pf_.o, *pf_.r1, *L.rms_ffn, *pf_.xn); }
-        // gate, up and their SwiGLU product: one launch for two FP8 weights of one type, else the three calls
+        // gate, up and their SwiGLU product: one launch for two weights of one type, else the three calls
         int fused = -1;
         if (rc == 0 && L.w_gate->getDataType() == L.w_up->getDataType())
         {

@@ -288,8 +288,9 @@ C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const voi
  * bf16(bf16(g * bf16(sigmoid g)) * u) (cccc/MatrixEx.cpp:756-762, hip_functions.cpp:722-732, :953-966) in one launch, with
  * the bits of the three calls it replaces -- or, with too few output tiles for the GPU (K >= 1024), the k range split over
  * workgroups and a second launch that adds the FP32 partial sums (workspace grown on demand) and writes the product with
- * the same roundings.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).
- * -1 (nothing launched, use the separate calls): other weight types, fewer than 17 tokens, K not a multiple of 64. */
+ * the same roundings.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).  FP4 block-scale
+ * weights (type 6) take part when both have a registered tiled copy of one block length, K is a multiple of 128 and
+ * ldw == K.  -1 (nothing launched, use the separate calls): other weight types, fewer than 17 tokens, K not a multiple of 64. */
 C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                                    float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);
 C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);

@@ -150,15 +150,19 @@ def test_linears_that_share_their_input_in_one_launch_equal_the_separate_calls(g
 @pytest.mark.parametrize("tokens,widths,K", [(60, (512, 256, 256), 256), (130, (1000, 72), 1024), (300, (2048, 512, 512), 512)])
 def test_fp4_linears_that_share_their_input_in_one_launch(gpu, oracle, block, tokens, widths, K):
     """hip_quant_gemm_segments on FP4 block-scale weights (tiled copies registered, which is what the FP4 GEMM reads) against
-    one hip_quant_gemm call per weight, byte for byte; without the tiled copies the call is refused."""
+    one hip_quant_gemm call per weight -- byte for byte where K is too short for a k split (under 1024), within the order of
+    the FP32 sums at K = 1024, where the joint launch splits its few tiles in two k ranges -- and against the exact
+    contraction; without the tiled copies the call is refused."""
     torch, dev, lib = gpu
     rng = np.random.default_rng(tokens + K + block)
     X = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
     xd = to_dev(torch, dev, X)
-    wds, sds, keep, sep, one = [], [], [], [], []
+    wds, sds, keep, sep, one, host_w, host_s = [], [], [], [], [], [], []
     for n_out in widths:
-        wds.append(to_dev(torch, dev, rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8)))
-        sds.append(to_dev(torch, dev, rng.integers(0x20, 0x40, size=(n_out, K // block), dtype=np.uint8)))
+        host_w.append(rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8))
+        host_s.append(rng.integers(0x20, 0x40, size=(n_out, K // block), dtype=np.uint8))
+        wds.append(to_dev(torch, dev, host_w[-1]))
+        sds.append(to_dev(torch, dev, host_s[-1]))
         sep.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
         one.append(torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev))
     n = len(widths)
@@ -178,10 +182,16 @@ def test_fp4_linears_that_share_their_input_in_one_launch(gpu, oracle, block, to
             assert lib.last_kernel() == "gemm_mfma_tiled"
         assert call() == 0
         assert lib.last_kernel() == "gemm_segments_tiled"
-        for y1, y3, n_out in zip(one, sep, widths):
+        for y1, y3, n_out, W, sc in zip(one, sep, widths, host_w, host_s):
             got = from_dev(y1, np.uint16)
             assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
-            assert np.array_equal(got, from_dev(y3, np.uint16))
+            if K < 1024:
+                assert np.array_equal(got, from_dev(y3, np.uint16))
+            have = oracle.bf16_to_f32(got[:tokens * n_out].reshape(tokens, n_out)).astype(np.float64)
+            other = oracle.bf16_to_f32(from_dev(y3, np.uint16)[:tokens * n_out].reshape(tokens, n_out)).astype(np.float64)
+            want = oracle.linear_exact(oracle.dequant_weight(W.reshape(-1), oracle.FP4, n_out, K, blk_sc=sc.reshape(-1), block=block), X)
+            check_rows(have, want, f"FP4 segment of {n_out} features")
+            assert (np.linalg.norm(have - other, axis=1) <= 2e-3 * np.linalg.norm(want, axis=1)).all()
     finally:
         for wd in wds:
             assert lib.weight_release(wd.data_ptr()) == 0
@@ -239,6 +249,50 @@ def test_gate_up_pair_gemm_with_swiglu_equals_the_three_calls(gpu, oracle, dec, 
     finally:
         if tiled:
             assert lib.weight_release(gd.data_ptr()) == 0 and lib.weight_release(ud.data_ptr()) == 0
+
+
+@pytest.mark.parametrize("block", [16, 32])
+@pytest.mark.parametrize("tokens,n_out,K", [(60, 512, 256), (130, 200, 1024), (300, 1536, 512)])
+def test_fp4_gate_up_pair_gemm_with_swiglu(gpu, oracle, dec, block, tokens, n_out, K):
+    """hip_quant_gemm_swiglu on FP4 block-scale weights (tiled copies registered) against two hip_quant_gemm calls and
+    hip_swiglu_bf16 -- byte for byte where K is too short for a k split (under 1024) -- and against the oracle's exact
+    contraction; without the tiled copies the call is refused."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + n_out + K + block)
+    X = oracle.f32_to_bf16(rng.standard_normal((tokens, K)).astype(np.float32))
+    xd = to_dev(torch, dev, X)
+    Wg, Wu = (rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8) for _ in range(2))
+    Sg, Su = (rng.integers(0x20, 0x40, size=(n_out, K // block), dtype=np.uint8) for _ in range(2))
+    gd, ud, sgd, sud = (to_dev(torch, dev, v) for v in (Wg, Wu, Sg, Su))
+    g, u, y3, y1 = (torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev) for _ in range(4))
+    call = lambda: lib.c.hip_quant_gemm_swiglu(n_out, tokens, K, ptr(gd), ptr(ud), oracle.FP4, K, ctypes.c_float(1.0), ctypes.c_float(1.0),
+                                               ptr(xd), K, ptr(y1), n_out)
+    assert call() == -1                                         # no tiled copies yet
+    keep = []
+    for wd, sd in ((gd, sgd), (ud, sud)):
+        t = torch.zeros(lib.tiled_size(oracle.FP4, n_out, K), dtype=torch.uint8, device=dev)
+        assert lib.weight_prepare_fp4(wd.data_ptr(), sd.data_ptr(), block, n_out, K, t.data_ptr()) == 0
+        keep.append(t)
+    try:
+        assert lib.linear(gd.data_ptr(), oracle.FP4, xd.data_ptr(), g.data_ptr(), n_out, tokens, K, 1.0, sgd.data_ptr(), block) == 0
+        assert lib.linear(ud.data_ptr(), oracle.FP4, xd.data_ptr(), u.data_ptr(), n_out, tokens, K, 1.0, sud.data_ptr(), block) == 0
+        assert lib.c.hip_swiglu_bf16(ptr(g), ptr(u), ptr(y3), tokens * n_out) == 0
+        assert call() == 0
+        assert lib.last_kernel() == "gemm_swiglu_tiled"
+        got = from_dev(y1, np.uint16)
+        assert got[:tokens * n_out].any() and not got[tokens * n_out:].any()
+        if K < 1024:
+            assert np.array_equal(got, from_dev(y3, np.uint16))
+        else:
+            assert np.mean(got != from_dev(y3, np.uint16)) < 0.02
+        deq = lambda W, S: oracle.dequant_weight(W.reshape(-1), oracle.FP4, n_out, K, blk_sc=S.reshape(-1), block=block)
+        gate = oracle.f32_to_bf16(oracle.linear_exact(deq(Wg, Sg), X).astype(np.float32))
+        up = oracle.f32_to_bf16(oracle.linear_exact(deq(Wu, Su), X).astype(np.float32))
+        want = dec.silu_mul(dec.f(gate), dec.f(up))
+        have = dec.f(got[:tokens * n_out].reshape(tokens, n_out))
+        assert np.linalg.norm(have - want) <= 1e-2 * np.linalg.norm(want)
+    finally:
+        assert lib.weight_release(gd.data_ptr()) == 0 and lib.weight_release(ud.data_ptr()) == 0
 
 
 @pytest.mark.parametrize("rows,inner", [(1, 256), (7, 4096), (130, 1024), (5, 136)])
