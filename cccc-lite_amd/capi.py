@@ -71,6 +71,7 @@ EXPORTS = (
     "hip_swiglu_bf16",
     "hip_add_rms_norm_bf16",
     "hip_quant_gemm_swiglu",
+    "hip_quant_gemm_add_rms_norm",
     "hip_quant_gemm_segments",
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
@@ -150,6 +151,8 @@ class QuantLibrary:
         L.hip_swiglu_bf16.argtypes = [vp, vp, vp, ctypes.c_ulonglong]
         L.hip_quant_gemm_segments.restype = i32
         L.hip_quant_gemm_segments.argtypes = [i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, i32]
+        L.hip_quant_gemm_add_rms_norm.restype = i32
+        L.hip_quant_gemm_add_rms_norm.argtypes = [i32, i32, i32, vp, i32, i32, ctypes.c_float, vp, i32, vp, vp, vp, vp, ctypes.c_float]
         L.hip_quant_gemm_swiglu.restype = i32
         L.hip_quant_gemm_swiglu.argtypes = [i32, i32, i32, vp, vp, i32, i32, ctypes.c_float, ctypes.c_float, vp, i32, vp, i32]
         L.hip_add_rms_norm_bf16.restype = i32

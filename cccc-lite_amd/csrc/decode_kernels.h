@@ -127,31 +127,6 @@ __device__ __forceinline__ void stage_issue(const FusedLinearArgs& a, StagedActi
     }
 }
 
-__device__ __forceinline__ float sumsq8(const u32x4& v)
-{
-    float s = 0.0f;
-#pragma unroll
-    for (int d = 0; d < 4; d++)
-    {
-        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu), hi = bf16_bits_to_f32(v[d] >> 16);
-        s += lo * lo + hi * hi;
-    }
-    return s;
-}
-
-__device__ __forceinline__ u32x4 normed8(const u32x4& v, const u32x4& w, float invstd)
-{
-    u32x4 out;
-#pragma unroll
-    for (int d = 0; d < 4; d++)
-    {
-        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu) * invstd * bf16_bits_to_f32(w[d] & 0xFFFFu);
-        const float hi = bf16_bits_to_f32(v[d] >> 16) * invstd * bf16_bits_to_f32(w[d] >> 16);
-        out[d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
-    }
-    return out;
-}
-
 // `red` holds THREADS / 64 floats.  Ends with a barrier: xs is complete for every thread.
 template <int THREADS, int PARTS = 2>
 __device__ __forceinline__ void stage_finish(const FusedLinearArgs& a, const StagedActivation& r, u32x4* xs, float* red)

@@ -641,6 +641,46 @@ int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, cons
     return finish("quant_gemm_swiglu");
 }
 
+int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const void* W, int w_type, int ldw, float inv_scale, const void* X, int ldx,
+                                const void* res, void* sum, const void* norm_w, void* y, float epsilon)
+{
+    const bool fp4 = w_type == DT_FP4;
+    if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
+    if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
+    if (n_out <= 0 || n_out % 8 != 0 || n_out > 4096 || tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K) { return -1; }
+    if (!W || !X || !res || !sum || !norm_w || !y || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
+    if (!aligned16(W) || !aligned16(X) || !aligned16(res) || !aligned16(sum) || !aligned16(norm_w) || !aligned16(y)) { return -1; }
+    LinearArgs a{};
+    a.W = (const uint8_t*)W;
+    a.X = (const uint16_t*)X;
+    a.ldw = ldw;
+    a.ldx = ldx;
+    a.y_stride_tok = n_out;
+    a.y_stride_out = 1;
+    a.n_out = n_out;
+    a.tokens = tokens;
+    a.K = K;
+    a.w_scale = inv_scale;
+    a.alpha = 1.0f;
+    a.beta = 0.0f;
+    const AddNormArgs e = { (const uint16_t*)res, (uint16_t*)sum, (const uint16_t*)norm_w, (uint16_t*)y, epsilon };
+    const uint8_t* tiled = ccq::lookup_tiled(W, w_type, n_out, K, ldw);
+    bool launched = false;
+    if (fp4)
+    {
+        if (!tiled) { return -1; }
+        const unsigned block = tiled_block_of(W);
+        a.block_size = block;
+        if (block == 16) { launched = gemm_mfma<DT_FP4, 16>(a, tiled, nullptr, &e); }
+        else if (block == 32) { launched = gemm_mfma<DT_FP4, 32>(a, tiled, nullptr, &e); }
+    }
+    else if (w_type == DT_E5M2) { launched = gemm_mfma<DT_E5M2, 0>(a, tiled, nullptr, &e); }
+    else { launched = gemm_mfma<DT_E4M3, 0>(a, tiled, nullptr, &e); }
+    if (!launched) { return -1; }                   // this shape does not split its k range: nothing to fold the add and the norm into
+    note_kernel(tiled ? "gemm_add_rms_norm_tiled" : "gemm_add_rms_norm");
+    return finish("quant_gemm_add_rms_norm");
+}
+
 int hip_quant_gemm_noalloc(int transA, int transB, int M, int N, int K, float alpha,
                            const void* A, int typeA, int lda, float invScaleA,
                            const void* B, int typeB, int ldb, float invScaleB,

@@ -950,9 +950,85 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
     }
 }
 
+// The combine launch of a k-split GEMM that also does what follows the linear in a transformer block: o = bf16(sum of the
+// partial tiles), r = bf16(res + o), y = rmsnorm(r) * w -- gemm_splitk_combine_kernel, the residual add and the row norm
+// in one launch, with their roundings and their order of sums (the sum of squares runs as in rms_norm_rows_kernel: lane l of
+// one wave adds the 8-value chunks l, l + 64, ... in turn, then the wave reduction), so the bits are those of the three
+// launches.  One 512-thread workgroup per token row, a thread per chunk of 8 features (n_out <= 4096, a multiple of 8);
+// the loads of up to MAXS partial tiles are all issued before the first add.
+template <int MAXS>
+__global__ __launch_bounds__(512) void gemm_splitk_combine_add_norm_kernel(const float* __restrict__ partial, const int splits, const LinearArgs a, const AddNormArgs e)
+{
+    __shared__ float sq[512];
+    __shared__ float s_invstd;
+    const int row = blockIdx.x, c = threadIdx.x;
+    const int n_chunks = a.n_out / 8;
+    const bool active = c < n_chunks;
+    const long long slice = (long long)a.tokens * a.n_out;
+    const size_t at = (size_t)row * a.n_out + (size_t)min(c, n_chunks - 1) * 8;
+    f32x4 lo[MAXS], hi[MAXS];
+#pragma unroll
+    for (int s = 0; s < MAXS; s++)
+    {
+        const float* p = partial + (long long)min(s, splits - 1) * slice + at;       // ranges past the last re-read it and are dropped
+        lo[s] = *(const f32x4*)p;
+        hi[s] = *(const f32x4*)(p + 4);
+    }
+    const u32x4 res = *(const u32x4*)(e.res + at), w = *(const u32x4*)(e.norm_w + (size_t)min(c, n_chunks - 1) * 8);
+    f32x4 r0 = lo[0], r1 = hi[0];
+#pragma unroll
+    for (int s = 1; s < MAXS; s++)
+    {
+        if (s < splits)
+        {
+            r0 += lo[s];
+            r1 += hi[s];
+        }
+    }
+    u32x4 v;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        const float o_lo = d < 2 ? r0[2 * d] : r1[2 * d - 4], o_hi = d < 2 ? r0[2 * d + 1] : r1[2 * d - 3];
+        const float x_lo = bf16_bits_to_f32(res[d] & 0xFFFFu) + bf16_bits_to_f32(finish_output_act<DT_BF16>(o_lo, a.alpha, 0.0f, nullptr));
+        const float x_hi = bf16_bits_to_f32(res[d] >> 16) + bf16_bits_to_f32(finish_output_act<DT_BF16>(o_hi, a.alpha, 0.0f, nullptr));
+        v[d] = f32_to_bf16_bits(x_lo) | (f32_to_bf16_bits(x_hi) << 16);
+    }
+    if (active) { *(u32x4*)(e.sum + at) = v; }
+    sq[c] = active ? sumsq8(v) : 0.0f;
+    __syncthreads();
+    if (c < 64)
+    {
+        float sumsq = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) { sumsq += sq[c + 64 * j]; }
+        const float invstd = rsqrtf(wave_sum(sumsq) / (float)a.n_out + e.eps);
+        if (c == 0) { s_invstd = invstd; }
+    }
+    __syncthreads();
+    if (active) { *(u32x4*)(e.y + at) = normed8(v, w, s_invstd); }
+}
+
+// the combine launch of a k-split GEMM: plain, or with the residual add and the norm behind the linear
+template <int AT>
+inline void launch_splitk_combine(const float* partial, int splits, const LinearArgs& a, const AddNormArgs* e)
+{
+    if (e)
+    {
+        if (splits <= 4) { gemm_splitk_combine_add_norm_kernel<4><<<a.tokens, 512, 0, stream()>>>(partial, splits, a, *e); }
+        else if (splits <= 8) { gemm_splitk_combine_add_norm_kernel<8><<<a.tokens, 512, 0, stream()>>>(partial, splits, a, *e); }
+        else { gemm_splitk_combine_add_norm_kernel<16><<<a.tokens, 512, 0, stream()>>>(partial, splits, a, *e); }
+        return;
+    }
+    const long long groups = (long long)a.tokens * (a.n_out / 4);
+    const long long blocks = (groups + 255) / 256;
+    const long long cap = (long long)cu_count() * 16;
+    gemm_splitk_combine_kernel<AT><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
+}
+
 // a.W = the tiled codes; splits > 1: `partial` holds splits * tokens * n_out floats
 template <int BLOCK, int MB, int NB = 4>
-void launch_gemm4_mfma_direct(const LinearArgs& a, const uint8_t* tiled_scales, int splits = 1, float* partial = nullptr)
+void launch_gemm4_mfma_direct(const LinearArgs& a, const uint8_t* tiled_scales, int splits = 1, float* partial = nullptr, const AddNormArgs* e = nullptr)
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
@@ -960,17 +1036,14 @@ void launch_gemm4_mfma_direct(const LinearArgs& a, const uint8_t* tiled_scales, 
     if (splits > 1)
     {
         gemm4_mfma_direct_kernel<BLOCK, MB, true, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, partial);
-        const long long groups = (long long)a.tokens * (a.n_out / 4);
-        const long long blocks = (groups + 255) / 256;
-        const long long cap = (long long)cu_count() * 16;
-        gemm_splitk_combine_kernel<DT_BF16><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
+        launch_splitk_combine<DT_BF16>(partial, splits, a, e);
     }
     else { gemm4_mfma_direct_kernel<BLOCK, MB, false, NB><<<grid, 256, 0, stream()>>>(a, tiled_scales, n_tiles, nullptr); }
 }
 
 // splits > 1: `partial` holds splits * tokens * n_out floats
 template <int WT, int MB, bool TILED, int AT = DT_BF16, int NB = 4>
-void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial = nullptr)
+void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial = nullptr, const AddNormArgs* e = nullptr)
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
@@ -980,10 +1053,7 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
     {
         if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
         else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
-        const long long groups = (long long)a.tokens * (a.n_out / 4);
-        const long long blocks = (groups + 255) / 256;
-        const long long cap = (long long)cu_count() * 16;
-        gemm_splitk_combine_kernel<AT><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, splits, a);
+        launch_splitk_combine<AT>(partial, splits, a, e);
     }
     else
     {
@@ -1302,8 +1372,10 @@ inline DirectPlan plan_direct_fp4(const LinearArgs& a, SplitScratch* scratch)
 // otherwise 128 x 64 tiles to put more workgroups on the machine.
 // `scratch`: see SplitScratch; nullptr = the stream's grow-on-demand workspace.  Returns false (nothing launched)
 // only when a fixed scratch buffer is too small for the k-split this shape takes.
+// `e`: the caller wants the residual add and the norm behind the linear in the combine launch of a k split; false
+// (nothing launched) when this shape does not split.
 template <int WT, int BLOCK, int AT = DT_BF16>
-bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch* scratch = nullptr)
+bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch* scratch = nullptr, const AddNormArgs* e = nullptr)
 {
     if constexpr (WT == DT_FP4 && AT == DT_BF16)
     {
@@ -1314,13 +1386,14 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
             d.W = tiled;
             const uint8_t* scales = tiled + (long long)((a.n_out + 15) / 16) * (a.K / 128) * 1024;
             const DirectPlan plan = plan_direct_fp4(a, scratch);
-            if (plan.refused) { return false; }
+            if (plan.refused || (e && plan.splits <= 1)) { return false; }
             if (plan.nb == 3) { plan.mb == 8 ? launch_gemm4_mfma_direct<BLOCK, 8, 3>(d, scales) : launch_gemm4_mfma_direct<BLOCK, 4, 3>(d, scales); }
-            else if (plan.mb == 8) { launch_gemm4_mfma_direct<BLOCK, 8>(d, scales, plan.splits, plan.partial); }
-            else { launch_gemm4_mfma_direct<BLOCK, 4>(d, scales, plan.splits, plan.partial); }
+            else if (plan.mb == 8) { launch_gemm4_mfma_direct<BLOCK, 8>(d, scales, plan.splits, plan.partial, e); }
+            else { launch_gemm4_mfma_direct<BLOCK, 4>(d, scales, plan.splits, plan.partial, e); }
             return true;
         }
     }
+    if constexpr (AT != DT_BF16) { if (e) { return false; } }
     if constexpr (WT != DT_FP4)
     {
         const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
@@ -1330,25 +1403,26 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }
             const DirectPlan plan = plan_direct(a, scratch, false, tiled == nullptr);
-            if (plan.refused) { return false; }
+            if (plan.refused || (e && plan.splits <= 1)) { return false; }
             const int nb = plan.nb, mb = plan.mb, splits = plan.splits;
             float* const partial = plan.partial;
             if (nb == 2) { tiled ? launch_gemm_mfma_direct<WT, 4, true, AT, 2>(d) : launch_gemm_mfma_direct<WT, 4, false, AT, 2>(d); }
             else if (tiled)
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, true, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, true, AT, 3>(d); }
-                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial); }
-                else { launch_gemm_mfma_direct<WT, 4, true, AT>(d, splits, partial); }
+                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial, e); }
+                else { launch_gemm_mfma_direct<WT, 4, true, AT>(d, splits, partial, e); }
             }
             else
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, false, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, false, AT, 3>(d); }
-                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial); }
-                else { launch_gemm_mfma_direct<WT, 4, false, AT>(d, splits, partial); }
+                else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial, e); }
+                else { launch_gemm_mfma_direct<WT, 4, false, AT>(d, splits, partial, e); }
             }
             return true;
         }
     }
+    if (e) { return false; }
     const long long tiles_big = (long long)((a.n_out + 127) / 128) * ((a.tokens + 127) / 128);
     if (tiles_big >= 2LL * cu_count())
     {

@@ -39,4 +39,15 @@ struct LinearArgs
     long long seg_y_stride_tok[3];
 };
 
+// What follows a k-split GEMM when its combine launch also carries the residual add and the RMSNorm behind it
+// (gemm_splitk_combine_add_norm_kernel): rows of n_out values, all dense.
+struct AddNormArgs
+{
+    const uint16_t* res;      // residual rows [tokens][n_out]
+    uint16_t* sum;            // bf16(res + bf16(W x))
+    const uint16_t* norm_w;   // [n_out]
+    uint16_t* y;              // rmsnorm(sum) * norm_w
+    float eps;
+};
+
 }    // namespace ccq

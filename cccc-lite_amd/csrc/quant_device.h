@@ -147,4 +147,32 @@ __device__ __forceinline__ float wave_sum(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
+// Sum of squares of eight BF16 values (one 16-byte chunk of a row), and the chunk scaled by 1 / rms and the norm weight:
+// the arithmetic of every row norm in the library, kept in one place so that the fused variants give the same bits.
+__device__ __forceinline__ float sumsq8(const u32x4& v)
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu), hi = bf16_bits_to_f32(v[d] >> 16);
+        s += lo * lo + hi * hi;
+    }
+    return s;
+}
+
+__device__ __forceinline__ u32x4 normed8(const u32x4& v, const u32x4& w, float invstd)
+{
+    u32x4 out;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+    {
+        const float lo = bf16_bits_to_f32(v[d] & 0xFFFFu) * invstd * bf16_bits_to_f32(w[d] & 0xFFFFu);
+        const float hi = bf16_bits_to_f32(v[d] >> 16) * invstd * bf16_bits_to_f32(w[d] >> 16);
+        out[d] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    }
+    return out;
+}
+
+
 }    // namespace ccq

@@ -440,6 +440,15 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         const int r = hip_add_bf16(a.data(), b.data(), sum.data(), (unsigned long long)n * c.hidden);
         return r != 0 ? r : norm(sum, y, w);
     };
+    // sum = res + W x and y = norm(sum): where the GEMM splits its k range the launch that adds the partial sums does the add
+    // and the norm as well (-1: this shape does not split, or the library has no such kernel for it)
+    auto linear_add_norm = [&](const Matrix& W, int n_out, int K, const Matrix& x, Matrix& res, Matrix& sum, Matrix& w, Matrix& y) {
+        int r = hip_quant_gemm_add_rms_norm(n_out, n, K, W.data(), (int)W.getDataType(), K, W.getQuantScale(), x.data(), K,
+                                            res.data(), sum.data(), w.data(), y.data(), c.eps);
+        if (r >= 0) { return r; }
+        r = linear(W, n_out, K, x, *pf_.o);
+        return r != 0 ? r : add_norm(res, *pf_.o, sum, w, y);
+    };
     if (rc == 0 && c.layers > 0) { rc = norm(*pf_.x, *pf_.xn, *layers_[0].rms_attn); }
     for (int li = 0; li < c.layers && rc == 0; li++)
     {
@@ -472,8 +481,8 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
             rc = hip_attention_prefill_bf16(pf_.q_rot->data(), k_cache_[li]->data(), v_cache_[li]->data(), pf_.att->data(),
                                             c.n_q, c.n_kv, c.head_dim, c.t_kv, n, pos0);
         }
-        if (rc == 0) { rc = linear(*L.wo, c.hidden, q_out, *pf_.att, *pf_.o); }
-        if (rc == 0) { rc = add_norm(*pf_.x, *pf_.o, *pf_.r1, *L.rms_ffn, *pf_.xn); }
+        // o, the residual add and the norm behind it: one call where the GEMM splits its k range (short prompts), else two
+        if (rc == 0) { rc = linear_add_norm(*L.wo, c.hidden, q_out, *pf_.att, *pf_.x, *pf_.r1, *L.rms_ffn, *pf_.xn); }
         // gate, up and their SwiGLU product: one launch for two weights of one type, else the three calls
         int fused = -1;
         if (rc == 0 && L.w_gate->getDataType() == L.w_up->getDataType())
@@ -488,10 +497,13 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
             if (rc == 0) { rc = linear(*L.w_up, c.inter, c.hidden, *pf_.xn, *pf_.up); }
             if (rc == 0) { rc = hip_swiglu_bf16(pf_.gate->data(), pf_.up->data(), pf_.gated->data(), (unsigned long long)n * c.inter); }
         }
-        if (rc == 0) { rc = linear(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.o); }
         // x = r1 + ffn, and the next layer's first norm with it (the head normalises the last token's row itself)
-        if (rc == 0 && li + 1 < c.layers) { rc = add_norm(*pf_.r1, *pf_.o, *pf_.x, *layers_[li + 1].rms_attn, *pf_.xn); }
-        else if (rc == 0) { rc = hip_add_bf16(pf_.r1->data(), pf_.o->data(), pf_.x->data(), (unsigned long long)n * c.hidden); }
+        if (rc == 0 && li + 1 < c.layers) { rc = linear_add_norm(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.r1, *pf_.x, *layers_[li + 1].rms_attn, *pf_.xn); }
+        else if (rc == 0)
+        {
+            rc = linear(*L.w_down, c.hidden, c.inter, *pf_.gated, *pf_.o);
+            if (rc == 0) { rc = hip_add_bf16(pf_.r1->data(), pf_.o->data(), pf_.x->data(), (unsigned long long)n * c.hidden); }
+        }
     }
     if (rc != 0 || !last) { return rc; }
     // the head runs on the last token's state: its greedy pick becomes the current token at position pos0 + n

@@ -282,6 +282,16 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
  * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
 C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
                                      void* const* Y, const int* ldy, int w_type, int tokens, int K, int ldw, const void* X, int ldx);
+/* A linear, the residual add behind it and the RMSNorm behind that, for the shapes whose GEMM splits its k range over
+ * workgroups (few output tiles: the o and down projections of a prompt of up to ~512 tokens): sum[t] = bf16(res[t] +
+ * bf16(W x_t)), y[t] = rmsnorm(sum[t]) * norm_w -- the launch that adds the FP32 partial sums does the add and the norm as
+ * well, with the bits of hip_quant_gemm + hip_add_bf16 + hip_rms_norm_fwd (hip_functions.cpp:895-908, :1121-1160).  FP8
+ * weights [n_out][K] (row pitch ldw; tiled copy used when registered) or FP4 block-scale weights with a registered tiled copy
+ * (K % 128 == 0, ldw == K); BF16 activations [tokens][K]; res, sum, y dense [tokens][n_out], n_out <= 4096 and a multiple
+ * of 8, everything 16-byte aligned.  -1 (nothing launched, use the separate calls): a shape that does not split, fewer than
+ * 17 tokens, anything else unsupported.  No counterpart in the reference. */
+C_EXPORT int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const void* W, int w_type, int ldw, float inv_scale,
+                                         const void* X, int ldx, const void* res, void* sum, const void* norm_w, void* y, float epsilon);
 /* y[t][o] = swiglu(gate[t][o], up[t][o]) with gate = bf16(W_gate x_t), up = bf16(W_up x_t): the gate and up linears of an
  * MLP block (two FP8 weights of one shape [n_out][K], row pitch ldw, dequantisation multipliers as in hip_quant_gemm; both
  * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product

@@ -295,6 +295,69 @@ def test_fp4_gate_up_pair_gemm_with_swiglu(gpu, oracle, dec, block, tokens, n_ou
         assert lib.weight_release(gd.data_ptr()) == 0 and lib.weight_release(ud.data_ptr()) == 0
 
 
+@pytest.mark.parametrize("w_type,tiled", [("e5m2", False), ("e4m3", True), ("fp4", True)])
+@pytest.mark.parametrize("tokens,n_out,K", [(20, 256, 1024), (60, 4096, 2048), (130, 1000, 4096), (300, 512, 8192)])
+def test_linear_residual_add_and_norm_in_the_combine_launch(gpu, oracle, w_type, tiled, tokens, n_out, K):
+    """hip_quant_gemm_add_rms_norm on shapes whose GEMM splits its k range against hip_quant_gemm, hip_add_bf16 and
+    hip_rms_norm_fwd on the same inputs: both outputs byte for byte, nothing written past them; a shape that does not
+    split and unsupported arguments return -1 and write nothing."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(tokens + n_out + K)
+    X = oracle.f32_to_bf16((rng.standard_normal((tokens, K)) * (0.05 if w_type == "e5m2" else 1.0)).astype(np.float32))
+    R = oracle.f32_to_bf16(rng.standard_normal((tokens, n_out)).astype(np.float32))
+    Wn = oracle.f32_to_bf16((1.0 + 0.1 * rng.standard_normal(n_out)).astype(np.float32))
+    xd, rd, nd = to_dev(torch, dev, X), to_dev(torch, dev, R), to_dev(torch, dev, Wn)
+    sd, block, sc = None, 16, 1.0
+    if w_type == "fp4":
+        wt = oracle.FP4
+        wd = to_dev(torch, dev, rng.integers(0, 256, size=(n_out, K // 2), dtype=np.uint8))
+        sd = to_dev(torch, dev, rng.integers(0x20, 0x40, size=(n_out, K // block), dtype=np.uint8))
+    else:
+        wt = oracle.E5M2 if w_type == "e5m2" else oracle.E4M3
+        sc = 1.0 if w_type == "e5m2" else 0.013
+        W = rng.integers(0, 256, size=(n_out, K), dtype=np.uint8)
+        if w_type == "e5m2": W[(W & 0x7C) == 0x7C] = 0x3C
+        else: W[(W & 0x7F) == 0x7F] = 0x38
+        wd = to_dev(torch, dev, W)
+    keep = None
+    if tiled:
+        keep = torch.zeros(lib.tiled_size(wt, n_out, K), dtype=torch.uint8, device=dev)
+        if w_type == "fp4": assert lib.weight_prepare_fp4(wd.data_ptr(), sd.data_ptr(), block, n_out, K, keep.data_ptr()) == 0
+        else: assert lib.weight_prepare(wd.data_ptr(), wt, n_out, K, K, keep.data_ptr()) == 0
+    try:
+        o, s3, y3, s1, y1 = (torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev) for _ in range(5))
+        if w_type == "fp4": assert lib.linear(wd.data_ptr(), wt, xd.data_ptr(), o.data_ptr(), n_out, tokens, K, 1.0, sd.data_ptr(), block) == 0
+        else: assert lib.linear(wd.data_ptr(), wt, xd.data_ptr(), o.data_ptr(), n_out, tokens, K, sc) == 0
+        assert lib.c.hip_add_bf16(ptr(rd), ptr(o), ptr(s3), tokens * n_out) == 0
+        assert lib.c.hip_rms_norm_fwd(oracle.BF16, ptr(s3), ptr(y3), ptr(nd), None, tokens, n_out, ctypes.c_float(1e-6)) == 0
+        call = lambda toks, n, k: lib.c.hip_quant_gemm_add_rms_norm(n, toks, k, ptr(wd), wt, K, ctypes.c_float(sc), ptr(xd), K,
+                                                                    ptr(rd), ptr(s1), ptr(nd), ptr(y1), ctypes.c_float(1e-6))
+        assert call(tokens, n_out, K) == 0
+        assert lib.last_kernel() == ("gemm_add_rms_norm_tiled" if tiled else "gemm_add_rms_norm")
+        got_s, got_y = from_dev(s1, np.uint16), from_dev(y1, np.uint16)
+        assert got_y[:tokens * n_out].any() and not got_y[tokens * n_out:].any() and not got_s[tokens * n_out:].any()
+        assert np.array_equal(got_s, from_dev(s3, np.uint16))
+        assert np.array_equal(got_y, from_dev(y3, np.uint16))
+        s1.zero_(); y1.zero_()
+        assert call(16, n_out, K) == -1 and call(tokens, n_out - 4, K) == -1 and call(tokens, n_out, K - 32) == -1
+        assert not from_dev(s1, np.uint16).any() and not from_dev(y1, np.uint16).any()
+    finally:
+        if tiled:
+            assert lib.weight_release(wd.data_ptr()) == 0
+
+
+def test_linear_add_norm_refuses_a_shape_that_does_not_split(gpu, oracle):
+    """2048 tokens x 4096 features fill the GPU without a k split: hip_quant_gemm_add_rms_norm returns -1 and launches nothing."""
+    torch, dev, lib = gpu
+    tokens, n_out, K = 2048, 4096, 256
+    w = torch.zeros(n_out * K, dtype=torch.uint8, device=dev)
+    x = torch.zeros(tokens * K, dtype=torch.int16, device=dev)
+    r, s, y = (torch.zeros(tokens * n_out, dtype=torch.int16, device=dev) for _ in range(3))
+    nw = torch.zeros(n_out, dtype=torch.int16, device=dev)
+    assert lib.c.hip_quant_gemm_add_rms_norm(n_out, tokens, K, ptr(w), oracle.E5M2, K, ctypes.c_float(1.0), ptr(x), K,
+                                             ptr(r), ptr(s), ptr(nw), ptr(y), ctypes.c_float(1e-6)) == -1
+
+
 @pytest.mark.parametrize("rows,inner", [(1, 256), (7, 4096), (130, 1024), (5, 136)])
 def test_add_and_rms_norm_in_one_pass_equals_the_two_calls(gpu, oracle, dec, rows, inner):
     """hip_add_rms_norm_bf16 against hip_add_bf16 followed by hip_rms_norm_fwd on the same inputs: both outputs byte for
