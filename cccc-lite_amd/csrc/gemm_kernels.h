@@ -281,7 +281,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // SEG: the launch covers up to three linears on the same activations (the q, k and v projections: the narrow ones alone
 // leave most CUs idle); a workgroup finds its segment from its feature tile and takes that segment's weight, output,
 // width and scale -- from there on it is the single-linear kernel.
-template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false>
+// PD: how many k-tiles ahead the weights are requested (the activations PD + 1 when PD > 1).  One is enough where two
+// workgroups share a CU and each k-tile carries 64 matrix-core instructions per wave; the k-split launches of a short
+// prompt (one 64-token tile, about one workgroup per CU) are bound by their weight bytes and run a k-tile per memory
+// latency with PD = 1 -- they take PD = 3.
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false, int PD = 1>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a_in, const int n_tiles, float* __restrict__ partial)
 {
     static_assert(!PAIR || (NB % 2 == 0 && AT == DT_BF16), "pair: an even number of feature blocks, BF16");
@@ -371,10 +375,12 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         x_store[i] = (q / CPR) * CPR + swizzled_chunk_n<CPR>(q / CPR, q % CPR);
     }
 
-    u32x4 wraw_a[NB], wraw_b[NB], xreg[X_PER_THREAD];
+    constexpr int RW = PD + 1;                  // weight register buffers: tile kt lives in wraw[kt % RW]
+    constexpr int RX = PD == 1 ? 1 : PD + 1;    // activation register buffers: tile kt travels in xring[kt % RX]
+    u32x4 wraw[RW][NB], xring[RX][X_PER_THREAD];
     // K is a multiple of 64 here and the k-tile index of a prefetch is clamped to the last one, so no load
     // or store in the loop needs a predicate or a branch: the wait counts stay exact
-    auto fetch_x = [&](int kt) {
+    auto fetch_x = [&](int kt, u32x4* xreg) {
         const int k0 = min(kt, n_kt - 1) * BK;
 #pragma unroll
         for (int i = 0; i < X_PER_THREAD; i++) { xreg[i] = *(const u32x4*)(x_begin + (size_t)k0 * 2 + (size_t)x_off[i]); }
@@ -384,21 +390,23 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) { wraw[nb] = *(const u32x4*)(w_begin + w_tile_base[nb] + k0 + (size_t)w_off[nb]); }
     };
-    auto stage = [&](int buf) {
+    auto stage = [&](int buf, const u32x4* xreg) {
 #pragma unroll
         for (int i = 0; i < X_PER_THREAD; i++) { xs[buf][x_store[i]] = xreg[i]; }
     };
 
-    // Order of one k-tile: barrier | request the next weights | first half of the matrix-core work |
-    // store the next activation tile to LDS and request the one after it | second half.  The LDS stores
+    // Order of one k-tile: barrier | request the weights of tile kt + PD | first half of the matrix-core work |
+    // store the next activation tile to LDS and request a later one into its registers | second half.  The LDS stores
     // and the global loads are thus a whole k-tile of work away from the instructions that wait for
     // them, and nothing but the barrier and the first fragment read stands between two k-tiles.
-    auto k_tile = [&](int kt, u32x4* wcur, u32x4* wnext) {
+    // wcur: tile kt; wnext: the buffer tile kt + PD goes to; xreg: tile kt + 1, replaced by tile kt + 1 + RX.
+    auto k_tile = [&](int kt, u32x4* wcur, u32x4* wnext, u32x4* xreg) {
         u32x4 wf[2][NB];
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) { dequant16_fp8<WT, SCALED, AT>(wcur[nb], PAIR && nb >= NBO ? a.w_scale_pair : a.w_scale, wf[0][nb], wf[1][nb]); }
-        __syncthreads();                                     // tile kt is in xs[kt & 1]; the other buffer is free
-        fetch_w(kt + 1, wnext);
+        if constexpr (PD == 1) { __syncthreads(); }          // tile kt is in xs[kt & 1]; the other buffer is free
+        else { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }    // LDS order only: the loads of later tiles stay in flight
+        fetch_w(kt + PD, wnext);
         const u32x4* xt = xs[kt & 1];
         // token fragments run AHEAD instructions in front of the matrix-core instructions that use them
         constexpr int AHEAD = 3, FRAGS = 2 * MB;
@@ -414,8 +422,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         {
             if (f == FRAGS / 2)
             {
-                stage((kt + 1) & 1);
-                fetch_x(kt + 2);
+                stage((kt + 1) & 1, xreg);
+                fetch_x(kt + 1 + RX, xreg);
             }
             if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
             const frag_t xf = __builtin_bit_cast(frag_t, ring[f % (AHEAD + 1)]);
@@ -444,14 +452,35 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         }
     };
 
-    fetch_x(0);
-    fetch_w(0, wraw_a);
-    stage(0);
-    fetch_x(1);
-    for (int kt = 0; kt < n_kt; kt += 2)
+    fetch_x(0, xring[0]);
+#pragma unroll
+    for (int t = 0; t < PD; t++) { fetch_w(t, wraw[t]); }
+    stage(0, xring[0]);
+#pragma unroll
+    for (int t = 1; t <= RX; t++) { fetch_x(t, xring[t % RX]); }
+    if constexpr (PD == 1)
     {
-        k_tile(kt, wraw_a, wraw_b);
-        if (kt + 1 < n_kt) { k_tile(kt + 1, wraw_b, wraw_a); }
+        for (int kt = 0; kt < n_kt; kt += 2)
+        {
+            k_tile(kt, wraw[0], wraw[1], xring[0]);
+            if (kt + 1 < n_kt) { k_tile(kt + 1, wraw[1], wraw[0], xring[0]); }
+        }
+    }
+    else
+    {
+        // whole rounds of the register ring without a branch between the tiles (behind a skipped tile the compiler has to
+        // assume that fewer loads are in flight and waits for all but a few), then the last 0 .. PD tiles
+        int kt = 0;
+        for (; kt + RW <= n_kt; kt += RW)
+        {
+#pragma unroll
+            for (int j = 0; j < RW; j++) { k_tile(kt + j, wraw[j], wraw[(j + PD) % RW], xring[(j + 1) % RX]); }
+        }
+#pragma unroll
+        for (int j = 0; j < PD; j++)
+        {
+            if (kt + j < n_kt) { k_tile(kt + j, wraw[j], wraw[(j + PD) % RW], xring[(j + 1) % RX]); }
+        }
     }
 
     const bool wide_store = SPLIT ? a.n_out % 4 == 0 : (a.y_stride_out == 1 && a.y_stride_tok % 4 == 0 && ((uintptr_t)a.Y & 7u) == 0);
@@ -1051,8 +1080,9 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
     const bool scaled = a.w_scale != 1.0f;
     if (splits > 1)
     {
-        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
-        else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT, NB><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        constexpr int PD = MB == 4 ? 3 : 1;          // 64-token tiles split k only up to 64 tokens: bound by the weight bytes
+        if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT, NB, false, false, PD><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+        else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT, NB, false, false, PD><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
         launch_splitk_combine<AT>(partial, splits, a, e);
     }
     else
@@ -1176,8 +1206,8 @@ void launch_gemm_mfma_direct_segments(LinearArgs a)
             }
             else
             {
-                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
-                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
             const long long blocks = ((long long)a.tokens * (n_all / 4) + 255) / 256, cap = (long long)cus * 16;
             gemm_splitk_combine_kernel<DT_BF16, true, false><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
@@ -1226,8 +1256,8 @@ void launch_gemm_mfma_direct_pair(const LinearArgs& a)
             }
             else
             {
-                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
-                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
             const long long blocks = ((long long)a.tokens * (a.n_out / 4) + 255) / 256, cap = (long long)cu_count() * 16;
             gemm_splitk_combine_kernel<DT_BF16, false, true><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
@@ -1254,7 +1284,7 @@ void launch_gemm_mfma(const LinearArgs& a)
 // evenly over the CUs (384 tiles on 256 CUs leave half of them with twice the work: 36 % of peak where 512 even tiles
 // reach 42 %), and 48-feature waves with 64-token tiles cost ~5 % against the larger tiles.  Too few tiles in every
 // shape: the k range is split over workgroups (256-feature tiles, about one workgroup per CU, 1024 elements of k or more
-// each) and a second kernel adds the partial sums.
+// each; 512 or more up to 64 tokens) and a second kernel adds the partial sums.
 struct DirectPlan
 {
     int nb, mb, splits;
