@@ -1080,7 +1080,7 @@ void launch_gemm_mfma_direct(const LinearArgs& a, int splits = 1, float* partial
     const bool scaled = a.w_scale != 1.0f;
     if (splits > 1)
     {
-        constexpr int PD = MB == 4 ? 3 : 1;          // 64-token tiles split k only up to 64 tokens: bound by the weight bytes
+        constexpr int PD = MB <= 4 ? 3 : 1;          // 64- and 32-token tiles split k only up to 64 tokens: bound by the weight bytes
         if (scaled) { gemm_mfma_direct_kernel<WT, true, MB, true, TILED, AT, NB, false, false, PD><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
         else { gemm_mfma_direct_kernel<WT, false, MB, true, TILED, AT, NB, false, false, PD><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
         launch_splitk_combine<AT>(partial, splits, a, e);
@@ -1190,7 +1190,7 @@ void launch_gemm_mfma_direct_segments(LinearArgs a)
             n_all += a.seg_n_out[sg];
             by4 = by4 && a.seg_n_out[sg] % 4 == 0;
         }
-        const int mb = a.tokens > 64 ? 8 : 4;
+        const int mb = a.tokens > 64 ? 8 : (a.tokens > 32 ? 4 : 2);
         const long long base = (long long)n_tiles * ((a.tokens + mb * 16 - 1) / (mb * 16));
         long long splits = cus / base;
         if (splits > (mb == 8 ? 8 : 16)) { splits = mb == 8 ? 8 : 16; }
@@ -1204,10 +1204,15 @@ void launch_gemm_mfma_direct_segments(LinearArgs a)
                 if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
                 else { gemm_mfma_direct_kernel<WT, false, 8, true, TILED, DT_BF16, 4, false, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
-            else
+            else if (mb == 4)
             {
                 if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
                 else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            else
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 2, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 2, true, TILED, DT_BF16, 4, false, true, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
             const long long blocks = ((long long)a.tokens * (n_all / 4) + 255) / 256, cap = (long long)cus * 16;
             gemm_splitk_combine_kernel<DT_BF16, true, false><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
@@ -1240,7 +1245,7 @@ void launch_gemm_mfma_direct_pair(const LinearArgs& a)
     // adds the gate and the up sums and writes the SwiGLU product with the same roundings (36-layer model, 128 tokens:
     // 8.0 -> 7.3 ms; from 129 tokens on, 192 workgroups or more, the split only costs).
     {
-        const int mb = a.tokens > 64 ? 8 : 4;
+        const int mb = a.tokens > 64 ? 8 : (a.tokens > 32 ? 4 : 2);
         const int m_split = (a.tokens + mb * 16 - 1) / (mb * 16);
         long long splits = cu_count() / ((long long)n_tiles * m_split);
         if (splits > 8) { splits = 8; }
@@ -1254,10 +1259,15 @@ void launch_gemm_mfma_direct_pair(const LinearArgs& a)
                 if (scaled) { gemm_mfma_direct_kernel<WT, true, 8, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
                 else { gemm_mfma_direct_kernel<WT, false, 8, true, TILED, DT_BF16, 4, true><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
-            else
+            else if (mb == 4)
             {
                 if (scaled) { gemm_mfma_direct_kernel<WT, true, 4, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
                 else { gemm_mfma_direct_kernel<WT, false, 4, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+            }
+            else
+            {
+                if (scaled) { gemm_mfma_direct_kernel<WT, true, 2, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
+                else { gemm_mfma_direct_kernel<WT, false, 2, true, TILED, DT_BF16, 4, true, false, 3><<<grid, 256, 0, stream()>>>(a, n_tiles, partial); }
             }
             const long long blocks = ((long long)a.tokens * (a.n_out / 4) + 255) / 256, cap = (long long)cu_count() * 16;
             gemm_splitk_combine_kernel<DT_BF16, false, true><<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(partial, (int)splits, a);
@@ -1361,7 +1371,7 @@ inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool f
         if (plan.splits > 1)
         {
             plan.nb = 4;
-            plan.mb = a.tokens > 64 ? 8 : 4;
+            plan.mb = a.tokens > 64 ? 8 : (a.tokens > 32 || fp4 ? 4 : 2);        // FP8, up to 32 tokens: a 32-token tile
         }
     }
     return plan;
@@ -1441,12 +1451,14 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, true, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, true, AT, 3>(d); }
                 else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, true, AT>(d, splits, partial, e); }
+                else if (mb == 2 && splits > 1) { launch_gemm_mfma_direct<WT, 2, true, AT>(d, splits, partial, e); }
                 else { launch_gemm_mfma_direct<WT, 4, true, AT>(d, splits, partial, e); }
             }
             else
             {
                 if (nb == 3) { mb == 8 ? launch_gemm_mfma_direct<WT, 8, false, AT, 3>(d) : launch_gemm_mfma_direct<WT, 4, false, AT, 3>(d); }
                 else if (mb == 8) { launch_gemm_mfma_direct<WT, 8, false, AT>(d, splits, partial, e); }
+                else if (mb == 2 && splits > 1) { launch_gemm_mfma_direct<WT, 2, false, AT>(d, splits, partial, e); }
                 else { launch_gemm_mfma_direct<WT, 4, false, AT>(d, splits, partial, e); }
             }
             return true;
