@@ -299,7 +299,7 @@ def llama_fp4_decode(ws: Workspace, steps: int, warmup: int, use_graph: bool, re
 
 def prompt_phase(ws: Workspace, model, token_counts=(512, 2048), reps: int = 3, layout: str = "row-major", c=None):
     """The prompt phase of the same model (DecodeModel::prefill, positions 0 .. T - 1): every linear is one quantized GEMM
-    with T columns -- BASELINE config 4's kernel on all seven shapes of a layer, on the row-major file bytes (a batch-1
+    with T columns -- the prefill-GEMM kernel of the `prefill` entry on all seven shapes of a layer, on the row-major file bytes (a batch-1
     DecodeModel keeps no tiled copies) -- with the row kernels and the causal attention between them.  Wall clock around the
     call, device synchronised on both sides; best of `reps` after one warm-up call (which also allocates the activations)."""
     import numpy as np
@@ -573,7 +573,7 @@ def same_gpu_comparators(ws, weights, K, N, M, max_ops=24):
 
 
 def prefill_cases(ws, by_shape):
-    """BASELINE config 4: W8A16 prefill GEMM, M in {512, 2048} x the two MLP shapes, with the plain BF16 GEMM
+    """The W8A16 prefill GEMM workload: M in {512, 2048} x the two MLP shapes, with the plain BF16 GEMM
     of the vendor library (torch.matmul) on the same shape beside it."""
     t = ws.torch
     out = []
@@ -609,7 +609,7 @@ def fp4_bytes(K, N, M, block):
 
 
 def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
-    """BASELINE config 3: Llama-3.1-8B-shaped FP4 block-scale GEMVs, block 16 (the reference's format) and 32, weights
+    """The FP4 workload: Llama-3.1-8B-shaped FP4 block-scale GEMVs, block 16 (the reference's format) and 32, weights
     rotating over at least 512 MiB of distinct buffers, with their load-time tiled copies registered as the host mirror
     registers them (unless --no-repack); M = 1 is the configuration's own row, 4 and 16 ride along.  Second list: the
     FP4 prefill GEMM on the two MLP shapes (FLOPs 2 M K N against the BF16 matrix-core peak)."""
