@@ -524,7 +524,7 @@ int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const*
     if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
     if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
     if (n_segments < 1 || n_segments > 3 || !n_out || !W || !inv_scale || !Y || !ldy) { return -1; }
-    if (tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
+    if (tokens < 2 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || !X || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
     LinearArgs a{};
     a.X = (const uint16_t*)X;
@@ -588,7 +588,7 @@ int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, cons
     const bool fp4 = w_type == DT_FP4;
     if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
     if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
-    if (n_out <= 0 || tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
+    if (n_out <= 0 || tokens < 2 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K || ldy < n_out) { return -1; }
     if (!W_gate || !W_up || !X || !Y || !aligned16(W_gate) || !aligned16(W_up) || !aligned16(X) || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if ((long long)n_out * ldw >= (1LL << 32) || (long long)tokens * ldx * 2 >= (1LL << 32)) { return -1; }
     LinearArgs a{};
@@ -647,7 +647,7 @@ int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const void* W, int
     const bool fp4 = w_type == DT_FP4;
     if (w_type != DT_E5M2 && w_type != DT_E4M3 && !fp4) { return -1; }
     if (fp4 && (K % 128 != 0 || ldw != K)) { return -1; }
-    if (n_out <= 0 || n_out % 8 != 0 || n_out > 4096 || tokens < 17 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K) { return -1; }
+    if (n_out <= 0 || n_out % 8 != 0 || n_out > 4096 || tokens < 2 || K <= 0 || K % 64 != 0 || ldw < K || ldx < K) { return -1; }
     if (!W || !X || !res || !sum || !norm_w || !y || ldw % 16 != 0 || ldx % 8 != 0) { return -1; }
     if (!aligned16(W) || !aligned16(X) || !aligned16(res) || !aligned16(sum) || !aligned16(norm_w) || !aligned16(y)) { return -1; }
     LinearArgs a{};

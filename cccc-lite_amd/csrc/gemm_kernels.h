@@ -1420,7 +1420,7 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
     if constexpr (WT == DT_FP4 && AT == DT_BF16)
     {
         // FP4 with a tiled copy (codes, then the scales behind all code KiBs): the register-fed kernel
-        if (tiled && a.K % 128 == 0 && a.tokens >= 17 && (long long)a.tokens * a.ldx * 2 < (1LL << 32))
+        if (tiled && a.K % 128 == 0 && a.tokens >= (e ? 2 : 17) && (long long)a.tokens * a.ldx * 2 < (1LL << 32))
         {
             LinearArgs d = a;
             d.W = tiled;
@@ -1438,7 +1438,7 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
     {
         const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
         // (HALF activations have no matrix-core GEMV: there the register-fed kernel also serves 5-16 tokens)
-        if (a.K % 64 == 0 && a.tokens >= (AT == DT_HALF ? 5 : 17) && small_offsets)
+        if (a.K % 64 == 0 && a.tokens >= (e ? 2 : (AT == DT_HALF ? 5 : 17)) && small_offsets)
         {
             LinearArgs d = a;
             if (tiled) { d.W = tiled; }

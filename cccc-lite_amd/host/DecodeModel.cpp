@@ -440,11 +440,15 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         const int r = hip_add_bf16(a.data(), b.data(), sum.data(), (unsigned long long)n * c.hidden);
         return r != 0 ? r : norm(sum, y, w);
     };
+    // The fused GEMM launches below are matrix-matrix kernels; up to 16 tokens the separate calls run the matrix-vector
+    // kernels, which stay ahead on tiled copies (16 tokens: 3.3 ms either way, 2 tokens 2.8 against 3.1) but not on the file
+    // layout from about 5 tokens on (16 tokens: 4.1 -> 3.7 ms of a 36-layer 4096-wide model, 6 tokens 3.9 -> 3.5)
+    const bool fuse_gemms = n >= (c.layers > 0 && layers_[0].wq->hasTiled() ? 17 : 5);
     // sum = res + W x and y = norm(sum): where the GEMM splits its k range the launch that adds the partial sums does the add
     // and the norm as well (-1: this shape does not split, or the library has no such kernel for it)
     auto linear_add_norm = [&](const Matrix& W, int n_out, int K, const Matrix& x, Matrix& res, Matrix& sum, Matrix& w, Matrix& y) {
-        int r = hip_quant_gemm_add_rms_norm(n_out, n, K, W.data(), (int)W.getDataType(), K, W.getQuantScale(), x.data(), K,
-                                            res.data(), sum.data(), w.data(), y.data(), c.eps);
+        int r = !fuse_gemms ? -1 : hip_quant_gemm_add_rms_norm(n_out, n, K, W.data(), (int)W.getDataType(), K, W.getQuantScale(), x.data(), K,
+                                                               res.data(), sum.data(), w.data(), y.data(), c.eps);
         if (r >= 0) { return r; }
         r = linear(W, n_out, K, x, *pf_.o);
         return r != 0 ? r : add_norm(res, *pf_.o, sum, w, y);
@@ -455,7 +459,7 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         Layer& L = layers_[li];
         // q, k, v: one launch for three weights of one type, else three calls
         int qkv = -1;
-        if (rc == 0 && L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
+        if (rc == 0 && fuse_gemms && L.wk->getDataType() == L.wq->getDataType() && L.wv->getDataType() == L.wq->getDataType())
         {
             const int widths[3] = { q_out, kv_out, kv_out };
             const void* const weights[3] = { L.wq->data(), L.wk->data(), L.wv->data() };
@@ -485,7 +489,7 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         if (rc == 0) { rc = linear_add_norm(*L.wo, c.hidden, q_out, *pf_.att, *pf_.x, *pf_.r1, *L.rms_ffn, *pf_.xn); }
         // gate, up and their SwiGLU product: one launch for two weights of one type, else the three calls
         int fused = -1;
-        if (rc == 0 && L.w_gate->getDataType() == L.w_up->getDataType())
+        if (rc == 0 && fuse_gemms && L.w_gate->getDataType() == L.w_up->getDataType())
         {
             fused = hip_quant_gemm_swiglu(c.inter, n, c.hidden, L.w_gate->data(), L.w_up->data(), (int)L.w_gate->getDataType(), c.hidden,
                                           L.w_gate->getQuantScale(), L.w_up->getQuantScale(), pf_.xn->data(), c.hidden, pf_.gated->data(), c.inter);

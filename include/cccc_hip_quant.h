@@ -277,7 +277,7 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
  * workgroups, the FP32 partial sums go to a workspace the library grows on demand and one more launch adds them for all
  * segments; otherwise the bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not split either.
  * FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
- * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 17 tokens, K not a
+ * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 2 tokens, K not a
  * multiple of 64.  No
  * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
 C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
@@ -289,7 +289,7 @@ C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const voi
  * weights [n_out][K] (row pitch ldw; tiled copy used when registered) or FP4 block-scale weights with a registered tiled copy
  * (K % 128 == 0, ldw == K); BF16 activations [tokens][K]; res, sum, y dense [tokens][n_out], n_out <= 4096 and a multiple
  * of 8, everything 16-byte aligned.  -1 (nothing launched, use the separate calls): a shape that does not split, fewer than
- * 17 tokens, anything else unsupported.  No counterpart in the reference. */
+ * 2 tokens, anything else unsupported.  No counterpart in the reference. */
 C_EXPORT int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const void* W, int w_type, int ldw, float inv_scale,
                                          const void* X, int ldx, const void* res, void* sum, const void* norm_w, void* y, float epsilon);
 /* y[t][o] = swiglu(gate[t][o], up[t][o]) with gate = bf16(W_gate x_t), up = bf16(W_up x_t): the gate and up linears of an
@@ -300,7 +300,9 @@ C_EXPORT int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const voi
  * workgroups and a second launch that adds the FP32 partial sums (workspace grown on demand) and writes the product with
  * the same roundings.  BF16 activations [tokens][K] (row pitch ldx) and output [tokens][n_out] (ldy).  FP4 block-scale
  * weights (type 6) take part when both have a registered tiled copy of one block length, K is a multiple of 128 and
- * ldw == K.  -1 (nothing launched, use the separate calls): other weight types, fewer than 17 tokens, K not a multiple of 64. */
+ * ldw == K.  -1 (nothing launched, use the separate calls): other weight types, fewer than 2 tokens, K not a multiple of 64.
+ * (Up to 16 tokens the separate calls are matrix-vector kernels; on the file layout the fused launches are ahead from about
+ * 5 tokens on, on tiled copies from 17.) */
 C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                                    float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);
 C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
