@@ -837,6 +837,7 @@ def main():
                     assert model.prepare_tiled(li, name)
             extra["prompt_phase"]["cases"] += prompt_phase(ws, model, token_counts=(32, 128, 512, 2048, DECODE_CTX), layout="tiled copies")
             extra["generate"] = generate_run(ws, model, use_graph)
+            extra["generate_short_prompt"] = generate_run(ws, model, use_graph, prompt_tokens=128)
             if not args.no_fp4_step:
                 # the Llama-3.1-8B-shaped FP4 model, whose linears were loaded with their tiled copies (the FP4 GEMM reads those)
                 extra["fp4_decode_step"]["prompt_phase"] = prompt_phase(ws, fp4_model, token_counts=(32, 128, 512, 2048), layout="tiled copies", c=LLAMA31_8B)
