@@ -270,18 +270,21 @@ C_EXPORT int hip_attention_prefill_bf16(const void* q, const void* k_cache, cons
 /* y = bf16(a + b) and y = bf16(bf16(gate * bf16(sigmoid(gate))) * up) over n BF16 elements (n % 8 == 0, 16-byte aligned):
  * the residual add and the SwiGLU product with the reference's roundings (cccc-hip/hip_functions.cpp:895-908, :722-732,
  * :953-966; cccc/MatrixEx.cpp:756-762). */
+C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
+C_EXPORT int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n);
+
 /* Up to three linears on the same activations in one launch: Y[s][t][o] = bf16(W[s] x_t), s < n_segments <= 3, FP8 weights
  * [n_out[s]][K] of one type, K and row pitch ldw (all on their registered tiled copies, or all on the file layout), BF16
  * activations [tokens][K] and outputs with row pitch ldy[s] -- the q, k and v projections of a prompt, whose narrow members
  * alone leave most of the GPU idle.  With too few output tiles for the GPU (FP8, K >= 1024) the k range is split over
  * workgroups, the FP32 partial sums go to a workspace the library grows on demand and one more launch adds them for all
  * segments; otherwise the bits of the separate hip_quant_gemm calls (alpha 1, beta 0) where those do not split either.
- * FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one
- * block length and K is a multiple of 128.  -1 (nothing launched): other weight types, fewer than 2 tokens, K not a
- * multiple of 64.  No
- * counterpart in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
+ * FP4 block-scale weights (type 6) take part when every one has a registered tiled copy of one block length and K is a
+ * multiple of 128.  -1 (nothing launched): other weight types, fewer than 2 tokens, K not a multiple of 64.  No counterpart
+ * in the reference, which issues one batchedMul per projection (scripts/convert_weights.py:492-500). */
 C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const void* const* W, const float* inv_scale,
                                      void* const* Y, const int* ldy, int w_type, int tokens, int K, int ldw, const void* X, int ldx);
+
 /* A linear, the residual add behind it and the RMSNorm behind that, for the shapes whose GEMM splits its k range over
  * workgroups (few output tiles: the o and down projections of a prompt of up to ~512 tokens): sum[t] = bf16(res[t] +
  * bf16(W x_t)), y[t] = rmsnorm(sum[t]) * norm_w -- the launch that adds the FP32 partial sums does the add and the norm as
@@ -292,6 +295,7 @@ C_EXPORT int hip_quant_gemm_segments(int n_segments, const int* n_out, const voi
  * 2 tokens, anything else unsupported.  No counterpart in the reference. */
 C_EXPORT int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const void* W, int w_type, int ldw, float inv_scale,
                                          const void* X, int ldx, const void* res, void* sum, const void* norm_w, void* y, float epsilon);
+
 /* y[t][o] = swiglu(gate[t][o], up[t][o]) with gate = bf16(W_gate x_t), up = bf16(W_up x_t): the gate and up linears of an
  * MLP block (two FP8 weights of one shape [n_out][K], row pitch ldw, dequantisation multipliers as in hip_quant_gemm; both
  * on their registered tiled copies or both on the file layout) and the reference's SwiGLU product
@@ -305,8 +309,7 @@ C_EXPORT int hip_quant_gemm_add_rms_norm(int n_out, int tokens, int K, const voi
  * 5 tokens on, on tiled copies from 17.) */
 C_EXPORT int hip_quant_gemm_swiglu(int n_out, int tokens, int K, const void* W_gate, const void* W_up, int w_type, int ldw,
                                    float inv_scale_gate, float inv_scale_up, const void* X, int ldx, void* Y, int ldy);
-C_EXPORT int hip_add_bf16(const void* a, const void* b, void* y, unsigned long long n);
-C_EXPORT int hip_swiglu_bf16(const void* gate, const void* up, void* y, unsigned long long n);
+
 /* sum = bf16(a + b) and y = rmsnorm(sum) * norm_w, rows of `inner` BF16 values (a multiple of 8, at most 4096; 16-byte
  * aligned pointers, else -1): hip_add_bf16 followed by hip_rms_norm_fwd in one pass, the same bits.  `sum` and `y` are
  * buffers of their own.  The residual add and the norm behind it in the reference's graph (hip_functions.cpp:895-908, :1506-1535). */
