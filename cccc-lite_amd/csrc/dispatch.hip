@@ -8,11 +8,17 @@
 //     FP8, tokens >= 17                            gemm_mfma: weights straight into the matrix-core operands when
 //                                                  tokens >= 17 and K % 64 == 0 (row-major or tiled copy, k split
 //                                                  over workgroups when the output has few tiles), else dequant-to-LDS
-//     FP4 block scales, tokens <= 16               gemv_dot2 in token groups of four
-//     FP4 block scales, tokens >= 17               gemm_mfma (dequant-to-LDS)
+//     FP4 block scales, tiled copy registered      tokens <= 16: gemv_mfma_tiled (matrix cores, one pass over the weight for
+//                                                  up to 16 tokens; one or two tokens of a short row stay on gemv_dot2);
+//                                                  tokens >= 17 and K % 128 == 0: gemm_mfma_tiled (codes and scales straight
+//                                                  into the matrix-core operands, k split when the output has few tiles)
+//     FP4 block scales, no tiled copy              gemv_dot2 in token groups of four; tokens >= 17: gemm_mfma (dequant-to-LDS)
 //     HALF activations                             the half instantiations of gemv_dot2 / gemm_mfma
 //     anything the fast kernels cannot take (transposed layouts, odd sizes, misaligned pointers,
 //     FP4 without block scales): generic
+// Also here, for a prompt's T tokens on the register-fed GEMM kernels: hip_quant_gemm_segments (q, k, v in one launch),
+// hip_quant_gemm_swiglu (gate, up and their SwiGLU product) and hip_quant_gemm_add_rms_norm (a k-split linear whose combine
+// launch adds the residual and norms the row).
 #include "../../include/cccc_hip_quant.h"
 #include "gemv_kernels.h"
 #include "dispatch_half.h"
