@@ -68,7 +68,29 @@ class BenchLibrary:
         L.cccc_bench_fp4_chain.argtypes = [i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_uint, i32, i32]
         L.cccc_decode_bench_gate_up.restype = ctypes.c_double
         L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
+        L.cccc_bench_floor_read.restype = ctypes.c_double
+        L.cccc_bench_floor_read.argtypes = [i32, ctypes.POINTER(vp), ctypes.c_ulonglong, i32, i32, i32]
+        L.cccc_bench_launch_us.restype = ctypes.c_double
+        L.cccc_bench_launch_us.argtypes = [i32, i32, i32]
         self.c, self.ctypes = L, ctypes
+
+    def floor_read_us(self, ptrs, nbytes, iters=None, wgs_per_cu=8) -> float:
+        """Microseconds per launch of a kernel that only streams `nbytes` with 16-byte loads, rotating over the buffers
+        `ptrs` (host/bench_kernels.hip): the floor of any weight-streaming launch of that size on this GPU."""
+        n = len(ptrs)
+        iters = iters or max(20, min(400, (4 << 30) // max(nbytes, 1)))
+        us = float(self.c.cccc_bench_floor_read(n, (self.ctypes.c_void_p * n)(*ptrs), nbytes, wgs_per_cu, iters, min(5, n)))
+        if us < 0:
+            raise RuntimeError(f"floor read failed: {us}")
+        return us
+
+    def launch_us(self, kind=0, n_launches=200, reps=20) -> float:
+        """Microseconds per launch of `n_launches` dependent launches inside one hipGraph (0: empty kernel, 1: one wave
+        with one dependent trip to memory)."""
+        us = float(self.c.cccc_bench_launch_us(n_launches, reps, kind))
+        if us < 0:
+            raise RuntimeError(f"launch timing failed: {us}")
+        return us
 
     def linear_chain(self, W, X, R, steps, warmup, use_graph) -> float:
         n = len(W)
@@ -103,28 +125,37 @@ class Workspace:
         self.repack = False
 
     def weight_e5m2(self, n_out, K):
+        return self.weight_fp8(n_out, K, E5M2)
+
+    def weight_fp8(self, n_out, K, dtype=E5M2, inv_scale=1.0):
+        """FP8 codes of N(0, 0.02) weights (bf16, then round to nearest).  inv_scale != 1: the codes are those of
+        w / inv_scale and the matrix carries inv_scale as its per-tensor dequantisation multiplier, as a weight quantized by
+        Matrix::quantizeWeights does (cccc/Matrix.cpp:338-352)."""
         t = self.torch
-        m = self.host.matrix(K, n_out, 1, 1, E5M2)
+        f8 = t.float8_e5m2 if dtype == E5M2 else t.float8_e4m3fn
+        m = self.host.matrix(K, n_out, 1, 1, dtype)
         rows = max(1, min(n_out, (1 << 27) // K))
         for r0 in range(0, n_out, rows):
             r = min(rows, n_out - r0)
-            w = (t.randn(r, K, device=self.dev, generator=self.gen) * 0.02).to(t.bfloat16).to(t.float8_e5m2)
-            assert self.lib.convert(w.data_ptr(), E5M2, m.data_ptr + r0 * K, E5M2, r * K, 1.0) == 0
+            w = ((t.randn(r, K, device=self.dev, generator=self.gen) * (0.02 / inv_scale)).to(t.bfloat16)).to(f8)
+            assert self.lib.convert(w.data_ptr(), dtype, m.data_ptr + r0 * K, dtype, r * K, 1.0) == 0
             t.cuda.synchronize()
+        if inv_scale != 1.0:
+            m.quant_scale = inv_scale
         if self.repack:
             m.prepare_tiled()        # what Matrix::loadQuantizedDirect does after uploading file bytes
         return m
 
-    def activation(self, tokens, K):
+    def activation(self, tokens, K, dtype=BF16):
         t = self.torch
-        m = self.host.matrix(K, tokens, 1, 1, BF16)
-        x = t.randn(tokens, K, device=self.dev, generator=self.gen).to(t.bfloat16)
-        assert self.lib.convert(x.data_ptr(), BF16, m.data_ptr, BF16, tokens * K * 2, 1.0) == 0
+        m = self.host.matrix(K, tokens, 1, 1, dtype)
+        x = t.randn(tokens, K, device=self.dev, generator=self.gen).to(t.bfloat16 if dtype == BF16 else t.float16)
+        assert self.lib.convert(x.data_ptr(), dtype, m.data_ptr, dtype, tokens * K * 2, 1.0) == 0
         t.cuda.synchronize()
         return m
 
-    def output(self, tokens, n_out):
-        return self.host.matrix(n_out, tokens, 1, 1, BF16)
+    def output(self, tokens, n_out, dtype=BF16):
+        return self.host.matrix(n_out, tokens, 1, 1, dtype)
 
 
 def build_decode_model(ws: Workspace, tokens: int):
@@ -178,10 +209,13 @@ def build_grouped_model(ws: Workspace, tokens: int):
 DECODE_CTX = 4096
 
 
-def build_decode_step(ws: Workspace, ctx: int):
+def build_decode_step(ws: Workspace, ctx: int, quantize_on_device: bool = False):
     """The full random-init Qwen3-8B W8A16 model of the C++ DecodeModel, tensors generated on the GPU:
     FP8_E5M2 linears from N(0, 0.02) (bf16, then round to nearest), norms near 1, BF16 embedding and
-    a KV cache already holding `ctx` positions of N(0, 1) keys and values."""
+    a KV cache already holding `ctx` positions of N(0, 1) keys and values.
+    quantize_on_device: the linears are generated as BF16 and quantized by Matrix::quantizeWeights, the reference's route for
+    a model stored unquantized (cccc/Matrix.cpp:301-355): truncating encoder, per-tensor scale absmax / 57344 -- every
+    linear then carries a dequantisation multiplier other than 1."""
     t, c = ws.torch, QWEN3_8B
     model = ws.pkg.host_api.DecodeModel(ws.host, c["layers"], c["hidden"], 32, 8, 128, c["inter"], c["vocab"], ctx)
 
@@ -192,6 +226,17 @@ def build_decode_step(ws: Workspace, ctx: int):
             w = (t.randn(r, K, device=ws.dev, generator=ws.gen) * 0.02).to(t.bfloat16).to(t.float8_e5m2)
             assert ws.lib.convert(w.data_ptr(), E5M2, ptr + r0 * K, E5M2, r * K, 1.0) == 0
             t.cuda.synchronize()
+
+    def quantize(li, name, n_out, K):
+        w = t.empty(n_out, K, dtype=t.bfloat16, device=ws.dev)
+        rows = max(1, min(n_out, (1 << 26) // K))
+        for r0 in range(0, n_out, rows):
+            r = min(rows, n_out - r0)
+            w[r0:r0 + r] = (t.randn(r, K, device=ws.dev, generator=ws.gen) * 0.02).to(t.bfloat16)
+        t.cuda.synchronize()
+        model.quantize_linear(li, name, w.data_ptr(), E5M2)
+        t.cuda.synchronize()
+        del w
 
     def fill_bf16(ptr, n, mean, std):
         step = 1 << 26
@@ -206,13 +251,19 @@ def build_decode_step(ws: Workspace, ctx: int):
               "w_down": (c["hidden"], c["inter"])}
     for li in range(c["layers"]):
         for name, (n_out, K) in shapes.items():
-            fill_fp8(model.tensor_ptr(li, name), n_out, K)
+            if quantize_on_device:
+                quantize(li, name, n_out, K)
+            else:
+                fill_fp8(model.tensor_ptr(li, name), n_out, K)
         for name, n in (("rms_attn", c["hidden"]), ("rms_ffn", c["hidden"]), ("q_norm", 128), ("k_norm", 128)):
             fill_bf16(model.tensor_ptr(li, name), n, 1.0, 0.1)
         for is_v in (False, True):
             fill_bf16(model.kv_ptr(li, is_v), 8 * ctx * 128, 0.0, 1.0)
-    fill_fp8(model.tensor_ptr(0, "lm_head"), c["vocab"], c["hidden"])
-    model.prepare_tiled(0, "lm_head")                  # what loading through set_tensor / load_named does
+    if quantize_on_device:
+        quantize(0, "lm_head", c["vocab"], c["hidden"])        # (quantizeLinear keeps the head's tiled copy itself)
+    else:
+        fill_fp8(model.tensor_ptr(0, "lm_head"), c["vocab"], c["hidden"])
+        model.prepare_tiled(0, "lm_head")              # what loading through set_tensor / load_named does
     fill_bf16(model.tensor_ptr(0, "rms_final"), c["hidden"], 1.0, 0.1)
     fill_bf16(model.tensor_ptr(0, "emb"), c["vocab"] * c["hidden"], 0.0, 1.0)
     return model
@@ -515,11 +566,13 @@ def time_chain(ws, ops, steps, warmup, use_graph):
     return ms
 
 
-def shape_sweep(ws, by_shape, token_counts, use_graph):
-    """Per-shape GEMV rates with weights rotating over distinct buffers (no cache reuse)."""
+def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
+    """Per-shape GEMV rates with weights rotating over distinct buffers (no cache reuse).  floor_us: a launch that only
+    streams the same weight buffers with 16-byte loads (host/bench_kernels.hip), i.e. what the memory side alone costs."""
     out = []
     for (K, N) in QWEN_SHAPES:
         weights = by_shape[(K, N)]
+        floor_us = ws.bench.floor_read_us([W.data_ptr for W in weights], K * N)
         for M in token_counts:
             X, Y = ws.activation(M, K), ws.output(M, N)
             reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
@@ -528,11 +581,48 @@ def shape_sweep(ws, by_shape, token_counts, use_graph):
             us = ms * 1000.0 / (3 * len(ops))
             gbs = gemv_bytes(K, N, M) / us * 1e-3
             assert ws.lib.linear(weights[0].data_ptr, E5M2, X.data_ptr, Y.data_ptr, N, M, K) == 0
-            row = {"K": K, "N": N, "M": M, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+            row = {"K": K, "N": N, "M": M, "us": round(us, 2), "floor_us": round(floor_us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
                    "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(K * N * len(weights) / 2 ** 20)}
-            if M == 1:
+            if M == 1 and comparators:
                 row.update(same_gpu_comparators(ws, weights, K, N, M))
             out.append(row)
+    return out
+
+
+SCALED_INV_SCALE = 0.1 / 57344.0       # absmax / max_code of a weight whose largest element is 0.1 (cccc/Matrix.cpp:338-352)
+
+
+def variant_sweep(ws, by_shape, token_counts=(1, 16)):
+    """The routes of the same GEMV that a model quantized by the reference takes instead of `sweep`'s (scale 1, E5M2, BF16):
+    "e5m2_scaled" -- the same E5M2 weights with a per-tensor dequantisation multiplier other than 1 (every weight
+    Matrix::quantizeWeights produces carries absmax / 57344, cccc/Matrix.cpp:338-352): the kernels then decode to FP32,
+    multiply and round to BF16 instead of one hardware conversion; "e4m3_scaled" -- FP8_E4M3 codes with a scale (the hy-mt2
+    files, scripts/convert_weights.py:272-313); "e5m2_half" -- HALF activations and outputs (the reference's Qwen3 inis
+    default to data_type = half, scripts/convert_weights.py:728-729; branch cccc/cublas_real.h:921-938).  Each row carries
+    the time of the plain route on the same shape (`base_us`, from `sweep`) when it was measured."""
+    out = []
+    for (K, N) in QWEN_SHAPES:
+        base = by_shape[(K, N)]
+        n_w = len(base) if K * N * len(base) <= (1 << 30) else max(1, (1 << 30) // (K * N))
+        e4 = [ws.weight_fp8(N, K, E4M3, SCALED_INV_SCALE * 128.0) for _ in range(n_w)]       # 448 instead of 57344
+        for route, weights, act in (("e5m2_scaled", base, BF16), ("e4m3_scaled", e4, BF16), ("e5m2_half", base, HALF)):
+            if route == "e5m2_scaled":
+                for W in weights:
+                    W.quant_scale = SCALED_INV_SCALE
+            for M in token_counts:
+                X, Y = ws.activation(M, K, act), ws.output(M, N, act)
+                reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
+                ops = [(W, X, Y, K, N) for W in weights] * reps
+                ms = time_chain(ws, ops, 3, 1, False)
+                us = ms * 1000.0 / (3 * len(ops))
+                gbs = gemv_bytes(K, N, M) / us * 1e-3
+                assert ws.lib.linear(weights[0].data_ptr, weights[0].dtype, X.data_ptr, Y.data_ptr, N, M, K, inv_scale=weights[0].quant_scale, act_type=act) == 0
+                out.append({"route": route, "K": K, "N": N, "M": M, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                            "kernel": ws.lib.last_kernel()})
+            if route == "e5m2_scaled":
+                for W in weights:
+                    W.quant_scale = 1.0
+        ws.keep.append(e4)                 # freed with everything else (freeing mid-run slows what runs next)
     return out
 
 
@@ -594,8 +684,16 @@ def prefill_cases(ws, by_shape):
                     y = x @ bf[i % 4].T
                 t.cuda.synchronize()
                 lib_us = (time.perf_counter() - t0) * 1e6 / 16
+            # the same launches with a per-tensor dequantisation multiplier (the route of a weight quantized on load)
+            for W in weights:
+                W.quant_scale = SCALED_INV_SCALE
+            us_scaled = time_chain(ws, ops, 10, 3, False) * 1000.0 / (10 * len(ops))
+            for W in weights:
+                W.quant_scale = 1.0
+            tf_scaled = 2.0 * M * K * N / us_scaled * 1e-6
             out.append({"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                        "kernel": ws.lib.last_kernel(), "vendor_bf16_gemm_us": round(lib_us, 2),
+                        "kernel": ws.lib.last_kernel(), "scaled_us": round(us_scaled, 2), "scaled_TFLOPs": round(tf_scaled, 1),
+                        "scaled_frac_of_bf16_mfma_peak": round(tf_scaled / MFMA_BF16_PEAK_TFLOPS, 4), "vendor_bf16_gemm_us": round(lib_us, 2),
                         "vendor_bf16_gemm_TFLOPs": round(2.0 * M * K * N / lib_us * 1e-6, 1)})
         del bf
     return out
@@ -698,12 +796,51 @@ def cpu_baseline(pkg, threads, unit):
     return out
 
 
+def north_star_summary(line):
+    """The headline figures of the line once more, compact and last, so that they survive a reader that keeps only the tail of
+    the output: fractions of the 8 TB/s HBM peak for the GEMVs (rows = K x N, columns = token counts), fractions of the
+    2.5 PFLOP/s BF16 matrix-core peak for the prefill GEMMs, the decode step against its HBM bound."""
+    def grid(rows, key="frac", extra=lambda r: True):
+        out = {}
+        for r in rows:
+            if extra(r):
+                out.setdefault(f"{r['K']}x{r['N']}", {})[f"M{r['M']}"] = r[key]
+        return out
+    # least important first: a reader that keeps only the last characters still gets the decode, GEMV and prefill figures
+    ns = {}
+    if "fp4_decode_step" in line:
+        ns["fp4_decode_tok_s"] = line["fp4_decode_step"]["tok_s"]
+    if "fp4_prefill" in line:
+        ns["fp4_prefill_frac"] = grid(line["fp4_prefill"], "frac_of_bf16_mfma_peak")
+    if "fp4_sweep" in line:
+        ns["fp4_b16_gemv_frac"] = grid(line["fp4_sweep"], extra=lambda r: r["block"] == 16)
+    if "sweep_variants" in line:
+        for route in ("e5m2_half", "e4m3_scaled", "e5m2_scaled"):
+            ns["gemv_frac_" + route] = grid(line["sweep_variants"], extra=lambda r, route=route: r["route"] == route)
+    if "sweep" in line:
+        ns["gemv_floor_us"] = {f"{r['K']}x{r['N']}": r["floor_us"] for r in line["sweep"] if r["M"] == 1}
+        ns["gemv_us"] = grid(line["sweep"], "us")
+    if "prefill" in line:
+        ns["prefill_frac_scaled"] = grid(line["prefill"], "scaled_frac_of_bf16_mfma_peak")
+        ns["prefill_frac"] = grid(line["prefill"], "frac_of_bf16_mfma_peak")
+    if "sweep" in line:
+        ns["gemv_frac"] = grid(line["sweep"])
+    if "quant_gemv" in line:
+        ns["gemv_chain_frac"] = line["quant_gemv"]["frac_of_hbm_peak"]
+        ns["gemv_chain_grouped_frac"] = line.get("quant_gemv_grouped", {}).get("frac_of_hbm_peak")
+    if "scaled_decode_step" in line:
+        ns["decode_ms_scaled_weights"] = line["scaled_decode_step"]["ms_per_step"]
+    ns.update({"decode_ms_exact_attention": line.get("ms_per_step_exact_attention"), "dominant_kernel_frac": line["roofline"]["frac"],
+               "decode_frac_of_hbm_bound": line.get("decode_step_frac_of_hbm_bound"), "decode_ms": line["ms_per_step"], "decode_tok_s": line["value"]})
+    return ns
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy", "prompt_attention"])
+    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy", "prompt_attention", "floor"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--weights", default="fp8", choices=["fp8", "fp4"], help="weight format of --workload gemv / prefill (fp4: E2M1 codes + E4M3 block scales)")
@@ -715,6 +852,7 @@ def main():
     ap.add_argument("--no-prompt", action="store_true", help="skip the prompt-phase (prefill) measurement of the decode model")
     ap.add_argument("--sweep-tokens", default="1,4,16", help="token counts of the per-shape GEMV sweep")
     ap.add_argument("--no-baselines", action="store_true", help="skip the same-GPU BF16 baselines of the decode step")
+    ap.add_argument("--no-scaled-step", action="store_true", help="skip the decode step on weights quantized on the device (per-tensor scales)")
     ap.add_argument("--no-repack", action="store_true", help="do not build the load-time tiled weight copies (tokens 3..16 then use the row-major kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -763,6 +901,25 @@ def main():
     ws.repack = not args.no_repack
     use_graph = not args.no_graph
     extra = {}
+    if args.workload == "floor":
+        # What a launch costs on this GPU when it only streams its bytes, for the byte counts of the GEMV sweeps (FP8 Qwen3-8B
+        # shapes, FP4 block-16 Llama-3.1-8B shapes), over rotating buffers of at least 512 MiB in total; and what a launch
+        # costs when it does nothing (dependent launches inside one hipGraph).
+        rows = []
+        sizes = [("fp8", K, N, K * N) for K, N in QWEN_SHAPES] + [("fp4_b16", K, N, K * N // 2 + K * N // 16) for K, N in LLAMA_SHAPES]
+        pool = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=ws.dev)
+        for fmt, K, N, nbytes in sizes:
+            span = (nbytes + 4095) // 4096 * 4096
+            n_buf = max(1, min(64, (1 << 30) // span))
+            ptrs = [pool.data_ptr() + i * span for i in range(n_buf)]
+            best = {w: round(min(ws.bench.floor_read_us(ptrs, nbytes, wgs_per_cu=w) for _ in range(2)), 2) for w in (2, 4, 8, 16)}
+            us = min(best.values())
+            rows.append({"weights": fmt, "K": K, "N": N, "bytes": nbytes, "floor_us": us, "GBps": round(nbytes / us * 1e-3, 1),
+                         "frac_of_hbm_peak": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4), "us_by_workgroups_per_cu": best})
+        print(json.dumps({"workload": "floor", "what": "streaming read of the sweep byte counts with 16-byte non-temporal loads, rotating buffers (1 GiB pool); "
+                                                       "empty and one-trip launches inside a hipGraph",
+                          "launch_us_empty": round(ws.bench.launch_us(0), 3), "launch_us_one_trip": round(ws.bench.launch_us(1), 3), "rows": rows}))
+        return
 
     metric, unit = "quant GEMV HBM GB/s (Qwen3-8B W8A16 decode linears, bs=1)", "GB/s"
     if args.workload == "decode_step":
@@ -790,6 +947,7 @@ def main():
         ms_step = ms / args.steps
         value = 1000.0 / ms_step
         extra["ms_per_step_exact_attention"] = round(ms_exact / args.steps, 4)
+        extra["launch_us"] = {"empty_in_graph": round(ws.bench.launch_us(0), 3), "one_trip_in_graph": round(ws.bench.launch_us(1), 3)}
         metric, unit = "decode tok/s Qwen3-8B W8A16 bs=1", "tok/s"
         step_bytes = decode_step_bytes(DECODE_CTX - (args.steps - 1) / 2.0)
         extra["launch_mode"] = "hipGraph" if use_graph else "stream"
@@ -800,11 +958,25 @@ def main():
         extra["launches_per_step"] = 6 * QWEN3_8B["layers"] + 2
         extra["last_token"] = model.token
         workload = ("full random-init Qwen3-8B W8A16 decode step, batch 1, greedy: 36 layers, hidden 4096, 32 q / 8 kv heads x 128, qk RMSNorm, "
-                    f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions")
+                    f"RoPE theta 1e6, SwiGLU 12288, vocab 151936, bf16 KV cache holding {DECODE_CTX} positions; FP8_E5M2 weights with scale 1; "
+                    "attention with FP32 softmax probabilities (ms_per_step_exact_attention: BF16 probabilities, the reference's rounding point)")
         # dominant kernel: the fused RMSNorm + gate/up SwiGLU launch (two 4096 x 12288 weights), timed over the 36 layers' distinct weights
         K, N, M = 4096, 2 * 12288, 1
         dom_us = ws.bench.gate_up_us(model, 10)
         dom_bytes = K * N + 2 * K + 2 * K + 2 * 12288
+        if not args.no_scaled_step:
+            # the same step on linears quantized on the device by Matrix::quantizeWeights (per-tensor scales absmax / 57344)
+            model_q = build_decode_step(ws, DECODE_CTX, quantize_on_device=True)
+            torch.cuda.synchronize()
+            model_q.reset(1, start)
+            if args.warmup:
+                model_q.run(args.warmup, use_graph)
+            ms_q = model_q.run(args.steps, use_graph) / args.steps
+            extra["scaled_decode_step"] = {"workload": "the same decode step with every linear quantized on the device by Matrix::quantizeWeights "
+                                                       "(FP8_E5M2, truncating encoder, per-tensor scale absmax / 57344): the reference's weight_data_type = fp8_e5m2 route",
+                                           "ms_per_step": round(ms_q, 4), "tok_s": round(1000.0 / ms_q, 1), "vs_scale_1": round(ms_q / ms_step, 4),
+                                           "example_scale": model_q.tensor_scale(0, "wq"), "last_token": model_q.token}
+            ws.keep.append(model_q)
         if not args.no_fp4_step:
             extra["fp4_decode_step"], fp4_model = llama_fp4_decode(ws, args.steps, args.warmup, use_graph, repack=not args.no_prompt)
         if not args.no_sweep:
@@ -817,6 +989,7 @@ def main():
             extra["quant_gemv"] = {"workload": "the 253 FP8_E5M2 linears of one decode token through Matrix::mulBatched", "ms_per_step": round(lin_ms, 4),
                                    "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
             extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
+            extra["sweep_variants"] = variant_sweep(ws, by_shape)
             extra["prefill"] = prefill_cases(ws, by_shape)
             gops = build_grouped_model(ws, 1)
             g_ms = time_chain(ws, gops, args.steps, args.warmup, use_graph) / args.steps
@@ -949,6 +1122,8 @@ def main():
         threads = min(16, len(os.sched_getaffinity(0)))
         line["cpu_baseline"] = cpu_baseline(pkg, threads, unit if args.workload != "prefill" else "GB/s")
     line.update(extra)
+    if args.workload == "decode_step":
+        line["north_star"] = north_star_summary(line)
     print(json.dumps(line))
 
 

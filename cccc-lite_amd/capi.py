@@ -78,6 +78,7 @@ EXPORTS = (
     "hip_argmax_pick_embed_bf16",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
+    "hip_quant_get_stream",
     "hip_quant_last_kernel",
 )
 
@@ -169,6 +170,8 @@ class QuantLibrary:
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32
         L.hip_quant_set_stream.argtypes = [vp]
+        L.hip_quant_get_stream.restype = vp
+        L.hip_quant_get_stream.argtypes = []
         L.hip_quant_last_kernel.restype = ctypes.c_char_p
         L.hip_quant_last_kernel.argtypes = []
         self.c = L
@@ -214,6 +217,9 @@ class QuantLibrary:
 
     def set_stream(self, stream_handle: int | None) -> int:
         return self.c.hip_quant_set_stream(stream_handle)
+
+    def get_stream(self) -> int:
+        return int(self.c.hip_quant_get_stream() or 0)
 
     def last_kernel(self) -> str:
         return (self.c.hip_quant_last_kernel() or b"").decode()

@@ -21,6 +21,7 @@
 // launch adds the residual and norms the row).
 #include "../../include/cccc_hip_quant.h"
 #include "gemv_kernels.h"
+#include "gemv_dispatch.h"
 #include "dispatch_half.h"
 #include "gemm_kernels.h"
 #include "runtime.h"
@@ -109,68 +110,6 @@ bool gemv8_dot2(const LinearArgs& a)
     case 4: return pick_gemv8_dot2<WT, 4, SCALED>(a);
     default: return false;
     }
-}
-
-template <int WT, bool SCALED>
-bool gemv8_mfma(const LinearArgs& a)
-{
-    const int cus = cu_count();
-    // row-major weight, 5..16 tokens: activations through LDS as on the tiled copy
-    if (a.n_out >= cus * 32) { gemv8_mfma_kernel<WT, 4, 2, 4, SCALED, false, true><<<(a.n_out + 63) / 64, 256, 0, stream()>>>(a); }
-    else { gemv8_mfma_kernel<WT, 1, 2, 8, SCALED, false, true><<<(a.n_out + 15) / 16, 512, 0, stream()>>>(a); }
-    return true;
-}
-
-// The same kernel on the load-time tiled copy: every load instruction of a wave covers one contiguous
-// KiB and a workgroup walks one contiguous row tile, which streams better than the row-major kernels
-// at every token count (lm_head, one token: 89.8 us against 92.7 for the dot2 kernel; 16 tokens:
-// 100 us against 125 for a variant that kept the activations in LDS).  Configurations tuned on
-// MI355X over the Qwen3-8B shapes with rotating weights.
-template <int WT, int RT, int U, int WAVES, bool SCALED, bool XLDS = false>
-void launch_ksplit_tiled(const LinearArgs& t)
-{
-    gemv8_mfma_kernel<WT, RT, U, WAVES, SCALED, true, XLDS><<<(t.n_out + 16 * RT - 1) / (16 * RT), WAVES * 64, 0, stream()>>>(t);
-}
-
-// From five tokens on the activation operand goes through LDS (XLDS, see the kernel): fetched in operand order it
-// costs 16 cache lines per 256 bytes, and at 16 tokens that, not HBM, bounds the kernel (K = 12288, 4096 rows:
-// 15.2 -> 13.3 us; K = 4096, 1024 rows: 6.4 -> 5.3 us).
-template <int WT, bool SCALED>
-bool gemv8_mfma_ksplit_tiled(const LinearArgs& a, const uint8_t* tiled)
-{
-    LinearArgs t = a;
-    t.W = tiled;
-    const int n_tiles = (a.n_out + 15) / 16;
-    const int tiles_per_cu = n_tiles / cu_count();
-    if (tiles_per_cu >= 16)
-    {
-        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 2, 2, 8, SCALED, true>(t); }
-        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED, true>(t); }
-    }
-    // projections stored together (gate + up: 24576 rows, q + k + v: 6144 rows), one or two tokens
-    else if (tiles_per_cu >= 4 && a.tokens <= 2) { launch_ksplit_tiled<WT, 2, 2, 16, SCALED>(t); }
-    else if (tiles_per_cu < 2 && a.K <= 8192 && a.tokens <= 2 && 2 * n_tiles >= 3 * cu_count()) { launch_ksplit_tiled<WT, 2, 4, 8, SCALED>(t); }
-    else if (tiles_per_cu >= 2)
-    {
-        if (a.tokens <= 2) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED>(t); }
-        else if (a.tokens <= 4) { launch_ksplit_tiled<WT, 2, 1, 8, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 1, 8, SCALED, true>(t); }
-        else { launch_ksplit_tiled<WT, 4, 2, 8, SCALED, true>(t); }
-    }
-    else if (a.K > 8192)
-    {
-        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 1, 4, 8, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED, true>(t); }
-        else { launch_ksplit_tiled<WT, 1, 4, 8, SCALED, true>(t); }
-    }
-    else
-    {
-        if (a.tokens <= 4) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED>(t); }
-        else if (a.tokens <= 8) { launch_ksplit_tiled<WT, 1, 2, 16, SCALED, true>(t); }
-        else { launch_ksplit_tiled<WT, 1, 4, 8, SCALED, true>(t); }
-    }
-    return true;
 }
 
 // ---- load-time repacked weights: caller's weight pointer -> tiled copy

@@ -1,5 +1,6 @@
 #include "dispatch_half.h"
 #include "gemm_kernels.h"
+#include "gemv_dispatch.h"
 #include "gemv_kernels.h"
 #include "runtime.h"
 
@@ -41,11 +42,28 @@ bool half_gemv(const LinearArgs& a)
     }
 }
 
+
+template <int WT>
+bool half_mfma_gemv(const LinearArgs& a, const uint8_t* tiled)
+{
+    const bool scaled = a.w_scale != 1.0f;
+    if (tiled) { return scaled ? gemv8_mfma_ksplit_tiled<WT, true, DT_HALF>(a, tiled) : gemv8_mfma_ksplit_tiled<WT, false, DT_HALF>(a, tiled); }
+    return scaled ? gemv8_mfma<WT, true, DT_HALF>(a) : gemv8_mfma<WT, false, DT_HALF>(a);
+}
+
 }    // namespace
 
+// Kernel choice as for BF16 activations (dispatch.hip): with a tiled copy the matrix-core GEMV on it for up to 16 tokens
+// (one or two tokens of a weight under 8 MiB stay on the dot2 kernel), else dot2 up to 4 tokens and the matrix-core GEMV
+// on the row-major bytes up to 16 (4096 x 12288 at 16 tokens: 16.3 us on the GEMM kernel this replaced there), the GEMM above.
 const char* half_linear(const LinearArgs& a, int w_type, SplitScratch* scratch)
 {
     const bool scaled = a.w_scale != 1.0f;
+    const uint8_t* tiled = lookup_tiled(a.W, w_type, a.n_out, a.K, a.ldw);
+    if (tiled && a.tokens <= 16 && (a.tokens >= 3 || (long long)a.n_out * a.K >= (8LL << 20)))
+    {
+        if (w_type == DT_E5M2 ? half_mfma_gemv<DT_E5M2>(a, tiled) : half_mfma_gemv<DT_E4M3>(a, tiled)) { return "gemv_mfma_tiled_half"; }
+    }
     if (a.tokens <= 4)
     {
         bool ok;
@@ -53,7 +71,10 @@ const char* half_linear(const LinearArgs& a, int w_type, SplitScratch* scratch)
         else { ok = scaled ? half_gemv<DT_E4M3, true>(a) : half_gemv<DT_E4M3, false>(a); }
         if (ok) { return "gemv_dot2_half"; }
     }
-    const uint8_t* tiled = lookup_tiled(a.W, w_type, a.n_out, a.K, a.ldw);
+    if (a.tokens <= 16)
+    {
+        if (w_type == DT_E5M2 ? half_mfma_gemv<DT_E5M2>(a, nullptr) : half_mfma_gemv<DT_E4M3>(a, nullptr)) { return "gemv_mfma_half"; }
+    }
     const bool launched = w_type == DT_E5M2 ? gemm_mfma<DT_E5M2, 0, DT_HALF>(a, tiled, scratch) : gemm_mfma<DT_E4M3, 0, DT_HALF>(a, tiled, scratch);
     return launched ? "gemm_mfma_half" : nullptr;
 }

@@ -529,7 +529,9 @@ namespace ccq
 // 8 (t / 8) + (p ^ (t % 8)) of a 256-byte row).  No workgroup barrier: a wave only reads what it wrote.
 __device__ __forceinline__ int xlds_slot(int t, int p) { return (t & 7) * 16 + ((t >> 3) * 8 + (p ^ (t & 7))); }
 
-template <int WT, int RT, int U, int WAVES, bool SCALED, bool TILED = false, bool XLDS = false>
+// AT: the 16-bit type of activations and outputs, DT_BF16 or DT_HALF (v_mfma_f32_16x16x32_f16; the weight entering a
+// product is then half(decode(w) * scale), cccc/cublas_real.h:921-938).
+template <int WT, int RT, int U, int WAVES, bool SCALED, bool TILED = false, bool XLDS = false, int AT = DT_BF16>
 __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs a)
 {
     __shared__ float partial[WAVES][RT][64][4];
@@ -628,12 +630,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs
 #pragma unroll
                 for (int h = 0; h < 2; h++)
                 {
-                    bf16x2 p0, p1, p2, p3;
-                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h], a.w_scale, p0, p1);
-                    fp8x4_to_bf16<WT, SCALED>(w[u][rt][2 * h + 1], a.w_scale, p2, p3);
-                    const bf16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
-                    const bf16x8 xb = __builtin_bit_cast(bf16x8, x[u][h]);
-                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb, acc[rt], 0, 0, 0);
+                    typename ActPair<AT>::type p0, p1, p2, p3;
+                    fp8x4_to_pairs<WT, SCALED, AT>(w[u][rt][2 * h], a.w_scale, p0, p1);
+                    fp8x4_to_pairs<WT, SCALED, AT>(w[u][rt][2 * h + 1], a.w_scale, p2, p3);
+                    if constexpr (AT == DT_HALF)
+                    {
+                        const f16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(f16x8, x[u][h]), acc[rt], 0, 0, 0);
+                    }
+                    else
+                    {
+                        const bf16x8 wa = { p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1] };
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, __builtin_bit_cast(bf16x8, x[u][h]), acc[rt], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -658,7 +667,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv8_mfma_kernel(const LinearArgs
         if (token < a.tokens && row < a.n_out)
         {
             uint16_t* y = a.Y + (long long)token * a.y_stride_tok + (long long)row * a.y_stride_out;
-            *y = finish_output(total, a.alpha, a.beta, y);
+            *y = finish_output_act<AT>(total, a.alpha, a.beta, y);
         }
     }
 }

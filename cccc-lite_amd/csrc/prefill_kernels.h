@@ -78,13 +78,15 @@ constexpr float PF_LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Two FP32 values rounded to BF16 (nearest even) into one dword, low half first.  Spelled as the instruction because the
-// compiler, seeing the halves used separately afterwards, converts each value with an instruction of its own.  Only for
-// results that VALU code consumes: fed straight into a matrix-core instruction the value arrived stale in some lanes (NaN
-// rows) -- the compiler keeps the wait states between a VALU write and a matrix-core read only for instructions it knows.
+// compiler, seeing the halves used separately afterwards, converts each value with an instruction of its own.  The compiler
+// keeps the wait states between a VALU write and a matrix-core read only for instructions it emits itself: a result of
+// this block consumed by the very next matrix-core instruction arrived stale in some lanes (NaN rows).  The block
+// therefore carries its own wait states behind the conversion, so that the result is safe for whichever instruction
+// follows; the callers here hand it to VALU code, and matrix-core operands are still built with (__bf16) casts.
 __device__ __forceinline__ uint32_t pf_pack_bf16(float lo, float hi)
 {
     uint32_t r;
-    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(lo), "v"(hi));
     return r;
 }
 

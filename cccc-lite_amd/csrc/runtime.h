@@ -19,8 +19,8 @@ int finish(const char* what);
 int cu_count();
 
 // Device scratch memory of at least `bytes` for the launches about to be enqueued on `stream()`: one
-// grow-only buffer per (device, stream), kept until the process ends, so kernels enqueued on one stream
-// reuse it in order.  Returns nullptr when it cannot be provided (allocation failure, or the buffer would
+// grow-only buffer per (host thread, device, stream), kept until the process ends, so kernels this thread
+// enqueues on one stream reuse it in order and no other thread can replace it under them.  Returns nullptr when it cannot be provided (allocation failure, or the buffer would
 // have to grow while the stream is being captured into a graph); callers then take a path that needs none.
 void* workspace(size_t bytes);
 

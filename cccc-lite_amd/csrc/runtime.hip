@@ -3,7 +3,6 @@
 #include <atomic>
 #include <cstdio>
 #include <map>
-#include <mutex>
 #include <utility>
 
 namespace ccq
@@ -47,14 +46,16 @@ int cu_count()
     return n;
 }
 
+// One grow-only buffer per (host thread, device, stream).  A buffer is only ever replaced by the thread that uses it,
+// after that thread has waited for the stream, so the pointer handed out stays valid until the same thread asks again:
+// no other thread can free it between this call and the launch that follows.  Two host threads that enqueue on one
+// stream each get a buffer of their own.
 void* workspace(size_t bytes)
 {
     struct Buffer { void* ptr; size_t bytes; };
-    static std::mutex mutex;
-    static std::map<std::pair<int, hipStream_t>, Buffer> buffers;
+    static thread_local std::map<std::pair<int, hipStream_t>, Buffer> buffers;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { return nullptr; }
-    std::lock_guard<std::mutex> lock(mutex);
     Buffer& b = buffers[{ dev, stream() }];
     if (b.bytes >= bytes) { return b.ptr; }
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -63,7 +64,7 @@ void* workspace(size_t bytes)
         (void)hipGetLastError();
         return nullptr;
     }
-    // work already enqueued on the stream may still be using the old buffer
+    // this thread's earlier launches on the stream may still be using the old buffer
     if (b.ptr && (hipStreamSynchronize(stream()) != hipSuccess || hipFree(b.ptr) != hipSuccess)) { (void)hipGetLastError(); }
     b = Buffer{ nullptr, 0 };
     const size_t want = bytes + bytes / 4;
@@ -91,5 +92,7 @@ int hip_quant_set_stream(void* s)
     ccq::g_stream = (hipStream_t)s;
     return 0;
 }
+
+void* hip_quant_get_stream(void) { return (void*)ccq::g_stream; }
 
 const char* hip_quant_last_kernel(void) { return ccq::g_last_kernel; }

@@ -128,6 +128,23 @@ int DecodeModel::setTensor(int layer, int which, const void* host, size_t bytes,
     return m->copyFromHost(host, bytes);
 }
 
+int DecodeModel::quantizeLinear(int layer, int which, const void* device_bf16, DataType to)
+{
+    const bool linear = which == WQ || which == WK || which == WV || which == WO || which == W_GATE || which == W_UP || which == W_DOWN ||
+                        (which == LM_HEAD && !tied_lm_head_);
+    Matrix* m = tensor(layer, which);
+    if (!m || !linear || !device_bf16 || !Rocblas::isQuantized(to)) { return -1; }
+    gpu_->setAsCurrent();
+    Matrix tmp(m->getWidth(), m->getHeight(), 1, 1, BFLOAT16, gpu_);
+    // only a tall FP8 weight (lm_head) is read through its tiled copy by the fused decode kernels
+    tmp.setAllowRepack(repack_linears_ || (which == LM_HEAD && to != FP4_E2M1));
+    if (GpuControl::copyDeviceToDevice(tmp.data(), device_bf16, (size_t)tmp.getDataSize() * 2) != 0) { return 1; }
+    tmp.quantizeWeights(to);
+    if (!Rocblas::isQuantized(tmp.getDataType())) { return -3; }
+    *m = tmp;
+    return 0;
+}
+
 int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, std::string* failed)
 {
     gpu_->setAsCurrent();
@@ -203,8 +220,6 @@ int DecodeModel::loadNamedWeights(const WeightFile& file, DataType quantize_to, 
             if (rc == 0 && (qk_norm_ || !head_norm)) { rc = load_plain(*m, prefix + n); }
         }
         for (auto& [m, prefix] : linear) { if (rc == 0) { rc = load_linear(*m, prefix + n); } }
-        // gate and up are decoded by one launch with one format
-        if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType()) { rc = fail("W_up_" + n, -3); }
     }
     return rc;
 }
@@ -354,8 +369,22 @@ int DecodeModel::step()
             rc = hip_quant_linear_fused(&o);
         }
         // 5. gated = silu(W_gate n) * (W_up n), n = rmsnorm(r1)
-        if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType()) { rc = -1; }    // the SwiGLU pair kernel decodes both with one format
-        if (rc == 0)
+        if (rc == 0 && L.w_up->getDataType() != L.w_gate->getDataType())
+        {
+            // the SwiGLU pair kernel decodes both weights with one format: two formats go out as two linears (each with the
+            // norm in front) and the product as a launch of its own, with the same roundings
+            if (!gate_) { gate_ = make(c.inter, 1, BFLOAT16, gpu_); up_ = make(c.inter, 1, BFLOAT16, gpu_); }
+            for (Matrix* w : { L.w_gate.get(), L.w_up.get() })
+            {
+                if (rc != 0) { break; }
+                hip_fused_linear one = linear_desc(*w, c.inter, c.hidden, r1_->data(), w == L.w_gate.get() ? gate_->data() : up_->data());
+                one.norm_weight = L.rms_ffn->data();
+                one.norm_eps = c.eps;
+                rc = hip_quant_linear_fused(&one);
+            }
+            if (rc == 0) { rc = hip_swiglu_bf16(gate_->data(), up_->data(), gated_->data(), (unsigned long long)c.inter); }
+        }
+        else if (rc == 0)
         {
             hip_fused_linear gu = linear_desc(*L.w_gate, c.inter, c.hidden, r1_->data(), gated_->data());
             gu.n_segments = 2;
@@ -421,6 +450,10 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
         for (auto* m : { &pf_.k, &pf_.v }) { *m = make(kv_out, n, BFLOAT16, gpu_); }
         for (auto* m : { &pf_.gate, &pf_.up, &pf_.gated }) { *m = make(c.inter, n, BFLOAT16, gpu_); }
     }
+    // Every kernel of the piece goes to the library's stream of this thread.  The host copies below are the mirror's blocking
+    // copies, which wait for that stream first (GpuControl::copyHostToDevice): nothing an earlier launch still reads
+    // (pf_.ids, the step state) is overwritten under it, and a copy has landed before anything is launched behind it.
+    const hipStream_t stream = (hipStream_t)hip_quant_get_stream();
     std::vector<float> ids(tokens, tokens + n);
     if (GpuControl::copyHostToDevice(pf_.ids->data(), ids.data(), (size_t)n * sizeof(float)) != 0) { return 1; }
     int rc = hip_embed_fwd((int)BFLOAT16, pf_.ids->data(), emb_->data(), pf_.x->data(), c.hidden, n, 1);
@@ -511,8 +544,9 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
     }
     if (rc != 0 || !last) { return rc; }
     // the head runs on the last token's state: its greedy pick becomes the current token at position pos0 + n
+    // (the row copy rides on the launch stream behind the last layer)
     const int state[2] = { tokens[n - 1], pos0 + n - 1 };
-    if (hipMemcpyAsync(x_->data(), (const char*)pf_.x->data() + (size_t)(n - 1) * c.hidden * 2, (size_t)c.hidden * 2, hipMemcpyDeviceToDevice, nullptr) != hipSuccess) { return 1; }
+    if (hipMemcpyAsync(x_->data(), (const char*)pf_.x->data() + (size_t)(n - 1) * c.hidden * 2, (size_t)c.hidden * 2, hipMemcpyDeviceToDevice, stream) != hipSuccess) { return 1; }
     if (GpuControl::copyHostToDevice(d_state_, state, sizeof(state)) != 0) { return 1; }
     return head();
 }

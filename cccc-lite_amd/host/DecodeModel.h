@@ -47,14 +47,22 @@ public:
     // FP4 linears: the E4M3 block scales that go with the packed codes (one byte per 16 elements).
     int setBlockScales(int layer, int which, const void* host, size_t n_scales);
 
+    // Quantizes one linear on the device from BF16 values already there ([n_out][K], the tensor's shape): the reference's
+    // on-the-fly route for a model stored unquantized (Net::quantizeWeights -> Matrix::quantizeWeights,
+    // cccc/Net.cpp:1142-1233, cccc/Matrix.cpp:301-355) -- FP8 with the per-tensor scale absmax / max_code and truncating
+    // encoders, FP4 with per-block E4M3 scales.  0 ok, -1 not a linear of this model / not a quantized type, -3 the
+    // tensor is too small to quantize (a side under 64).
+    int quantizeLinear(int layer, int which, const void* device_bf16, DataType to);
+
     // Loads every tensor from a converted model file by the converter's names (scripts/convert_weights.py:142-166):
     // W_emb, W_rms_final, W_lm_head (absent: tied embeddings, the head then reads W_emb in BF16), W_rms_attn_<i>, W_q_<i>, W_k_<i>, W_v_<i>, W_o_<i>,
     // W_qnorm_<i>, W_knorm_<i> (a file without them loads as a model without per-head norms), W_rms_ffn_<i>, W_gate_<i>,
     // W_up_<i>, W_down_<i>.  FP8 and FP4 linears are taken as stored;
     // linears stored as BF16 / HALF / FLOAT are quantized on load to `quantize_to` with a per-tensor absmax scale
     // (the reference's weight_data_type route, cccc/Matrix.cpp:301-355).  0 ok; otherwise `failed` names the tensor:
-    // -1 missing, -2 wrong size, -3 something the fused decode kernels do not take (FP4 without block scales, gate and
-    // up in two formats, a tensor too small to quantize).  FP4_E2M1 linears load with their blockscale_<name> entries.
+    // -1 missing, -2 wrong size, -3 something the fused decode kernels do not take (FP4 without block scales, a tensor too
+    // small to quantize).  Every tensor keeps the format the file gives it (cccc/Net.cpp:1444-1481 resolves each by
+    // itself): projections that share a launch but not a format (q, k, v; gate, up) go out as separate launches.  FP4_E2M1 linears load with their blockscale_<name> entries.
     int loadNamedWeights(const WeightFile& file, DataType quantize_to = FP8_E5M2, std::string* failed = nullptr);
 
     // Writes every tensor under the same names, as Net::saveNamedWeights does (cccc/Net.cpp:1235-1314): the header
@@ -112,6 +120,7 @@ private:
     std::unique_ptr<Matrix> emb_, rms_final_, lm_head_, logits_, cos_, sin_;
     std::vector<std::unique_ptr<Matrix>> k_cache_, v_cache_;
     std::unique_ptr<Matrix> x_, r1_, q_, k_, v_, att_, gated_, attn_ws_, argmax_ws_;
+    std::unique_ptr<Matrix> gate_, up_;     // only for a layer whose gate and up weights differ in format (allocated on first use)
     // activations of a prompt piece, grown on demand: [tokens][features] BF16, and the token ids as floats (hip_embed_fwd's input)
     struct PromptBuffers
     {

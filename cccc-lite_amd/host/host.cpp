@@ -84,9 +84,28 @@ size_t GpuControl::allocatedBytes() const
     return total;
 }
 
-int GpuControl::copyHostToDevice(void* dst, const void* src, size_t bytes) { return hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) == hipSuccess ? 0 : 1; }
-int GpuControl::copyDeviceToHost(void* dst, const void* src, size_t bytes) { return hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) == hipSuccess ? 0 : 1; }
-int GpuControl::copyDeviceToDevice(void* dst, const void* src, size_t bytes) { return hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice) == hipSuccess ? 0 : 1; }
+// The reference reads and writes device memory with blocking copies behind kernels on the null stream
+// (cccc/MatrixData.cpp:155-165).  Here the kernels of a host thread may run on a stream of its own
+// (hip_quant_set_stream), possibly one the null stream does not order with, so every blocking copy of the mirror first
+// waits for that stream: the copy then sees what the launches before it wrote, and overwrites nothing they still read.
+static bool drain_launch_stream()
+{
+    hipStream_t s = (hipStream_t)hip_quant_get_stream();
+    return s == nullptr || hipStreamSynchronize(s) == hipSuccess;
+}
+
+int GpuControl::copyHostToDevice(void* dst, const void* src, size_t bytes)
+{
+    return drain_launch_stream() && hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) == hipSuccess ? 0 : 1;
+}
+int GpuControl::copyDeviceToHost(void* dst, const void* src, size_t bytes)
+{
+    return drain_launch_stream() && hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) == hipSuccess ? 0 : 1;
+}
+int GpuControl::copyDeviceToDevice(void* dst, const void* src, size_t bytes)
+{
+    return drain_launch_stream() && hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice) == hipSuccess ? 0 : 1;
+}
 
 // ------------------------------------------------------------------ Rocblas
 

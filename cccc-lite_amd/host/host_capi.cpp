@@ -61,6 +61,8 @@ int cccc_matrix_dtype(void* m) { return (int)((Matrix*)m)->getDataType(); }
 
 float cccc_matrix_quant_scale(void* m) { return ((Matrix*)m)->getQuantScale(); }
 
+void cccc_matrix_set_quant_scale(void* m, float scale) { ((Matrix*)m)->setQuantScale(scale); }
+
 const void* cccc_matrix_block_scale_data(void* m) { return ((Matrix*)m)->getBlockScaleData(); }
 
 long long cccc_matrix_get_block_scale(void* m, void* host, long long capacity)
@@ -184,6 +186,17 @@ void* cccc_decode_tensor_data(void* m, int layer, int which)
 {
     Matrix* t = ((DecodeModel*)m)->tensor(layer, which);
     return t ? t->data() : nullptr;
+}
+
+int cccc_decode_quantize_linear(void* m, int layer, int which, const void* device_bf16, int to)
+{
+    return ((DecodeModel*)m)->quantizeLinear(layer, which, device_bf16, (DataType)to);
+}
+
+float cccc_decode_tensor_scale(void* m, int layer, int which)
+{
+    Matrix* t = ((DecodeModel*)m)->tensor(layer, which);
+    return t ? t->getQuantScale() : 0.0f;
 }
 
 int cccc_decode_tensor_prepare(void* m, int layer, int which)

@@ -32,6 +32,7 @@ class HostLibrary:
         L.cccc_matrix_prepare_tiled.restype = i32; L.cccc_matrix_prepare_tiled.argtypes = [vp]
         L.cccc_matrix_dtype.restype = i32; L.cccc_matrix_dtype.argtypes = [vp]
         L.cccc_matrix_quant_scale.restype = f32; L.cccc_matrix_quant_scale.argtypes = [vp]
+        L.cccc_matrix_set_quant_scale.restype = None; L.cccc_matrix_set_quant_scale.argtypes = [vp, f32]
         L.cccc_matrix_block_scale_data.restype = vp; L.cccc_matrix_block_scale_data.argtypes = [vp]
         L.cccc_matrix_get_block_scale.restype = i64; L.cccc_matrix_get_block_scale.argtypes = [vp, vp, i64]
         L.cccc_matrix_mul.restype = i32; L.cccc_matrix_mul.argtypes = [vp, vp, vp, f32, f32, i32, i32]
@@ -75,6 +76,8 @@ class HostLibrary:
         L.cccc_decode_set_tied_lm_head.restype = None; L.cccc_decode_set_tied_lm_head.argtypes = [vp, i32]
         L.cccc_decode_tied_lm_head.restype = i32; L.cccc_decode_tied_lm_head.argtypes = [vp]
         L.cccc_decode_tensor_prepare.restype = i32; L.cccc_decode_tensor_prepare.argtypes = [vp, i32, i32]
+        L.cccc_decode_quantize_linear.restype = i32; L.cccc_decode_quantize_linear.argtypes = [vp, i32, i32, vp, i32]
+        L.cccc_decode_tensor_scale.restype = f32; L.cccc_decode_tensor_scale.argtypes = [vp, i32, i32]
         L.cccc_decode_kv_data.restype = vp; L.cccc_decode_kv_data.argtypes = [vp, i32, i32]
         self.c = L
 
@@ -153,6 +156,11 @@ class HostMatrix:
     @property
     def quant_scale(self) -> float:
         return self.lib.c.cccc_matrix_quant_scale(self.handle)
+
+    @quant_scale.setter
+    def quant_scale(self, scale: float) -> None:
+        """Matrix::setQuantScale: the per-tensor dequantisation multiplier that goes with the codes already in the storage."""
+        self.lib.c.cccc_matrix_set_quant_scale(self.handle, scale)
 
     @property
     def block_scale_ptr(self):
@@ -261,6 +269,16 @@ class DecodeModel:
         """Builds the tiled copy of a linear whose bytes were written through tensor_ptr (set_tensor and
         load_named do this themselves)."""
         return self.lib.c.cccc_decode_tensor_prepare(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))) == 0
+
+    def quantize_linear(self, layer: int, name: str, device_bf16_ptr: int, to: int = 5) -> None:
+        """Quantizes a linear on the device from BF16 values ([n_out][K]) already in device memory (DecodeModel::quantizeLinear:
+        per-tensor absmax scale for FP8, block scales for FP4)."""
+        rc = self.lib.c.cccc_decode_quantize_linear(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name)), device_bf16_ptr, to)
+        if rc != 0:
+            raise ValueError(f"quantize_linear({layer}, {name}) failed: {rc}")
+
+    def tensor_scale(self, layer: int, name: str) -> float:
+        return float(self.lib.c.cccc_decode_tensor_scale(self.handle, layer, LAYER_TENSORS.get(name, GLOBAL_TENSORS.get(name))))
 
     def load(self, model: dict, fp8_dtype: int = 5) -> None:
         """model: the dict layout of oracle.decode_oracle.make_model (uint8 codes / uint16 bf16 bits); a quantized

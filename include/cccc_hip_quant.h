@@ -339,9 +339,12 @@ C_EXPORT int hip_argmax_pick_embed_bf16(const void* workspace, unsigned int n, v
  *   hip_quant_set_sync(1)   : hipDeviceSynchronize + error check after every launch of this thread
  *                             (parity/debug); returns the previous setting
  *   hip_quant_set_stream(s) : this thread's launches go to hipStream_t `s` (NULL = null stream)
+ *   hip_quant_get_stream()  : the hipStream_t this thread's launches currently go to (NULL = null stream), for a
+ *                             caller that has copies of its own to order with them
  *   hip_quant_last_kernel() : name of the kernel family the last hip_quant_gemm call dispatched to
  *                             ("gemv_dot2", "gemv_mfma", "gemm_mfma", "generic", ...)
  */
 C_EXPORT int hip_quant_set_sync(int enabled);
 C_EXPORT int hip_quant_set_stream(void* stream);
+C_EXPORT void* hip_quant_get_stream(void);
 C_EXPORT const char* hip_quant_last_kernel(void);

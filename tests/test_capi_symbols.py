@@ -53,6 +53,8 @@ def test_argument_checks_need_no_gpu(pkg):
     assert lib.quant_gemm(1, 3, 16, 1, 16, 1.0, p, D.FP8_E5M2, 16, 1.0, p, D.BFLOAT16, 16, 1.0, 0.0, p, D.BFLOAT16, 16) == -1
     assert lib.quant_gemm(1, 0, 16, 1, 16, 1.0, None, D.FP8_E5M2, 16, 1.0, p, D.BFLOAT16, 16, 1.0, 0.0, p, D.BFLOAT16, 16) == -1
     assert lib.quant_gemm(1, 0, 0, 1, 16, 1.0, p, D.FP8_E5M2, 16, 1.0, p, D.BFLOAT16, 16, 1.0, 0.0, p, D.BFLOAT16, 16) == 0
-    assert lib.set_sync(True) == 0 and lib.set_sync(False) == 1 and lib.set_sync(False) == 0      # returns the previous setting
-    assert lib.set_stream(None) == 0
+    before = lib.set_sync(True)                                          # returns the previous setting
+    assert before in (0, 1) and lib.set_sync(False) == 1 and lib.set_sync(False) == 0
+    lib.set_sync(bool(before))
+    assert lib.set_stream(None) == 0 and lib.get_stream() == 0
     assert not buf.any()

@@ -32,7 +32,8 @@ def check_half(got_bits, exact, alpha=1.0, extra=None, label=""):
 
 
 @pytest.mark.parametrize("w_type", [E5M2, E4M3])
-@pytest.mark.parametrize("tokens,kernel", [(1, "gemv_dot2_half"), (3, "gemv_dot2_half"), (4, "gemv_dot2_half"), (7, "gemm_mfma_half"), (40, "gemm_mfma_half"), (200, "gemm_mfma_half")])
+@pytest.mark.parametrize("tokens,kernel", [(1, "gemv_dot2_half"), (3, "gemv_dot2_half"), (4, "gemv_dot2_half"), (7, "gemv_mfma_half"), (16, "gemv_mfma_half"),
+                                           (17, "gemm_mfma_half"), (40, "gemm_mfma_half"), (200, "gemm_mfma_half")])
 @pytest.mark.parametrize("scale", [1.0, 0.37])
 def test_half_activations(gpu, oracle, w_type, tokens, kernel, scale):
     torch, dev, lib = gpu
@@ -74,6 +75,32 @@ def test_half_gemm_with_weights_kept_out_of_lds(gpu, oracle, w_type, tokens):
         outs.append(out[:tokens * n_out].reshape(tokens, n_out))
         check_half(outs[-1], exact, label=f"{w_type} {tokens} tiled={tiled}")
     assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("w_type", [E5M2, E4M3])
+@pytest.mark.parametrize("n_out,K", [(328, 1024), (4200, 2112), (1040, 8448)])
+def test_half_matrix_core_gemv_on_the_tiled_copy(gpu, oracle, w_type, n_out, K):
+    """1..16 tokens of HALF activations on a weight with a registered tiled copy: the matrix-core GEMV reads the copy (from
+    three tokens on for a weight this small), with and without a per-tensor scale, alpha / beta included; every
+    configuration of its launch table that these shapes reach (few / many row tiles, short / long rows)."""
+    torch, dev, lib = gpu
+    rng = np.random.default_rng(n_out + w_type)
+    for tokens, scale, alpha, beta in ((3, 1.0, 1.0, 0.0), (4, 0.37, 1.0, 0.0), (8, 0.37, 0.5, -2.0), (16, 1.0, 1.0, 0.0), (13, 0.37, 1.0, 0.0)):
+        codes, x, exact = make_case(oracle, rng, w_type, n_out, K, tokens, scale)
+        c0 = rng.standard_normal((tokens, n_out)).astype(np.float16)
+        wd, xd = to_dev(torch, dev, codes), to_dev(torch, dev, x.view(np.uint16))
+        td = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
+        assert lib.weight_prepare(wd.data_ptr(), w_type, n_out, K, K, td.data_ptr()) == 0
+        try:
+            y = to_dev(torch, dev, np.concatenate([c0.view(np.uint16).ravel(), np.zeros(16, dtype=np.uint16)]))
+            assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), y.data_ptr(), n_out, tokens, K, inv_scale=scale, alpha=alpha, beta=beta, act_type=HALF) == 0
+            assert lib.last_kernel() == "gemv_mfma_tiled_half"
+        finally:
+            assert lib.weight_release(wd.data_ptr()) == 0
+        out = from_dev(y, np.uint16)
+        assert not out[tokens * n_out:].any()
+        check_half(out[:tokens * n_out].reshape(tokens, n_out), exact, alpha=alpha, extra=beta * c0.astype(np.float64) if beta else None,
+                   label=f"{w_type} {n_out}x{K} {tokens} tokens")
 
 
 def test_half_alpha_beta_tall_and_generic(gpu, oracle):

@@ -492,3 +492,43 @@ def test_prompt_in_pieces_and_bad_arguments(gpu, pkg, oracle, dec):
         a.prefill([3, cfg.vocab, 4])
     with pytest.raises(RuntimeError):
         a.prefill([1, 2], pos0=63)
+
+
+def test_prompt_and_steps_on_a_non_blocking_stream(gpu, pkg, oracle, dec):
+    """The prompt phase and the decode steps behind it with the library's launches on a stream created with
+    hipStreamNonBlocking (which the null stream's blocking copies do not order with) and no device synchronisation after the
+    launches: cache rows, logits and tokens equal those of the same model driven on the null stream.  A prompt in two pieces
+    and a reset between steps go through the host copies (token ids, step state, last row) that must be ordered with the
+    launches by the model itself."""
+    torch, dev, lib = gpu
+    host = pkg.host_api.host()
+    host.init(0)
+    cfg = dec.DecodeConfig(layers=2, hidden=256, n_q=4, n_kv=2, inter=512, vocab=1000, t_kv=96)
+    weights = dec.make_model(cfg, 71)
+    prompt = [int(t) for t in np.random.default_rng(9).integers(0, cfg.vocab, size=70)]
+
+    def drive(model):
+        model.load(weights)
+        out = [model.prefill(prompt[:40]), model.prefill(prompt[40:], pos0=40)]
+        for _ in range(3):
+            out.append(model.step())
+        model.reset(out[-1], model.pos)
+        out.append(model.step())
+        return out, model.logits().copy(), [model.kv(li, v).copy() for li in range(cfg.layers) for v in (False, True)]
+
+    want = drive(_fresh(pkg, host, cfg))
+    stream = torch.cuda.Stream(device=dev)                     # torch creates its streams non-blocking
+    lib.set_sync(False)
+    try:
+        assert lib.set_stream(stream.cuda_stream) == 0
+        assert lib.get_stream() == stream.cuda_stream
+        got = drive(_fresh(pkg, host, cfg))
+        stream.synchronize()
+    finally:
+        lib.set_stream(None)
+        lib.set_sync(True)
+    assert lib.get_stream() == 0
+    assert got[0] == want[0]
+    assert np.array_equal(got[1], want[1])
+    for a, b in zip(got[2], want[2]):
+        assert np.array_equal(a[:, :75], b[:, :75])
