@@ -572,7 +572,7 @@ def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
     out = []
     for (K, N) in QWEN_SHAPES:
         weights = by_shape[(K, N)]
-        floor_us = ws.bench.floor_read_us([W.data_ptr for W in weights], K * N)
+        floor_us = min(ws.bench.floor_read_us([W.data_ptr for W in weights], K * N, wgs_per_cu=w) for w in (2, 8))
         for M in token_counts:
             X, Y = ws.activation(M, K), ws.output(M, N)
             reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
@@ -581,7 +581,8 @@ def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
             us = ms * 1000.0 / (3 * len(ops))
             gbs = gemv_bytes(K, N, M) / us * 1e-3
             assert ws.lib.linear(weights[0].data_ptr, E5M2, X.data_ptr, Y.data_ptr, N, M, K) == 0
-            row = {"K": K, "N": N, "M": M, "us": round(us, 2), "floor_us": round(floor_us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+            row = {"K": K, "N": N, "M": M, "us": round(us, 2), "floor_us": round(floor_us, 2), "floor_over_us": round(floor_us / us, 3),
+                   "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "launch_mode": "hipGraph" if use_graph else "stream",
                    "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(K * N * len(weights) / 2 ** 20)}
             if M == 1 and comparators:
                 row.update(same_gpu_comparators(ws, weights, K, N, M))
@@ -592,7 +593,7 @@ def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
 SCALED_INV_SCALE = 0.1 / 57344.0       # absmax / max_code of a weight whose largest element is 0.1 (cccc/Matrix.cpp:338-352)
 
 
-def variant_sweep(ws, by_shape, token_counts=(1, 16)):
+def variant_sweep(ws, by_shape, token_counts=(1, 16), use_graph=False):
     """The routes of the same GEMV that a model quantized by the reference takes instead of `sweep`'s (scale 1, E5M2, BF16):
     "e5m2_scaled" -- the same E5M2 weights with a per-tensor dequantisation multiplier other than 1 (every weight
     Matrix::quantizeWeights produces carries absmax / 57344, cccc/Matrix.cpp:338-352): the kernels then decode to FP32,
@@ -613,7 +614,7 @@ def variant_sweep(ws, by_shape, token_counts=(1, 16)):
                 X, Y = ws.activation(M, K, act), ws.output(M, N, act)
                 reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
                 ops = [(W, X, Y, K, N) for W in weights] * reps
-                ms = time_chain(ws, ops, 3, 1, False)
+                ms = time_chain(ws, ops, 3, 1, use_graph)
                 us = ms * 1000.0 / (3 * len(ops))
                 gbs = gemv_bytes(K, N, M) / us * 1e-3
                 assert ws.lib.linear(weights[0].data_ptr, weights[0].dtype, X.data_ptr, Y.data_ptr, N, M, K, inv_scale=weights[0].quant_scale, act_type=act) == 0
@@ -818,7 +819,7 @@ def north_star_summary(line):
         for route in ("e5m2_half", "e4m3_scaled", "e5m2_scaled"):
             ns["gemv_frac_" + route] = grid(line["sweep_variants"], extra=lambda r, route=route: r["route"] == route)
     if "sweep" in line:
-        ns["gemv_floor_us"] = {f"{r['K']}x{r['N']}": r["floor_us"] for r in line["sweep"] if r["M"] == 1}
+        ns["gemv_floor_us"] = {f"{r['K']}x{r['N']}": r["floor_us"] for r in line["sweep"] if r["M"] == line["sweep"][0]["M"]}
         ns["gemv_us"] = grid(line["sweep"], "us")
     if "prefill" in line:
         ns["prefill_frac_scaled"] = grid(line["prefill"], "scaled_frac_of_bf16_mfma_peak")
@@ -988,8 +989,8 @@ def main():
             lin_ms = time_chain(ws, ops, args.steps, args.warmup, use_graph) / args.steps
             extra["quant_gemv"] = {"workload": "the 253 FP8_E5M2 linears of one decode token through Matrix::mulBatched", "ms_per_step": round(lin_ms, 4),
                                    "GBps": round(lin_bytes / lin_ms * 1e-6, 1), "frac_of_hbm_peak": round(lin_bytes / lin_ms * 1e-6 / HBM_PEAK_GBS, 4)}
-            extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), False)
-            extra["sweep_variants"] = variant_sweep(ws, by_shape)
+            extra["sweep"] = shape_sweep(ws, by_shape, tuple(int(v) for v in args.sweep_tokens.split(",")), use_graph)
+            extra["sweep_variants"] = variant_sweep(ws, by_shape, use_graph=use_graph)
             extra["prefill"] = prefill_cases(ws, by_shape)
             gops = build_grouped_model(ws, 1)
             g_ms = time_chain(ws, gops, args.steps, args.warmup, use_graph) / args.steps

@@ -76,6 +76,7 @@ EXPORTS = (
     "hip_argmax_workspace_bytes",
     "hip_argmax_bf16",
     "hip_argmax_pick_embed_bf16",
+    "hip_quant_workspace_reserve",
     "hip_quant_set_sync",
     "hip_quant_set_stream",
     "hip_quant_get_stream",
@@ -170,6 +171,8 @@ class QuantLibrary:
         L.hip_quant_set_sync.argtypes = [i32]
         L.hip_quant_set_stream.restype = i32
         L.hip_quant_set_stream.argtypes = [vp]
+        L.hip_quant_workspace_reserve.restype = i32
+        L.hip_quant_workspace_reserve.argtypes = [ctypes.c_ulonglong]
         L.hip_quant_get_stream.restype = vp
         L.hip_quant_get_stream.argtypes = []
         L.hip_quant_last_kernel.restype = ctypes.c_char_p
@@ -217,6 +220,9 @@ class QuantLibrary:
 
     def set_stream(self, stream_handle: int | None) -> int:
         return self.c.hip_quant_set_stream(stream_handle)
+
+    def workspace_reserve(self, nbytes: int) -> int:
+        return self.c.hip_quant_workspace_reserve(nbytes)
 
     def get_stream(self) -> int:
         return int(self.c.hip_quant_get_stream() or 0)

@@ -33,6 +33,8 @@ int hip_attention_prefill_bf16(const void* q, const void* k_cache, const void* v
     if (pos0 < 0 || (long long)pos0 + n_tokens > t_kv || n_kv_heads > 65535) { return -1; }
     if (!q || !k_cache || !v_cache || !y || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) { return -1; }
     if ((long long)((n_tokens + 15) / 16) * n_kv_heads > 0x7FFFFFFFLL) { return -1; }
+    // the kernel addresses cache rows with 32-bit byte offsets inside a KV head (row * 256)
+    if ((long long)pos0 + n_tokens > (1LL << 24)) { return -1; }
     const dim3 grid((unsigned)((n_tokens + 15) / 16) * n_kv_heads);
     const float scale = 1.0f / sqrtf(128.0f);
 #define CCQ_ATTN_PREFILL(G)                                                                                                                  \

@@ -93,6 +93,18 @@ int hip_quant_set_stream(void* s)
     return 0;
 }
 
+int hip_quant_workspace_reserve(unsigned long long bytes)
+{
+    if (bytes == 0) { return 0; }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ccq::stream(), &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+    {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return ccq::workspace((size_t)bytes) ? 0 : 1;
+}
+
 void* hip_quant_get_stream(void) { return (void*)ccq::g_stream; }
 
 const char* hip_quant_last_kernel(void) { return ccq::g_last_kernel; }

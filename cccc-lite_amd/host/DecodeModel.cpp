@@ -476,6 +476,23 @@ int DecodeModel::prefillPiece(const int* tokens, int n, int pos0, bool last)
     // The fused GEMM launches below are matrix-matrix kernels; up to 16 tokens the separate calls run the matrix-vector
     // kernels, which stay ahead on tiled copies (16 tokens: 3.3 ms either way, 2 tokens 2.8 against 3.1) but not on the file
     // layout from about 5 tokens on (16 tokens: 4.1 -> 3.7 ms of a 36-layer 4096-wide model, 6 tokens 3.9 -> 3.5)
+    // FP4 linears reach the register-fed GEMM and its fused launches only through their tiled copies (codes and scales in
+    // matrix-core operand order; the two-operand kernel on the file layout runs at half the rate).  A model loaded without
+    // them builds them when a prompt of 17 tokens or more first needs them: 1.125x the FP4 weight memory from then on.
+    if (n >= 17)
+    {
+        for (auto& L : layers_)
+        {
+            for (Matrix* w : { L.wq.get(), L.wk.get(), L.wv.get(), L.wo.get(), L.w_gate.get(), L.w_up.get(), L.w_down.get() })
+            {
+                if (w->getDataType() == FP4_E2M1 && !w->hasTiled() && w->getWidth() % 128 == 0)
+                {
+                    w->setAllowRepack(true);
+                    w->prepareTiled();
+                }
+            }
+        }
+    }
     const bool fuse_gemms = n >= (c.layers > 0 && layers_[0].wq->hasTiled() ? 17 : 5);
     // sum = res + W x and y = norm(sum): where the GEMM splits its k range the launch that adds the partial sums does the add
     // and the norm as well (-1: this shape does not split, or the library has no such kernel for it)

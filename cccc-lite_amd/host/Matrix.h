@@ -41,16 +41,28 @@ public:
     {
         return shared_data_->block_scale_data_ ? (const uint8_t*)shared_data_->block_scale_data_ + scale_offset_ : nullptr;
     }
-    int64_t getBlockScaleCount() const { return shared_data_->block_scale_count_; }
-    // Uploads the FP4 block scales; a [K x n_out] linear weight then gets its tiled copy (codes + scales)
+    // Block scales this tensor owns: all of the storage's, or, for a row view, those of its own rows
+    int64_t getBlockScaleCount() const
+    {
+        if (!rows_view_) { return shared_data_->block_scale_count_; }
+        return shared_data_->block_scale_data_ ? (getDataSize() + fp4BlockSize() - 1) / fp4BlockSize() : 0;
+    }
+    // Uploads the FP4 block scales; a [K x n_out] linear weight then gets its tiled copy (codes + scales).  A row view
+    // does neither: the scale array and the tiled copy belong to the whole storage, under the storage's own dims.
     void setBlockScaleFromHost(const void* src, int64_t n_scales)
     {
+        if (rows_view_) { return; }
         shared_data_->setBlockScaleFromHost(src, n_scales);
         if (number_ == 1 && channel_ == 1 && getDataType() == FP4_E2M1) { shared_data_->prepareTiled(height_, width_); }
     }
-    void getBlockScaleToHost(void* dst) const { shared_data_->getBlockScaleToHost(dst); }
+    void getBlockScaleToHost(void* dst) const
+    {
+        if (!rows_view_) { shared_data_->getBlockScaleToHost(dst); }
+        else if (getBlockScaleCount() > 0) { GpuControl::copyDeviceToHost(dst, getBlockScaleData(), (size_t)getBlockScaleCount()); }
+    }
     static unsigned int fp4BlockSize() { return MatrixData::fp4_block_size_; }
-    void prepareTiled() { if (shared_data_ && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); } }
+    void prepareTiled() { if (shared_data_ && !rows_view_ && number_ == 1 && channel_ == 1) { shared_data_->prepareTiled(height_, width_); } }
+    bool isRowsView() const { return rows_view_; }
     void setAllowRepack(bool allow) { if (shared_data_) { shared_data_->allow_repack_ = allow; } }
     bool hasTiled() const { return shared_data_ && shared_data_->tiled_data_ != nullptr; }
     float getInputScale() const { return shared_data_ ? shared_data_->input_scale_ : 0.0f; }
@@ -84,6 +96,7 @@ private:
     std::shared_ptr<MatrixData> shared_data_;
     void* data_ = nullptr;
     int64_t scale_offset_ = 0;    // first block scale of this view within the storage's scale array
+    bool rows_view_ = false;      // made by rowsView(): a row range of a larger storage
     int width_ = 0, height_ = 0, channel_ = 0, number_ = 0, row_ = 0;
 };
 

@@ -244,6 +244,7 @@ Matrix Matrix::rowsView(int row0, int n_rows) const
     m.setDim(width_, n_rows, 1, 1);
     m.data_ = (char*)data_ + (dt == FP4_E2M1 ? first / 2 : first * (int64_t)Rocblas::elemBytes(dt));
     m.scale_offset_ = scale_offset_ + (dt == FP4_E2M1 ? first / fp4BlockSize() : 0);
+    m.rows_view_ = rows_view_ || n_rows != height_;
     return m;
 }
 

@@ -88,11 +88,11 @@ C_EXPORT int hip_absmax(const void* src, int src_type, unsigned int n, void* d_r
  * C of type HALF; the weight is dequantised to half, FP32 accumulation, one rounding to half).
  * `act_scale` is accepted and ignored (it only drives the W8A8 route, cccc/cublas_real.h:871-873).
  * Anything else (both operands quantized, FP4 with HALF, mixed 16-bit types, other C types) returns -1.
- * Device memory: the one case in which the library allocates is an FP8 GEMM of 17 tokens or more whose
- * output has too few tiles to fill the GPU; it then splits K over workgroups and keeps FP32 partial sums in a
- * scratch buffer per (device, stream) that grows on demand and lives until the process ends (at most
- * 8 * M * N * 4 bytes).  While the stream is being captured into a graph the buffer is never grown: the
- * call then runs without the split.
+ * Device memory: the one case in which the library allocates is a GEMM of 17 tokens or more (FP8, FP4 on a tiled
+ * copy, or HALF activations) whose output has too few tiles to fill the GPU; it then splits K over workgroups and keeps
+ * FP32 partial sums in a scratch buffer per (host thread, device, stream) that grows on demand and lives until the
+ * process ends (at most 16 * M * N * 4 bytes).  While the stream is being captured into a graph the buffer is never
+ * grown: the call then runs without the split (see hip_quant_workspace_reserve).
  */
 C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
                             const void* A, int typeA, int lda, float invScaleA,
@@ -107,8 +107,9 @@ C_EXPORT int hip_quant_gemm(int transA, int transB, int M, int N, int K, float a
  * partial sums: in a static device array of HIP_QUANT_NOALLOC_SCRATCH_BYTES inside the library (one per
  * GPU the library runs on, held until the process ends) instead of a buffer grown on demand.  The call
  * never allocates or frees device memory.  A shape whose k-split needs more than that (splits * M * N * 4
- * bytes, splits <= 16; only FP8 GEMMs of 17 tokens or more with few output tiles split at all) returns -1
- * with a message on stderr and launches nothing; 32 MiB covers 512 tokens x 4096 features.
+ * bytes, splits <= 16) returns -1 with a message on stderr and launches nothing; 32 MiB covers 512 tokens x 4096
+ * features.  The routes that split K, all with few output tiles for the GPU: FP8 GEMMs of 17 tokens or more (K % 64 == 0),
+ * FP4 GEMMs of 17 tokens or more on a registered tiled copy (K % 128 == 0), and HALF-activation GEMMs of 17 tokens or more.
  * Every call on a GPU shares the one array: calls that overlap on one GPU (two streams, two host
  * threads) race on it and must be ordered by the caller.  Nothing in it needs clearing between calls:
  * each call overwrites every partial sum it later reads.
@@ -344,6 +345,20 @@ C_EXPORT int hip_argmax_pick_embed_bf16(const void* workspace, unsigned int n, v
  *   hip_quant_last_kernel() : name of the kernel family the last hip_quant_gemm call dispatched to
  *                             ("gemv_dot2", "gemv_mfma", "gemm_mfma", "generic", ...)
  */
+/*
+ * Workspace of the k-split launches (no counterpart in the reference, whose grow-only workspaces live in its BLAS
+ * wrapper, cccc/cublas_real.h:1174-1225).  A GEMM whose output has too few tiles for the GPU splits K over workgroups and
+ * keeps FP32 partial sums in a buffer per (host thread, device, stream) that grows on demand and lives until the process
+ * ends.  The buffer is never grown while the stream is being captured into a graph: a call that would need a larger one
+ * then runs without the split (hip_quant_gemm, hip_quant_gemm_segments, hip_quant_gemm_swiglu: same result up to the FP32
+ * summation order) or returns -1 (hip_quant_gemm_add_rms_norm).  A caller that captures such launches either runs each
+ * shape once eagerly on the same stream first, or reserves the bytes up front with
+ *   hip_quant_workspace_reserve(bytes) : grows this thread's buffer for the current device and stream to at least
+ *                                        `bytes` (16 * tokens * n_out * 4 covers every split; a gate / up pair twice that).
+ *                                        0 ok, 1 allocation failed, -1 the stream is being captured.
+ */
+C_EXPORT int hip_quant_workspace_reserve(unsigned long long bytes);
+
 C_EXPORT int hip_quant_set_sync(int enabled);
 C_EXPORT int hip_quant_set_stream(void* stream);
 C_EXPORT void* hip_quant_get_stream(void);

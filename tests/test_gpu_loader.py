@@ -252,7 +252,9 @@ def test_fp4_matrix_saves_packed_codes_and_block_scales(tmp_path, gpu, pkg, host
 
 def test_mixed_fp8_formats_in_one_file(tmp_path, gpu, pkg, host, oracle, dec):
     """k stored as FP8_E4M3 with a scale next to E5M2 q and v: the step decodes each projection with its own format
-    (three launches instead of one).  Gate and up in two formats are refused by name."""
+    (three launches instead of one).  Gate and up in two formats likewise: every tensor keeps the format the file gives
+    it (cccc/Net.cpp:1444-1481), the step runs the two linears and the SwiGLU product as launches of their own, and the
+    prompt phase takes its separate calls."""
     cfg = dec.DecodeConfig(layers=1, hidden=256, n_q=4, n_kv=2, inter=512, vocab=300, t_kv=16)
     weights = dec.make_model(cfg, 31)
     path = tmp_path / "mixed.bin"
@@ -293,9 +295,38 @@ def test_mixed_fp8_formats_in_one_file(tmp_path, gpu, pkg, host, oracle, dec):
         got = dec.f(model.logits())
         assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
     up_f32 = oracle.decode_table(oracle.E5M2)[weights["layers"][0]["w_up"]]
-    bad = rewrite("weight_fp8_e5m2_W_up_0", "weight_fp8_e4m3_W_up_0", oracle.encode_e4m3_rne((up_f32 / np.float32(scale)).astype(np.float32)), "scale_W_up_0")
-    with pytest.raises(ValueError, match="W_up_0"):
-        make_model(pkg, host, cfg).load_named(pkg.host_api.WeightFile(host, bad))
+    up_scale = float(np.abs(up_f32).max()) / 448.0
+    up_e4m3 = oracle.encode_e4m3_rne((up_f32 / np.float32(up_scale)).astype(np.float32))
+    scale = up_scale
+    both = rewrite("weight_fp8_e5m2_W_up_0", "weight_fp8_e4m3_W_up_0", up_e4m3, "scale_W_up_0")
+
+    class MixedUpOracle(dec.DecodeOracle):
+        def deq(self, layer, name):
+            if name == "w_up":
+                return oracle.dequant_fp8_to_bf16(up_e4m3, oracle.E4M3, up_scale).reshape(up_e4m3.shape)
+            return super().deq(layer, name)
+
+    model = make_model(pkg, host, cfg)
+    model.load_named(pkg.host_api.WeightFile(host, both))
+    model.set_exact_attention(True)
+    orc = MixedUpOracle(cfg, weights)
+    token = 4
+    for pos in range(3):
+        model.reset(token, pos)
+        model.step()
+        want_logits, token = orc.step(token, pos)
+        got = dec.f(model.logits())
+        assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits), pos
+        gated = dec.f(model.activation("gated"))
+        assert np.isfinite(gated).all()
+    # the prompt phase of the same model (separate gate / up calls), then a step behind it
+    orc = MixedUpOracle(cfg, weights)
+    prompt = [5, 17, 250, 3, 9, 11]
+    for pos, tok in enumerate(prompt):
+        want_logits, want_next = orc.step(tok, pos)
+    model.prefill(prompt)
+    got = dec.f(model.logits())
+    assert np.linalg.norm(got - want_logits) <= 1e-2 * np.linalg.norm(want_logits)
 
 
 def test_decode_model_from_an_fp4_file(tmp_path, gpu, pkg, host, oracle, dec):
@@ -400,6 +431,23 @@ def test_projections_sharing_an_input_load_into_one_storage(tmp_path, gpu, pkg, 
             assert pkg.host_api.mul_batched(view, xm, yv, ta=1, tb=0) == 0
             check_rows(oracle.bf16_to_f32(yv.download(np.uint16, tokens * n).reshape(tokens, n)).astype(np.float64), oracle.linear_exact(Wd, X), name + " view")
             row0 += n
+    # A row view saved under a name of its own holds exactly its rows: codes, and for FP4 the block scales of those rows
+    # (not the storage's whole scale array); a view can neither replace the storage's scales nor build a tiled copy.
+    row0 = rows[0]
+    view = group.rows_view(row0, rows[1])
+    saved = tmp_path / f"view_{fmt}.bin"
+    view.save_named("W_k_0", saved)
+    codes, sc = packed[1]
+    key = "weight_fp4_e2m1_W_k_0" if sc is not None else "weight_fp8_e5m2_W_k_0"
+    assert weight_file.read_entry(saved, key) == codes.tobytes()
+    if sc is not None:
+        assert weight_file.read_entry(saved, "blockscale_W_k_0") == sc.tobytes()
+        assert np.array_equal(view.block_scales(), sc.ravel())
+        all_scales = group.block_scales()
+        view.set_block_scale(np.zeros(sc.size, np.uint8))          # ignored on a view
+        assert np.array_equal(group.block_scales(), all_scales)
+    had = group.prepare_tiled()
+    assert view.prepare_tiled() == had                              # (reports the storage's copy; builds none of its own)
     # members of different types or scales, a missing name, a storage of the wrong size
     if fmt == "fp8_e5m2":
         assert f.load_named_group(host.matrix(K, 512 + 128, 1, 1, BF16), ("W_q_0", "W_other")) == -1
