@@ -590,7 +590,7 @@ def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
     return out
 
 
-SCALED_INV_SCALE = 0.1 / 57344.0       # absmax / max_code of a weight whose largest element is 0.1 (cccc/Matrix.cpp:338-352)
+SCALED_INV_SCALE = 0.2 / 57344.0       # absmax / max_code of a weight whose largest element is 0.2 (cccc/Matrix.cpp:338-352): ten sigma, no Inf codes
 
 
 def variant_sweep(ws, by_shape, token_counts=(1, 16), use_graph=False):

@@ -211,6 +211,31 @@ bool pick_gemv4_dot2(const LinearArgs& a)
     return launch_gemv4_dot2<MT, 2, 4, 4, 4, BLOCK>(a);
 }
 
+// Rows of K % 32 == 16 elements (blocks of 16): the ragged instantiation, one shape for every size
+template <int MT>
+bool launch_gemv4_dot2_ragged(const LinearArgs& a)
+{
+    const size_t lds = (size_t)MT * ((a.K + 2047) / 2048) * 4096;
+    auto kernel = gemv4_dot2_kernel<MT, 1, 2, 8, 16, true>;
+    if (!allow_big_lds(kernel, lds)) { return false; }
+    const int want = (a.n_out + 7) / 8;
+    const int cap = cu_count() * (lds > 80 * 1024 ? 1 : 2);
+    kernel<<<want < cap ? want : cap, 512, lds, stream()>>>(a);
+    return true;
+}
+
+bool gemv4_dot2_ragged(const LinearArgs& a)
+{
+    switch (a.tokens)
+    {
+    case 1: return launch_gemv4_dot2_ragged<1>(a);
+    case 2: return launch_gemv4_dot2_ragged<2>(a);
+    case 3: return launch_gemv4_dot2_ragged<3>(a);
+    case 4: return launch_gemv4_dot2_ragged<4>(a);
+    default: return false;
+    }
+}
+
 template <int BLOCK>
 bool gemv4_dot2(const LinearArgs& a)
 {
@@ -371,6 +396,21 @@ int quant_gemm(int transA, int transB, int M, int N, int K, float alpha,
         {
             const bool ok = x_ok && a.blk_sc && (a.block_size == 16 || a.block_size == 32) && K % 32 == 0 && a.ldw % 32 == 0 &&
                             aligned16(a.W) && ((uintptr_t)a.blk_sc & 1u) == 0;
+            // blocks of 16 over the flat index with K % 32 == 16 (dense rows): the ragged dot2 kernel, up to 16 tokens
+            const bool ragged = !ok && x_ok && a.blk_sc && a.block_size == 16 && K % 32 == 16 && a.ldw == K && aligned16(a.W) && a.tokens <= 16;
+            if (ragged)
+            {
+                launched = true;
+                for (int t0 = 0; t0 < g.tokens && launched; t0 += 4)
+                {
+                    LinearArgs s = a;
+                    s.tokens = (g.tokens - t0 < 4) ? g.tokens - t0 : 4;
+                    s.X = a.X + (long long)t0 * a.ldx;
+                    s.Y = a.Y + (long long)t0 * a.y_stride_tok;
+                    launched = gemv4_dot2_ragged(s);
+                }
+                if (launched) { note_kernel("gemv_dot2"); }
+            }
             if (ok && a.tokens <= 16)
             {
                 const uint8_t* tiled = fp4_tiled_pays(a) ? find_tiled_fp4(a) : nullptr;

@@ -380,10 +380,15 @@ __device__ __forceinline__ float e4m3_byte_to_f32(uint32_t word, int byte_index)
     return byte_index == 0 ? __builtin_amdgcn_cvt_f32_fp8(word, 0) : __builtin_amdgcn_cvt_f32_fp8(word, 1);
 }
 
-template <int MT, int R, int U, int WAVES, int BLOCK>
+// RAGGED (BLOCK 16 only): K % 32 == 16, legal in the reference, whose blocks of 16 run over the flat element index
+// (cccc-cuda/cuda_functions.cu:2926-2939).  Every other row then starts 8 bytes off a 16-byte boundary and at an odd
+// scale byte, and a row's last load covers 16 elements of this row and 16 of the next: codes are fetched as two 8-byte
+// halves and scales as single bytes, and the half that belongs to the next row is neither read nor used.
+template <int MT, int R, int U, int WAVES, int BLOCK, bool RAGGED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv4_dot2_kernel(const LinearArgs a)
 {
     static_assert(BLOCK == 16 || BLOCK == 32, "block scale length");
+    static_assert(!RAGGED || BLOCK == 16, "ragged rows: blocks of 16 only (blocks of 32 would straddle rows)");
     extern __shared__ u32x4 xs[];
     const int n_steps = (a.K + 2047) / 2048;
     stage_activations<MT, 4>(a, xs, n_steps, WAVES * 64);
@@ -424,7 +429,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv4_dot2_kernel(const LinearArgs
                 {
                     w[u][r] = u32x4{ 0u, 0u, 0u, 0u };
                     sc[u][r] = 0u;
-                    if (k < a.K)
+                    if constexpr (RAGGED)
+                    {
+                        if (k < a.K)
+                        {
+                            const uint8_t* wp = wrow[r] + (s0 + u) * 1024;
+                            const uint8_t* sp = srow[r] + (s0 + u) * 128;
+                            const u32x2 lo = __builtin_nontemporal_load((const u32x2*)wp);
+                            u32x2 hi = { 0u, 0u };
+                            uint32_t s_hi = 0u;
+                            if (k + 32 <= a.K)
+                            {
+                                hi = __builtin_nontemporal_load((const u32x2*)(wp + 8));
+                                s_hi = sp[1];
+                            }
+                            w[u][r] = u32x4{ lo[0], lo[1], hi[0], hi[1] };
+                            sc[u][r] = (uint32_t)sp[0] | (s_hi << 8);
+                        }
+                    }
+                    else if (k < a.K)
                     {
                         w[u][r] = __builtin_nontemporal_load((const u32x4*)(wrow[r] + (s0 + u) * 1024));
                         if (BLOCK == 16) { sc[u][r] = *(const uint16_t*)(srow[r] + (s0 + u) * 128); }

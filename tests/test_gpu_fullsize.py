@@ -84,6 +84,52 @@ def test_tiled_gemv_at_the_qwen3_8b_shapes(gpu, pkg, oracle, K, n_out):
         assert lib.weight_release(wd.data_ptr()) == 0
 
 
+def draw_fp8_scaled(torch, dev, gen, n_out, K, w_type, inv_scale):
+    """uint8 codes [n_out, K] of w / inv_scale for N(0, 0.02) weights w: what a weight quantized with the per-tensor scale
+    inv_scale holds (cccc/Matrix.cpp:338-352), rounded to nearest."""
+    f8 = torch.float8_e5m2 if w_type == E5M2 else torch.float8_e4m3fn
+    out = torch.empty(n_out, K, dtype=torch.uint8, device=dev)
+    rows = max(1, (1 << 27) // K)
+    for r0 in range(0, n_out, rows):
+        r = min(rows, n_out - r0)
+        out[r0:r0 + r] = (torch.randn(r, K, device=dev, generator=gen) * (0.02 / inv_scale)).to(torch.bfloat16).to(f8).view(torch.uint8)
+    return out
+
+
+@pytest.mark.parametrize("w_type,inv_scale", [(E5M2, 0.2 / 57344.0), (E4M3, 0.2 / 448.0)])      # ten sigma of headroom: no Inf / NaN codes
+@pytest.mark.parametrize("K,n_out", QWEN_SHAPES)
+def test_scaled_weights_at_the_qwen3_8b_shapes(gpu, pkg, oracle, K, n_out, w_type, inv_scale):
+    """The routes of the benchmark's `sweep_variants` and scaled prefill rows at full size: weights with a per-tensor
+    dequantisation multiplier (every weight Matrix::quantizeWeights makes carries absmax / 57344 or / 448), E5M2 and E4M3,
+    1 and 16 tokens on the tiled copy, and 512 tokens (the register-fed GEMM; the two MLP shapes only) -- the weight that
+    enters a product is bf16(decode(code) * inv_scale), rounded once, as the oracle rounds it."""
+    torch, dev, lib = gpu
+    gen = torch.Generator(device=dev).manual_seed(K + n_out + w_type)
+    wd = draw_fp8_scaled(torch, dev, gen, n_out, K, w_type, inv_scale)
+    td = torch.zeros(lib.tiled_size(w_type, n_out, K), dtype=torch.uint8, device=dev)
+    assert lib.weight_prepare(wd.data_ptr(), w_type, n_out, K, K, td.data_ptr()) == 0
+    try:
+        rows = np.sort(np.random.default_rng(n_out + w_type).choice(n_out, size=193, replace=False))
+        W_rows = wd[torch.from_numpy(rows).to(dev)].cpu().numpy()
+        Wd_rows = oracle.dequant_fp8_to_bf16(W_rows, oracle.E5M2 if w_type == E5M2 else oracle.E4M3, inv_scale).reshape(W_rows.shape)
+        counts = (1, 16, 512) if (K, n_out) in ((4096, 12288), (12288, 4096)) else (1, 16)
+        for tokens in counts:
+            X = synth.activations(n_out + tokens + w_type, tokens, K)
+            xd = to_dev(torch, dev, X)
+            yd = torch.zeros(tokens * n_out + 64, dtype=torch.int16, device=dev)
+            assert lib.linear(wd.data_ptr(), w_type, xd.data_ptr(), yd.data_ptr(), n_out, tokens, K, inv_scale=inv_scale) == 0
+            small = tokens <= 2 and n_out * K < (8 << 20)
+            assert lib.last_kernel() == ("gemm_mfma_tiled" if tokens > 16 else "gemv_dot2" if small else "gemv_mfma_tiled")
+            out = from_dev(yd, np.uint16)
+            assert not out[tokens * n_out:].any(), "wrote past the end"
+            y = out[:tokens * n_out].reshape(tokens, n_out)
+            want = oracle.linear_exact(Wd_rows, X)
+            check_rows(bf16_f64(oracle, y[:, rows]), want, f"scaled type {w_type} {n_out}x{K} M={tokens}")
+            check_bf16_close(y[:, rows], want, "scaled", slack_ulp=1.0, abs_floor=2e-5)
+    finally:
+        assert lib.weight_release(wd.data_ptr()) == 0
+
+
 # ------------------------------------------------------------------------------------------ FP4
 
 FP4_BOUNDS = (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0)

@@ -140,6 +140,30 @@ def test_fp4_gemv_vs_oracle(gpu, pkg, oracle, tokens, n_out, K, block):
     assert kernel == "gemv_dot2"
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 4, 7, 16])
+@pytest.mark.parametrize("n_out,K", [(8, 48), (257, 144), (130, 2064), (64, 4112)])
+def test_fp4_rows_of_half_a_load_more(gpu, pkg, oracle, tokens, n_out, K):
+    """K % 32 == 16 with blocks of 16 -- legal in the reference, whose blocks run over the flat element index
+    (cccc-cuda/cuda_functions.cu:2926-2939): every other row starts in the middle of a 16-byte load and at an odd scale
+    byte, and a row's last load is half this row, half the next.  Up to 16 tokens stay on the dot2 kernel; the neighbours'
+    codes and scales must not leak in (the buffers end with the last row: nothing past them may be read either), and
+    blocks of 32 on such rows, which straddle rows, take the generic kernel."""
+    seed = synth.seed_for(3, 700 + tokens + n_out % 11)
+    X = synth.activations(seed, tokens, K)
+    nib, sc = synth.pack_fp4_blockscale(synth.weights_f32(seed, n_out, K), 16)
+    y, kernel = run_linear(gpu, pkg, nib, oracle.FP4, X, n_out, tokens, K, blk_sc=sc, block=16)
+    assert kernel == "gemv_dot2"
+    Wd = oracle.dequant_weight(nib, oracle.FP4, n_out, K, blk_sc=sc, block=16)
+    want = oracle.linear_exact(Wd, X)
+    check_rows(bf16_f64(oracle, y), want, f"ragged fp4 {tokens}x{n_out}x{K}")
+    check_bf16_close(y, want, kernel, slack_ulp=1.0, abs_floor=2e-5)
+    if tokens == 1 and (n_out * K) % 32 == 0:
+        nib32, sc32 = synth.pack_fp4_blockscale(synth.weights_f32(seed, n_out, K), 32)
+        y, kernel = run_linear(gpu, pkg, nib32, oracle.FP4, X, n_out, tokens, K, blk_sc=sc32, block=32)
+        assert kernel == "generic"
+        check_rows(bf16_f64(oracle, y), oracle.linear_exact(oracle.dequant_weight(nib32, oracle.FP4, n_out, K, blk_sc=sc32, block=32), X), "ragged block 32")
+
+
 def test_fp4_every_nibble_and_scale_inside_the_gemv(gpu, pkg, oracle):
     """x = one-hot: the output is bf16(fp4 * e4m3 scale) exactly, for all 16 nibbles x all finite
     scale bytes."""
