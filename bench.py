@@ -72,7 +72,20 @@ class BenchLibrary:
         L.cccc_bench_floor_read.argtypes = [i32, ctypes.POINTER(vp), ctypes.c_ulonglong, i32, i32, i32]
         L.cccc_bench_launch_us.restype = ctypes.c_double
         L.cccc_bench_launch_us.argtypes = [i32, i32, i32]
+        L.cccc_bench_gemm_variant.restype = ctypes.c_double
+        L.cccc_bench_gemm_variant.argtypes = [i32, i32, i32, ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_float, vp, i32, i32, ctypes.POINTER(ctypes.c_double)]
         self.c, self.ctypes = L, ctypes
+
+    def gemm_variant(self, variant, tile, tiled_ptrs, X_ptr, Y_ptr, n_out, tokens, K, inv_scale=1.0, partial_ptr=None, iters=64, warmup=8):
+        """Microseconds per launch of one experimental variant of the FP8 prefill GEMM (host/bench_gemm_variants.hip)
+        and, for the tracing variants, the share of a workgroup's ticks spent converting / at the barrier / in the rest."""
+        n = len(tiled_ptrs)
+        phases = (self.ctypes.c_double * 4)()
+        us = float(self.c.cccc_bench_gemm_variant(variant, tile, n, (self.ctypes.c_void_p * n)(*tiled_ptrs), X_ptr, Y_ptr, n_out, tokens, K,
+                                                  inv_scale, partial_ptr, iters, warmup, phases))
+        if us < 0:
+            raise RuntimeError(f"gemm variant {variant}/{tile} failed: {us}")
+        return us, ([round(phases[j] / phases[3], 4) for j in range(3)] if (variant & 4) and phases[3] > 0 else None)
 
     def floor_read_us(self, ptrs, nbytes, iters=None, wgs_per_cu=8) -> float:
         """Microseconds per launch of a kernel that only streams `nbytes` with 16-byte loads, rotating over the buffers
@@ -674,8 +687,9 @@ def prefill_cases(ws, by_shape):
         for M in (512, 2048):
             X, Y = ws.activation(M, K), ws.output(M, N)
             ops = [(W, X, Y, K, N) for W in weights]
-            ms = time_chain(ws, ops, 10, 3, False)
-            us = ms * 1000.0 / (10 * len(ops))
+            steps = 40 if M <= 512 else 12                  # 30 ms or more per figure: shorter bursts run at other clocks
+            ms = time_chain(ws, ops, steps, steps // 4, False)
+            us = ms * 1000.0 / (steps * len(ops))
             tf = 2.0 * M * K * N / us * 1e-6
             x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
             for rep in range(2):
@@ -688,7 +702,7 @@ def prefill_cases(ws, by_shape):
             # the same launches with a per-tensor dequantisation multiplier (the route of a weight quantized on load)
             for W in weights:
                 W.quant_scale = SCALED_INV_SCALE
-            us_scaled = time_chain(ws, ops, 10, 3, False) * 1000.0 / (10 * len(ops))
+            us_scaled = time_chain(ws, ops, steps, steps // 4, False) * 1000.0 / (steps * len(ops))
             for W in weights:
                 W.quant_scale = 1.0
             tf_scaled = 2.0 * M * K * N / us_scaled * 1e-6
@@ -841,7 +855,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy", "prompt_attention", "floor"])
+    ap.add_argument("--workload", default="decode_step", choices=["decode_step", "decode_linears", "gemv", "prefill", "copy", "prompt_attention", "floor", "prefill_variants"])
     ap.add_argument("--shape", default="4096,12288", help="K,N for --workload gemv / prefill")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--weights", default="fp8", choices=["fp8", "fp4"], help="weight format of --workload gemv / prefill (fp4: E2M1 codes + E4M3 block scales)")
@@ -920,6 +934,57 @@ def main():
         print(json.dumps({"workload": "floor", "what": "streaming read of the sweep byte counts with 16-byte non-temporal loads, rotating buffers (1 GiB pool); "
                                                        "empty and one-trip launches inside a hipGraph",
                           "launch_us_empty": round(ws.bench.launch_us(0), 3), "launch_us_one_trip": round(ws.bench.launch_us(1), 3), "rows": rows}))
+        return
+
+    if args.workload == "prefill_variants":
+        # The FP8 prefill GEMM against the variants of it that were tried and not adopted (host/bench_gemm_variants.hip):
+        # conversions spread between the matrix-core instructions, a 4 x 2 blocking of the tiles over the XCDs, other
+        # tile shapes; and where a workgroup's time goes (wave 0's clock: conversion + wait for weight bytes / barrier /
+        # rest of the k-tile).  Same weights (tiled copies of 8 distinct E5M2 matrices), activations and launch count
+        # for every row; every variant's output is compared with its tile's "block" variant (bit for bit) and the product entry's.
+        rows = []
+        for (K, N) in ((4096, 12288), (12288, 4096)):
+            codes = [torch.randn(N, K, device=ws.dev, generator=ws.gen).mul_(0.02).to(torch.bfloat16).to(torch.float8_e5m2) for _ in range(8)]
+            tiled = [torch.empty(ws.lib.tiled_size(E5M2, N, K), dtype=torch.uint8, device=ws.dev) for _ in codes]
+            for c_, t_ in zip(codes, tiled):
+                assert ws.lib.weight_prepare(c_.data_ptr(), E5M2, N, K, K, t_.data_ptr()) == 0
+            ptrs = [t_.data_ptr() for t_ in tiled]
+            for M in (512, 2048):
+                x = torch.randn(M, K, device=ws.dev, generator=ws.gen).to(torch.bfloat16)
+                y, y_ref = torch.zeros(M, N, device=ws.dev, dtype=torch.bfloat16), torch.zeros(M, N, device=ws.dev, dtype=torch.bfloat16)
+                partial = torch.empty(4 * M * N, device=ws.dev, dtype=torch.float32)
+                rm_ptrs = [c_.data_ptr() for c_ in codes]
+                n_it = 600 if M <= 512 else 200                 # 30 ms or more per figure: shorter bursts run at other clocks
+                us, _ = ws.bench.gemm_variant(8, 0, rm_ptrs, x.data_ptr(), y_ref.data_ptr(), N, M, K, iters=n_it, warmup=n_it // 4)
+                row = {"K": K, "N": N, "M": M, "product_us": round(us, 2), "product_kernel": ws.lib.last_kernel(), "variants": {}}
+                names = {0: "block", 1: "spread", 2: "raster4x2", 3: "spread+raster4x2"}
+                tiles = {0: "128x256", 3: "64x256", 4: "128x192", 1: "64x192", 5: "128x256_split2", 6: "64x256_split2", 2: "128x256_split4"}
+                for tile in tiles:
+                    if tile in (1, 4) and N % 192 != 0:
+                        continue
+                    for variant in (0, 1, 2, 3):
+                        y.zero_()
+                        us, _ = ws.bench.gemm_variant(variant, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=n_it, warmup=n_it // 4)
+                        if variant == 0:
+                            y_block = y.clone()         # same k order for every variant of one tile: they must agree bit for bit
+                        row["variants"][f"{tiles[tile]}/{names[variant]}"] = {
+                            "us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
+                            "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
+                    for variant in (4, 5):
+                        _, ph = ws.bench.gemm_variant(variant, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=8, warmup=2)
+                        row["variants"][f"{tiles[tile]}/{names[variant - 4]}"]["ticks_cvt_barrier_rest"] = ph
+                us0, _ = ws.bench.gemm_variant(0, 0, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, inv_scale=SCALED_INV_SCALE, iters=n_it, warmup=n_it // 4)
+                us1, _ = ws.bench.gemm_variant(1, 0, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, inv_scale=SCALED_INV_SCALE, iters=n_it, warmup=n_it // 4)
+                row["scaled_128x256"] = {"block_us": round(us0, 2), "spread_us": round(us1, 2)}
+                us, _ = ws.bench.gemm_variant(8, 0, rm_ptrs, x.data_ptr(), y_ref.data_ptr(), N, M, K, iters=n_it, warmup=n_it // 4)
+                row["product_us_after_the_variants"] = round(us, 2)
+                rows.append(row)
+                del x, y, y_ref, partial
+            for c_ in codes:
+                ws.lib.weight_release(c_.data_ptr())
+            del codes, tiled
+        print(json.dumps({"workload": "prefill_variants", "what": "W8A16 prefill GEMM: the product kernel and the variants measured against it "
+                          "(us per launch over 600 (M 512) / 200 (M 2048) launches on 8 distinct weights; ticks = shares of wave 0's clock per workgroup)", "rows": rows}))
         return
 
     metric, unit = "quant GEMV HBM GB/s (Qwen3-8B W8A16 decode linears, bs=1)", "GB/s"
