@@ -306,6 +306,45 @@ bool launch_tile(int tile, bool scaled, const LinearArgs& a, float* partial, uns
     }
 }
 
+// the product kernel itself with a tile shape, k split and prefetch distance of the caller's choice
+template <int MB, int NB, bool SPLIT, int PD>
+void launch_product_kernel(const LinearArgs& a, int splits, float* partial)
+{
+    const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
+    const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, splits);
+    gemm_mfma_direct_kernel<DT_E5M2, false, MB, SPLIT, true, DT_BF16, NB, false, false, PD><<<grid, 256, 0, nullptr>>>(a, n_tiles, SPLIT ? partial : nullptr);
+    if (SPLIT) { launch_splitk_combine<DT_BF16>(partial, splits, a, nullptr); }
+}
+
+// tile 100 + 10 * shape + PD: shape 0 = 64 x 192, 1 = 64 x 256, 2 = 128 x 192, 3 = 64 x 256 split 4, 4 = 128 x 256 split 4,
+// 5 = 64 x 256 split 2, 6 = 64 x 256 split 3, 7 = 128 x 192 split 2 ... ; PD 1 .. 3 (128-token tiles: 1 or 2)
+bool launch_product_tile(int tile, const LinearArgs& a, float* partial)
+{
+    switch (tile)
+    {
+    case 101: launch_product_kernel<4, 3, false, 1>(a, 1, partial); return true;
+    case 102: launch_product_kernel<4, 3, false, 2>(a, 1, partial); return true;
+    case 103: launch_product_kernel<4, 3, false, 3>(a, 1, partial); return true;
+    case 111: launch_product_kernel<4, 4, false, 1>(a, 1, partial); return true;
+    case 112: launch_product_kernel<4, 4, false, 2>(a, 1, partial); return true;
+    case 113: launch_product_kernel<4, 4, false, 3>(a, 1, partial); return true;
+    case 121: launch_product_kernel<8, 3, false, 1>(a, 1, partial); return true;
+    case 122: launch_product_kernel<8, 3, false, 2>(a, 1, partial); return true;
+    case 131: launch_product_kernel<4, 4, true, 1>(a, 4, partial); return true;
+    case 132: launch_product_kernel<4, 4, true, 2>(a, 4, partial); return true;
+    case 133: launch_product_kernel<4, 4, true, 3>(a, 4, partial); return true;
+    case 141: launch_product_kernel<8, 4, true, 1>(a, 4, partial); return true;
+    case 151: launch_product_kernel<4, 4, true, 1>(a, 2, partial); return true;
+    case 153: launch_product_kernel<4, 4, true, 3>(a, 2, partial); return true;
+    case 161: launch_product_kernel<4, 4, true, 1>(a, 3, partial); return true;
+    case 163: launch_product_kernel<4, 4, true, 3>(a, 3, partial); return true;
+    case 171: launch_product_kernel<8, 3, true, 1>(a, 2, partial); return true;
+    case 172: launch_product_kernel<8, 3, true, 2>(a, 2, partial); return true;
+    default: return false;
+    }
+}
+
 }    // namespace
 
 extern "C" {
@@ -321,7 +360,7 @@ extern "C" {
 double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, const void* X, void* Y, int n_out, int tokens, int K,
                                float inv_scale, float* partial, int iters, int warmup, double* phases)
 {
-    const bool wide3 = tile == 1 || tile == 4;
+    const bool wide3 = tile == 1 || tile == 4 || (tile >= 100 && (tile / 10 == 10 || tile / 10 == 12 || tile / 10 == 17));
     if (n_w <= 0 || !W_tiled || !X || !Y || iters <= 0 || K % 64 != 0 || tokens % 128 != 0 || n_out % (wide3 ? 192 : 256) != 0) { return -1.0; }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
@@ -350,6 +389,11 @@ double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, c
         if (i == warmup) { (void)hipEventRecord(e0, nullptr); }
         a.W = (const uint8_t*)W_tiled[i % n_w];
         const bool scaled = inv_scale != 1.0f;
+        if (tile >= 100)
+        {
+            ok = variant == 0 && !scaled && launch_product_tile(tile, a, partial);
+            continue;
+        }
         switch (variant)
         {
         case 0: ok = launch_tile<false, false, false>(tile, scaled, a, partial, trace, &n_wgs); break;
