@@ -1346,7 +1346,10 @@ inline DirectPlan plan_direct(const LinearArgs& a, SplitScratch* scratch, bool f
         if (sh.mb == 8 && (a.tokens <= 64 || (sh.nb == 4 && !big_tile))) { continue; }
         const long long tiles = (long long)((a.n_out + 64 * sh.nb - 1) / (64 * sh.nb)) * ((a.tokens + 16 * sh.mb - 1) / (16 * sh.mb));
         const double balance = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
-        const double occupancy = tiles >= 2LL * cus ? 1.0 : (tiles > cus ? 0.95 : 0.85);
+        double occupancy = tiles >= 2LL * cus ? 1.0 : (tiles > cus ? 0.95 : 0.85);
+        // one 128 x 256 tile on (nearly) every CU and a long K: ahead of two 64-token tiles per CU, which convert every weight
+        // twice (2048 tokens x 4096 features, K 12288, tiled copy: 160 against 168-170 us; K 4096: level)
+        if (sh.nb == 4 && sh.mb == 8 && !row_major && a.K >= 8192 && tiles * 8 > 7LL * cus && tiles <= cus) { occupancy = 1.02; }
         const double score = sh.quality * balance * occupancy;
         if (score > best + 1e-9)
         {
