@@ -1440,7 +1440,7 @@ bool gemm_mfma(const LinearArgs& a, const uint8_t* tiled = nullptr, SplitScratch
     if constexpr (WT != DT_FP4)
     {
         const bool small_offsets = (long long)a.n_out * a.ldw < (1LL << 32) && (long long)a.tokens * a.ldx * 2 < (1LL << 32);
-        // (HALF activations have no matrix-core GEMV: there the register-fed kernel also serves 5-16 tokens)
+        // (HALF activations: the register-fed kernel also serves 5-16 tokens where the matrix-core GEMV refuses the shape)
         if (a.K % 64 == 0 && a.tokens >= (e ? 2 : (AT == DT_HALF ? 5 : 17)) && small_offsets)
         {
             LinearArgs d = a;
