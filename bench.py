@@ -72,9 +72,21 @@ class BenchLibrary:
         L.cccc_bench_floor_read.argtypes = [i32, ctypes.POINTER(vp), ctypes.c_ulonglong, i32, i32, i32]
         L.cccc_bench_launch_us.restype = ctypes.c_double
         L.cccc_bench_launch_us.argtypes = [i32, i32, i32]
+        L.cccc_bench_gemm_ablation.restype = ctypes.c_double
+        L.cccc_bench_gemm_ablation.argtypes = [i32, i32, i32, ctypes.POINTER(i32)]
         L.cccc_bench_gemm_variant.restype = ctypes.c_double
         L.cccc_bench_gemm_variant.argtypes = [i32, i32, i32, ctypes.POINTER(vp), vp, vp, i32, i32, i32, ctypes.c_float, vp, i32, i32, ctypes.POINTER(ctypes.c_double)]
         self.c, self.ctypes = L, ctypes
+
+    def gemm_ablation_tflops(self, flags: int, trips=2048, launches=40) -> float:
+        """TFLOP/s of the prefill GEMM's k-tile with only some of its ingredients (host/bench_gemm_variants.hip,
+        gemm_ablation_kernel): 0 = the 64 matrix-core instructions on register operands; +1 FP8 -> BF16 conversions,
+        +2 fragment reads from LDS, +4 barrier, +8 LDS stores, +16 weight loads, +32 activation loads (L2-resident windows)."""
+        n = self.ctypes.c_int(0)
+        us = float(self.c.cccc_bench_gemm_ablation(flags, trips, launches, self.ctypes.byref(n)))
+        if us < 0:
+            raise RuntimeError(f"gemm ablation {flags} failed: {us}")
+        return n.value * 4.0 * trips * 64 * 16384 / us * 1e-6
 
     def gemm_variant(self, variant, tile, tiled_ptrs, X_ptr, Y_ptr, n_out, tokens, K, inv_scale=1.0, partial_ptr=None, iters=64, warmup=8):
         """Microseconds per launch of one experimental variant of the FP8 prefill GEMM (host/bench_gemm_variants.hip)
@@ -728,10 +740,15 @@ def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
     FP4 prefill GEMM on the two MLP shapes (FLOPs 2 M K N against the BF16 matrix-core peak)."""
     t = ws.torch
     out, prefill, keep = [], [], []                 # buffers stay allocated until the sweep is over (freeing slows what runs next)
+    pool = t.randint(0, 255, (800 << 20,), dtype=t.uint8, device=ws.dev)        # what the streaming floor reads
+    keep.append(([], [], [pool]))
     for (K, N) in LLAMA_SHAPES:
         for block in (16, 32):
             per = K * N // 2 + K * N // block
             n_w = max(2, min(48, (768 << 20) // per))
+            span = (per + 4095) // 4096 * 4096
+            floor_ptrs = [pool.data_ptr() + i * span for i in range(max(1, min(n_w, (800 << 20) // span)))]
+            floor_us = min(ws.bench.floor_read_us(floor_ptrs, per, wgs_per_cu=w) for w in (2, 8))
             nib = [t.randint(0, 256, (N, K // 2), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             tiled = []
@@ -750,7 +767,8 @@ def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
                 us = ms * 1000.0 / n_it
                 if M <= 16:
                     gbs = fp4_bytes(K, N, M, block) / us * 1e-3
-                    out.append({"K": K, "N": N, "M": M, "block": block, "us": round(us, 2), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                    out.append({"K": K, "N": N, "M": M, "block": block, "us": round(us, 2), "floor_us": round(floor_us, 2), "floor_over_us": round(floor_us / us, 3),
+                                "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
                                 "kernel": ws.lib.last_kernel(), "distinct_weight_MB": round(per * n_w / 2 ** 20)})
                 else:
                     tf = 2.0 * M * K * N / us * 1e-6
@@ -970,6 +988,11 @@ def main():
                         row["variants"][f"{tiles[tile]}/{names[variant]}"] = {
                             "us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
                             "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
+                    if tile in (0, 1, 2, 3, 4):
+                        y.zero_()
+                        us, _ = ws.bench.gemm_variant(16, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=n_it, warmup=n_it // 4)
+                        row["variants"][f"{tiles[tile]}/memory_spread"] = {"us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
+                                                                           "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
                     for variant in (4, 5):
                         _, ph = ws.bench.gemm_variant(variant, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=8, warmup=2)
                         row["variants"][f"{tiles[tile]}/{names[variant - 4]}"]["ticks_cvt_barrier_rest"] = ph
@@ -992,7 +1015,14 @@ def main():
             for c_ in codes:
                 ws.lib.weight_release(c_.data_ptr())
             del codes, tiled
-        print(json.dumps({"workload": "prefill_variants", "what": "W8A16 prefill GEMM: the product kernel and the variants measured against it "
+        names = {0: "mfma_only", 1: "+conversions", 3: "+fragment_reads_from_lds", 7: "+barrier", 15: "+lds_stores (all four mid-tile)",
+                 31: "+weight_loads (all four behind the barrier)", 63: "+activation_loads (all four mid-tile) = the whole k-tile, memory instructions in bursts",
+                 1307: "the whole k-tile in the product's order (one memory instruction per token block)",
+                 1507: "the same with 5 fragments read ahead instead of 3", 6: "mfma+fragment_reads+barrier", 17: "mfma+conversions+weight_loads"}
+        ceiling = {"TFLOPs": {names[f]: round(ws.bench.gemm_ablation_tflops(f), 1) for f in names},
+                   "what": "the 128 x 256 tile's k-tile (64 matrix-core instructions per wave, two workgroups per CU, operands in registers or in "
+                           "windows that stay in L2: no HBM traffic) with its ingredients switched on one after the other, ~30-50 ms per figure"}
+        print(json.dumps({"workload": "prefill_variants", "k_tile_ablation": ceiling, "what": "W8A16 prefill GEMM: the product kernel and the variants measured against it "
                           "(us per launch over 600 (M 512) / 200 (M 2048) launches on 8 distinct weights; ticks = shares of wave 0's clock per workgroup)", "rows": rows}))
         return
 

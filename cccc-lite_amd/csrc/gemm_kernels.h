@@ -395,10 +395,12 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         for (int i = 0; i < X_PER_THREAD; i++) { xs[buf][x_store[i]] = xreg[i]; }
     };
 
-    // Order of one k-tile: barrier | request the weights of tile kt + PD | first half of the matrix-core work |
-    // store the next activation tile to LDS and request a later one into its registers | second half.  The LDS stores
-    // and the global loads are thus a whole k-tile of work away from the instructions that wait for
-    // them, and nothing but the barrier and the first fragment read stands between two k-tiles.
+    // Order of one k-tile: barrier | the matrix-core work, token block by token block, with one memory instruction in
+    // front of each block: the NB weight pieces of tile kt + PD with the first blocks, from the middle on the stores of
+    // the next activation tile to LDS, each followed one block later by the load that refills its register.  The LDS
+    // stores and the global loads are thus a whole k-tile of work away from the instructions that wait for them, nothing
+    // but the barrier and the first fragment read stands between two k-tiles, and no burst of memory instructions holds
+    // up the fragment reads queued behind it (all of them in one place each: 1-3 % slower on the benchmark shapes).
     // wcur: tile kt; wnext: the buffer tile kt + PD goes to; xreg: tile kt + 1, replaced by tile kt + 1 + RX.
     auto k_tile = [&](int kt, u32x4* wcur, u32x4* wnext, u32x4* xreg) {
         u32x4 wf[2][NB];
@@ -406,7 +408,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         for (int nb = 0; nb < NB; nb++) { dequant16_fp8<WT, SCALED, AT>(wcur[nb], PAIR && nb >= NBO ? a.w_scale_pair : a.w_scale, wf[0][nb], wf[1][nb]); }
         if constexpr (PD == 1) { __syncthreads(); }          // tile kt is in xs[kt & 1]; the other buffer is free
         else { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }    // LDS order only: the loads of later tiles stay in flight
-        fetch_w(kt + PD, wnext);
+        const int w_k0 = min(kt + PD, n_kt - 1) * (TILED ? 1024 : BK);
+        const int x_k0 = min(kt + 1 + RX, n_kt - 1) * BK;
         const u32x4* xt = xs[kt & 1];
         // token fragments run AHEAD instructions in front of the matrix-core instructions that use them
         constexpr int AHEAD = 3, FRAGS = 2 * MB;
@@ -417,13 +420,16 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
         u32x4 ring[AHEAD + 1];
 #pragma unroll
         for (int f = 0; f < AHEAD; f++) { ring[f] = read_frag(f); }
+        static_assert(NB <= FRAGS && FRAGS / 2 + 1 + X_PER_THREAD <= FRAGS, "one slot per memory instruction");
 #pragma unroll
         for (int f = 0; f < FRAGS; f++)
         {
-            if (f == FRAGS / 2)
+            if (f < NB) { wnext[f] = *(const u32x4*)(w_begin + w_tile_base[f] + w_k0 + (size_t)w_off[f]); }
+            if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { xs[(kt + 1) & 1][x_store[f - FRAGS / 2]] = xreg[f - FRAGS / 2]; }
+            if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD)
             {
-                stage((kt + 1) & 1, xreg);
-                fetch_x(kt + 1 + RX, xreg);
+                const int i = f - FRAGS / 2 - 1;
+                xreg[i] = *(const u32x4*)(x_begin + (size_t)x_k0 * 2 + (size_t)x_off[i]);
             }
             if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
             const frag_t xf = __builtin_bit_cast(frag_t, ring[f % (AHEAD + 1)]);
@@ -437,16 +443,13 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearAr
             }
         }
         // pin the order: the scheduler otherwise pulls every read down to just before its first use
-        __builtin_amdgcn_sched_group_barrier(0x020, NB, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
 #pragma unroll
         for (int f = 0; f < FRAGS; f++)
         {
-            if (f == FRAGS / 2)
-            {
-                __builtin_amdgcn_sched_group_barrier(0x200, X_PER_THREAD, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, X_PER_THREAD, 0);
-            }
+            if (f < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+            if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+            if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
             if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
             __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
         }

@@ -1,6 +1,8 @@
 // Variants of the register-fed FP8 prefill GEMM (csrc/gemm_kernels.h: gemm_mfma_direct_kernel on the tiled copy) that were
 // measured against it and not adopted, kept runnable so that the measurements can be repeated (bench.py --workload
 // prefill_variants).  Built into libcccc_bench.so, which only bench.py loads; the product library does not carry them.
+//   MEMSPREAD  one memory instruction per token block (the order the product kernel adopted from here); without it the
+//           weight loads follow the barrier in one burst and the stores and activation loads sit together mid-tile
 //   SPREAD  the FP8 -> BF16 conversions issued between the matrix-core instructions (the high halves of tile kt while
 //           its first step is multiplied, the low halves of tile kt + 1 during its second step) instead of in a block
 //           in front of the k-tile's barrier
@@ -9,6 +11,7 @@
 //   TRACE   wave 0 of every workgroup adds up the clock ticks it spends (a) converting, which includes the wait for the
 //           weight bytes, (b) at the k-tile's barrier and (c) between the barrier and the end of the k-tile
 // Everything else -- tile shapes, operand layouts, LDS swizzle, prefetch distances, epilogue -- is the product kernel's.
+// gemm_ablation_kernel: the k-tile's ingredients one by one on operands that need no HBM.
 #include "../csrc/gemm_kernels.h"
 #include "../../include/cccc_hip_quant.h"
 #include <hip/hip_runtime.h>
@@ -31,7 +34,7 @@ struct Raster
     int P, Q;
 };
 
-template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE>
+template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, bool MEMSPREAD = false>
 __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a, const int n_tiles, const int m_tiles, float* __restrict__ partial,
                                                               const Raster rast, unsigned long long* __restrict__ trace)
 {
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
         }
         __syncthreads();
         if constexpr (TRACE) { c2 = ticks(); }
-        if constexpr (!SPREAD) { fetch_w(kt + 1, wnext); }
+        if constexpr (!SPREAD && !MEMSPREAD) { fetch_w(kt + 1, wnext); }
         const u32x4* xt = xs[kt & 1];
         auto read_frag = [&](int f) {
             const int row = (f % MB) * 16 + i16;
@@ -155,7 +158,23 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
         for (int f = 0; f < FRAGS; f++)
         {
             if constexpr (SPREAD) { __builtin_amdgcn_sched_barrier(0); }
-            if (f == FRAGS / 2)
+            if constexpr (MEMSPREAD)
+            {
+                // one memory instruction per token block: the weight pieces from the start, the stores from the middle, each
+                // activation load one block behind the store that frees its register
+                if (f < NB)
+                {
+                    const int k0 = min(kt + 1, n_kt - 1) * 1024;
+                    wnext[f] = *(const u32x4*)(w_begin + w_tile_base[f] + k0 + (size_t)w_off);
+                }
+                if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { xs[(kt + 1) & 1][x_store[f - FRAGS / 2]] = xreg[f - FRAGS / 2]; }
+                if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD)
+                {
+                    const int i = f - FRAGS / 2 - 1;
+                    xreg[i] = *(const u32x4*)(x_begin + (size_t)(min(kt + 2, n_kt - 1) * BK) * 2 + (size_t)x_off[i]);
+                }
+            }
+            if (!MEMSPREAD && f == FRAGS / 2)
             {
                 stage((kt + 1) & 1);
                 fetch_x(kt + 2);
@@ -194,6 +213,20 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
             }
         }
         if constexpr (SPREAD) { __builtin_amdgcn_sched_barrier(0); }
+        else if constexpr (MEMSPREAD)
+        {
+            static_assert(FRAGS / 2 + 1 + X_PER_THREAD <= FRAGS && NB <= FRAGS, "spread slots");
+            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+            for (int f = 0; f < FRAGS; f++)
+            {
+                if (f < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+                if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+                if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+                if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+                __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
+            }
+        }
         else
         {
             __builtin_amdgcn_sched_group_barrier(0x020, NB, 0);
@@ -270,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
     }
 }
 
-template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE>
+template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, bool MEMSPREAD = false>
 void launch_variant(const LinearArgs& a, int splits, float* partial, unsigned long long* trace, unsigned* n_wgs)
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
@@ -278,12 +311,26 @@ void launch_variant(const LinearArgs& a, int splits, float* partial, unsigned lo
     const Raster rast = { 4, 2 };
     const unsigned gx = RAST ? 8u * ((m_tiles + rast.P - 1) / rast.P) * ((n_tiles + rast.Q - 1) / rast.Q) : (unsigned)(((n_tiles + 7) & ~7) * m_tiles);
     *n_wgs = gx * (unsigned)splits;
-    gemm_variant_kernel<SCALED, MB, SPLIT, NB, SPREAD, RAST, TRACE><<<dim3(gx, splits), 256, 0, nullptr>>>(a, n_tiles, m_tiles, partial, rast, trace);
+    gemm_variant_kernel<SCALED, MB, SPLIT, NB, SPREAD, RAST, TRACE, MEMSPREAD><<<dim3(gx, splits), 256, 0, nullptr>>>(a, n_tiles, m_tiles, partial, rast, trace);
     if (SPLIT) { launch_splitk_combine<DT_BF16>(partial, splits, a, nullptr); }
 }
 
 // tile: 0 = 128 tokens x 256 features, 1 = 64 x 192, 2 = 128 x 256 with the k range split in four, 3 = 64 x 256,
 // 4 = 128 x 192, 5 = 128 x 256 split in two, 6 = 64 x 256 split in two
+// the memory instructions of a k-tile one per token block (tiles 0, 1, 3, 4 and the k split of 4)
+bool launch_tile_memspread(int tile, const LinearArgs& a, float* partial, unsigned* n_wgs)
+{
+    switch (tile)
+    {
+    case 0: launch_variant<false, 8, false, 4, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
+    case 1: launch_variant<false, 4, false, 3, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
+    case 2: launch_variant<false, 8, true, 4, false, false, false, true>(a, 4, partial, nullptr, n_wgs); return true;
+    case 3: launch_variant<false, 4, false, 4, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
+    case 4: launch_variant<false, 8, false, 3, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
+    default: return false;
+    }
+}
+
 template <bool SPREAD, bool RAST, bool TRACE>
 bool launch_tile(int tile, bool scaled, const LinearArgs& a, float* partial, unsigned long long* trace, unsigned* n_wgs)
 {
@@ -304,6 +351,166 @@ bool launch_tile(int tile, bool scaled, const LinearArgs& a, float* partial, uns
     case 6: launch_variant<false, 4, true, 4, SPREAD, RAST, TRACE>(a, 2, partial, trace, n_wgs); return true;
     default: return false;
     }
+}
+
+// What the k-tile of the 128 x 256 tile costs piece by piece: its 64 matrix-core instructions per wave (32 accumulator
+// blocks, two workgroups per CU) on operands that never leave the registers, then with the other ingredients of the
+// product loop switched on one by one (FLAGS):
+//   1  CVT   the k-tile's sixteen FP8 -> BF16 dword conversions, on raw words that change every trip
+//   2  LDSR  the sixteen activation fragments read from LDS, three instructions ahead of their use, as the product does
+//   4  BAR   the workgroup barrier of the k-tile
+//   8  LDSW  the four 16-byte stores per thread of the next activation tile
+//   16 GW    the four 16-byte weight loads per lane (KiB-contiguous per wave, from a 4 MiB window that stays in L2)
+//   32 GX    the four 16-byte activation loads per thread (from a 1 MiB window)
+// No result is meaningful; the operands are finite and the accumulators are kept alive by a store that never happens.
+// SCHED: 0 = memory instructions in bursts (the weight loads behind the barrier, the stores and the activation loads in
+// the middle of the k-tile); bit 0 = the four stores one per token block from the middle on; bit 1 = the four weight
+// loads one per token block from the start on; bit 2 = the activation loads one per token block behind the stores;
+// 7 = the product kernel's order.  AHEAD: fragments read ahead of their use.
+template <int FLAGS, int AHEAD = 3, int SCHED = 0>
+__global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, const uint32_t seed, const uint8_t* __restrict__ wbuf,
+                                                               const uint8_t* __restrict__ xbuf, float* __restrict__ sink)
+{
+    constexpr bool CVT = FLAGS & 1, LDSR = FLAGS & 2, BAR = FLAGS & 4, LDSW = FLAGS & 8, GW = FLAGS & 16, GX = FLAGS & 32;
+    constexpr int MB = 8, NB = 4, CPR = 8, BTOK = 128, X_PER_THREAD = 4, FRAGS = 2 * MB;
+    constexpr bool ST1 = SCHED & 1, WL1 = SCHED & 2, XL1 = SCHED & 4;
+    __shared__ u32x4 xs[2][BTOK * CPR];
+    const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    f32x4 acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { acc[mb][nb] = f32x4{ 0.0f, 0.0f, 0.0f, 0.0f }; }
+    u32x4 raw[NB], wf[2][NB], xreg[X_PER_THREAD], xconst[4];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+    {
+        const uint32_t r = (seed + tid * 7u + nb) & 0x3b3b3b3bu;           // small finite E5M2 codes
+        raw[nb] = u32x4{ r, r ^ 0x01010101u, r ^ 0x02020202u, r ^ 0x03030303u };
+        wf[0][nb] = u32x4{ 0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u };
+        wf[1][nb] = wf[0][nb];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+    {
+        xconst[i] = u32x4{ 0x3a003a00u + i, 0x3a003a00u, 0x3a003a00u, 0x3a003a00u };
+        xreg[i] = xconst[i];
+    }
+    int x_store[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; i++)
+    {
+        const int q = tid + i * 256;
+        x_store[i] = (q / CPR) * CPR + swizzled_chunk_n<CPR>(q / CPR, q % CPR);
+        xs[0][x_store[i]] = xconst[i];
+        xs[1][x_store[i]] = xconst[i];
+    }
+    __syncthreads();
+    const uint8_t* const w_wave = wbuf + (size_t)((blockIdx.x * 4 + wave) & 15) * (256 << 10) + (size_t)lane * 16;      // 16 windows of 256 KiB
+    const uint8_t* const x_wg = xbuf + (size_t)(blockIdx.x & 7) * (128 << 10) + (size_t)tid * 16;                     // 8 windows of 128 KiB
+    for (int t = 0; t < trips; t++)
+    {
+        if constexpr (CVT)
+        {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+            {
+                if constexpr (!GW) { raw[nb][0] ^= (uint32_t)(t & 1); }
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                {
+                    bf16x2 p, q;
+                    fp8x4_to_bf16<DT_E5M2, false>(raw[nb][d] & 0x3b3b3b3bu, 1.0f, p, q);
+                    wf[d / 2][nb][2 * (d & 1)] = __builtin_bit_cast(uint32_t, p);
+                    wf[d / 2][nb][2 * (d & 1) + 1] = __builtin_bit_cast(uint32_t, q);
+                }
+            }
+        }
+        if constexpr (BAR) { __syncthreads(); }
+        u32x4 rawn[NB];
+        auto load_w = [&](int nb) { rawn[nb] = *(const u32x4*)(w_wave + (size_t)(((t + 1) & 15) * NB + nb) * 4096 + (size_t)(nb * 1024)); };
+        auto store_x = [&](int i) { xs[(t + 1) & 1][x_store[i]] = xreg[i] & u32x4{ 0x3b7f3b7fu, 0x3b7f3b7fu, 0x3b7f3b7fu, 0x3b7f3b7fu }; };
+        auto load_x = [&](int i) { xreg[i] = *(const u32x4*)(x_wg + (size_t)((t + 2) & 7) * 16384 + (size_t)i * 4096); };
+        if constexpr (GW && !WL1)
+        {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) { load_w(nb); }
+        }
+        const u32x4* xt = xs[t & 1];
+        auto read_frag = [&](int f) {
+            if constexpr (!LDSR) { return xconst[f % 4]; }
+            const int row = (f % MB) * 16 + i16;
+            return xt[row * CPR + swizzled_chunk_n<CPR>(row, 2 * g + f / MB)];
+        };
+        u32x4 ring[AHEAD + 1];
+#pragma unroll
+        for (int f = 0; f < AHEAD; f++) { ring[f] = read_frag(f); }
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++)
+        {
+            if constexpr (GW && WL1) { if (f < NB) { load_w(f); } }
+            if (f == FRAGS / 2)
+            {
+                if constexpr (LDSW && !ST1)
+                {
+#pragma unroll
+                    for (int i = 0; i < X_PER_THREAD; i++) { store_x(i); }
+                }
+                if constexpr (GX && !XL1)
+                {
+#pragma unroll
+                    for (int i = 0; i < X_PER_THREAD; i++) { load_x(i); }
+                }
+            }
+            if constexpr (LDSW && ST1) { if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { store_x(f - FRAGS / 2); } }
+            if constexpr (GX && XL1) { if (f >= FRAGS / 2 + (ST1 ? 1 : 0) && f < FRAGS / 2 + (ST1 ? 1 : 0) + X_PER_THREAD) { load_x(f - FRAGS / 2 - (ST1 ? 1 : 0)); } }
+            if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
+            const bf16x8 xf = __builtin_bit_cast(bf16x8, ring[f % (AHEAD + 1)]);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+            {
+                acc[f % MB][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[f / MB][nb]), xf, acc[f % MB][nb], 0, 0, 0);
+            }
+        }
+        if constexpr (GW)
+        {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) { raw[nb] = rawn[nb]; }
+        }
+        if constexpr (LDSR)
+        {
+            // pin the order written above: the scheduler otherwise sinks every read to just before its use
+            if constexpr (GW && !WL1) { __builtin_amdgcn_sched_group_barrier(0x020, NB, 0); }
+            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+            for (int f = 0; f < FRAGS; f++)
+            {
+                if constexpr (GW && WL1) { if (f < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
+                if (f == FRAGS / 2)
+                {
+                    if constexpr (LDSW && !ST1) { __builtin_amdgcn_sched_group_barrier(0x200, X_PER_THREAD, 0); }
+                    if constexpr (GX && !XL1) { __builtin_amdgcn_sched_group_barrier(0x020, X_PER_THREAD, 0); }
+                }
+                if constexpr (LDSW && ST1) { if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); } }
+                if constexpr (GX && XL1) { if (f >= FRAGS / 2 + (ST1 ? 1 : 0) && f < FRAGS / 2 + (ST1 ? 1 : 0) + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
+                if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+                __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
+            }
+        }
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { total += acc[mb][nb][0] + acc[mb][nb][1] + acc[mb][nb][2] + acc[mb][nb][3]; }
+    if (total == -1.0f) { sink[0] = total + (float)xreg[0][0]; }           // keeps everything alive; never true for these operands
+}
+
+template <int FLAGS, int AHEAD = 3, int SCHED = 0>
+void launch_ablation(int wgs, int trips, uint32_t seed, const uint8_t* wbuf, const uint8_t* xbuf, float* sink)
+{
+    gemm_ablation_kernel<FLAGS, AHEAD, SCHED><<<wgs, 256, 0, nullptr>>>(trips, seed, wbuf, xbuf, sink);
 }
 
 // the product kernel itself with a tile shape, k split and prefetch distance of the caller's choice
@@ -351,12 +558,79 @@ extern "C" {
 
 // Times `iters` launches of one variant on the tiled copies W_tiled[0 .. n_w) of E5M2 weights [n_out][K] (rotated),
 // BF16 activations X [tokens][K], BF16 output Y [tokens][n_out] (n_out and tokens multiples of the tile).
-// variant: bit 0 = SPREAD, bit 1 = RAST (4 x 2), bit 2 = TRACE; 8 = the product entry (hip_quant_gemm, W_tiled then holds
+// variant: bit 0 = SPREAD, bit 1 = RAST (4 x 2), bit 2 = TRACE; 16 = the memory instructions spread; 8 = the product entry (hip_quant_gemm, W_tiled then holds
 // the row-major weights whose tiled copies are registered) in the same loop.  tile: see launch_tile.  inv_scale != 1: the scaled
 // conversion (tile 0, no raster, no trace).  partial: tokens * n_out * 4 floats for tile 2.  Returns microseconds per
 // launch (the combine launch of tile 2 included) or < 0; with TRACE, phases[0..3] receive the averages over all
 // workgroups of the ticks spent converting (and waiting for weight bytes), at the barrier, in the rest of the k-tiles,
 // and in the whole kernel.
+// Microseconds per launch of gemm_ablation_kernel<flags>: 2 workgroups per CU, `trips` k-tiles per wave (each 64
+// instructions of 16384 FLOPs), `launches` launches after two of warm-up.  flags: one of 0, 1, 3, 7, 15, 31, 63 (each adds
+// one ingredient to the one before) or 2, 4, 16, 18 (single ingredients on the bare loop).
+// FLOPs per launch = *n_workgroups * 4 * trips * 64 * 16384.
+double cccc_bench_gemm_ablation(int flags, int trips, int launches, int* n_workgroups)
+{
+    if (trips <= 0 || launches <= 0 || !n_workgroups) { return -1.0; }
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { return -1.0; }
+    const int wgs = 2 * prop.multiProcessorCount;
+    *n_workgroups = wgs;
+    uint8_t* mem = nullptr;
+    const size_t w_bytes = (size_t)16 * (256 << 10) + (1 << 20), x_bytes = (size_t)8 * (128 << 10) + (1 << 20);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipMalloc(&mem, w_bytes + x_bytes + 256) != hipSuccess || hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -3.0; }
+    (void)hipMemset(mem, 0x3a, w_bytes + x_bytes + 256);          // finite FP8 codes and BF16 values
+    float* sink = (float*)(mem + w_bytes + x_bytes);
+    bool ok = true;
+    for (int i = 0; i < launches + 2 && ok; i++)
+    {
+        if (i == 2) { (void)hipEventRecord(e0, nullptr); }
+        const uint32_t seed = 0x12345u + i;
+        switch (flags)
+        {
+        case 0: launch_ablation<0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1: launch_ablation<1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 3: launch_ablation<3>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 7: launch_ablation<7>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 15: launch_ablation<15>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 31: launch_ablation<31>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 63: launch_ablation<63>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 2: launch_ablation<2>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4: launch_ablation<4>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 16: launch_ablation<16>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 17: launch_ablation<17>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 6: launch_ablation<6>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        // the whole k-tile under other schedules: 1000 + 100 * AHEAD + SCHED
+        case 1301: launch_ablation<63, 3, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1302: launch_ablation<63, 3, 2>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1303: launch_ablation<63, 3, 3>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1307: launch_ablation<63, 3, 7>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1500: launch_ablation<63, 5, 0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1503: launch_ablation<63, 5, 3>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1507: launch_ablation<63, 5, 7>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 1200: launch_ablation<63, 2, 0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 2301: launch_ablation<15, 3, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;      // up to the stores only
+        case 2501: launch_ablation<15, 5, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 2500: launch_ablation<15, 5, 0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        default: ok = false; break;
+        }
+    }
+    (void)hipEventRecord(e1, nullptr);
+    double result = -2.0;
+    if (ok && hipEventSynchronize(e1) == hipSuccess && hipGetLastError() == hipSuccess)
+    {
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        result = (double)ms * 1000.0 / launches;
+    }
+    (void)hipDeviceSynchronize();
+    (void)hipFree(mem);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return result;
+}
+
 double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, const void* X, void* Y, int n_out, int tokens, int K,
                                float inv_scale, float* partial, int iters, int warmup, double* phases)
 {
@@ -402,6 +676,7 @@ double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, c
         case 3: ok = launch_tile<true, true, false>(tile, scaled, a, partial, trace, &n_wgs); break;
         case 4: ok = launch_tile<false, false, true>(tile, scaled, a, partial, trace, &n_wgs); break;
         case 5: ok = launch_tile<true, false, true>(tile, scaled, a, partial, trace, &n_wgs); break;
+        case 16: ok = !scaled && launch_tile_memspread(tile, a, partial, &n_wgs); break;
         case 8:
             ok = hip_quant_gemm(1, 0, n_out, tokens, K, 1.0f, a.W, (int)DT_E5M2, K, inv_scale, X, (int)DT_BF16, K, 1.0f, 0.0f, Y, (int)DT_BF16, n_out, 0.0f,
                                 nullptr, nullptr, 0) == 0;
