@@ -988,11 +988,13 @@ def main():
                         row["variants"][f"{tiles[tile]}/{names[variant]}"] = {
                             "us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
                             "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
-                    if tile in (0, 1, 2, 3, 4):
+                    for code, label in ((16, "memory_spread"), (17, "memory_spread_wide"), (18, "memory_spread_weights_first")):
+                        if tile not in (0, 1, 2, 3, 4):
+                            continue
                         y.zero_()
-                        us, _ = ws.bench.gemm_variant(16, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=n_it, warmup=n_it // 4)
-                        row["variants"][f"{tiles[tile]}/memory_spread"] = {"us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
-                                                                           "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
+                        us, _ = ws.bench.gemm_variant(code, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=n_it, warmup=n_it // 4)
+                        row["variants"][f"{tiles[tile]}/{label}"] = {"us": round(us, 2), "equal_to_block_variant": bool(torch.equal(y, y_block)),
+                                                                     "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
                     for variant in (4, 5):
                         _, ph = ws.bench.gemm_variant(variant, tile, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=8, warmup=2)
                         row["variants"][f"{tiles[tile]}/{names[variant - 4]}"]["ticks_cvt_barrier_rest"] = ph

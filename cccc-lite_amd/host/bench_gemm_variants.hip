@@ -34,7 +34,7 @@ struct Raster
     int P, Q;
 };
 
-template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, bool MEMSPREAD = false>
+template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, int MEMSPREAD = 0>
 __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a, const int n_tiles, const int m_tiles, float* __restrict__ partial,
                                                               const Raster rast, unsigned long long* __restrict__ trace)
 {
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
         }
         __syncthreads();
         if constexpr (TRACE) { c2 = ticks(); }
-        if constexpr (!SPREAD && !MEMSPREAD) { fetch_w(kt + 1, wnext); }
+        if constexpr (!SPREAD && MEMSPREAD == 0) { fetch_w(kt + 1, wnext); }
         const u32x4* xt = xs[kt & 1];
         auto read_frag = [&](int f) {
             const int row = (f % MB) * 16 + i16;
@@ -158,23 +158,26 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
         for (int f = 0; f < FRAGS; f++)
         {
             if constexpr (SPREAD) { __builtin_amdgcn_sched_barrier(0); }
-            if constexpr (MEMSPREAD)
+            if constexpr (MEMSPREAD != 0)
             {
-                // one memory instruction per token block: the weight pieces from the start, the stores from the middle, each
-                // activation load one block behind the store that frees its register
-                if (f < NB)
+                // one memory instruction per token block.  1: the weight pieces with the first blocks, the stores from the
+                // middle on, each activation load one block behind the store that frees its register; 2: weights, stores
+                // and loads each spread over the whole k-tile; 3: weights first, stores and loads spread over the whole k-tile
+                constexpr int WS = MEMSPREAD == 2 ? FRAGS / NB : 1;
+                constexpr int S0 = MEMSPREAD == 1 ? FRAGS / 2 : 2, SS = MEMSPREAD == 1 ? 1 : 4;
+                if (f % WS == 0 && f / WS < NB)
                 {
                     const int k0 = min(kt + 1, n_kt - 1) * 1024;
-                    wnext[f] = *(const u32x4*)(w_begin + w_tile_base[f] + k0 + (size_t)w_off);
+                    wnext[f / WS] = *(const u32x4*)(w_begin + w_tile_base[f / WS] + k0 + (size_t)w_off);
                 }
-                if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { xs[(kt + 1) & 1][x_store[f - FRAGS / 2]] = xreg[f - FRAGS / 2]; }
-                if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD)
+                if (f >= S0 && (f - S0) % SS == 0 && (f - S0) / SS < X_PER_THREAD) { xs[(kt + 1) & 1][x_store[(f - S0) / SS]] = xreg[(f - S0) / SS]; }
+                if (f >= S0 + 1 && (f - S0 - 1) % SS == 0 && (f - S0 - 1) / SS < X_PER_THREAD)
                 {
-                    const int i = f - FRAGS / 2 - 1;
+                    const int i = (f - S0 - 1) / SS;
                     xreg[i] = *(const u32x4*)(x_begin + (size_t)(min(kt + 2, n_kt - 1) * BK) * 2 + (size_t)x_off[i]);
                 }
             }
-            if (!MEMSPREAD && f == FRAGS / 2)
+            if (MEMSPREAD == 0 && f == FRAGS / 2)
             {
                 stage((kt + 1) & 1);
                 fetch_x(kt + 2);
@@ -213,16 +216,18 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
             }
         }
         if constexpr (SPREAD) { __builtin_amdgcn_sched_barrier(0); }
-        else if constexpr (MEMSPREAD)
+        else if constexpr (MEMSPREAD != 0)
         {
-            static_assert(FRAGS / 2 + 1 + X_PER_THREAD <= FRAGS && NB <= FRAGS, "spread slots");
+            constexpr int WS = MEMSPREAD == 2 ? FRAGS / NB : 1;
+            constexpr int S0 = MEMSPREAD == 1 ? FRAGS / 2 : 2, SS = MEMSPREAD == 1 ? 1 : 4;
+            static_assert(S0 + 1 + (X_PER_THREAD - 1) * SS < FRAGS && (NB - 1) * WS < FRAGS, "spread slots");
             __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
 #pragma unroll
             for (int f = 0; f < FRAGS; f++)
             {
-                if (f < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
-                if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
-                if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+                if (f % WS == 0 && f / WS < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+                if (f >= S0 && (f - S0) % SS == 0 && (f - S0) / SS < X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+                if (f >= S0 + 1 && (f - S0 - 1) % SS == 0 && (f - S0 - 1) / SS < X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
                 if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
                 __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
             }
@@ -303,7 +308,7 @@ __global__ __launch_bounds__(256, 2) void gemm_variant_kernel(const LinearArgs a
     }
 }
 
-template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, bool MEMSPREAD = false>
+template <bool SCALED, int MB, bool SPLIT, int NB, bool SPREAD, bool RAST, bool TRACE, int MEMSPREAD = 0>
 void launch_variant(const LinearArgs& a, int splits, float* partial, unsigned long long* trace, unsigned* n_wgs)
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
@@ -318,15 +323,16 @@ void launch_variant(const LinearArgs& a, int splits, float* partial, unsigned lo
 // tile: 0 = 128 tokens x 256 features, 1 = 64 x 192, 2 = 128 x 256 with the k range split in four, 3 = 64 x 256,
 // 4 = 128 x 192, 5 = 128 x 256 split in two, 6 = 64 x 256 split in two
 // the memory instructions of a k-tile one per token block (tiles 0, 1, 3, 4 and the k split of 4)
+template <int MODE>
 bool launch_tile_memspread(int tile, const LinearArgs& a, float* partial, unsigned* n_wgs)
 {
     switch (tile)
     {
-    case 0: launch_variant<false, 8, false, 4, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
-    case 1: launch_variant<false, 4, false, 3, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
-    case 2: launch_variant<false, 8, true, 4, false, false, false, true>(a, 4, partial, nullptr, n_wgs); return true;
-    case 3: launch_variant<false, 4, false, 4, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
-    case 4: launch_variant<false, 8, false, 3, false, false, false, true>(a, 1, partial, nullptr, n_wgs); return true;
+    case 0: launch_variant<false, 8, false, 4, false, false, false, MODE>(a, 1, partial, nullptr, n_wgs); return true;
+    case 1: launch_variant<false, 4, false, 3, false, false, false, MODE>(a, 1, partial, nullptr, n_wgs); return true;
+    case 2: launch_variant<false, 8, true, 4, false, false, false, MODE>(a, 4, partial, nullptr, n_wgs); return true;
+    case 3: launch_variant<false, 4, false, 4, false, false, false, MODE>(a, 1, partial, nullptr, n_wgs); return true;
+    case 4: launch_variant<false, 8, false, 3, false, false, false, MODE>(a, 1, partial, nullptr, n_wgs); return true;
     default: return false;
     }
 }
@@ -367,9 +373,9 @@ bool launch_tile(int tile, bool scaled, const LinearArgs& a, float* partial, uns
 // the middle of the k-tile); bit 0 = the four stores one per token block from the middle on; bit 1 = the four weight
 // loads one per token block from the start on; bit 2 = the activation loads one per token block behind the stores;
 // 7 = the product kernel's order.  AHEAD: fragments read ahead of their use.
-template <int FLAGS, int AHEAD = 3, int SCHED = 0>
-__global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, const uint32_t seed, const uint8_t* __restrict__ wbuf,
-                                                               const uint8_t* __restrict__ xbuf, float* __restrict__ sink)
+template <int FLAGS, int AHEAD, int SCHED, int WS = 1, int S0 = 8, int SS = 1>
+__device__ __forceinline__ void gemm_ablation_body(const int trips, const uint32_t seed, const uint8_t* __restrict__ wbuf,
+                                                   const uint8_t* __restrict__ xbuf, float* __restrict__ sink)
 {
     constexpr bool CVT = FLAGS & 1, LDSR = FLAGS & 2, BAR = FLAGS & 4, LDSW = FLAGS & 8, GW = FLAGS & 16, GX = FLAGS & 32;
     constexpr int MB = 8, NB = 4, CPR = 8, BTOK = 128, X_PER_THREAD = 4, FRAGS = 2 * MB;
@@ -449,7 +455,7 @@ __global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, 
 #pragma unroll
         for (int f = 0; f < FRAGS; f++)
         {
-            if constexpr (GW && WL1) { if (f < NB) { load_w(f); } }
+            if constexpr (GW && WL1) { if (f % WS == 0 && f / WS < NB) { load_w(f / WS); } }
             if (f == FRAGS / 2)
             {
                 if constexpr (LDSW && !ST1)
@@ -463,8 +469,8 @@ __global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, 
                     for (int i = 0; i < X_PER_THREAD; i++) { load_x(i); }
                 }
             }
-            if constexpr (LDSW && ST1) { if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { store_x(f - FRAGS / 2); } }
-            if constexpr (GX && XL1) { if (f >= FRAGS / 2 + (ST1 ? 1 : 0) && f < FRAGS / 2 + (ST1 ? 1 : 0) + X_PER_THREAD) { load_x(f - FRAGS / 2 - (ST1 ? 1 : 0)); } }
+            if constexpr (LDSW && ST1) { if (f >= S0 && (f - S0) % SS == 0 && (f - S0) / SS < X_PER_THREAD) { store_x((f - S0) / SS); } }
+            if constexpr (GX && XL1) { if (f >= S0 + 1 && (f - S0 - 1) % SS == 0 && (f - S0 - 1) / SS < X_PER_THREAD) { load_x((f - S0 - 1) / SS); } }
             if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
             const bf16x8 xf = __builtin_bit_cast(bf16x8, ring[f % (AHEAD + 1)]);
 #pragma unroll
@@ -486,14 +492,14 @@ __global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, 
 #pragma unroll
             for (int f = 0; f < FRAGS; f++)
             {
-                if constexpr (GW && WL1) { if (f < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
+                if constexpr (GW && WL1) { if (f % WS == 0 && f / WS < NB) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
                 if (f == FRAGS / 2)
                 {
                     if constexpr (LDSW && !ST1) { __builtin_amdgcn_sched_group_barrier(0x200, X_PER_THREAD, 0); }
                     if constexpr (GX && !XL1) { __builtin_amdgcn_sched_group_barrier(0x020, X_PER_THREAD, 0); }
                 }
-                if constexpr (LDSW && ST1) { if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); } }
-                if constexpr (GX && XL1) { if (f >= FRAGS / 2 + (ST1 ? 1 : 0) && f < FRAGS / 2 + (ST1 ? 1 : 0) + X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
+                if constexpr (LDSW && ST1) { if (f >= S0 && (f - S0) % SS == 0 && (f - S0) / SS < X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); } }
+                if constexpr (GX && XL1) { if (f >= S0 + 1 && (f - S0 - 1) % SS == 0 && (f - S0 - 1) / SS < X_PER_THREAD) { __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); } }
                 if (f + AHEAD < FRAGS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
                 __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
             }
@@ -507,10 +513,17 @@ __global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, 
     if (total == -1.0f) { sink[0] = total + (float)xreg[0][0]; }           // keeps everything alive; never true for these operands
 }
 
-template <int FLAGS, int AHEAD = 3, int SCHED = 0>
+template <int FLAGS, int AHEAD = 3, int SCHED = 0, int WS = 1, int S0 = 8, int SS = 1>
+__global__ __launch_bounds__(256, 2) void gemm_ablation_kernel(const int trips, const uint32_t seed, const uint8_t* __restrict__ wbuf,
+                                                               const uint8_t* __restrict__ xbuf, float* __restrict__ sink)
+{
+    gemm_ablation_body<FLAGS, AHEAD, SCHED, WS, S0, SS>(trips, seed, wbuf, xbuf, sink);
+}
+
+template <int FLAGS, int AHEAD = 3, int SCHED = 0, int WS = 1, int S0 = 8, int SS = 1>
 void launch_ablation(int wgs, int trips, uint32_t seed, const uint8_t* wbuf, const uint8_t* xbuf, float* sink)
 {
-    gemm_ablation_kernel<FLAGS, AHEAD, SCHED><<<wgs, 256, 0, nullptr>>>(trips, seed, wbuf, xbuf, sink);
+    gemm_ablation_kernel<FLAGS, AHEAD, SCHED, WS, S0, SS><<<wgs, 256, 0, nullptr>>>(trips, seed, wbuf, xbuf, sink);
 }
 
 // the product kernel itself with a tile shape, k split and prefetch distance of the caller's choice
@@ -558,7 +571,7 @@ extern "C" {
 
 // Times `iters` launches of one variant on the tiled copies W_tiled[0 .. n_w) of E5M2 weights [n_out][K] (rotated),
 // BF16 activations X [tokens][K], BF16 output Y [tokens][n_out] (n_out and tokens multiples of the tile).
-// variant: bit 0 = SPREAD, bit 1 = RAST (4 x 2), bit 2 = TRACE; 16 = the memory instructions spread; 8 = the product entry (hip_quant_gemm, W_tiled then holds
+// variant: bit 0 = SPREAD, bit 1 = RAST (4 x 2), bit 2 = TRACE; 16 / 17 / 18 = the memory instructions spread (three placements); 8 = the product entry (hip_quant_gemm, W_tiled then holds
 // the row-major weights whose tiled copies are registered) in the same loop.  tile: see launch_tile.  inv_scale != 1: the scaled
 // conversion (tile 0, no raster, no trace).  partial: tokens * n_out * 4 floats for tile 2.  Returns microseconds per
 // launch (the combine launch of tile 2 included) or < 0; with TRACE, phases[0..3] receive the averages over all
@@ -609,6 +622,15 @@ double cccc_bench_gemm_ablation(int flags, int trips, int launches, int* n_workg
         case 1500: launch_ablation<63, 5, 0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
         case 1503: launch_ablation<63, 5, 3>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
         case 1507: launch_ablation<63, 5, 7>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        // the product's order with other slots: weight loads every WS-th token block, stores from block S0 every SS-th
+        case 4001: launch_ablation<63, 3, 7, 2, 8, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4002: launch_ablation<63, 3, 7, 4, 8, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4003: launch_ablation<63, 3, 7, 1, 4, 3>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4004: launch_ablation<63, 3, 7, 1, 11, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4005: launch_ablation<63, 3, 7, 1, 2, 4>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4006: launch_ablation<63, 3, 7, 4, 2, 4>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4007: launch_ablation<63, 3, 7, 2, 7, 2>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
+        case 4008: launch_ablation<63, 3, 7, 1, 4, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
         case 1200: launch_ablation<63, 2, 0>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
         case 2301: launch_ablation<15, 3, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;      // up to the stores only
         case 2501: launch_ablation<15, 5, 1>(wgs, trips, seed, mem, mem + w_bytes, sink); break;
@@ -676,7 +698,9 @@ double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, c
         case 3: ok = launch_tile<true, true, false>(tile, scaled, a, partial, trace, &n_wgs); break;
         case 4: ok = launch_tile<false, false, true>(tile, scaled, a, partial, trace, &n_wgs); break;
         case 5: ok = launch_tile<true, false, true>(tile, scaled, a, partial, trace, &n_wgs); break;
-        case 16: ok = !scaled && launch_tile_memspread(tile, a, partial, &n_wgs); break;
+        case 16: ok = !scaled && launch_tile_memspread<1>(tile, a, partial, &n_wgs); break;
+        case 17: ok = !scaled && launch_tile_memspread<2>(tile, a, partial, &n_wgs); break;
+        case 18: ok = !scaled && launch_tile_memspread<3>(tile, a, partial, &n_wgs); break;
         case 8:
             ok = hip_quant_gemm(1, 0, n_out, tokens, K, 1.0f, a.W, (int)DT_E5M2, K, inv_scale, X, (int)DT_BF16, K, 1.0f, 0.0f, Y, (int)DT_BF16, n_out, 0.0f,
                                 nullptr, nullptr, 0) == 0;
