@@ -285,8 +285,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const LinearArgs a, cons
 // workgroups share a CU and each k-tile carries 64 matrix-core instructions per wave; the k-split launches of a short
 // prompt (one 64-token tile, about one workgroup per CU) are bound by their weight bytes and run a k-tile per memory
 // latency with PD = 1 -- they take PD = 3.
-template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false, int PD = 1>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_direct_kernel(const LinearArgs a_in, const int n_tiles, float* __restrict__ partial)
+template <int WT, bool SCALED, int MB, bool SPLIT, bool TILED, int AT = DT_BF16, int NB = 4, bool PAIR = false, bool SEG = false, int PD = 1, int WGS_PER_CU = 2>
+__global__ __launch_bounds__(256, WGS_PER_CU) void gemm_mfma_direct_kernel(const LinearArgs a_in, const int n_tiles, float* __restrict__ partial)
 {
     static_assert(!PAIR || (NB % 2 == 0 && AT == DT_BF16), "pair: an even number of feature blocks, BF16");
     static_assert(!SEG || !PAIR, "segments: single linears");
@@ -683,7 +683,7 @@ __device__ __forceinline__ u32x4 dequant8_fp4_blocks(uint32_t w, float s_lo, flo
 // PAIR: as in the FP8 kernel -- a.W = gate, a.W_pair = up, two tiled copies of one shape (so the up weight's codes and scale
 // bytes sit at the same offsets behind a.W_pair as the gate's behind a.W); a wave's first NB / 2 feature blocks are gate
 // rows, the others the same rows of up; SwiGLU product in the epilogue, or in the combine launch when the k range is split.
-template <int BLOCK, int MB, bool SPLIT, int NB = 4, bool SEG = false, bool PAIR = false>
+template <int BLOCK, int MB, bool SPLIT, int NB = 4, bool SEG = false, bool PAIR = false, bool MEM_BURSTS = false>
 __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direct_kernel(const LinearArgs a_in, const uint8_t* scales_in, const int n_tiles,
                                                                                         float* __restrict__ partial)
 {
@@ -824,9 +824,12 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
     u32x4 wf_a[NB], wf_b[NB];
     auto k_tile = [&](int kt, int h, const u32x4* wcur, const u32x2* scur, u32x4* wnext, u32x2* snext) {
         __syncthreads();                                     // tile kt is in xs[kt & 1]; the other buffer is free
-        if (h == 0) { fetch_w(kt / 2 + 1, wnext, snext); }
+        if constexpr (MEM_BURSTS) { if (h == 0) { fetch_w(kt / 2 + 1, wnext, snext); } }
         const u32x4* xt = xs[kt & 1];
         constexpr int FRAGS = 2 * MB;
+        static_assert(NB <= FRAGS && FRAGS / 2 + 1 + X_PER_THREAD <= FRAGS, "one token block per memory instruction");
+        const long long w_cc = min(kt / 2 + 1, n_chunks - 1);
+        const int x_k0 = min(kt + 2, n_kt - 1) * BK;
         constexpr int PIECES = 2 * NB;                       // per step
         auto read_frag = [&](int f) {
             const int row = (f % MB) * 16 + i16;
@@ -839,11 +842,39 @@ __global__ __launch_bounds__(256, (MB * NB >= 32) ? 1 : 2) void gemm4_mfma_direc
         for (int f = 0; f < FRAGS; f++)
         {
             __builtin_amdgcn_sched_barrier(0);
-            if (f == FRAGS / 2)
+            if constexpr (MEM_BURSTS)
             {
-                stage((kt + 1) & 1);
-                fetch_x(kt + 2);
-                __builtin_amdgcn_sched_barrier(0);
+                if (f == FRAGS / 2)
+                {
+                    stage((kt + 1) & 1);
+                    fetch_x(kt + 2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            else
+            {
+                // one memory instruction (pair) per token block, as in the FP8 kernel: the next chunk's codes and scales
+                // with the first blocks of a chunk's first half, the stores of the next activation tile from the middle
+                // on, each followed one block later by the load that refills its register
+                if (h == 0 && f < NB)
+                {
+                    wnext[f] = *(const u32x4*)(a.W + w_base[f] + w_cc * 1024 + (size_t)w_off);
+                    const uint8_t* sp = tiled_scales + s_base[f] + w_cc * (16 * NS) + (size_t)s_off;
+                    if constexpr (NS == 8) { snext[f] = *(const u32x2*)sp; }
+                    else { snext[f] = u32x2{ *(const uint32_t*)sp, 0u }; }
+                }
+                if (f >= FRAGS / 2 && f < FRAGS / 2 + X_PER_THREAD)
+                {
+                    const int i = f - FRAGS / 2;
+                    u32x2* dst = (u32x2*)xs[(kt + 1) & 1];
+                    dst[x_store + i * (32 * CPR * 2)] = u32x2{ xreg[i][0], xreg[i][1] };
+                    dst[(x_store ^ 2) + i * (32 * CPR * 2)] = u32x2{ xreg[i][2], xreg[i][3] };
+                }
+                if (f >= FRAGS / 2 + 1 && f < FRAGS / 2 + 1 + X_PER_THREAD)
+                {
+                    const int i = f - FRAGS / 2 - 1;
+                    xreg[i] = *(const u32x4*)(x_begin + (size_t)x_k0 * 2 + (size_t)x_off[i]);
+                }
             }
             if (f + AHEAD < FRAGS) { ring[(f + AHEAD) % (AHEAD + 1)] = read_frag(f + AHEAD); }
             const bf16x8 xf = __builtin_bit_cast(bf16x8, ring[f % (AHEAD + 1)]);

@@ -527,18 +527,19 @@ void launch_ablation(int wgs, int trips, uint32_t seed, const uint8_t* wbuf, con
 }
 
 // the product kernel itself with a tile shape, k split and prefetch distance of the caller's choice
-template <int MB, int NB, bool SPLIT, int PD>
+template <int MB, int NB, bool SPLIT, int PD, int WGS_PER_CU = 2>
 void launch_product_kernel(const LinearArgs& a, int splits, float* partial)
 {
     const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
     const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
     const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, splits);
-    gemm_mfma_direct_kernel<DT_E5M2, false, MB, SPLIT, true, DT_BF16, NB, false, false, PD><<<grid, 256, 0, nullptr>>>(a, n_tiles, SPLIT ? partial : nullptr);
+    gemm_mfma_direct_kernel<DT_E5M2, false, MB, SPLIT, true, DT_BF16, NB, false, false, PD, WGS_PER_CU><<<grid, 256, 0, nullptr>>>(a, n_tiles, SPLIT ? partial : nullptr);
     if (SPLIT) { launch_splitk_combine<DT_BF16>(partial, splits, a, nullptr); }
 }
 
 // tile 100 + 10 * shape + PD: shape 0 = 64 x 192, 1 = 64 x 256, 2 = 128 x 192, 3 = 64 x 256 split 4, 4 = 128 x 256 split 4,
-// 5 = 64 x 256 split 2, 6 = 64 x 256 split 3, 7 = 128 x 192 split 2 ... ; PD 1 .. 3 (128-token tiles: 1 or 2)
+// 5 = 64 x 256 split 2, 6 = 64 x 256 split 3, 7 = 128 x 192 split 2, 8 = 128 x 256 compiled for one workgroup per CU,
+// 9 = the same split 4; PD 1 .. 3 (128-token tiles at two workgroups per CU: 1 or 2)
 bool launch_product_tile(int tile, const LinearArgs& a, float* partial)
 {
     switch (tile)
@@ -559,10 +560,28 @@ bool launch_product_tile(int tile, const LinearArgs& a, float* partial)
     case 153: launch_product_kernel<4, 4, true, 3>(a, 2, partial); return true;
     case 161: launch_product_kernel<4, 4, true, 1>(a, 3, partial); return true;
     case 163: launch_product_kernel<4, 4, true, 3>(a, 3, partial); return true;
+    // 128 x 256 compiled for one workgroup per CU (512 registers per wave): unsplit and split in four
+    case 181: launch_product_kernel<8, 4, false, 1, 1>(a, 1, partial); return true;
+    case 182: launch_product_kernel<8, 4, false, 2, 1>(a, 1, partial); return true;
+    case 183: launch_product_kernel<8, 4, false, 3, 1>(a, 1, partial); return true;
+    case 191: launch_product_kernel<8, 4, true, 1, 1>(a, 4, partial); return true;
+    case 192: launch_product_kernel<8, 4, true, 2, 1>(a, 4, partial); return true;
+    case 193: launch_product_kernel<8, 4, true, 3, 1>(a, 4, partial); return true;
     case 171: launch_product_kernel<8, 3, true, 1>(a, 2, partial); return true;
     case 172: launch_product_kernel<8, 3, true, 2>(a, 2, partial); return true;
     default: return false;
     }
+}
+
+// the FP4 prefill kernel with its memory instructions in bursts (MEM_BURSTS) or one per token block
+template <int MB, int NB, bool SPLIT, bool BURSTS>
+void launch_fp4_kernel(const LinearArgs& a, const uint8_t* scales, int splits, float* partial)
+{
+    const int n_tiles = (a.n_out + 64 * NB - 1) / (64 * NB);
+    const int m_tiles = (a.tokens + MB * 16 - 1) / (MB * 16);
+    const dim3 grid(((n_tiles + 7) & ~7) * m_tiles, splits);
+    gemm4_mfma_direct_kernel<16, MB, SPLIT, NB, false, false, BURSTS><<<grid, 256, 0, nullptr>>>(a, scales, n_tiles, SPLIT ? partial : nullptr);
+    if (SPLIT) { launch_splitk_combine<DT_BF16>(partial, splits, a, nullptr); }
 }
 
 }    // namespace
@@ -648,6 +667,61 @@ double cccc_bench_gemm_ablation(int flags, int trips, int launches, int* n_workg
     }
     (void)hipDeviceSynchronize();
     (void)hipFree(mem);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return result;
+}
+
+// Times the FP4 (block 16) prefill kernel on the tiled copies W_tiled[0 .. n_w) (codes, then the scale bytes behind all
+// code KiBs, as hip_quant_weight_prepare_fp4 writes them) of weights [n_out][K].  shape: 0 = 128 tokens x 256 features
+// (one workgroup per CU), 1 = 64 x 256, 2 = 128 x 192, 3 = 128 x 256 with the k range split in `splits`.  bursts != 0: the
+// memory instructions of a k-tile in two bursts instead of one per token block.  Microseconds per launch or < 0.
+double cccc_bench_gemm4_variant(int shape, int bursts, int splits, int n_w, void** W_tiled, const void* X, void* Y, int n_out, int tokens, int K,
+                                float* partial, int iters, int warmup)
+{
+    if (n_w <= 0 || !W_tiled || !X || !Y || iters <= 0 || K % 128 != 0 || tokens % 128 != 0 || n_out % (shape == 2 ? 192 : 256) != 0) { return -1.0; }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
+    LinearArgs a{};
+    a.X = (const uint16_t*)X;
+    a.Y = (uint16_t*)Y;
+    a.ldw = K;
+    a.ldx = K;
+    a.y_stride_tok = n_out;
+    a.y_stride_out = 1;
+    a.n_out = n_out;
+    a.tokens = tokens;
+    a.K = K;
+    a.w_scale = 1.0f;
+    a.alpha = 1.0f;
+    a.beta = 0.0f;
+    bool ok = true;
+    for (int i = 0; i < warmup + iters && ok; i++)
+    {
+        if (i == warmup) { (void)hipEventRecord(e0, nullptr); }
+        a.W = (const uint8_t*)W_tiled[i % n_w];
+        const uint8_t* scales = a.W + (long long)((n_out + 15) / 16) * (K / 128) * 1024;
+        switch (shape * 2 + (bursts ? 1 : 0))
+        {
+        case 0: launch_fp4_kernel<8, 4, false, false>(a, scales, 1, partial); break;
+        case 1: launch_fp4_kernel<8, 4, false, true>(a, scales, 1, partial); break;
+        case 2: launch_fp4_kernel<4, 4, false, false>(a, scales, 1, partial); break;
+        case 3: launch_fp4_kernel<4, 4, false, true>(a, scales, 1, partial); break;
+        case 4: launch_fp4_kernel<8, 3, false, false>(a, scales, 1, partial); break;
+        case 5: launch_fp4_kernel<8, 3, false, true>(a, scales, 1, partial); break;
+        case 6: launch_fp4_kernel<8, 4, true, false>(a, scales, splits, partial); break;
+        case 7: launch_fp4_kernel<8, 4, true, true>(a, scales, splits, partial); break;
+        default: ok = false; break;
+        }
+    }
+    (void)hipEventRecord(e1, nullptr);
+    double result = -2.0;
+    if (ok && hipEventSynchronize(e1) == hipSuccess && hipGetLastError() == hipSuccess)
+    {
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        result = (double)ms * 1000.0 / iters;
+    }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     return result;
