@@ -1000,13 +1000,13 @@ def main():
                         row["variants"][f"{tiles[tile]}/{names[variant - 4]}"]["ticks_cvt_barrier_rest"] = ph
                 # the product kernel with other tile shapes, k splits and weight prefetch distances (PD k-tiles ahead)
                 shapes = {0: "64x192", 1: "64x256", 2: "128x192", 3: "64x256_split4", 4: "128x256_split4", 5: "64x256_split2", 6: "64x256_split3", 7: "128x192_split2",
-                          8: "128x256_one_wg_per_cu", 9: "128x256_split4_one_wg_per_cu"}
+                          8: "128x256_one_wg_per_cu", 9: "128x256_split4_one_wg_per_cu", 20: "128x128_split4", 21: "128x128"}
                 row["product_kernel_by_tile_and_prefetch"] = {}
-                for code in (101, 102, 103, 111, 112, 113, 121, 122, 131, 132, 133, 141, 151, 153, 161, 163, 171, 172, 181, 182, 183, 191, 192, 193):
-                    if (code // 10) % 10 in (0, 2, 7) and N % 192 != 0:
+                for code in (101, 102, 103, 111, 112, 113, 121, 122, 131, 132, 133, 141, 151, 153, 161, 163, 171, 172, 181, 182, 183, 191, 192, 193, 201, 202, 211):
+                    if code < 200 and (code // 10) % 10 in (0, 2, 7) and N % 192 != 0:
                         continue
                     us, _ = ws.bench.gemm_variant(0, code, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, partial_ptr=partial.data_ptr(), iters=n_it, warmup=n_it // 4)
-                    row["product_kernel_by_tile_and_prefetch"][f"{shapes[(code // 10) % 10]}/pd{code % 10}"] = {
+                    row["product_kernel_by_tile_and_prefetch"][f"{shapes[(code // 10) % 10 if code < 200 else code // 10]}/pd{code % 10}"] = {
                         "us": round(us, 2), "max_abs_diff_to_product": float((y.float() - y_ref.float()).abs().max())}
                 us0, _ = ws.bench.gemm_variant(0, 0, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, inv_scale=SCALED_INV_SCALE, iters=n_it, warmup=n_it // 4)
                 us1, _ = ws.bench.gemm_variant(1, 0, ptrs, x.data_ptr(), y.data_ptr(), N, M, K, inv_scale=SCALED_INV_SCALE, iters=n_it, warmup=n_it // 4)

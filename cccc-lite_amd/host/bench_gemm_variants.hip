@@ -567,6 +567,9 @@ bool launch_product_tile(int tile, const LinearArgs& a, float* partial)
     case 191: launch_product_kernel<8, 4, true, 1, 1>(a, 4, partial); return true;
     case 192: launch_product_kernel<8, 4, true, 2, 1>(a, 4, partial); return true;
     case 193: launch_product_kernel<8, 4, true, 3, 1>(a, 4, partial); return true;
+    case 201: launch_product_kernel<8, 2, true, 1>(a, 4, partial); return true;       // 128 x 128, k split in 4
+    case 202: launch_product_kernel<8, 2, true, 2>(a, 4, partial); return true;
+    case 211: launch_product_kernel<8, 2, false, 1>(a, 1, partial); return true;      // 128 x 128 unsplit
     case 171: launch_product_kernel<8, 3, true, 1>(a, 2, partial); return true;
     case 172: launch_product_kernel<8, 3, true, 2>(a, 2, partial); return true;
     default: return false;
@@ -731,7 +734,8 @@ double cccc_bench_gemm_variant(int variant, int tile, int n_w, void** W_tiled, c
                                float inv_scale, float* partial, int iters, int warmup, double* phases)
 {
     const bool wide3 = tile == 1 || tile == 4 || (tile >= 100 && (tile / 10 == 10 || tile / 10 == 12 || tile / 10 == 17));
-    if (n_w <= 0 || !W_tiled || !X || !Y || iters <= 0 || K % 64 != 0 || tokens % 128 != 0 || n_out % (wide3 ? 192 : 256) != 0) { return -1.0; }
+    const bool narrow = tile >= 200;           // 128-feature tiles
+    if (n_w <= 0 || !W_tiled || !X || !Y || iters <= 0 || K % 64 != 0 || tokens % 128 != 0 || n_out % (wide3 ? 192 : (narrow ? 128 : 256)) != 0) { return -1.0; }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { return -1.0; }
     unsigned long long* trace = nullptr;
