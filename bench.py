@@ -685,45 +685,55 @@ def same_gpu_comparators(ws, weights, K, N, M, max_ops=24):
             y = x @ bf[i % n_bf].T
         t.cuda.synchronize()
         out["bf16_gemm_us"] = round((time.perf_counter() - t0) * 1e6 / (4 * n_bf), 2)
+    ws.keep.append((wsb, bf, x))           # freed with everything else (freeing GBs mid-run slows what is timed next)
     return out
 
 
 def prefill_cases(ws, by_shape):
     """The W8A16 prefill GEMM workload: M in {512, 2048} x the two MLP shapes, with the plain BF16 GEMM
-    of the vendor library (torch.matmul) on the same shape beside it."""
+    of the vendor library (torch.matmul) on the same shape beside it.  Three passes over the four cases -- this build's
+    kernel, the same with a per-tensor multiplier, the vendor GEMM -- because seconds of dense vendor GEMMs, and freeing
+    their operands, depress whatever is timed next by several per cent; nothing is freed until the last case is done."""
     t = ws.torch
-    out = []
-    for (K, N) in ((4096, 12288), (12288, 4096)):
+    cases = [(K, N, M) for (K, N) in ((4096, 12288), (12288, 4096)) for M in (512, 2048)]
+    rows, chains = {}, {}
+    for (K, N, M) in cases:
         weights = by_shape[(K, N)][:16]
-        bf = [t.randn(N, K, device=ws.dev, generator=ws.gen).to(t.bfloat16) for _ in range(4)]
-        for M in (512, 2048):
-            X, Y = ws.activation(M, K), ws.output(M, N)
-            ops = [(W, X, Y, K, N) for W in weights]
-            steps = 40 if M <= 512 else 12                  # 30 ms or more per figure: shorter bursts run at other clocks
-            ms = time_chain(ws, ops, steps, steps // 4, False)
-            us = ms * 1000.0 / (steps * len(ops))
-            tf = 2.0 * M * K * N / us * 1e-6
-            x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
-            for rep in range(2):
-                t.cuda.synchronize()
-                t0 = time.perf_counter()
-                for i in range(16):
-                    y = x @ bf[i % 4].T
-                t.cuda.synchronize()
-                lib_us = (time.perf_counter() - t0) * 1e6 / 16
-            # the same launches with a per-tensor dequantisation multiplier (the route of a weight quantized on load)
-            for W in weights:
-                W.quant_scale = SCALED_INV_SCALE
-            us_scaled = time_chain(ws, ops, steps, steps // 4, False) * 1000.0 / (steps * len(ops))
-            for W in weights:
-                W.quant_scale = 1.0
-            tf_scaled = 2.0 * M * K * N / us_scaled * 1e-6
-            out.append({"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                        "kernel": ws.lib.last_kernel(), "scaled_us": round(us_scaled, 2), "scaled_TFLOPs": round(tf_scaled, 1),
-                        "scaled_frac_of_bf16_mfma_peak": round(tf_scaled / MFMA_BF16_PEAK_TFLOPS, 4), "vendor_bf16_gemm_us": round(lib_us, 2),
-                        "vendor_bf16_gemm_TFLOPs": round(2.0 * M * K * N / lib_us * 1e-6, 1)})
-        del bf
-    return out
+        X, Y = ws.activation(M, K), ws.output(M, N)
+        ops = [(W, X, Y, K, N) for W in weights]
+        steps = 40 if M <= 512 else 12                  # 30 ms or more per figure: shorter bursts run at other clocks
+        chains[(K, N, M)] = (ops, steps, weights)
+        us = time_chain(ws, ops, steps, steps // 4, False) * 1000.0 / (steps * len(ops))
+        tf = 2.0 * M * K * N / us * 1e-6
+        rows[(K, N, M)] = {"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                           "kernel": ws.lib.last_kernel()}
+    # the same launches with a per-tensor dequantisation multiplier (the route of a weight quantized on load)
+    for (K, N, M) in cases:
+        ops, steps, weights = chains[(K, N, M)]
+        for W in weights:
+            W.quant_scale = SCALED_INV_SCALE
+        us_scaled = time_chain(ws, ops, steps, steps // 4, False) * 1000.0 / (steps * len(ops))
+        for W in weights:
+            W.quant_scale = 1.0
+        tf_scaled = 2.0 * M * K * N / us_scaled * 1e-6
+        rows[(K, N, M)].update({"scaled_us": round(us_scaled, 2), "scaled_TFLOPs": round(tf_scaled, 1),
+                                "scaled_frac_of_bf16_mfma_peak": round(tf_scaled / MFMA_BF16_PEAK_TFLOPS, 4)})
+    bf = {}
+    for (K, N, M) in cases:
+        if (K, N) not in bf:
+            bf[(K, N)] = [t.randn(N, K, device=ws.dev, generator=ws.gen).to(t.bfloat16) for _ in range(4)]
+        x = t.randn(M, K, device=ws.dev, generator=ws.gen).to(t.bfloat16)
+        for rep in range(2):
+            t.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(16):
+                y = x @ bf[(K, N)][i % 4].T
+            t.cuda.synchronize()
+            lib_us = (time.perf_counter() - t0) * 1e6 / 16
+        rows[(K, N, M)].update({"vendor_bf16_gemm_us": round(lib_us, 2), "vendor_bf16_gemm_TFLOPs": round(2.0 * M * K * N / lib_us * 1e-6, 1)})
+        ws.keep.append((x, y))
+    ws.keep.append((bf, chains))
+    return [rows[c] for c in cases]
 
 
 LLAMA_SHAPES = [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (4096, 128256)]     # (K, N)
