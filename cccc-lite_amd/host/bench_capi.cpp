@@ -134,7 +134,8 @@ double cccc_bench_fp4_chain(int n_w, void** W, void** S, void* X, void* Y, int n
 }
 
 // Times `reps` passes over every layer's fused gate/up launch of a DecodeModel (RMSNorm + SwiGLU pair, distinct
-// weights per layer) with events on the launch stream; returns the average microseconds per launch or < 0.
+// weights per layer), the pass captured once and replayed as a hipGraph the way the decode step runs, with events on the
+// launch stream; returns the average microseconds per launch or < 0.
 double cccc_decode_bench_gate_up(void* model, int reps)
 {
     DecodeModel* m = (DecodeModel*)model;
@@ -142,10 +143,8 @@ double cccc_decode_bench_gate_up(void* model, int reps)
     if (reps <= 0 || cfg.layers <= 0) { return -2.0; }
     TimingScope timing;
     if (!timing.ok) { return -1.0; }
-    bool ok = true;
-    for (int rep = -1; rep < reps; rep++)    // pass -1 is the warm-up
-    {
-        if (rep == 0) { (void)hipEventRecord(timing.e0, nullptr); }
+    auto one_pass = [&]() -> bool {
+        bool ok = true;
         for (int li = 0; li < cfg.layers; li++)
         {
             Matrix *gate = m->tensor(li, DecodeModel::W_GATE), *up = m->tensor(li, DecodeModel::W_UP);
@@ -162,11 +161,32 @@ double cccc_decode_bench_gate_up(void* model, int reps)
             gu.norm_eps = cfg.eps;
             ok = (hip_quant_linear_fused(&gu) == 0) && ok;
         }
-    }
-    (void)hipEventRecord(timing.e1, nullptr);
-    ok = (hipEventSynchronize(timing.e1) == hipSuccess) && ok;
+        return ok;
+    };
+    if (!one_pass() || hipDeviceSynchronize() != hipSuccess) { return -3.0; }          // warm-up
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (hipStreamCreate(&stream) != hipSuccess) { return -4.0; }
+    hip_quant_set_stream(stream);
+    bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) == hipSuccess;
+    if (ok) { ok = one_pass(); }
+    ok = (hipStreamEndCapture(stream, &graph) == hipSuccess) && ok;
+    hip_quant_set_stream(nullptr);
+    if (ok) { ok = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess; }
+    if (ok) { ok = hipGraphLaunch(exec, stream) == hipSuccess && hipStreamSynchronize(stream) == hipSuccess; }
     float ms = 0;
+    if (ok)
+    {
+        (void)hipEventRecord(timing.e0, stream);
+        for (int rep = 0; rep < reps; rep++) { (void)hipGraphLaunch(exec, stream); }
+        (void)hipEventRecord(timing.e1, stream);
+        ok = hipEventSynchronize(timing.e1) == hipSuccess;
+    }
     if (ok) { (void)hipEventElapsedTime(&ms, timing.e0, timing.e1); }
+    if (exec) { (void)hipGraphExecDestroy(exec); }
+    if (graph) { (void)hipGraphDestroy(graph); }
+    (void)hipStreamDestroy(stream);
     return ok ? (double)ms * 1000.0 / ((double)reps * cfg.layers) : -3.0;
 }
 
