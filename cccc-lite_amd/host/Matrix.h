@@ -2,6 +2,7 @@
 // shared storage: the part of the reference's Matrix (cccc/Matrix.h, cccc/Matrix.cpp) that the
 // quantized linear path touches, HIP only.
 #pragma once
+#include <cstdio>
 #include "MatrixData.h"
 #include <memory>
 #include <vector>
@@ -51,7 +52,11 @@ public:
     // does neither: the scale array and the tiled copy belong to the whole storage, under the storage's own dims.
     void setBlockScaleFromHost(const void* src, int64_t n_scales)
     {
-        if (rows_view_) { return; }
+        if (rows_view_)
+        {
+            fprintf(stderr, "cccc host: setBlockScaleFromHost on a row view is refused (upload the scales through the storage that owns them)\n");
+            return;
+        }
         shared_data_->setBlockScaleFromHost(src, n_scales);
         if (number_ == 1 && channel_ == 1 && getDataType() == FP4_E2M1) { shared_data_->prepareTiled(height_, width_); }
     }
