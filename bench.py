@@ -69,7 +69,7 @@ class BenchLibrary:
         L.cccc_decode_bench_gate_up.restype = ctypes.c_double
         L.cccc_decode_bench_gate_up.argtypes = [vp, i32]
         L.cccc_bench_floor_read.restype = ctypes.c_double
-        L.cccc_bench_floor_read.argtypes = [i32, ctypes.POINTER(vp), ctypes.c_ulonglong, i32, i32, i32]
+        L.cccc_bench_floor_read.argtypes = [i32, ctypes.POINTER(vp), ctypes.c_ulonglong, i32, i32, i32, i32, i32]
         L.cccc_bench_launch_us.restype = ctypes.c_double
         L.cccc_bench_launch_us.argtypes = [i32, i32, i32]
         L.cccc_bench_gemm_ablation.restype = ctypes.c_double
@@ -99,15 +99,22 @@ class BenchLibrary:
             raise RuntimeError(f"gemm variant {variant}/{tile} failed: {us}")
         return us, ([round(phases[j] / phases[3], 4) for j in range(3)] if (variant & 4) and phases[3] > 0 else None)
 
-    def floor_read_us(self, ptrs, nbytes, iters=None, wgs_per_cu=8) -> float:
+    def floor_read_us(self, ptrs, nbytes, iters=None, wgs_per_cu=8, contiguous=False, pipelined=True) -> float:
         """Microseconds per launch of a kernel that only streams `nbytes` with 16-byte loads, rotating over the buffers
-        `ptrs` (host/bench_kernels.hip): the floor of any weight-streaming launch of that size on this GPU."""
+        `ptrs` (host/bench_kernels.hip): the floor of any weight-streaming launch of that size on this GPU.  contiguous:
+        every workgroup reads one contiguous range instead of KiB pieces at a grid stride; pipelined: eight KiB pieces
+        in flight per wave instead of four."""
         n = len(ptrs)
         iters = iters or max(20, min(400, (4 << 30) // max(nbytes, 1)))
-        us = float(self.c.cccc_bench_floor_read(n, (self.ctypes.c_void_p * n)(*ptrs), nbytes, wgs_per_cu, iters, min(5, n)))
+        us = float(self.c.cccc_bench_floor_read(n, (self.ctypes.c_void_p * n)(*ptrs), nbytes, wgs_per_cu, iters, min(5, n), 1 if contiguous else 0, 1 if pipelined else 0))
         if us < 0:
             raise RuntimeError(f"floor read failed: {us}")
         return us
+
+    def floor_us(self, ptrs, nbytes) -> float:
+        """The fastest of the streaming-read forms: 2, 4 or 8 workgroups per CU, pieces at a grid stride or one contiguous
+        range per workgroup, four or eight KiB pieces in flight per wave."""
+        return min(self.floor_read_us(ptrs, nbytes, wgs_per_cu=w, contiguous=c, pipelined=p) for w in (2, 4, 8) for c in (False, True) for p in (False, True))
 
     def launch_us(self, kind=0, n_launches=200, reps=20) -> float:
         """Microseconds per launch of `n_launches` dependent launches inside one hipGraph (0: empty kernel, 1: one wave
@@ -597,7 +604,7 @@ def shape_sweep(ws, by_shape, token_counts, use_graph, comparators=True):
     out = []
     for (K, N) in QWEN_SHAPES:
         weights = by_shape[(K, N)]
-        floor_us = min(ws.bench.floor_read_us([W.data_ptr for W in weights], K * N, wgs_per_cu=w) for w in (2, 8))
+        floor_us = ws.bench.floor_us([W.data_ptr for W in weights], K * N)
         for M in token_counts:
             X, Y = ws.activation(M, K), ws.output(M, N)
             reps = max(1, min(8, (2 << 30) // (K * N * len(weights))))
@@ -758,7 +765,7 @@ def fp4_sweep(ws, token_counts=(1, 4, 16), prefill_tokens=(512, 2048)):
             n_w = max(2, min(48, (768 << 20) // per))
             span = (per + 4095) // 4096 * 4096
             floor_ptrs = [pool.data_ptr() + i * span for i in range(max(1, min(n_w, (800 << 20) // span)))]
-            floor_us = min(ws.bench.floor_read_us(floor_ptrs, per, wgs_per_cu=w) for w in (2, 8))
+            floor_us = ws.bench.floor_us(floor_ptrs, per)
             nib = [t.randint(0, 256, (N, K // 2), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             sc = [t.randint(0x10, 0x40, (N, K // block), dtype=t.uint8, device=ws.dev, generator=ws.gen) for _ in range(n_w)]
             tiled = []
@@ -949,17 +956,19 @@ def main():
         # shapes, FP4 block-16 Llama-3.1-8B shapes), over rotating buffers of at least 512 MiB in total; and what a launch
         # costs when it does nothing (dependent launches inside one hipGraph).
         rows = []
-        sizes = [("fp8", K, N, K * N) for K, N in QWEN_SHAPES] + [("fp4_b16", K, N, K * N // 2 + K * N // 16) for K, N in LLAMA_SHAPES]
+        sizes = ([("fp8", K, N, K * N) for K, N in QWEN_SHAPES] + [("fp8 q,k,v together", 4096, 6144, 4096 * 6144), ("fp8 gate,up together", 4096, 24576, 4096 * 24576)]
+                 + [("fp4_b16", K, N, K * N // 2 + K * N // 16) for K, N in LLAMA_SHAPES])
         pool = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=ws.dev)
         for fmt, K, N, nbytes in sizes:
             span = (nbytes + 4095) // 4096 * 4096
             n_buf = max(1, min(64, (1 << 30) // span))
             ptrs = [pool.data_ptr() + i * span for i in range(n_buf)]
-            best = {w: round(min(ws.bench.floor_read_us(ptrs, nbytes, wgs_per_cu=w) for _ in range(2)), 2) for w in (2, 4, 8, 16)}
+            best = {f"{'contiguous' if c else 'strided'}_{'8' if p else '4'}KiB_{w}": round(min(ws.bench.floor_read_us(ptrs, nbytes, wgs_per_cu=w, contiguous=c, pipelined=p) for _ in range(2)), 2)
+                    for c in (False, True) for p in (True, False) for w in (2, 4, 8)}
             us = min(best.values())
             rows.append({"weights": fmt, "K": K, "N": N, "bytes": nbytes, "floor_us": us, "GBps": round(nbytes / us * 1e-3, 1),
-                         "frac_of_hbm_peak": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4), "us_by_workgroups_per_cu": best})
-        print(json.dumps({"workload": "floor", "what": "streaming read of the sweep byte counts with 16-byte non-temporal loads, rotating buffers (1 GiB pool); "
+                         "frac_of_hbm_peak": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4), "us_by_pattern_bytes_in_flight_per_wave_and_workgroups_per_cu": best})
+        print(json.dumps({"workload": "floor", "what": "streaming read of the sweep byte counts with 16-byte non-temporal loads, KiB pieces at a grid stride or one contiguous range per workgroup, rotating buffers (1 GiB pool); "
                                                        "empty and one-trip launches inside a hipGraph",
                           "launch_us_empty": round(ws.bench.launch_us(0), 3), "launch_us_one_trip": round(ws.bench.launch_us(1), 3), "rows": rows}))
         return
