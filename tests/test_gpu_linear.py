@@ -667,3 +667,39 @@ def test_fp4_prefill_without_whole_chunks_stays_on_the_two_operand_kernel(gpu, p
         check_rows(bf16_f64(oracle, from_dev(y, np.uint16).reshape(tokens, n_out)), want, "fp4 K=160")
     finally:
         assert lib.weight_release(nd.data_ptr()) == 0
+
+
+def test_reserved_workspace_keeps_the_k_split_under_capture(gpu, pkg, oracle):
+    """hip_quant_workspace_reserve: a k-split GEMM captured into a graph on a stream whose scratch buffer was sized
+    beforehand gives the bits of the eager call (same kernels, same FP32 order); the library allocates nothing while
+    the stream is capturing, and the reserve call itself is refused there."""
+    torch, dev, lib = gpu
+    tokens, n_out, K = 512, 4096, 4096                  # 64 tiles of 128 x 256 on 256 CUs: the k range splits in four
+    seed = synth.seed_for(7, 33)
+    W, X = synth.weights_e5m2(seed, n_out, K), synth.activations(seed, tokens, K)
+    wd, xd = to_dev(torch, dev, W), to_dev(torch, dev, X)
+    y_eager = torch.zeros(tokens * n_out, dtype=torch.int16, device=dev)
+    y_graph = torch.zeros_like(y_eager)
+    assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y_eager.data_ptr(), n_out, tokens, K) == 0
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream(device=dev)
+    graph = torch.cuda.CUDAGraph()
+    lib.set_sync(False)
+    try:
+        assert lib.set_stream(stream.cuda_stream) == 0
+        assert lib.workspace_reserve(8 * tokens * n_out * 4) == 0        # this thread's buffer for this stream
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream, capture_error_mode="thread_local"):
+            assert lib.workspace_reserve(1 << 30) == -1                   # never while capturing
+            assert lib.linear(wd.data_ptr(), oracle.E5M2, xd.data_ptr(), y_graph.data_ptr(), n_out, tokens, K) == 0
+        for _ in range(2):
+            y_graph.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_graph, y_eager)
+    finally:
+        lib.set_stream(None)
+        lib.set_sync(True)
+    want = oracle.linear_exact(oracle.dequant_weight(W, oracle.E5M2, n_out, K), X[:16])
+    check_rows(bf16_f64(oracle, from_dev(y_graph, np.uint16).reshape(tokens, n_out)[:16]), want, "captured k-split GEMM")
